@@ -1,0 +1,70 @@
+"""ctypes binding of libaussm_hip.so (declarations: include/aussm_hip.h).
+
+The library is the only compute path of this package: if it is missing or a
+call fails, an exception is raised — there is no fallback.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import c_char_p, c_int, c_void_p
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libaussm_hip.so")
+
+F32, BF16 = 0, 1
+TILE = 32
+MAX_STATE = 64
+
+_lib = None
+
+_P = c_void_p
+_I = c_int
+
+# name -> argtypes; every entry point returns int
+_SIGNATURES = {
+    "aussm_version": [],
+    "aussm_num_checkpoints": [_I, _I],
+    "aussm_bwd_checkpoint_interval": [_I],
+    "aussm_unitary_fwd": [_P] * 11 + [_I] * 6 + [_P],
+    "aussm_unitary_bwd": [_P] * 16 + [_I] * 6 + [_P],
+    "aussm_complex_fwd": [_P] * 12 + [_I] * 6 + [_P],
+    "aussm_real_fwd": [_P] * 8 + [_I] + [_P] * 4 + [_I] * 6 + [_P],
+}
+
+EXPORTED = tuple(_SIGNATURES) + ("aussm_error_string",)
+
+
+class AussmError(RuntimeError):
+    pass
+
+
+def load() -> ctypes.CDLL:
+    """Load the HIP library (once).  Raises AussmError if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise AussmError(
+            f"{LIB_PATH} not found: build it with `python -m aussm_amd.build` "
+            "(the HIP library is required; there is no CPU fallback)")
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, argtypes in _SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.argtypes = argtypes
+        fn.restype = c_int
+    lib.aussm_error_string.argtypes = [c_int]
+    lib.aussm_error_string.restype = c_char_p
+    _lib = lib
+    return lib
+
+
+def check(code: int, what: str) -> None:
+    if code != 0:
+        msg = load().aussm_error_string(code).decode()
+        raise AussmError(f"{what} failed with code {code}: {msg}")
+
+
+def ptr(t) -> c_void_p | None:
+    """Device pointer of a tensor (None -> NULL)."""
+    return None if t is None else c_void_p(t.data_ptr())

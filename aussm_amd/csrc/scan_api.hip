@@ -1,0 +1,165 @@
+// C ABI of libaussm_hip.so: argument checks, kernel selection and launches.
+// Declarations and tensor layouts: include/aussm_hip.h.
+#include "../../include/aussm_hip.h"
+
+#include <hip/hip_runtime.h>
+
+#include "scan_bwd_unitary.h"
+#include "scan_common.h"
+#include "scan_fwd.h"
+
+using namespace aussm;
+
+namespace {
+
+constexpr int NT_DEFAULT = 256;
+
+// states per wavefront for a 4-wavefront workgroup
+inline int pick_nw(int N) {
+  if (N <= 4) return 1;
+  if (N <= 8) return 2;
+  if (N <= 16) return 4;
+  if (N <= 32) return 8;
+  return 16;
+}
+
+inline int check_common(int B, int D, int N, int L, int ck, int in_dtype) {
+  if (B < 1 || D < 1 || N < 1 || L < 1) return AUSSM_E_SHAPE;
+  if (N > AUSSM_MAX_STATE) return AUSSM_E_SHAPE;
+  if ((long long)B * ((D + CH - 1) / CH) > 0x7fffffffLL) return AUSSM_E_SHAPE;
+  if (ck < AUSSM_TILE || ck % AUSSM_TILE != 0) return AUSSM_E_CK;
+  if (in_dtype != AUSSM_F32 && in_dtype != AUSSM_BF16) return AUSSM_E_DTYPE;
+  return AUSSM_OK;
+}
+
+inline bool misaligned(const void* p, size_t a) { return p && (reinterpret_cast<uintptr_t>(p) % a) != 0; }
+
+inline int launch_status() {
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? AUSSM_OK : (int)e;
+}
+
+inline void zero_async(float* p, size_t n, hipStream_t s) {
+  if (!p || n == 0) return;
+  size_t blocks = (n + 255) / 256;
+  if (blocks > 4096) blocks = 4096;
+  hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)blocks), dim3(256), 0, s, p, n);
+}
+
+template <int VAR, typename Tin>
+int launch_fwd_t(const FwdArgs& a, hipStream_t s) {
+  const dim3 grid((unsigned)(a.B * a.ncg)), block(NT_DEFAULT);
+  switch (pick_nw(a.N)) {
+    case 1: hipLaunchKernelGGL((core_fwd_kernel<VAR, 1, NT_DEFAULT, Tin>), grid, block, 0, s, a); break;
+    case 2: hipLaunchKernelGGL((core_fwd_kernel<VAR, 2, NT_DEFAULT, Tin>), grid, block, 0, s, a); break;
+    case 4: hipLaunchKernelGGL((core_fwd_kernel<VAR, 4, NT_DEFAULT, Tin>), grid, block, 0, s, a); break;
+    case 8: hipLaunchKernelGGL((core_fwd_kernel<VAR, 8, NT_DEFAULT, Tin>), grid, block, 0, s, a); break;
+    default: hipLaunchKernelGGL((core_fwd_kernel<VAR, 16, NT_DEFAULT, Tin>), grid, block, 0, s, a); break;
+  }
+  return launch_status();
+}
+
+template <int VAR>
+int launch_fwd(const FwdArgs& a, int in_dtype, hipStream_t s) {
+  return in_dtype == AUSSM_BF16 ? launch_fwd_t<VAR, bf16_t>(a, s) : launch_fwd_t<VAR, float>(a, s);
+}
+
+template <typename Tin>
+int launch_unitary_bwd_t(const UniBwdArgs& a, hipStream_t s) {
+  const dim3 grid((unsigned)(a.B * a.ncg)), block(NT_DEFAULT);
+  switch (pick_nw(a.N)) {
+    case 1: hipLaunchKernelGGL((unitary_bwd_kernel<1, NT_DEFAULT, Tin>), grid, block, 0, s, a); break;
+    case 2: hipLaunchKernelGGL((unitary_bwd_kernel<2, NT_DEFAULT, Tin>), grid, block, 0, s, a); break;
+    case 4: hipLaunchKernelGGL((unitary_bwd_kernel<4, NT_DEFAULT, Tin>), grid, block, 0, s, a); break;
+    case 8: hipLaunchKernelGGL((unitary_bwd_kernel<8, NT_DEFAULT, Tin>), grid, block, 0, s, a); break;
+    default: hipLaunchKernelGGL((unitary_bwd_kernel<16, NT_DEFAULT, Tin>), grid, block, 0, s, a); break;
+  }
+  return launch_status();
+}
+
+}  // namespace
+
+extern "C" {
+
+int aussm_version(void) { return 100; }
+
+const char* aussm_error_string(int code) {
+  switch (code) {
+    case AUSSM_OK: return "ok";
+    case AUSSM_E_NULL: return "a required pointer is NULL";
+    case AUSSM_E_SHAPE: return "dimension out of the supported range (B,D,N,L >= 1, N <= 64)";
+    case AUSSM_E_CK: return "checkpoint interval must be a multiple of 32 accepted by this function";
+    case AUSSM_E_DTYPE: return "in_dtype must be AUSSM_F32 or AUSSM_BF16";
+    case AUSSM_E_ALIGN: return "pointer not aligned to its element size";
+    default: return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown aussm error";
+  }
+}
+
+int aussm_num_checkpoints(int L, int ck) { return (L < 1 || ck < 1) ? 0 : (L + ck - 1) / ck; }
+
+int aussm_bwd_checkpoint_interval(int variant) { return variant == VAR_UNITARY ? 0 : AUSSM_TILE; }
+
+int aussm_unitary_fwd(const void* u, const void* delta, const float* theta, const void* Bc, const void* Cc,
+                      const float* Dskip, const float* z, const float* h0, float* y, float* hL, float* hck,
+                      int B, int D, int N, int L, int ck, int in_dtype, void* stream) {
+  if (int e = check_common(B, D, N, L, ck, in_dtype)) return e;
+  if (!u || !delta || !theta || !Bc || !Cc) return AUSSM_E_NULL;
+  const size_t ca = in_dtype == AUSSM_BF16 ? 4 : 8;
+  if (misaligned(Bc, ca) || misaligned(Cc, ca)) return AUSSM_E_ALIGN;
+  FwdArgs a{};
+  a.u = u; a.delta = delta; a.theta = theta; a.Bm = Bc; a.Cm = Cc; a.Dskip = Dskip; a.z = z;
+  a.h0 = h0; a.y = y; a.hL = hL; a.hck = hck;
+  a.B = B; a.D = D; a.N = N; a.L = L; a.ck = ck; a.nck = (L + ck - 1) / ck; a.ncg = (D + CH - 1) / CH;
+  return launch_fwd<VAR_UNITARY>(a, in_dtype, (hipStream_t)stream);
+}
+
+int aussm_complex_fwd(const void* u, const void* delta, const float* rho, const float* theta, const void* Bc,
+                      const void* Cc, const float* Dskip, const float* z, const float* h0, float* y, float* hL,
+                      float* hck, int B, int D, int N, int L, int ck, int in_dtype, void* stream) {
+  if (int e = check_common(B, D, N, L, ck, in_dtype)) return e;
+  if (!u || !delta || !rho || !theta || !Bc || !Cc) return AUSSM_E_NULL;
+  const size_t ca = in_dtype == AUSSM_BF16 ? 4 : 8;
+  if (misaligned(Bc, ca) || misaligned(Cc, ca)) return AUSSM_E_ALIGN;
+  FwdArgs a{};
+  a.u = u; a.delta = delta; a.rho = rho; a.theta = theta; a.Bm = Bc; a.Cm = Cc; a.Dskip = Dskip; a.z = z;
+  a.h0 = h0; a.y = y; a.hL = hL; a.hck = hck;
+  a.B = B; a.D = D; a.N = N; a.L = L; a.ck = ck; a.nck = (L + ck - 1) / ck; a.ncg = (D + CH - 1) / CH;
+  return launch_fwd<VAR_COMPLEX>(a, in_dtype, (hipStream_t)stream);
+}
+
+int aussm_real_fwd(const void* u, const void* delta, const float* A, const void* Bm, const void* Cm,
+                   const float* Dskip, const float* z, const float* delta_bias, int delta_softplus,
+                   const float* h0, float* y, float* hL, float* hck,
+                   int B, int D, int N, int L, int ck, int in_dtype, void* stream) {
+  if (int e = check_common(B, D, N, L, ck, in_dtype)) return e;
+  if (!u || !delta || !A || !Bm || !Cm) return AUSSM_E_NULL;
+  FwdArgs a{};
+  a.u = u; a.delta = delta; a.A = A; a.Bm = Bm; a.Cm = Cm; a.Dskip = Dskip; a.z = z;
+  a.delta_bias = delta_bias; a.delta_softplus = delta_softplus;
+  a.h0 = h0; a.y = y; a.hL = hL; a.hck = hck;
+  a.B = B; a.D = D; a.N = N; a.L = L; a.ck = ck; a.nck = (L + ck - 1) / ck; a.ncg = (D + CH - 1) / CH;
+  return launch_fwd<VAR_REAL>(a, in_dtype, (hipStream_t)stream);
+}
+
+int aussm_unitary_bwd(const float* dy, const float* dhL, const void* u, const void* delta, const float* theta,
+                      const void* Bc, const void* Cc, const float* Dskip, const float* hck,
+                      float* du, float* ddelta, float* dtheta, float* dB, float* dC, float* dD, float* dh0,
+                      int B, int D, int N, int L, int ck, int in_dtype, void* stream) {
+  if (int e = check_common(B, D, N, L, ck, in_dtype)) return e;
+  if (!dy || !u || !delta || !theta || !Bc || !Cc || !hck || !du || !ddelta || !dtheta || !dB || !dC)
+    return AUSSM_E_NULL;
+  const size_t ca = in_dtype == AUSSM_BF16 ? 4 : 8;
+  if (misaligned(Bc, ca) || misaligned(Cc, ca)) return AUSSM_E_ALIGN;
+  hipStream_t s = (hipStream_t)stream;
+  UniBwdArgs a{};
+  a.dy = dy; a.dhL = dhL; a.u = u; a.delta = delta; a.theta = theta; a.Bm = Bc; a.Cm = Cc; a.Dskip = Dskip;
+  a.hck = hck; a.du = du; a.ddelta = ddelta; a.dtheta = dtheta; a.dB = dB; a.dC = dC; a.dD = dD; a.dh0 = dh0;
+  a.B = B; a.D = D; a.N = N; a.L = L; a.ck = ck; a.nck = (L + ck - 1) / ck; a.ncg = (D + CH - 1) / CH;
+  const size_t nbc = (size_t)B * N * L * 2;
+  zero_async(dB, nbc, s);
+  zero_async(dC, nbc, s);
+  zero_async(dD, (size_t)D, s);
+  return in_dtype == AUSSM_BF16 ? launch_unitary_bwd_t<bf16_t>(a, s) : launch_unitary_bwd_t<float>(a, s);
+}
+
+}  // extern "C"

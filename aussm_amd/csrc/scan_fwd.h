@@ -1,0 +1,203 @@
+// Forward core scan for the three variants (adaptive-unitary, complex, real/S6).
+//
+// Reference semantics: extension-cpp/extension_cpp/ops.py:215-223 (unitary loop),
+// :270-291 (complex loop), :349-356 (real loop) and the selective-scan call at
+// ai-modules/wavesAI/model/aussm.py:791-802.
+#pragma once
+#include "scan_common.h"
+
+namespace aussm {
+
+struct FwdArgs {
+  const void* u;            // [B,D,L]  Tin
+  const void* delta;        // [B,D,L]  Tin
+  const float* theta;       // [B,D,L]  (unitary, complex)
+  const float* rho;         // [B,D,L]  (complex)
+  const float* A;           // [D,N]    (real)
+  const void* Bm;           // [B,N,L(,2)] Tin
+  const void* Cm;           // [B,N,L(,2)] Tin
+  const float* Dskip;       // [D] or null
+  const float* z;           // [B,D,L] or null
+  const float* delta_bias;  // [D] or null (real)
+  const float* h0;          // [B,D,N,C] or null
+  float* y;                 // [B,D,L] or null
+  float* hL;                // [B,D,N,C] or null
+  float* hck;               // [B,nck,N,C,D] or null
+  int B, D, N, L, ck, nck, ncg, delta_softplus;
+};
+
+// VAR: variant.  NW: states per wavefront.  NT: threads per workgroup.  Tin: float or bf16_t.
+template <int VAR, int NW, int NT, typename Tin>
+__global__ __launch_bounds__(NT) void core_fwd_kernel(const FwdArgs p) {
+  constexpr int C = (VAR == VAR_REAL) ? 1 : 2;   // floats per state
+  constexpr int NWV = NT / 64;                   // wavefronts per workgroup
+  constexpr int E = CH * T / NT;                 // tile elements per thread in the staging phases
+  constexpr int RSTEP = NT / T;                  // channel-row step between a thread's elements
+
+  __shared__ float4 s_in[T * TS];                // per (t, channel): unitary/complex (Re a, Im a, delta*u, -)
+                                                 //                   real            (delta, delta*u, -, -)
+  __shared__ float s_part[NWV * T * TS];         // per wavefront partial read-outs  sum_n Re(C h)
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = wave_index();
+  const int wg = xcd_remap(blockIdx.x, gridDim.x);
+  const int b = wg / p.ncg, d0 = (wg % p.ncg) * CH;
+  const int N = p.N, L = p.L, D = p.D;
+  const int n0 = wave * NW;
+  const bool active = n0 < N;                    // wave-uniform
+  const int nwa = (N + NW - 1) / NW;             // wavefronts that own states
+  const int d = d0 + lane;
+  const bool dok = d < D;
+
+  const Tin* __restrict__ gu = static_cast<const Tin*>(p.u);
+  const Tin* __restrict__ gdl = static_cast<const Tin*>(p.delta);
+  const Tin* __restrict__ gB = static_cast<const Tin*>(p.Bm);
+  const Tin* __restrict__ gC = static_cast<const Tin*>(p.Cm);
+
+  // ---- scan-side state (lane == channel)
+  float hr[NW], hi[NW], a2[NW];
+#pragma unroll
+  for (int k = 0; k < NW; ++k) {
+    const int n = n0 + k;
+    hr[k] = 0.f; hi[k] = 0.f; a2[k] = 0.f;
+    if (dok && n < N) {
+      if (p.h0) {
+        const size_t o = (((size_t)b * D + d) * N + n) * C;
+        hr[k] = p.h0[o];
+        if (C == 2) hi[k] = p.h0[o + C - 1];
+      }
+      if (VAR == VAR_REAL) a2[k] = p.A[(size_t)d * N + n] * LOG2E;
+    }
+  }
+
+  // ---- staging-side mapping (lanes run along time)
+  const int col = tid % T, row0 = tid / T;
+  float ru[E], rdl[E], rth[E], rrho[E], rz[E], dsk[E], dbias[E];
+  size_t goff[E];
+  bool rowok[E];
+#pragma unroll
+  for (int k = 0; k < E; ++k) {
+    const int dd = d0 + row0 + k * RSTEP;
+    rowok[k] = dd < D;
+    goff[k] = ((size_t)b * D + (rowok[k] ? dd : 0)) * L;
+    dsk[k] = (p.Dskip && rowok[k]) ? p.Dskip[dd] : 0.f;
+    dbias[k] = (VAR == VAR_REAL && p.delta_bias && rowok[k]) ? p.delta_bias[dd] : 0.f;
+    rth[k] = 0.f; rrho[k] = 0.f; rz[k] = 0.f;
+  }
+
+  auto load_tile = [&](int l0) {
+#pragma unroll
+    for (int k = 0; k < E; ++k) {
+      const int ll = l0 + col;
+      const bool ok = rowok[k] && ll < L;
+      const size_t o = goff[k] + (ok ? ll : 0);
+      ru[k] = ok ? to_f32(gu[o]) : 0.f;
+      rdl[k] = ok ? to_f32(gdl[o]) : 0.f;
+      if (VAR != VAR_REAL) rth[k] = ok ? p.theta[o] : 0.f;
+      if (VAR == VAR_COMPLEX) rrho[k] = ok ? p.rho[o] : 0.f;
+      if (p.z) rz[k] = ok ? p.z[o] : 0.f;
+    }
+  };
+  load_tile(0);
+
+  for (int l0 = 0; l0 < L; l0 += T) {
+    // ---- stage: convert this tile once per (channel, t) and transpose into LDS
+    float yin[E], gate[E];
+#pragma unroll
+    for (int k = 0; k < E; ++k) {
+      const float uu = ru[k];
+      float dl = rdl[k];
+      float4 rec;
+      if (VAR == VAR_REAL) {
+        dl += dbias[k];
+        if (p.delta_softplus) dl = softplusf_(dl);
+        rec = make_float4(dl, dl * uu, 0.f, 0.f);
+      } else {
+        float sn, cs;
+        sincosf(rth[k], &sn, &cs);
+        if (VAR == VAR_COMPLEX) { const float r = expf(rrho[k]); cs *= r; sn *= r; }
+        rec = make_float4(cs, sn, dl * uu, 0.f);
+      }
+      s_in[col * TS + row0 + k * RSTEP] = rec;
+      yin[k] = dsk[k] * uu;
+      gate[k] = rz[k];
+    }
+    __syncthreads();
+    if (l0 + T < L) load_tile(l0 + T);           // next tile's loads fly during the scan
+
+    // ---- scan: lane == channel, sequential over the tile's timesteps
+    const int tmax = (L - l0 < T) ? (L - l0) : T;
+    if (active) {
+      const size_t brow = ((size_t)b * N + n0) * L + l0;
+#pragma unroll 4
+      for (int t = 0; t < tmax; ++t) {
+        const float4 v = s_in[t * TS + lane];
+        float yacc = 0.f;
+#pragma unroll
+        for (int k = 0; k < NW; ++k) {
+          if (n0 + k < N) {                      // wave-uniform
+            const size_t bi = brow + (size_t)k * L + t;
+            if (VAR == VAR_REAL) {
+              const float bv = ld_r(gB, bi), cv = ld_r(gC, bi);
+              const float a = __builtin_amdgcn_exp2f(v.x * a2[k]);
+              hr[k] = fmaf(a, hr[k], bv * v.y);
+              yacc = fmaf(cv, hr[k], yacc);
+            } else {
+              const float2 bv = ld_c(gB, bi), cv = ld_c(gC, bi);
+              const float nr = fmaf(v.x, hr[k], fmaf(-v.y, hi[k], bv.x * v.z));
+              const float ni = fmaf(v.x, hi[k], fmaf(v.y, hr[k], bv.y * v.z));
+              hr[k] = nr; hi[k] = ni;
+              yacc = fmaf(cv.x, nr, yacc);
+              yacc = fmaf(-cv.y, ni, yacc);
+            }
+          }
+        }
+        s_part[(wave * T + t) * TS + lane] = yacc;
+      }
+    }
+    __syncthreads();
+
+    // ---- epilogue: add the wavefronts' partial read-outs, skip term and gate; coalesced store
+    if (p.y) {
+#pragma unroll
+      for (int k = 0; k < E; ++k) {
+        const int ll = l0 + col;
+        if (rowok[k] && ll < L) {
+          float acc = yin[k];
+          for (int w = 0; w < nwa; ++w) acc += s_part[(w * T + col) * TS + row0 + k * RSTEP];
+          if (p.z) acc *= siluf_(gate[k]);
+          p.y[goff[k] + ll] = acc;
+        }
+      }
+    }
+    // ---- checkpoint at the end of every ck-step block (and at the end of the sequence)
+    if (p.hck && active && dok && (((l0 + T) % p.ck) == 0 || l0 + T >= L)) {
+      const int kb = l0 / p.ck;
+#pragma unroll
+      for (int k = 0; k < NW; ++k) {
+        const int n = n0 + k;
+        if (n < N) {
+          const size_t o = ((((size_t)b * p.nck + kb) * N + n) * C) * D + d;
+          p.hck[o] = hr[k];
+          if (C == 2) p.hck[o + D] = hi[k];
+        }
+      }
+    }
+    // No third barrier: the next stage only writes s_in (all scan reads of it are behind the
+    // barrier above) and the next scan writes s_part only after the next barrier, by which time
+    // every wavefront has finished this epilogue.
+  }
+
+  if (p.hL && active && dok) {
+#pragma unroll
+    for (int k = 0; k < NW; ++k) {
+      const int n = n0 + k;
+      if (n < N) {
+        const size_t o = (((size_t)b * D + d) * N + n) * C;
+        p.hL[o] = hr[k];
+        if (C == 2) p.hL[o + 1] = hi[k];
+      }
+    }
+  }
+}
+
+}  // namespace aussm

@@ -1,0 +1,185 @@
+"""Core selective scans on MI355X: Python host over the C ABI of libaussm_hip.so.
+
+Three operators, each differentiable through torch.autograd:
+
+    unitary_scan(u, delta, theta, Bc, Cc, D, z, h0)        a_l = exp(i theta_l)
+    complex_scan(u, delta, rho, theta, Bc, Cc, D, z, h0)   a_l = exp(rho_l + i theta_l)
+    selective_scan_fn(u, delta, A, B, C, D, z, delta_bias, delta_softplus, return_last_state)
+                                                            a_l = exp(delta_l A)   (Mamba S6)
+
+    h_l[b,d,n] = a_l h_{l-1}[b,d,n] + delta_l[b,d] B_l[b,n] u_l[b,d]
+    y_l[b,d]   = Re sum_n C_l[b,n] h_l[b,d,n] + D[d] u_l[b,d]          (* silu(z_l[b,d]))
+
+selective_scan_fn keeps the argument names and meaning of the call at
+ai-modules/wavesAI/model/aussm.py:791-802 of the reference; the unitary/complex
+recurrences are those of extension-cpp/extension_cpp/ops.py:215-223 and :270-291.
+
+Tensors must live on the GPU.  u, delta, B, C may be float32 or bfloat16 (both
+the same); everything else is float32 and the state is accumulated in float32.
+Complex B_t/C_t are torch.complex64 tensors (b, n, l) or, for bfloat16, real
+tensors (b, n, l, 2) holding (re, im).
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+import torch.nn.functional as F
+
+from . import _lib
+from ._lib import check, ptr
+
+Tensor = torch.Tensor
+
+# Checkpoint interval (timesteps) of the forward pass.  The unitary backward pass regenerates the
+# states by running the recurrence in reverse and only uses checkpoints to stop rounding drift,
+# so a long interval is enough; the complex and real backward passes recompute every tile from
+# its checkpoint and need one per tile.
+UNITARY_CK = 256
+TILE_CK = _lib.TILE
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _in_dtype(t: Tensor) -> int:
+    if t.dtype == torch.float32:
+        return _lib.F32
+    if t.dtype == torch.bfloat16:
+        return _lib.BF16
+    raise RuntimeError(f"expected float32 or bfloat16 scan input, got {t.dtype}")
+
+
+def _f32(t: Optional[Tensor], name: str, shape=None) -> Optional[Tensor]:
+    if t is None:
+        return None
+    if t.dtype != torch.float32:
+        raise RuntimeError(f"expected {name} to be float32, got {t.dtype}")
+    if shape is not None and tuple(t.shape) != tuple(shape):
+        raise RuntimeError(f"expected {name} of shape {tuple(shape)}, got {tuple(t.shape)}")
+    return t.contiguous()
+
+
+def _check_bdl(u: Tensor, delta: Tensor):
+    if u.dim() != 3:
+        raise RuntimeError(f"expected u of shape (b, d, l), got {tuple(u.shape)}")
+    if not u.is_cuda:
+        raise RuntimeError("scan inputs must be on the GPU (no CPU implementation is shipped)")
+    if delta.shape != u.shape or delta.dtype != u.dtype:
+        raise RuntimeError("delta must match u in shape and dtype")
+    return u.shape
+
+
+def _complex_as_real(t: Tensor, name: str, b: int, l: int, dtype: torch.dtype) -> Tensor:
+    """(b, n, l) complex64 or (b, n, l, 2) real -> contiguous real (b, n, l, 2) of `dtype`."""
+    if t.is_complex():
+        if t.dtype != torch.complex64:
+            raise RuntimeError(f"expected {name} to be complex64, got {t.dtype}")
+        t = torch.view_as_real(t)
+    if t.dim() != 4 or t.shape[0] != b or t.shape[2] != l or t.shape[3] != 2:
+        raise RuntimeError(f"expected {name} of shape (b, n, l) complex or (b, n, l, 2), got {tuple(t.shape)}")
+    if t.dtype != dtype:
+        raise RuntimeError(f"{name} must have the dtype of u ({dtype}), got {t.dtype}")
+    return t.contiguous()
+
+
+def num_checkpoints(L: int, ck: int) -> int:
+    return (L + ck - 1) // ck
+
+
+# --------------------------------------------------------------------------------------------
+# raw launches (no autograd)
+# --------------------------------------------------------------------------------------------
+
+def unitary_fwd_raw(u, delta, theta, Bri, Cri, D=None, z=None, h0=None, want_state=False, ck=0):
+    """Launch aussm_unitary_fwd.  Bri/Cri are real views (b, n, l, 2).  Returns (y, hL, hck);
+    hL is (b, d, n, 2) or None, hck is the checkpoint tensor when ck > 0."""
+    lib = _lib.load()
+    b, d, l = u.shape
+    n = Bri.shape[1]
+    y = torch.empty((b, d, l), device=u.device, dtype=torch.float32)
+    hL = torch.empty((b, d, n, 2), device=u.device, dtype=torch.float32) if want_state else None
+    hck = None
+    if ck:
+        hck = torch.empty((b, num_checkpoints(l, ck), n, 2, d), device=u.device, dtype=torch.float32)
+    check(lib.aussm_unitary_fwd(ptr(u), ptr(delta), ptr(theta), ptr(Bri), ptr(Cri), ptr(D), ptr(z), ptr(h0),
+                                ptr(y), ptr(hL), ptr(hck), b, d, n, l, ck or _lib.TILE, _in_dtype(u), _stream()),
+          "aussm_unitary_fwd")
+    return y, hL, hck
+
+
+def unitary_bwd_raw(dy, dhL, u, delta, theta, Bri, Cri, D, hck, ck, want_dD=True, want_dh0=False):
+    lib = _lib.load()
+    b, d, l = u.shape
+    n = Bri.shape[1]
+    f32 = dict(device=u.device, dtype=torch.float32)
+    du, ddelta, dtheta = (torch.empty((b, d, l), **f32) for _ in range(3))
+    dB = torch.empty((b, n, l, 2), **f32)
+    dC = torch.empty((b, n, l, 2), **f32)
+    dD = torch.empty((d,), **f32) if (want_dD and D is not None) else None
+    dh0 = torch.empty((b, d, n, 2), **f32) if want_dh0 else None
+    check(lib.aussm_unitary_bwd(ptr(dy), ptr(dhL), ptr(u), ptr(delta), ptr(theta), ptr(Bri), ptr(Cri), ptr(D),
+                                ptr(hck), ptr(du), ptr(ddelta), ptr(dtheta), ptr(dB), ptr(dC), ptr(dD), ptr(dh0),
+                                b, d, n, l, ck, _in_dtype(u), _stream()),
+          "aussm_unitary_bwd")
+    return du, ddelta, dtheta, dB, dC, dD, dh0
+
+
+# --------------------------------------------------------------------------------------------
+# autograd
+# --------------------------------------------------------------------------------------------
+
+class _UnitaryScanFn(torch.autograd.Function):
+    """y, hL = scan(u, delta, theta, B, C, D, h0) with all tensors real (complex ones as (..., 2))."""
+
+    @staticmethod
+    def forward(ctx, u, delta, theta, Bri, Cri, D, h0):
+        y, hL, hck = unitary_fwd_raw(u, delta, theta, Bri, Cri, D, None, h0, want_state=True, ck=UNITARY_CK)
+        ctx.save_for_backward(u, delta, theta, Bri, Cri, D, hck)
+        ctx.has_h0 = h0 is not None
+        return y, hL
+
+    @staticmethod
+    def backward(ctx, dy, dhL):
+        u, delta, theta, Bri, Cri, D, hck = ctx.saved_tensors
+        dy = dy.contiguous()
+        dhL = None if dhL is None else dhL.contiguous()
+        du, ddelta, dtheta, dB, dC, dD, dh0 = unitary_bwd_raw(
+            dy, dhL, u, delta, theta, Bri, Cri, D, hck, UNITARY_CK,
+            want_dD=D is not None and ctx.needs_input_grad[5], want_dh0=ctx.has_h0 and ctx.needs_input_grad[6])
+        return (du.to(u.dtype), ddelta.to(delta.dtype), dtheta, dB.to(Bri.dtype), dC.to(Cri.dtype), dD, dh0)
+
+
+def unitary_scan(u: Tensor, delta: Tensor, theta: Tensor, Bc: Tensor, Cc: Tensor, D: Optional[Tensor] = None,
+                 z: Optional[Tensor] = None, h0: Optional[Tensor] = None, return_last_state: bool = False):
+    """Adaptive-unitary scan.  u, delta, theta, z: (b, d, l); Bc, Cc: (b, n, l) complex64 (or
+    (b, n, l, 2) real); D: (d,); h0: (b, d, n) complex64.  Returns y (b, d, l) float32, and the final
+    state (b, d, n) complex64 if return_last_state."""
+    b, d, l = _check_bdl(u, delta)
+    u = u.contiguous()
+    delta = delta.contiguous()
+    theta = _f32(theta, "theta", (b, d, l))
+    Bri = _complex_as_real(Bc, "B", b, l, u.dtype)
+    Cri = _complex_as_real(Cc, "C", b, l, u.dtype)
+    n = Bri.shape[1]
+    if Cri.shape[1] != n:
+        raise RuntimeError("B and C must have the same state size")
+    D = _f32(D, "D", (d,))
+    z = _f32(z, "z", (b, d, l))
+    h0r = None
+    if h0 is not None:
+        if h0.dtype != torch.complex64 or tuple(h0.shape) != (b, d, n):
+            raise RuntimeError(f"expected h0 complex64 of shape {(b, d, n)}")
+        h0r = torch.view_as_real(h0).contiguous()
+    needs_grad = torch.is_grad_enabled() and any(
+        t is not None and t.requires_grad for t in (u, delta, theta, Bri, Cri, D, z, h0r))
+    if needs_grad:
+        y, hL = _UnitaryScanFn.apply(u, delta, theta, Bri, Cri, D, h0r)
+        if z is not None:
+            y = y * F.silu(z)
+    else:
+        y, hL, _ = unitary_fwd_raw(u, delta, theta, Bri, Cri, D, z, h0r, want_state=return_last_state)
+    if return_last_state:
+        return y, torch.view_as_complex(hL)
+    return y

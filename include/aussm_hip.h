@@ -1,0 +1,141 @@
+/*
+ * aussm_hip.h — C ABI of libaussm_hip.so, the MI355X (gfx950) selective-scan library.
+ *
+ * Every pointer is a DEVICE pointer unless stated otherwise.  Tensors are dense,
+ * row-major, in the shapes given per function.  Functions enqueue work on the HIP
+ * stream passed as `stream` (a hipStream_t cast to void*; NULL = default stream),
+ * never synchronise, never allocate, and return 0 on success, a negative
+ * AUSSM_E_* code for a rejected argument, or a positive hipError_t from the launch.
+ *
+ * Layout conventions
+ *   B, D, N, L        batch, channels, state size per channel, sequence length
+ *   u, delta, theta, rho, z, y, dy and their gradients      [B, D, L]
+ *   complex B_t / C_t (unitary, complex variants)           [B, N, L, 2]  (re, im interleaved,
+ *                                                            i.e. a torch complex64 [B,N,L] tensor)
+ *   real B_t / C_t (real variant)                            [B, N, L]
+ *   h0, hL, dh0, dhL  start / final state and their cotangents
+ *                                                            [B, D, N, 2] complex, [B, D, N] real
+ *   hck               checkpointed states at the END of every `ck`-step block,
+ *                     [B, nck, N, C, D] with nck = ceil(L / ck), C = 2 (complex state) or 1;
+ *                     channel index fastest so that a wavefront stores it coalesced.
+ *                     The last block holds the final state.
+ *   in_dtype          element type of u, delta, B_t, C_t: AUSSM_F32 or AUSSM_BF16.
+ *                     Everything else (phases, skip, gate, states, outputs, gradients) is fp32
+ *                     and the recurrence always accumulates in fp32.
+ *
+ * Reference interfaces these entry points replace are cited per function as
+ * path:line inside the reference tree (arjunkaruvally/AUSSM).
+ */
+#ifndef AUSSM_HIP_H
+#define AUSSM_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define AUSSM_F32 0
+#define AUSSM_BF16 1
+
+#define AUSSM_OK 0
+#define AUSSM_E_NULL (-1)      /* a required pointer is NULL                         */
+#define AUSSM_E_SHAPE (-2)     /* a dimension is out of the supported range          */
+#define AUSSM_E_CK (-3)        /* checkpoint interval not accepted by this function  */
+#define AUSSM_E_DTYPE (-4)     /* unknown in_dtype                                   */
+#define AUSSM_E_ALIGN (-5)     /* a pointer is not aligned to its element size       */
+
+#define AUSSM_TILE 32          /* timesteps per staged tile; ck must be a multiple   */
+#define AUSSM_MAX_STATE 64     /* largest N accepted                                  */
+
+/* Library version (major*10000 + minor*100 + patch). No reference counterpart. */
+int aussm_version(void);
+
+/* Human-readable text for a return code of this library (host pointer, static storage). */
+const char* aussm_error_string(int code);
+
+/* nck = ceil(L / ck): number of checkpoint blocks the hck buffer must hold. */
+int aussm_num_checkpoints(int L, int ck);
+
+/* The checkpoint interval the backward pass of a variant requires (0 = any multiple of
+ * AUSSM_TILE).  variant: 0 unitary, 1 complex, 2 real. */
+int aussm_bwd_checkpoint_interval(int variant);
+
+/* ---------------------------------------------------------------------------------------
+ * Core adaptive-unitary scan
+ *     h_l[b,d,n] = exp(i*theta_l[b,d]) * h_{l-1}[b,d,n] + delta_l[b,d] * B_l[b,n] * u_l[b,d]
+ *     y_l[b,d]   = Re sum_n C_l[b,n] * h_l[b,d,n] + Dskip[d] * u_l[b,d]      (* silu(z_l[b,d]))
+ * Replaces the recurrence of extension-cpp/extension_cpp/ops.py:215-223 (sequential scan) and
+ * the device scan of extension-cpp/extension_cpp/csrc/cuda/ssm_adaptive_unitary_forward.cu:113-181
+ * for a phase that is given per (b,d,l).
+ * Optional (NULL allowed): Dskip, z, h0, y (NULL = states only), hL, hck.
+ * ------------------------------------------------------------------------------------- */
+int aussm_unitary_fwd(const void* u, const void* delta, const float* theta,
+                      const void* Bc, const void* Cc, const float* Dskip, const float* z,
+                      const float* h0, float* y, float* hL, float* hck,
+                      int B, int D, int N, int L, int ck, int in_dtype, void* stream);
+
+/* Reverse scan for aussm_unitary_fwd called WITHOUT a gate (z == NULL).  Recomputes the states
+ * by running the (norm-preserving, hence invertible) recurrence backwards from the checkpoints
+ * in hck, which must come from aussm_unitary_fwd on the same inputs with the same ck.
+ * Replaces extension-cpp/extension_cpp/csrc/cuda/ssm_adaptive_unitary_backward.cu:22-491.
+ * dB, dC use the convention dRe + i*dIm (what torch returns for a complex leaf).
+ * Required: dy, u, delta, theta, Bc, Cc, hck, du, ddelta, dtheta, dB, dC.
+ * Optional: dhL, Dskip, h0 (unused, may be NULL), dD, dh0.
+ * dB, dC and dD are zeroed by this call before being accumulated into. */
+int aussm_unitary_bwd(const float* dy, const float* dhL,
+                      const void* u, const void* delta, const float* theta,
+                      const void* Bc, const void* Cc, const float* Dskip, const float* hck,
+                      float* du, float* ddelta, float* dtheta, float* dB, float* dC,
+                      float* dD, float* dh0,
+                      int B, int D, int N, int L, int ck, int in_dtype, void* stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Complex scan:  a_l = exp(rho_l[b,d] + i*theta_l[b,d]), otherwise as the unitary scan.
+ * Replaces extension-cpp/extension_cpp/ops.py:270-291 (loop) and the semantics of
+ * extension-cpp/extension_cpp/csrc/cuda/ssm_adaptive_complex.cu:181-293 / :358-660.
+ * The backward pass needs hck written with ck == aussm_bwd_checkpoint_interval(1).
+ * ------------------------------------------------------------------------------------- */
+int aussm_complex_fwd(const void* u, const void* delta, const float* rho, const float* theta,
+                      const void* Bc, const void* Cc, const float* Dskip, const float* z,
+                      const float* h0, float* y, float* hL, float* hck,
+                      int B, int D, int N, int L, int ck, int in_dtype, void* stream);
+
+int aussm_complex_bwd(const float* dy, const float* dhL,
+                      const void* u, const void* delta, const float* rho, const float* theta,
+                      const void* Bc, const void* Cc, const float* Dskip,
+                      const float* h0, const float* hck,
+                      float* du, float* ddelta, float* drho, float* dtheta, float* dB, float* dC,
+                      float* dD, float* dh0,
+                      int B, int D, int N, int L, int ck, int in_dtype, void* stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Real (Mamba S6) selective scan:
+ *     dl = delta (+ delta_bias[d]) (softplus if delta_softplus)
+ *     h_l[b,d,n] = exp(dl_l[b,d]*A[d,n]) * h_{l-1} + dl_l[b,d] * B_l[b,n] * u_l[b,d]
+ *     y_l[b,d]   = sum_n C_l[b,n] h_l[b,d,n] + Dskip[d] u_l[b,d]              (* silu(z_l))
+ * Replaces the third-party selective_scan_fn called at
+ * ai-modules/wavesAI/model/aussm.py:791-802 (same argument meaning: u, delta, A, B, C, D, z,
+ * delta_bias, delta_softplus) and the real-state loop of extension-cpp/extension_cpp/ops.py:349-356.
+ * ddelta is the gradient w.r.t. the RAW delta input (before bias and softplus).
+ * ------------------------------------------------------------------------------------- */
+int aussm_real_fwd(const void* u, const void* delta, const float* A,
+                   const void* Bm, const void* Cm, const float* Dskip, const float* z,
+                   const float* delta_bias, int delta_softplus,
+                   const float* h0, float* y, float* hL, float* hck,
+                   int B, int D, int N, int L, int ck, int in_dtype, void* stream);
+
+int aussm_real_bwd(const float* dy, const float* dhL,
+                   const void* u, const void* delta, const float* A,
+                   const void* Bm, const void* Cm, const float* Dskip,
+                   const float* delta_bias, int delta_softplus,
+                   const float* h0, const float* hck,
+                   float* du, float* ddelta, float* dA, float* dB, float* dC,
+                   float* dD, float* dh0,
+                   int B, int D, int N, int L, int ck, int in_dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* AUSSM_HIP_H */
