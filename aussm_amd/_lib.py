@@ -44,6 +44,10 @@ def load() -> ctypes.CDLL:
     global _lib
     if _lib is not None:
         return _lib
+    # PyTorch ships its own HIP runtime.  It has to be in the process before this library is
+    # opened so that both resolve to the same runtime (two runtimes in one process do not share
+    # a device context).
+    import torch  # noqa: F401
     if not os.path.exists(LIB_PATH):
         raise AussmError(
             f"{LIB_PATH} not found: build it with `python -m aussm_amd.build` "

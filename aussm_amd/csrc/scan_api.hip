@@ -39,13 +39,6 @@ inline int launch_status() {
   return e == hipSuccess ? AUSSM_OK : (int)e;
 }
 
-inline void zero_async(float* p, size_t n, hipStream_t s) {
-  if (!p || n == 0) return;
-  size_t blocks = (n + 255) / 256;
-  if (blocks > 4096) blocks = 4096;
-  hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)blocks), dim3(256), 0, s, p, n);
-}
-
 template <int VAR, typename Tin>
 int launch_fwd_t(const FwdArgs& a, hipStream_t s) {
   const dim3 grid((unsigned)(a.B * a.ncg)), block(NT_DEFAULT);
@@ -155,10 +148,6 @@ int aussm_unitary_bwd(const float* dy, const float* dhL, const void* u, const vo
   a.dy = dy; a.dhL = dhL; a.u = u; a.delta = delta; a.theta = theta; a.Bm = Bc; a.Cm = Cc; a.Dskip = Dskip;
   a.hck = hck; a.du = du; a.ddelta = ddelta; a.dtheta = dtheta; a.dB = dB; a.dC = dC; a.dD = dD; a.dh0 = dh0;
   a.B = B; a.D = D; a.N = N; a.L = L; a.ck = ck; a.nck = (L + ck - 1) / ck; a.ncg = (D + CH - 1) / CH;
-  const size_t nbc = (size_t)B * N * L * 2;
-  zero_async(dB, nbc, s);
-  zero_async(dC, nbc, s);
-  zero_async(dD, (size_t)D, s);
   return in_dtype == AUSSM_BF16 ? launch_unitary_bwd_t<bf16_t>(a, s) : launch_unitary_bwd_t<float>(a, s);
 }
 

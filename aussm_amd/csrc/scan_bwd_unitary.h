@@ -26,8 +26,8 @@ struct UniBwdArgs {
   const float* Dskip;   // [D] or null
   const float* hck;     // [B,nck,N,2,D]
   float *du, *ddelta, *dtheta;   // [B,D,L]
-  float *dB, *dC;       // [B,N,L,2]  (zeroed before launch; accumulated with atomics over channel groups)
-  float* dD;            // [D] or null (zeroed before launch)
+  float *dB, *dC;       // [B,N,L,2]  accumulated into with atomics (caller zero-fills)
+  float* dD;            // [D] or null, accumulated into
   float* dh0;           // [B,D,N,2] or null
   int B, D, N, L, ck, nck, ncg;
 };
@@ -68,7 +68,7 @@ __global__ __launch_bounds__(NT) void unitary_bwd_kernel(const UniBwdArgs p) {
 
   __shared__ float4 s_in[T * TS];                // (Re a, Im a, delta*u, dy) per (t, channel)
   __shared__ float2 s_part[NWV * T * TS];        // per wavefront partial (dw, dtheta)
-  __shared__ float s_red[NWV * 64 * (NV + 4)];   // transpose scratch
+  __shared__ __align__(16) float s_red[NWV * 64 * (NV + 4)];   // transpose scratch
   __shared__ float s_acc[NWV * T * AS];          // per wavefront dB/dC of the current tile
 
   const int tid = threadIdx.x, lane = tid & 63, wave = wave_index();

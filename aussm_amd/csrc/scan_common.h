@@ -79,10 +79,4 @@ __device__ __forceinline__ float half_wave_sum(float v) {
   return v;
 }
 
-__global__ void fill_zero_kernel(float* __restrict__ p, size_t n) {
-  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-  const size_t stride = (size_t)gridDim.x * blockDim.x;
-  for (; i < n; i += stride) p[i] = 0.0f;
-}
-
 }  // namespace aussm

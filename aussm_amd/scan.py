@@ -115,9 +115,10 @@ def unitary_bwd_raw(dy, dhL, u, delta, theta, Bri, Cri, D, hck, ck, want_dD=True
     n = Bri.shape[1]
     f32 = dict(device=u.device, dtype=torch.float32)
     du, ddelta, dtheta = (torch.empty((b, d, l), **f32) for _ in range(3))
-    dB = torch.empty((b, n, l, 2), **f32)
-    dC = torch.empty((b, n, l, 2), **f32)
-    dD = torch.empty((d,), **f32) if (want_dD and D is not None) else None
+    # accumulated into with atomics by the kernel: start from zero
+    dB = torch.zeros((b, n, l, 2), **f32)
+    dC = torch.zeros((b, n, l, 2), **f32)
+    dD = torch.zeros((d,), **f32) if (want_dD and D is not None) else None
     dh0 = torch.empty((b, d, n, 2), **f32) if want_dh0 else None
     check(lib.aussm_unitary_bwd(ptr(dy), ptr(dhL), ptr(u), ptr(delta), ptr(theta), ptr(Bri), ptr(Cri), ptr(D),
                                 ptr(hck), ptr(du), ptr(ddelta), ptr(dtheta), ptr(dB), ptr(dC), ptr(dD), ptr(dh0),

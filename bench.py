@@ -1,0 +1,168 @@
+#!/usr/bin/env python3
+"""Headline benchmark: adaptive-unitary core scan, forward + backward, fp32,
+B=32 D=512 N=16 L=2048, on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu]
+
+One "step" = one forward launch (y, checkpoints) + zero-fill of the accumulated gradients +
+one backward launch (du, ddelta, dtheta, dB, dC, dD) on synthetic inputs that are already
+resident in HBM.  Prints ONE JSON line.
+
+  value          (b,d,l) samples per second over forward+backward (B*D*L / step time)
+  roofline       dominant kernel (the backward scan): algorithmic bytes (28E + 32S + 4D,
+                 E = B*D*L, S = B*N*L) / its average launch duration, measured here with HIP
+                 events on the launch stream, against the 8 TB/s HBM peak
+  cpu_baseline   the CPU oracle (sequential-loop PyTorch scan + autograd) timed on this host's
+                 cores on a bounded slice of the batch
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+SHAPE = dict(B=32, D=512, N=16, L=2048)
+
+
+def cpu_baseline(B_sample: int):
+    """Oracle forward+backward on a slice of the batch (same D, N, L)."""
+    import torch
+    from oracle import scan_oracle as O
+    D, N, L = SHAPE["D"], SHAPE["N"], SHAPE["L"]
+    cores = os.cpu_count() or 1
+    threads = min(cores, 16)
+    torch.set_num_threads(threads)
+    p = O.make_core_inputs(B_sample, D, N, L, seed=0)
+    leaves = [p[k].clone().requires_grad_(True) for k in ("u", "delta", "theta", "Bc", "Cc", "Dskip")]
+    t0 = time.perf_counter()
+    y, _ = O.unitary_core_loop(*leaves)
+    (y * p["dy"]).sum().backward()
+    dt = time.perf_counter() - t0
+    return {
+        "value": B_sample * D * L / dt,
+        "unit": "(b,d,l) samples/s, forward+backward",
+        "cores": threads,
+        "kind": "port",
+        "sample": f"B={B_sample} of {SHAPE['B']} batch elements at D={D} N={N} L={L}, one run, {dt:.1f} s wall, "
+                  f"torch {threads} threads on a host with {cores} cores",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cpu-batch", type=int, default=16)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU; --gpus must be 1 (no multi-GPU path exists)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from aussm_amd import scan
+    from oracle import scan_oracle as O
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    B, D, N, L = SHAPE["B"], SHAPE["D"], SHAPE["N"], SHAPE["L"]
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    p = {k: v.to(dev) for k, v in O.make_core_inputs(B, D, N, L, seed=0).items()}
+    Bri = torch.view_as_real(p["Bc"]).contiguous()
+    Cri = torch.view_as_real(p["Cc"]).contiguous()
+    ck = scan.UNITARY_CK
+
+    def step():
+        y, _, hck = scan.unitary_fwd_raw(p["u"], p["delta"], p["theta"], Bri, Cri, p["Dskip"], None, None,
+                                         want_state=False, ck=ck)
+        return scan.unitary_bwd_raw(p["dy"], None, p["u"], p["delta"], p["theta"], Bri, Cri, p["Dskip"], hck, ck)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / args.steps
+
+    # ---- per-kernel durations with HIP events on the launch stream (torch's current stream)
+    lib = scan._lib.load()
+    ptr, stream = scan.ptr, scan._stream()
+    f32 = dict(device=dev, dtype=torch.float32)
+    y = torch.empty((B, D, L), **f32)
+    hck = torch.empty((B, scan.num_checkpoints(L, ck), N, 2, D), **f32)
+    du, ddl, dth = (torch.empty((B, D, L), **f32) for _ in range(3))
+    dB, dC, dD = torch.zeros((B, N, L, 2), **f32), torch.zeros((B, N, L, 2), **f32), torch.zeros((D,), **f32)
+
+    def fwd_only():
+        scan.check(lib.aussm_unitary_fwd(ptr(p["u"]), ptr(p["delta"]), ptr(p["theta"]), ptr(Bri), ptr(Cri),
+                                         ptr(p["Dskip"]), None, None, ptr(y), None, ptr(hck),
+                                         B, D, N, L, ck, 0, stream), "fwd")
+
+    def bwd_only():
+        scan.check(lib.aussm_unitary_bwd(ptr(p["dy"]), None, ptr(p["u"]), ptr(p["delta"]), ptr(p["theta"]), ptr(Bri),
+                                         ptr(Cri), ptr(p["Dskip"]), ptr(hck), ptr(du), ptr(ddl), ptr(dth),
+                                         ptr(dB), ptr(dC), ptr(dD), None, B, D, N, L, ck, 0, stream), "bwd")
+
+    def kernel_us(fn, reps):
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
+        fn()
+        torch.cuda.synchronize()
+        for s, e in evs:
+            s.record()
+            fn()
+            e.record()
+        torch.cuda.synchronize()
+        return sum(s.elapsed_time(e) for s, e in evs) / reps * 1e3
+
+    reps = max(10, min(args.steps, 50))
+    t_fwd = kernel_us(fwd_only, reps)
+    t_bwd = kernel_us(bwd_only, reps)
+    E, S = B * D * L, B * N * L
+    bytes_fwd = 16 * E + 16 * S + 4 * D
+    bytes_bwd = 28 * E + 32 * S + 4 * D
+    ach = bytes_bwd / (t_bwd * 1e-6) / 1e9
+
+    out = {
+        "metric": "unitary scan fwd+bwd elements/s + achieved HBM GB/s (% peak), B32 D512 N16 L2048",
+        "value": B * D * L / dt,
+        "unit": "(b,d,l) samples/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": dt * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "unitary core scan fwd+bwd, B=32 D=512 N=16 L=2048, fp32 (BASELINE configs[3], unitary, fp32)",
+                   "B": B, "D": D, "N": N, "L": L, "checkpoint_interval": ck},
+        "state_updates_per_s": B * D * N * L / dt,
+        "fwd_bwd_algorithmic_GBps": (bytes_fwd + bytes_bwd) / ((t_fwd + t_bwd) * 1e-6) / 1e9,
+        "fwd_bwd_frac_of_hbm_peak": (bytes_fwd + bytes_bwd) / ((t_fwd + t_bwd) * 1e-6) / 1e9 / HBM_PEAK_GBS,
+        "kernels_us": {"unitary_fwd": t_fwd, "unitary_bwd": t_bwd},
+        "roofline": {"bound": "hbm", "kernel": "unitary_bwd_kernel", "achieved": ach, "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": ach / HBM_PEAK_GBS, "traffic": None,
+                     "algorithmic_bytes": bytes_bwd,
+                     "fwd_kernel": {"achieved": bytes_fwd / (t_fwd * 1e-6) / 1e9,
+                                    "frac": bytes_fwd / (t_fwd * 1e-6) / 1e9 / HBM_PEAK_GBS,
+                                    "algorithmic_bytes": bytes_fwd}},
+    }
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(args.cpu_batch)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -83,7 +83,9 @@ int aussm_unitary_fwd(const void* u, const void* delta, const float* theta,
  * dB, dC use the convention dRe + i*dIm (what torch returns for a complex leaf).
  * Required: dy, u, delta, theta, Bc, Cc, hck, du, ddelta, dtheta, dB, dC.
  * Optional: dhL, Dskip, h0 (unused, may be NULL), dD, dh0.
- * dB, dC and dD are zeroed by this call before being accumulated into. */
+ * dB, dC and dD are ACCUMULATED into (several channel groups add into the same element with
+ * float atomics): the caller zero-fills them for a plain gradient, as the reference's host
+ * launcher does (ssm_adaptive_unitary_backward.cu:531-543).  All other outputs are overwritten. */
 int aussm_unitary_bwd(const float* dy, const float* dhL,
                       const void* u, const void* delta, const float* theta,
                       const void* Bc, const void* Cc, const float* Dskip, const float* hck,
