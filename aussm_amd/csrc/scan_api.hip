@@ -3,6 +3,8 @@
 #include "../../include/aussm_hip.h"
 
 #include <hip/hip_runtime.h>
+#include <stdio.h>
+#include <stdlib.h>
 
 #include "scan_bwd_unitary.h"
 #include "scan_common.h"
@@ -12,15 +14,24 @@ using namespace aussm;
 
 namespace {
 
-constexpr int NT_DEFAULT = 256;
+// ---- kernel configuration -------------------------------------------------------------------
+// A workgroup of NT threads (NT/64 wavefronts) owns 64 channels; each wavefront owns NW states.
+// The scalar loads of B_t/C_t are issued one "turn" ahead; with two or more wavefronts per SIMD
+// the turn of another wavefront doubles that distance, so for a given N the configuration with
+// MORE wavefronts (smaller NW) is preferred as long as the launch still fits one workgroup.
+struct Cfg { int nw, nt; };
 
-// states per wavefront for a 4-wavefront workgroup
-inline int pick_nw(int N) {
-  if (N <= 4) return 1;
-  if (N <= 8) return 2;
-  if (N <= 16) return 4;
-  if (N <= 32) return 8;
-  return 16;
+inline Cfg pick_cfg(int N, int max_waves) {
+  // test/tuning override: AUSSM_CFG="NW,NT" (must be one of the compiled configurations)
+  if (const char* e = getenv("AUSSM_CFG")) {
+    Cfg c{0, 0};
+    if (sscanf(e, "%d,%d", &c.nw, &c.nt) == 2 && c.nw > 0 && c.nw * (c.nt / 64) >= N) return c;
+  }
+  const Cfg table[] = {{1, 256}, {1, 512}, {2, 512}, {4, 512}, {8, 512},
+                       {2, 256}, {4, 256}, {8, 256}, {16, 256}};
+  for (const Cfg& c : table)
+    if (c.nw * (c.nt / 64) >= N && c.nt / 64 <= max_waves) return c;
+  return Cfg{16, 256};
 }
 
 inline int check_common(int B, int D, int N, int L, int ck, int in_dtype) {
@@ -39,17 +50,20 @@ inline int launch_status() {
   return e == hipSuccess ? AUSSM_OK : (int)e;
 }
 
+#define AUSSM_FWD_CASE(NW_, NT_)                                                                     \
+  if (c.nw == NW_ && c.nt == NT_) {                                                                  \
+    hipLaunchKernelGGL((core_fwd_kernel<VAR, NW_, NT_, Tin>), grid, dim3(NT_), 0, s, a);             \
+    return launch_status();                                                                          \
+  }
+
 template <int VAR, typename Tin>
 int launch_fwd_t(const FwdArgs& a, hipStream_t s) {
-  const dim3 grid((unsigned)(a.B * a.ncg)), block(NT_DEFAULT);
-  switch (pick_nw(a.N)) {
-    case 1: hipLaunchKernelGGL((core_fwd_kernel<VAR, 1, NT_DEFAULT, Tin>), grid, block, 0, s, a); break;
-    case 2: hipLaunchKernelGGL((core_fwd_kernel<VAR, 2, NT_DEFAULT, Tin>), grid, block, 0, s, a); break;
-    case 4: hipLaunchKernelGGL((core_fwd_kernel<VAR, 4, NT_DEFAULT, Tin>), grid, block, 0, s, a); break;
-    case 8: hipLaunchKernelGGL((core_fwd_kernel<VAR, 8, NT_DEFAULT, Tin>), grid, block, 0, s, a); break;
-    default: hipLaunchKernelGGL((core_fwd_kernel<VAR, 16, NT_DEFAULT, Tin>), grid, block, 0, s, a); break;
-  }
-  return launch_status();
+  const dim3 grid((unsigned)(a.B * a.ncg));
+  const Cfg c = pick_cfg(a.N, 8);
+  AUSSM_FWD_CASE(1, 256) AUSSM_FWD_CASE(2, 256) AUSSM_FWD_CASE(4, 256) AUSSM_FWD_CASE(8, 256)
+  AUSSM_FWD_CASE(16, 256) AUSSM_FWD_CASE(1, 512) AUSSM_FWD_CASE(2, 512) AUSSM_FWD_CASE(4, 512)
+  AUSSM_FWD_CASE(8, 512)
+  return AUSSM_E_SHAPE;
 }
 
 template <int VAR>
@@ -57,17 +71,23 @@ int launch_fwd(const FwdArgs& a, int in_dtype, hipStream_t s) {
   return in_dtype == AUSSM_BF16 ? launch_fwd_t<VAR, bf16_t>(a, s) : launch_fwd_t<VAR, float>(a, s);
 }
 
+// The backward workgroup keeps a (dw, dtheta) slab per wavefront in LDS: four wavefronts afford
+// 32-step tiles, eight wavefronts 16-step tiles.
+#define AUSSM_UBWD_CASE(NW_, NT_, TT_)                                                               \
+  if (c.nw == NW_ && c.nt == NT_) {                                                                  \
+    hipLaunchKernelGGL((unitary_bwd_kernel<NW_, NT_, TT_, Tin>), grid, dim3(NT_), 0, s, a);          \
+    return launch_status();                                                                          \
+  }
+
 template <typename Tin>
 int launch_unitary_bwd_t(const UniBwdArgs& a, hipStream_t s) {
-  const dim3 grid((unsigned)(a.B * a.ncg)), block(NT_DEFAULT);
-  switch (pick_nw(a.N)) {
-    case 1: hipLaunchKernelGGL((unitary_bwd_kernel<1, NT_DEFAULT, Tin>), grid, block, 0, s, a); break;
-    case 2: hipLaunchKernelGGL((unitary_bwd_kernel<2, NT_DEFAULT, Tin>), grid, block, 0, s, a); break;
-    case 4: hipLaunchKernelGGL((unitary_bwd_kernel<4, NT_DEFAULT, Tin>), grid, block, 0, s, a); break;
-    case 8: hipLaunchKernelGGL((unitary_bwd_kernel<8, NT_DEFAULT, Tin>), grid, block, 0, s, a); break;
-    default: hipLaunchKernelGGL((unitary_bwd_kernel<16, NT_DEFAULT, Tin>), grid, block, 0, s, a); break;
-  }
-  return launch_status();
+  const dim3 grid((unsigned)(a.B * a.ncg));
+  const Cfg c = pick_cfg(a.N, 8);
+  AUSSM_UBWD_CASE(1, 256, 32) AUSSM_UBWD_CASE(2, 256, 32) AUSSM_UBWD_CASE(4, 256, 32)
+  AUSSM_UBWD_CASE(8, 256, 32) AUSSM_UBWD_CASE(16, 256, 32)
+  AUSSM_UBWD_CASE(1, 512, 16) AUSSM_UBWD_CASE(2, 512, 16) AUSSM_UBWD_CASE(4, 512, 16)
+  AUSSM_UBWD_CASE(8, 512, 16)
+  return AUSSM_E_SHAPE;
 }
 
 }  // namespace

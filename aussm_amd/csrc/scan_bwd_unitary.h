@@ -10,6 +10,13 @@
 //     dtheta_l = -sum_n Im(conj(g_l) a_l h_{l-1})
 // Gradient formulas: the recurrence form of
 // extension-cpp/extension_cpp/csrc/cuda/ssm_adaptive_unitary_backward.cu:154-403.
+//
+// dB/dC are sums over channels, i.e. over the lanes of a wavefront and over the workgroups of
+// one batch element.  The lane sum is an LDS transpose (every lane writes its products as a row,
+// then reads one column), the sum over workgroups uses float atomics on the output.
+// dw and dtheta are sums over states, i.e. over the wavefronts of a workgroup: every wavefront
+// writes its partial sums to its own LDS slab and the epilogue adds the slabs in a fixed order
+// (LDS float atomics were measured to be several times slower than this).
 #pragma once
 #include "scan_common.h"
 
@@ -32,44 +39,48 @@ struct UniBwdArgs {
   int B, D, N, L, ck, nck, ncg;
 };
 
-// Sum NV per-lane values over the 64 lanes (channels) of a wavefront through an LDS transpose.
-// After the call lane c (< NV) holds the total of value c.  `red` is this wavefront's private
-// scratch of 64 * RS floats.
-template <int NV>
-__device__ __forceinline__ float lane_transpose_sum(const float (&vals)[NV], float* red, int lane) {
-  constexpr int RS = NV + 4;            // row stride in floats (keeps 16-byte alignment)
-  constexpr int PARTS = 64 / NV;        // lanes per column
-  float4* row = reinterpret_cast<float4*>(red + lane * RS);
+constexpr int RED_COLS = 4 * TG;        // products per lane per turn: TG x (dB re, dB im) then TG x (dC re, dC im)
+constexpr int RED_RS = RED_COLS + 4;    // padded row stride (floats), keeps rows 16-byte aligned
+
+// Column sums over the 64 lanes of a wavefront.  Each lane passes RED_COLS values; afterwards
+// lane c (< RED_COLS) holds the sum of value c over all lanes.  `red` = this wavefront's scratch.
+// LDS operations of one wavefront execute in order, so the column reads see the row writes of
+// the other lanes without a wait; the wave barriers only pin the compiler's ordering.
+__device__ __forceinline__ float lane_transpose_sum32(const float (&vals)[RED_COLS], float* red, int lane) {
+  float4* row = reinterpret_cast<float4*>(red + lane * RED_RS);
 #pragma unroll
-  for (int j = 0; j < NV / 4; ++j) row[j] = make_float4(vals[4 * j], vals[4 * j + 1], vals[4 * j + 2], vals[4 * j + 3]);
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  for (int j = 0; j < RED_COLS / 4; ++j)
+    row[j] = make_float4(vals[4 * j], vals[4 * j + 1], vals[4 * j + 2], vals[4 * j + 3]);
   __builtin_amdgcn_wave_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-  const int c = lane % NV, part = lane / NV;
-  float acc = 0.f;
+  const int c = lane & (RED_COLS - 1), half = lane >> 5;
+  const float* colp = red + (half * 32) * RED_RS + c;
+  float v[32];
 #pragma unroll
-  for (int i = 0; i < NV; ++i) acc += red[(i * PARTS + part) * RS + c];
+  for (int i = 0; i < 32; ++i) v[i] = colp[i * RED_RS];
+  sched_fence();                       // all 32 reads in flight before the first add
 #pragma unroll
-  for (int o = NV; o < 64; o <<= 1) acc += __shfl_xor(acc, o, 64);
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  for (int s = 16; s >= 1; s >>= 1)
+#pragma unroll
+    for (int i = 0; i < s; ++i) v[i] += v[i + s];
+  float acc = v[0];
+  acc += __shfl_xor(acc, 32, 64);
   __builtin_amdgcn_wave_barrier();
   return acc;
 }
 
-template <int NW, int NT, typename Tin>
+// TT: timesteps per staged tile (16 or 32; the checkpoint interval is a multiple of 32 either way).
+template <int NW, int NT, int TT, typename Tin>
 __global__ __launch_bounds__(NT) void unitary_bwd_kernel(const UniBwdArgs p) {
   constexpr int NWV = NT / 64;
-  constexpr int E = CH * T / NT;
-  constexpr int RSTEP = NT / T;
-  constexpr int NG = (NW < 4) ? NW : 4;          // states reduced per transpose batch
-  constexpr int NV = 4 * NG;                     // values per batch: (dB re, dB im, dC re, dC im) per state
-  constexpr int NB = NW / NG;                    // batches per step
-  constexpr int AS = 4 * NW + 1;                 // padded row stride of the tile accumulator
+  constexpr int E = CH * TT / NT;
+  constexpr int RSTEP = NT / TT;
+  constexpr int NGRP = TT / TG;
+  static_assert(RED_COLS == 32, "the lane transpose assumes 32 columns");
+  static_assert(E >= 1 && NGRP >= 1, "tile too small for this workgroup size");
 
-  __shared__ float4 s_in[T * TS];                // (Re a, Im a, delta*u, dy) per (t, channel)
-  __shared__ float2 s_part[NWV * T * TS];        // per wavefront partial (dw, dtheta)
-  __shared__ __align__(16) float s_red[NWV * 64 * (NV + 4)];   // transpose scratch
-  __shared__ float s_acc[NWV * T * AS];          // per wavefront dB/dC of the current tile
+  __shared__ float4 s_in[TT * TS];                         // (Re a, Im a, delta*u, dy) per (t, channel)
+  __shared__ float2 s_part[NWV * TT * TS];                 // per wavefront partial (dw, dtheta)
+  __shared__ __align__(16) float s_red[NWV * 64 * RED_RS]; // lane-transpose scratch, one slab per wavefront
 
   const int tid = threadIdx.x, lane = tid & 63, wave = wave_index();
   const int wg = xcd_remap(blockIdx.x, gridDim.x);
@@ -77,6 +88,7 @@ __global__ __launch_bounds__(NT) void unitary_bwd_kernel(const UniBwdArgs p) {
   const int N = p.N, L = p.L, D = p.D;
   const int n0 = wave * NW;
   const bool active = n0 < N;
+  const bool full_group = active && n0 + NW <= N;
   const int nwa = (N + NW - 1) / NW;
   const int d = d0 + lane;
   const bool dok = d < D;
@@ -85,8 +97,8 @@ __global__ __launch_bounds__(NT) void unitary_bwd_kernel(const UniBwdArgs p) {
   const Tin* __restrict__ gdl = static_cast<const Tin*>(p.delta);
   const Tin* __restrict__ gB = static_cast<const Tin*>(p.Bm);
   const Tin* __restrict__ gC = static_cast<const Tin*>(p.Cm);
-  float* red = s_red + wave * 64 * (NV + 4);
-  float* acc = s_acc + wave * T * AS;
+  float* red = s_red + wave * 64 * RED_RS;
+  float2* part = s_part + wave * TT * TS;
 
   auto load_ck = [&](int kb, float (&xr)[NW], float (&xi)[NW]) {
 #pragma unroll
@@ -114,8 +126,8 @@ __global__ __launch_bounds__(NT) void unitary_bwd_kernel(const UniBwdArgs p) {
     }
   }
 
-  // ---- staging-side mapping
-  const int col = tid % T, row0 = tid / T;
+  // ---- staging-side mapping (lanes run along time)
+  const int col = tid % TT, row0 = tid / TT;
   float ru[E], rdl[E], rth[E], rgy[E], dsk[E], accD[E];
   size_t goff[E];
   bool rowok[E];
@@ -140,84 +152,155 @@ __global__ __launch_bounds__(NT) void unitary_bwd_kernel(const UniBwdArgs p) {
     }
   };
 
-  const int ntiles = (L + T - 1) / T;
-  load_tile((ntiles - 1) * T);
+  const int ntiles = (L + TT - 1) / TT;
+  load_tile((ntiles - 1) * TT);
+
+  // scalar-cache warm-up of the B_t/C_t lines, one tile ahead of the scan (see the forward kernel)
+  constexpr bool WARM = NW <= 4;
+  constexpr int RB = (int)sizeof(Tin) * 2;
+  const size_t row_base = ((size_t)b * N + n0) * L;
+  TileWarm<WARM ? NW : 1, RB, TT> warm;
+  if (WARM && full_group && ntiles * TT == L) {
+    warm.issue(gB, gC, row_base + (size_t)(ntiles - 1) * TT, L);
+    warm.retire();
+  }
 
   for (int it = ntiles - 1; it >= 0; --it) {
-    const int l0 = it * T;
+    const int l0 = it * TT;
+    const int tmax = (L - l0 < TT) ? (L - l0) : TT;
+    const bool warm_next = WARM && full_group && it > 0;
+    if (warm_next) warm.issue(gB, gC, row_base + l0 - TT, L);
+
+    // ---- stage
     float eu[E], edl[E], egy[E];
 #pragma unroll
     for (int k = 0; k < E; ++k) {
       float sn, cs;
-      sincosf(rth[k], &sn, &cs);
+      fast_sincosf(rth[k], &sn, &cs);
       s_in[col * TS + row0 + k * RSTEP] = make_float4(cs, sn, rdl[k] * ru[k], rgy[k]);
       eu[k] = ru[k]; edl[k] = rdl[k]; egy[k] = rgy[k];
     }
+    if (warm_next) warm.retire();
     __syncthreads();
-    if (it > 0) load_tile(l0 - T);
+    if (it > 0) load_tile(l0 - TT);
 
-    const int tmax = (L - l0 < T) ? (L - l0) : T;
-    if (active) {
-      const size_t brow = ((size_t)b * N + n0) * L + l0;
-      for (int t = tmax - 1; t >= 0; --t) {
-        const float4 v = s_in[t * TS + lane];
-        const float cs = v.x, sn = v.y, w = v.z, gy = v.w;
-        float kacc = 0.f, qacc = 0.f;
+    const size_t brow = row_base + l0;
+    if (full_group && tmax == TT) {
+      // ---- fast path: groups of TG timesteps right to left; inside a group the wavefront's
+      // state rows take turns, each turn consuming ONE scalar load of B_t and one of C_t that
+      // was issued a turn earlier.
+      float rc[TG], rs[TG], rw[TG], rg[TG];
 #pragma unroll
-        for (int bt = 0; bt < NB; ++bt) {
-          float vals[NV];
+      for (int t = 0; t < TG; ++t) {
+        const float4 v = s_in[(TT - TG + t) * TS + lane];
+        rc[t] = v.x; rs[t] = v.y; rw[t] = v.z; rg[t] = v.w;
+      }
+      f32x16 bn = ld_c8(gB, brow + (TT - TG)), cn = ld_c8(gC, brow + (TT - TG));
 #pragma unroll
-          for (int j = 0; j < NG; ++j) {
-            const int k = bt * NG + j;
-            float2 bv = make_float2(0.f, 0.f), cv = make_float2(0.f, 0.f);
-            if (n0 + k < N) {
-              const size_t bi = brow + (size_t)k * L + t;
-              bv = ld_c(gB, bi); cv = ld_c(gC, bi);
+      for (int g = NGRP - 1; g >= 0; --g) {
+        float kacc[TG], qacc[TG], nc[TG], ns[TG], nw_[TG], ng[TG];
+#pragma unroll
+        for (int t = 0; t < TG; ++t) { kacc[t] = 0.f; qacc[t] = 0.f; }
+#pragma unroll
+        for (int k = 0; k < NW; ++k) {
+          const f32x16 bc = bn, cc = cn;
+          touch_uniform(bc[0]);
+          touch_uniform(cc[0]);
+          sched_fence();
+          if (k + 1 < NW) {
+            bn = ld_c8(gB, brow + (size_t)(k + 1) * L + g * TG);
+            cn = ld_c8(gC, brow + (size_t)(k + 1) * L + g * TG);
+          } else if (g > 0) {
+            bn = ld_c8(gB, brow + (g - 1) * TG);
+            cn = ld_c8(gC, brow + (g - 1) * TG);
+          }
+          if (k == 0 && g > 0) {
+#pragma unroll
+            for (int t = 0; t < TG; ++t) {
+              const float4 v = s_in[((g - 1) * TG + t) * TS + lane];
+              nc[t] = v.x; ns[t] = v.y; nw_[t] = v.z; ng[t] = v.w;
             }
-            // adjoint of the read-out
-            gr[k] = fmaf(cv.x, gy, gr[k]);
-            gi[k] = fmaf(-cv.y, gy, gi[k]);
-            vals[4 * j + 0] = w * gr[k];
-            vals[4 * j + 1] = w * gi[k];
-            vals[4 * j + 2] = gy * hr[k];
-            vals[4 * j + 3] = -gy * hi[k];
-            kacc = fmaf(bv.x, gr[k], kacc);
-            kacc = fmaf(bv.y, gi[k], kacc);
-            // p = a_l h_{l-1} = h_l - B_l w_l
-            const float pr = fmaf(-bv.x, w, hr[k]);
-            const float pi = fmaf(-bv.y, w, hi[k]);
-            qacc = fmaf(gi[k], pr, qacc);
-            qacc = fmaf(-gr[k], pi, qacc);
-            // h_{l-1} = conj(a) p ;  adjoint carried to l-1 = conj(a) g
+          }
+          sched_fence();
+          float vals[RED_COLS];
+#pragma unroll
+          for (int t = TG - 1; t >= 0; --t) {
+            const float br = bc[2 * t], bi = bc[2 * t + 1], cr = cc[2 * t], ci = cc[2 * t + 1];
+            const float w = rw[t], gy = rg[t], cs = rc[t], sn = rs[t];
+            gr[k] = fmaf(cr, gy, gr[k]);
+            gi[k] = fmaf(-ci, gy, gi[k]);
+            vals[2 * t] = w * gr[k];
+            vals[2 * t + 1] = w * gi[k];
+            vals[2 * TG + 2 * t] = gy * hr[k];
+            vals[2 * TG + 2 * t + 1] = -gy * hi[k];
+            kacc[t] = fmaf(br, gr[k], kacc[t]);
+            kacc[t] = fmaf(bi, gi[k], kacc[t]);
+            const float pr = fmaf(-br, w, hr[k]);
+            const float pi = fmaf(-bi, w, hi[k]);
+            qacc[t] = fmaf(gi[k], pr, qacc[t]);
+            qacc[t] = fmaf(-gr[k], pi, qacc[t]);
             hr[k] = fmaf(cs, pr, sn * pi);
             hi[k] = fmaf(cs, pi, -sn * pr);
             const float tg = fmaf(cs, gr[k], sn * gi[k]);
             gi[k] = fmaf(cs, gi[k], -sn * gr[k]);
             gr[k] = tg;
           }
-          const float tot = lane_transpose_sum<NV>(vals, red, lane);
-          if (lane < NV) acc[t * AS + bt * NV + lane] = tot;
-        }
-        s_part[(wave * T + t) * TS + lane] = make_float2(kacc, qacc);
-      }
-      // ---- flush this wavefront's dB/dC tile: lane = (t, re/im) -> 256 contiguous bytes per state row
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-      __builtin_amdgcn_wave_barrier();
-      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-      const int ft = lane >> 1, fc = lane & 1;
-      if (ft < tmax) {
-#pragma unroll
-        for (int k = 0; k < NW; ++k) {
-          if (n0 + k < N) {
-            const size_t o = ((brow + (size_t)k * L + ft) << 1) + fc;
-            atomicAdd(p.dB + o, acc[ft * AS + 4 * k + fc]);
-            atomicAdd(p.dC + o, acc[ft * AS + 4 * k + 2 + fc]);
+          // lanes 0..15: dB of (row, t0..t0+7) as 16 consecutive floats; lanes 16..31: dC likewise
+          const float tot = lane_transpose_sum32(vals, red, lane);
+          if (lane < RED_COLS) {
+            float* dst = (lane < 2 * TG) ? p.dB : p.dC;
+            atomicAdd(dst + 2 * (brow + (size_t)k * L + g * TG) + (lane & (2 * TG - 1)), tot);
           }
         }
+#pragma unroll
+        for (int t = 0; t < TG; ++t) {
+          part[(g * TG + t) * TS + lane] = make_float2(kacc[t], qacc[t]);
+          if (g > 0) { rc[t] = nc[t]; rs[t] = ns[t]; rw[t] = nw_[t]; rg[t] = ng[t]; }
+        }
       }
-      // ---- re-synchronise the regenerated state with the forward pass's checkpoint
-      if (l0 > 0 && (l0 % p.ck) == 0) load_ck(l0 / p.ck - 1, hr, hi);
+    } else if (active) {
+      // ---- general path (ragged tile or partial state group): one timestep at a time
+      for (int t = tmax - 1; t >= 0; --t) {
+        const float4 v = s_in[t * TS + lane];
+        const float cs = v.x, sn = v.y, w = v.z, gy = v.w;
+        float kacc = 0.f, qacc = 0.f;
+#pragma unroll
+        for (int k = 0; k < NW; ++k) {
+          float2 bv = make_float2(0.f, 0.f), cv = make_float2(0.f, 0.f);
+          const bool nok = n0 + k < N;
+          const size_t bi = brow + (size_t)k * L + t;
+          if (nok) { bv = ld_c(gB, bi); cv = ld_c(gC, bi); }
+          gr[k] = fmaf(cv.x, gy, gr[k]);
+          gi[k] = fmaf(-cv.y, gy, gi[k]);
+          float vals[RED_COLS];
+#pragma unroll
+          for (int j = 0; j < RED_COLS; ++j) vals[j] = 0.f;
+          vals[0] = w * gr[k];
+          vals[1] = w * gi[k];
+          vals[2] = gy * hr[k];
+          vals[3] = -gy * hi[k];
+          kacc = fmaf(bv.x, gr[k], kacc);
+          kacc = fmaf(bv.y, gi[k], kacc);
+          const float pr = fmaf(-bv.x, w, hr[k]);
+          const float pi = fmaf(-bv.y, w, hi[k]);
+          qacc = fmaf(gi[k], pr, qacc);
+          qacc = fmaf(-gr[k], pi, qacc);
+          hr[k] = fmaf(cs, pr, sn * pi);
+          hi[k] = fmaf(cs, pi, -sn * pr);
+          const float tg = fmaf(cs, gr[k], sn * gi[k]);
+          gi[k] = fmaf(cs, gi[k], -sn * gr[k]);
+          gr[k] = tg;
+          const float tot = lane_transpose_sum32(vals, red, lane);
+          if (nok && lane < 4) {
+            float* dst = (lane < 2) ? p.dB : p.dC;
+            atomicAdd(dst + 2 * bi + (lane & 1), tot);
+          }
+        }
+        part[t * TS + lane] = make_float2(kacc, qacc);
+      }
     }
+    // ---- re-synchronise the regenerated state with the forward pass's checkpoint
+    if (active && l0 > 0 && (l0 % p.ck) == 0) load_ck(l0 / p.ck - 1, hr, hi);
     __syncthreads();
 
     // ---- epilogue: channel-wise gradients, coalesced along time
@@ -227,7 +310,7 @@ __global__ __launch_bounds__(NT) void unitary_bwd_kernel(const UniBwdArgs p) {
       if (rowok[k] && ll < L) {
         float kk = 0.f, qq = 0.f;
         for (int w = 0; w < nwa; ++w) {
-          const float2 pv = s_part[(w * T + col) * TS + row0 + k * RSTEP];
+          const float2 pv = s_part[(w * TT + col) * TS + row0 + k * RSTEP];
           kk += pv.x; qq += pv.y;
         }
         const size_t o = goff[k] + ll;
@@ -237,6 +320,8 @@ __global__ __launch_bounds__(NT) void unitary_bwd_kernel(const UniBwdArgs p) {
         accD[k] = fmaf(egy[k], eu[k], accD[k]);
       }
     }
+    // No barrier here: the next stage writes only s_in (its readers are behind the barrier above)
+    // and the next scan writes s_part only after the next barrier.
   }
 
   if (p.dh0 && active && dok) {
@@ -250,9 +335,12 @@ __global__ __launch_bounds__(NT) void unitary_bwd_kernel(const UniBwdArgs p) {
     }
   }
   if (p.dD) {
+    // the TT lanes that share a channel row are consecutive: sum them with xor-shuffles
 #pragma unroll
     for (int k = 0; k < E; ++k) {
-      const float s = half_wave_sum(accD[k]);
+      float s = accD[k];
+#pragma unroll
+      for (int o = TT / 2; o >= 1; o >>= 1) s += __shfl_xor(s, o, 64);
       if (col == 0 && rowok[k]) atomicAdd(p.dD + d0 + row0 + k * RSTEP, s);
     }
   }

@@ -48,6 +48,30 @@ __device__ __forceinline__ float dsiluf_(float v) { float s = sigmoidf_(v); retu
 // softplus with torch's threshold of 20 (F.softplus default)
 __device__ __forceinline__ float softplusf_(float v) { return v > 20.0f ? v : log1pf(__expf(v)); }
 
+// sin and cos of one argument, about 25 VALU instructions and no branch on the common path.
+// Cody-Waite reduction by pi/2 in three fused steps, then minimax polynomials on [-pi/4, pi/4]
+// (max error ~1 ulp of 1.0 for |x| < 1e4, which covers accumulated phases of practical length).
+// Larger arguments take the library routine.
+__device__ __forceinline__ void fast_sincosf(float x, float* sn, float* cs) {
+  if (__builtin_expect(fabsf(x) > 1.0e4f, 0)) { sincosf(x, sn, cs); return; }
+  const float kf = rintf(x * 0.636619772367581343f);
+  float r = fmaf(-kf, 1.57079637050628662109375f, x);
+  r = fmaf(-kf, -4.37113900018624283e-8f, r);
+  r = fmaf(-kf, -1.71512449782676e-15f, r);
+  const float r2 = r * r;
+  float ps = fmaf(-1.9515295891e-4f, r2, 8.3321608736e-3f);
+  ps = fmaf(ps, r2, -1.6666654611e-1f);
+  const float s = fmaf(r * r2, ps, r);
+  float pc = fmaf(2.443315711809948e-5f, r2, -1.388731625493765e-3f);
+  pc = fmaf(pc, r2, 4.166664568298827e-2f);
+  const float c = fmaf(r2 * r2, pc, fmaf(-0.5f, r2, 1.0f));
+  const int q = (int)kf;
+  const float s1 = (q & 1) ? c : s;
+  const float c1 = (q & 1) ? s : c;
+  *sn = (q & 2) ? -s1 : s1;
+  *cs = ((q + 1) & 2) ? -c1 : c1;
+}
+
 // wave-uniform loads of B_t / C_t.  idx is uniform across the wavefront.  The tensors are inputs
 // that no kernel of this library writes, so they are read through the constant address space:
 // that lets the compiler select scalar (SMEM) loads whose results sit in SGPRs and feed the FMAs
@@ -71,6 +95,82 @@ __device__ __forceinline__ float ld_r(const bf16_t* __restrict__ p, size_t idx) 
   const uint32_t raw = const_as<uint32_t>(p)[idx >> 1];
   return __uint_as_float((idx & 1) ? (raw & 0xffff0000u) : (raw << 16));
 }
+
+// ---- eight consecutive timesteps of one state row in one scalar load (one 64-byte line for
+// complex fp32).  TG is the number of timesteps the scan consumes per row "turn".
+constexpr int TG = 8;
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x8 __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x8 __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+struct __attribute__((aligned(8))) f32x16_a8 { f32x16 v; };
+struct __attribute__((aligned(4))) f32x8_a4 { f32x8 v; };
+struct __attribute__((aligned(4))) u32x8_a4 { u32x8 v; };
+struct __attribute__((aligned(4))) u32x4_a4 { u32x4 v; };
+
+// complex rows: idx counts (re, im) records; result = re0, im0, re1, im1, ...
+__device__ __forceinline__ f32x16 ld_c8(const float* __restrict__ p, size_t idx) {
+  return const_as<f32x16_a8>(p + 2 * idx)->v;
+}
+__device__ __forceinline__ f32x16 ld_c8(const bf16_t* __restrict__ p, size_t idx) {
+  const u32x8 raw = const_as<u32x8_a4>(p + 2 * idx)->v;
+  f32x16 r;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    r[2 * i] = __uint_as_float(raw[i] << 16);
+    r[2 * i + 1] = __uint_as_float(raw[i] & 0xffff0000u);
+  }
+  return r;
+}
+// real rows.  For bf16 the caller guarantees an even idx (4-byte aligned address).
+__device__ __forceinline__ f32x8 ld_r8(const float* __restrict__ p, size_t idx) {
+  return const_as<f32x8_a4>(p + idx)->v;
+}
+__device__ __forceinline__ f32x8 ld_r8(const bf16_t* __restrict__ p, size_t idx) {
+  const u32x4 raw = const_as<u32x4_a4>(p + idx)->v;
+  f32x8 r;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    r[2 * i] = __uint_as_float(raw[i] << 16);
+    r[2 * i + 1] = __uint_as_float(raw[i] & 0xffff0000u);
+  }
+  return r;
+}
+
+// Orders the instruction stream at this point: nothing is scheduled across it.
+__device__ __forceinline__ void sched_fence() { __builtin_amdgcn_sched_barrier(0); }
+// A use of a wave-uniform value that emits no instruction: makes the compiler place its
+// "scalar loads have landed" wait here rather than at the first arithmetic use.
+__device__ __forceinline__ void touch_uniform(float v) { asm volatile("" ::"s"(v)); }
+__device__ __forceinline__ void touch_uniform(uint32_t v) { asm volatile("" ::"s"(v)); }
+
+// One dword of record `idx` of a row tensor (REC_BYTES per record) through the scalar cache.  Its
+// only purpose is to pull the record's 64-byte line into the scalar cache well before the scan
+// asks for it; the value itself is discarded (pass it to touch_uniform before the next barrier).
+template <int REC_BYTES>
+__device__ __forceinline__ uint32_t ld_touch(const void* p, size_t idx) {
+  return *const_as<uint32_t>(static_cast<const char*>(p) + ((idx * REC_BYTES) & ~(size_t)3));
+}
+
+// Warm the scalar cache with the B_t/C_t lines of the NW state rows starting at record `row`
+// (row stride L records) for one tile of TT timesteps.
+template <int NW, int REC_BYTES, int TT = T>
+struct TileWarm {
+  uint32_t v[2 * NW * (TT / TG)];
+  __device__ __forceinline__ void issue(const void* gB, const void* gC, size_t row, int L) {
+#pragma unroll
+    for (int k = 0; k < NW; ++k)
+#pragma unroll
+      for (int g = 0; g < TT / TG; ++g) {
+        v[(2 * k) * (TT / TG) + g] = ld_touch<REC_BYTES>(gB, row + (size_t)k * L + g * TG);
+        v[(2 * k + 1) * (TT / TG) + g] = ld_touch<REC_BYTES>(gC, row + (size_t)k * L + g * TG);
+      }
+  }
+  __device__ __forceinline__ void retire() {
+#pragma unroll
+    for (int i = 0; i < 2 * NW * (TT / TG); ++i) touch_uniform(v[i]);
+  }
+};
 
 // Sum `v` over the lanes of each aligned group of 32 lanes; result valid in every lane.
 __device__ __forceinline__ float half_wave_sum(float v) {

@@ -99,7 +99,21 @@ __global__ __launch_bounds__(NT) void core_fwd_kernel(const FwdArgs p) {
   };
   load_tile(0);
 
+  // The scan consumes every B_t/C_t line exactly once, so each of its scalar loads would miss
+  // the scalar cache and pay the full memory latency.  Instead the lines of the NEXT tile are
+  // touched here, a whole tile ahead, while the vector ALUs are busy with the staging maths.
+  constexpr bool WARM = NW <= 4;
+  constexpr int RB = (int)sizeof(Tin) * C;
+  const bool full_group = active && n0 + NW <= N;
+  TileWarm<WARM ? NW : 1, RB> warm;
+  if (WARM && full_group && T <= L) {
+    warm.issue(gB, gC, ((size_t)b * N + n0) * L, L);
+    warm.retire();
+  }
+
   for (int l0 = 0; l0 < L; l0 += T) {
+    const bool warm_next = WARM && full_group && l0 + 2 * T <= L;
+    if (warm_next) warm.issue(gB, gC, ((size_t)b * N + n0) * L + l0 + T, L);
     // ---- stage: convert this tile once per (channel, t) and transpose into LDS
     float yin[E], gate[E];
 #pragma unroll
@@ -113,7 +127,7 @@ __global__ __launch_bounds__(NT) void core_fwd_kernel(const FwdArgs p) {
         rec = make_float4(dl, dl * uu, 0.f, 0.f);
       } else {
         float sn, cs;
-        sincosf(rth[k], &sn, &cs);
+        fast_sincosf(rth[k], &sn, &cs);
         if (VAR == VAR_COMPLEX) { const float r = expf(rrho[k]); cs *= r; sn *= r; }
         rec = make_float4(cs, sn, dl * uu, 0.f);
       }
@@ -121,13 +135,115 @@ __global__ __launch_bounds__(NT) void core_fwd_kernel(const FwdArgs p) {
       yin[k] = dsk[k] * uu;
       gate[k] = rz[k];
     }
+    if (warm_next) warm.retire();
     __syncthreads();
     if (l0 + T < L) load_tile(l0 + T);           // next tile's loads fly during the scan
 
     // ---- scan: lane == channel, sequential over the tile's timesteps
     const int tmax = (L - l0 < T) ? (L - l0) : T;
-    if (active) {
-      const size_t brow = ((size_t)b * N + n0) * L + l0;
+    const size_t brow = ((size_t)b * N + n0) * L + l0;
+    // fast path: a full tile and a full group of states.  (bf16 real rows need an even offset
+    // so that the 8-element scalar load is 4-byte aligned.)
+    const bool fast = tmax == T && n0 + NW <= N &&
+                      !(VAR == VAR_REAL && sizeof(Tin) == 2 && (L & 1));
+    if (active && fast) {
+      // The tile is walked in groups of TG timesteps; inside a group the wavefront's states take
+      // turns.  One turn = one state row x TG timesteps: its B_t and C_t values are ONE scalar
+      // load each, issued a full turn ahead so the load latency hides behind the previous turn's
+      // arithmetic.  The (channel, timestep) records of the next group are read from LDS a group
+      // ahead for the same reason.
+      float rx[TG], ry[TG], rz[TG];
+#pragma unroll
+      for (int t = 0; t < TG; ++t) {
+        const float4 v = s_in[t * TS + lane];
+        rx[t] = v.x; ry[t] = v.y; rz[t] = v.z;
+      }
+      if constexpr (VAR == VAR_REAL) {
+        f32x8 bn = ld_r8(gB, brow), cn = ld_r8(gC, brow);
+#pragma unroll
+        for (int g = 0; g < T / TG; ++g) {
+          float yacc[TG], nx[TG], ny[TG];
+#pragma unroll
+          for (int t = 0; t < TG; ++t) yacc[t] = 0.f;
+#pragma unroll
+          for (int k = 0; k < NW; ++k) {
+            const f32x8 bc = bn, cc = cn;
+            touch_uniform(bc[0]);
+            touch_uniform(cc[0]);
+            sched_fence();
+            if (k + 1 < NW) {
+              bn = ld_r8(gB, brow + (size_t)(k + 1) * L + g * TG);
+              cn = ld_r8(gC, brow + (size_t)(k + 1) * L + g * TG);
+            } else if (g + 1 < T / TG) {
+              bn = ld_r8(gB, brow + (g + 1) * TG);
+              cn = ld_r8(gC, brow + (g + 1) * TG);
+            }
+            if (k == 0 && g + 1 < T / TG) {
+#pragma unroll
+              for (int t = 0; t < TG; ++t) {
+                const float4 v = s_in[((g + 1) * TG + t) * TS + lane];
+                nx[t] = v.x; ny[t] = v.y;
+              }
+            }
+            sched_fence();
+#pragma unroll
+            for (int t = 0; t < TG; ++t) {
+              const float a = __builtin_amdgcn_exp2f(rx[t] * a2[k]);
+              hr[k] = fmaf(a, hr[k], bc[t] * ry[t]);
+              yacc[t] = fmaf(cc[t], hr[k], yacc[t]);
+            }
+          }
+#pragma unroll
+          for (int t = 0; t < TG; ++t) {
+            s_part[(wave * T + g * TG + t) * TS + lane] = yacc[t];
+            if (g + 1 < T / TG) { rx[t] = nx[t]; ry[t] = ny[t]; }
+          }
+        }
+      } else {
+        f32x16 bn = ld_c8(gB, brow), cn = ld_c8(gC, brow);
+#pragma unroll
+        for (int g = 0; g < T / TG; ++g) {
+          float yacc[TG], nx[TG], ny[TG], nz[TG];
+#pragma unroll
+          for (int t = 0; t < TG; ++t) yacc[t] = 0.f;
+#pragma unroll
+          for (int k = 0; k < NW; ++k) {
+            const f32x16 bc = bn, cc = cn;
+            touch_uniform(bc[0]);
+            touch_uniform(cc[0]);
+            sched_fence();
+            if (k + 1 < NW) {
+              bn = ld_c8(gB, brow + (size_t)(k + 1) * L + g * TG);
+              cn = ld_c8(gC, brow + (size_t)(k + 1) * L + g * TG);
+            } else if (g + 1 < T / TG) {
+              bn = ld_c8(gB, brow + (g + 1) * TG);
+              cn = ld_c8(gC, brow + (g + 1) * TG);
+            }
+            if (k == 0 && g + 1 < T / TG) {
+#pragma unroll
+              for (int t = 0; t < TG; ++t) {
+                const float4 v = s_in[((g + 1) * TG + t) * TS + lane];
+                nx[t] = v.x; ny[t] = v.y; nz[t] = v.z;
+              }
+            }
+            sched_fence();
+#pragma unroll
+            for (int t = 0; t < TG; ++t) {
+              const float nr = fmaf(rx[t], hr[k], fmaf(-ry[t], hi[k], bc[2 * t] * rz[t]));
+              const float ni = fmaf(rx[t], hi[k], fmaf(ry[t], hr[k], bc[2 * t + 1] * rz[t]));
+              hr[k] = nr; hi[k] = ni;
+              yacc[t] = fmaf(cc[2 * t], nr, yacc[t]);
+              yacc[t] = fmaf(-cc[2 * t + 1], ni, yacc[t]);
+            }
+          }
+#pragma unroll
+          for (int t = 0; t < TG; ++t) {
+            s_part[(wave * T + g * TG + t) * TS + lane] = yacc[t];
+            if (g + 1 < T / TG) { rx[t] = nx[t]; ry[t] = ny[t]; rz[t] = nz[t]; }
+          }
+        }
+      }
+    } else if (active) {
 #pragma unroll 4
       for (int t = 0; t < tmax; ++t) {
         const float4 v = s_in[t * TS + lane];
