@@ -42,31 +42,34 @@ struct UniBwdArgs {
 constexpr int RED_COLS = 4 * TG;        // products per lane per turn: TG x (dB re, dB im) then TG x (dC re, dC im)
 constexpr int RED_RS = RED_COLS + 4;    // padded row stride (floats), keeps rows 16-byte aligned
 
-// Column sums over the 64 lanes of a wavefront.  Each lane passes RED_COLS values; afterwards
-// lane c (< RED_COLS) holds the sum of value c over all lanes.  `red` = this wavefront's scratch.
+// Column sums over the lanes of a wavefront through an LDS transpose, split in two halves so that
+// the LDS latency overlaps the next turn's arithmetic:
+//   issue()   every lane writes its RED_COLS products as a row, then starts reading column
+//             (lane % 32) over the 32 rows of its half of the wavefront;
+//   finish()  adds the 32 values.  Lanes c and c + 32 then hold the two half sums of column c.
 // LDS operations of one wavefront execute in order, so the column reads see the row writes of
-// the other lanes without a wait; the wave barriers only pin the compiler's ordering.
-__device__ __forceinline__ float lane_transpose_sum32(const float (&vals)[RED_COLS], float* red, int lane) {
-  float4* row = reinterpret_cast<float4*>(red + lane * RED_RS);
-#pragma unroll
-  for (int j = 0; j < RED_COLS / 4; ++j)
-    row[j] = make_float4(vals[4 * j], vals[4 * j + 1], vals[4 * j + 2], vals[4 * j + 3]);
-  __builtin_amdgcn_wave_barrier();
-  const int c = lane & (RED_COLS - 1), half = lane >> 5;
-  const float* colp = red + (half * 32) * RED_RS + c;
+// the other lanes, and a later issue() cannot overtake these reads.
+struct LaneTranspose {
   float v[32];
+  __device__ __forceinline__ void issue(const float (&vals)[RED_COLS], float* red, int lane) {
+    float4* row = reinterpret_cast<float4*>(red + lane * RED_RS);
 #pragma unroll
-  for (int i = 0; i < 32; ++i) v[i] = colp[i * RED_RS];
-  sched_fence();                       // all 32 reads in flight before the first add
+    for (int j = 0; j < RED_COLS / 4; ++j)
+      row[j] = make_float4(vals[4 * j], vals[4 * j + 1], vals[4 * j + 2], vals[4 * j + 3]);
+    __builtin_amdgcn_wave_barrier();
+    const float* colp = red + ((lane >> 5) * 32) * RED_RS + (lane & 31);
 #pragma unroll
-  for (int s = 16; s >= 1; s >>= 1)
+    for (int i = 0; i < 32; ++i) v[i] = colp[i * RED_RS];
+    sched_fence();
+  }
+  __device__ __forceinline__ float finish() {
 #pragma unroll
-    for (int i = 0; i < s; ++i) v[i] += v[i + s];
-  float acc = v[0];
-  acc += __shfl_xor(acc, 32, 64);
-  __builtin_amdgcn_wave_barrier();
-  return acc;
-}
+    for (int s = 16; s >= 1; s >>= 1)
+#pragma unroll
+      for (int i = 0; i < s; ++i) v[i] += v[i + s];
+    return v[0];
+  }
+};
 
 // TT: timesteps per staged tile (16 or 32; the checkpoint interval is a multiple of 32 either way).
 template <int NW, int NT, int TT, typename Tin>
@@ -99,6 +102,10 @@ __global__ __launch_bounds__(NT) void unitary_bwd_kernel(const UniBwdArgs p) {
   const Tin* __restrict__ gC = static_cast<const Tin*>(p.Cm);
   float* red = s_red + wave * 64 * RED_RS;
   float2* part = s_part + wave * TT * TS;
+  // lane -> element of the (row, 8 timesteps) output block of a turn: columns 0..15 are dB
+  // (re, im interleaved), 16..31 dC; both halves of the wavefront add their half sum.
+  float* const red_dst = ((lane & 31) < 2 * TG) ? p.dB : p.dC;
+  const int red_off = lane & (2 * TG - 1);
 
   auto load_ck = [&](int kb, float (&xr)[NW], float (&xi)[NW]) {
 #pragma unroll
@@ -128,7 +135,12 @@ __global__ __launch_bounds__(NT) void unitary_bwd_kernel(const UniBwdArgs p) {
 
   // ---- staging-side mapping (lanes run along time)
   const int col = tid % TT, row0 = tid / TT;
-  float ru[E], rdl[E], rth[E], rgy[E], dsk[E], accD[E];
+  // Raw inputs travel through two register sets: `rdy` holds the tile that is staged next and
+  // `fly` the tile after it, whose loads are still in flight.  Loads are issued TWO tiles ahead
+  // and collected one tile later, right after a barrier (see the forward kernel).
+  struct RawTile { Tin u[E], dl[E]; float th[E], gy[E]; };
+  RawTile rdy, fly;
+  float dsk[E], accD[E];
   size_t goff[E];
   bool rowok[E];
 #pragma unroll
@@ -138,22 +150,31 @@ __global__ __launch_bounds__(NT) void unitary_bwd_kernel(const UniBwdArgs p) {
     goff[k] = ((size_t)b * D + (rowok[k] ? dd : 0)) * L;
     dsk[k] = (p.Dskip && rowok[k]) ? p.Dskip[dd] : 0.f;
     accD[k] = 0.f;
+    fly.u[k] = fly.dl[k] = Tin(0);
+    fly.th[k] = fly.gy[k] = 0.f;
   }
-  auto load_tile = [&](int l0) {
+  auto load_tile = [&](RawTile& r, int l0) {
 #pragma unroll
     for (int k = 0; k < E; ++k) {
-      const int ll = l0 + col;
-      const bool ok = rowok[k] && ll < L;
-      const size_t o = goff[k] + (ok ? ll : 0);
-      ru[k] = ok ? to_f32(gu[o]) : 0.f;
-      rdl[k] = ok ? to_f32(gdl[o]) : 0.f;
-      rth[k] = ok ? p.theta[o] : 0.f;
-      rgy[k] = ok ? p.dy[o] : 0.f;
+      // unconditional loads from a clamped address; out-of-range elements are zeroed at staging
+      const int ll = (l0 + col < L) ? l0 + col : L - 1;
+      const size_t o = goff[k] + ll;
+      r.u[k] = gu[o];
+      r.dl[k] = gdl[o];
+      r.th[k] = p.theta[o];
+      r.gy[k] = p.dy[o];
     }
+  };
+  // A use of every register of a set: the compiler puts its wait for the loads here.
+  auto collect_tile = [&](RawTile& r) {
+#pragma unroll
+    for (int k = 0; k < E; ++k) { touch_vgpr(r.u[k]); touch_vgpr(r.dl[k]); touch_vgpr(r.th[k]); touch_vgpr(r.gy[k]); }
   };
 
   const int ntiles = (L + TT - 1) / TT;
-  load_tile((ntiles - 1) * TT);
+  load_tile(rdy, (ntiles - 1) * TT);
+  collect_tile(rdy);
+  if (ntiles > 1) load_tile(fly, (ntiles - 2) * TT);
 
   // scalar-cache warm-up of the B_t/C_t lines, one tile ahead of the scan (see the forward kernel)
   constexpr bool WARM = NW <= 4;
@@ -175,20 +196,25 @@ __global__ __launch_bounds__(NT) void unitary_bwd_kernel(const UniBwdArgs p) {
     float eu[E], edl[E], egy[E];
 #pragma unroll
     for (int k = 0; k < E; ++k) {
+      const bool ok = rowok[k] && l0 + col < L;
+      eu[k] = ok ? to_f32(rdy.u[k]) : 0.f;
+      edl[k] = ok ? to_f32(rdy.dl[k]) : 0.f;
+      egy[k] = ok ? rdy.gy[k] : 0.f;
       float sn, cs;
-      fast_sincosf(rth[k], &sn, &cs);
-      s_in[col * TS + row0 + k * RSTEP] = make_float4(cs, sn, rdl[k] * ru[k], rgy[k]);
-      eu[k] = ru[k]; edl[k] = rdl[k]; egy[k] = rgy[k];
+      fast_sincosf(ok ? rdy.th[k] : 0.f, &sn, &cs);
+      s_in[col * TS + row0 + k * RSTEP] = make_float4(cs, sn, edl[k] * eu[k], egy[k]);
     }
     if (warm_next) warm.retire();
     __syncthreads();
-    if (it > 0) load_tile(l0 - TT);
 
     const size_t brow = row_base + l0;
-    if (full_group && tmax == TT) {
+    const bool fast = full_group && tmax == TT;
+    float rres[NGRP * NW];      // finished dB/dC sums of this tile's turns (fast path)
+    if (fast) {
       // ---- fast path: groups of TG timesteps right to left; inside a group the wavefront's
       // state rows take turns, each turn consuming ONE scalar load of B_t and one of C_t that
-      // was issued a turn earlier.
+      // was issued a turn earlier.  The channel reduction of a turn's dB/dC products is started
+      // at the end of the turn and collected at the end of the NEXT turn.
       float rc[TG], rs[TG], rw[TG], rg[TG];
 #pragma unroll
       for (int t = 0; t < TG; ++t) {
@@ -196,6 +222,7 @@ __global__ __launch_bounds__(NT) void unitary_bwd_kernel(const UniBwdArgs p) {
         rc[t] = v.x; rs[t] = v.y; rw[t] = v.z; rg[t] = v.w;
       }
       f32x16 bn = ld_c8(gB, brow + (TT - TG)), cn = ld_c8(gC, brow + (TT - TG));
+      LaneTranspose xp;
 #pragma unroll
       for (int g = NGRP - 1; g >= 0; --g) {
         float kacc[TG], qacc[TG], nc[TG], ns[TG], nw_[TG], ng[TG];
@@ -245,12 +272,11 @@ __global__ __launch_bounds__(NT) void unitary_bwd_kernel(const UniBwdArgs p) {
             gi[k] = fmaf(cs, gi[k], -sn * gr[k]);
             gr[k] = tg;
           }
-          // lanes 0..15: dB of (row, t0..t0+7) as 16 consecutive floats; lanes 16..31: dC likewise
-          const float tot = lane_transpose_sum32(vals, red, lane);
-          if (lane < RED_COLS) {
-            float* dst = (lane < 2 * TG) ? p.dB : p.dC;
-            atomicAdd(dst + 2 * (brow + (size_t)k * L + g * TG) + (lane & (2 * TG - 1)), tot);
-          }
+          sched_fence();
+          // collect the previous turn's sums (turn (g, k-1), or (g+1, NW-1) across a group)
+          if (k > 0) rres[g * NW + k - 1] = xp.finish();
+          else if (g < NGRP - 1) rres[(g + 1) * NW + NW - 1] = xp.finish();
+          xp.issue(vals, red, lane);
         }
 #pragma unroll
         for (int t = 0; t < TG; ++t) {
@@ -258,6 +284,7 @@ __global__ __launch_bounds__(NT) void unitary_bwd_kernel(const UniBwdArgs p) {
           if (g > 0) { rc[t] = nc[t]; rs[t] = ns[t]; rw[t] = nw_[t]; rg[t] = ng[t]; }
         }
       }
+      rres[NW - 1] = xp.finish();   // the last turn was (g = 0, k = NW-1)
     } else if (active) {
       // ---- general path (ragged tile or partial state group): one timestep at a time
       for (int t = tmax - 1; t >= 0; --t) {
@@ -290,29 +317,58 @@ __global__ __launch_bounds__(NT) void unitary_bwd_kernel(const UniBwdArgs p) {
           const float tg = fmaf(cs, gr[k], sn * gi[k]);
           gi[k] = fmaf(cs, gi[k], -sn * gr[k]);
           gr[k] = tg;
-          const float tot = lane_transpose_sum32(vals, red, lane);
-          if (nok && lane < 4) {
-            float* dst = (lane < 2) ? p.dB : p.dC;
+          LaneTranspose xs;
+          xs.issue(vals, red, lane);
+          const float tot = xs.finish();
+          if (nok && (lane & 31) < 4) {
+            float* dst = ((lane & 31) < 2) ? p.dB : p.dC;
             atomicAdd(dst + 2 * bi + (lane & 1), tot);
           }
         }
         part[t * TS + lane] = make_float2(kacc, qacc);
       }
     }
-    // ---- re-synchronise the regenerated state with the forward pass's checkpoint
-    if (active && l0 > 0 && (l0 % p.ck) == 0) load_ck(l0 / p.ck - 1, hr, hi);
     __syncthreads();
 
+    // ---- the tile's vector-memory traffic, in ONE burst.  Loads, stores and atomics share one
+    // in-order completion counter and the compiler can only wait for "everything": so the wait
+    // comes first, when every outstanding operation is a whole tile old, then the new loads,
+    // then this tile's atomics and stores.
+    // (re-synchronise the regenerated state with the forward pass's checkpoint first, so that
+    // its rare load is part of the same wait)
+    if (active && l0 > 0 && (l0 % p.ck) == 0) {
+      load_ck(l0 / p.ck - 1, hr, hi);
+#pragma unroll
+      for (int k = 0; k < NW; ++k) { touch_vgpr(hr[k]); touch_vgpr(hi[k]); }
+    }
+    if (it > 0) { collect_tile(fly); rdy = fly; }          // tile it-1 has arrived
+    sched_fence();
+    if (it > 1) load_tile(fly, l0 - 2 * TT);               // request tile it-2
+    sched_fence();
+    if (fast) {
+#pragma unroll
+      for (int g = 0; g < NGRP; ++g)
+#pragma unroll
+        for (int k = 0; k < NW; ++k)
+          atomicAdd(red_dst + 2 * (brow + (size_t)k * L + g * TG) + red_off, rres[g * NW + k]);
+    }
+
     // ---- epilogue: channel-wise gradients, coalesced along time
+    // all partial sums are fetched before the first add, so their LDS latencies overlap
+    float2 pv[E][NWV];
+#pragma unroll
+    for (int k = 0; k < E; ++k)
+#pragma unroll
+      for (int w = 0; w < NWV; ++w)
+        pv[k][w] = (w < nwa) ? s_part[(w * TT + col) * TS + row0 + k * RSTEP] : make_float2(0.f, 0.f);
+    sched_fence();
 #pragma unroll
     for (int k = 0; k < E; ++k) {
       const int ll = l0 + col;
+      float kk = 0.f, qq = 0.f;
+#pragma unroll
+      for (int w = 0; w < NWV; ++w) { kk += pv[k][w].x; qq += pv[k][w].y; }
       if (rowok[k] && ll < L) {
-        float kk = 0.f, qq = 0.f;
-        for (int w = 0; w < nwa; ++w) {
-          const float2 pv = s_part[(w * TT + col) * TS + row0 + k * RSTEP];
-          kk += pv.x; qq += pv.y;
-        }
         const size_t o = goff[k] + ll;
         p.du[o] = fmaf(kk, edl[k], dsk[k] * egy[k]);
         p.ddelta[o] = kk * eu[k];

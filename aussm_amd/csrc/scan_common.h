@@ -143,6 +143,12 @@ __device__ __forceinline__ void sched_fence() { __builtin_amdgcn_sched_barrier(0
 // "scalar loads have landed" wait here rather than at the first arithmetic use.
 __device__ __forceinline__ void touch_uniform(float v) { asm volatile("" ::"s"(v)); }
 __device__ __forceinline__ void touch_uniform(uint32_t v) { asm volatile("" ::"s"(v)); }
+// The same for a per-lane value.  Vector loads, stores and atomics share ONE in-order counter on
+// this architecture, and the compiler waits for "everything" whenever control flow hides how many
+// younger stores follow a load.  Touching prefetched values at a point where the count is known
+// (or where nothing younger is in flight) keeps that wait from also draining recent stores.
+__device__ __forceinline__ void touch_vgpr(float v) { asm volatile("" ::"v"(v)); }
+__device__ __forceinline__ void touch_vgpr(bf16_t v) { asm volatile("" ::"v"((uint32_t)v)); }
 
 // One dword of record `idx` of a row tensor (REC_BYTES per record) through the scalar cache.  Its
 // only purpose is to pull the record's 64-byte line into the scalar cache well before the scan

@@ -71,7 +71,13 @@ __global__ __launch_bounds__(NT) void core_fwd_kernel(const FwdArgs p) {
 
   // ---- staging-side mapping (lanes run along time)
   const int col = tid % T, row0 = tid / T;
-  float ru[E], rdl[E], rth[E], rrho[E], rz[E], dsk[E], dbias[E];
+  // Raw inputs travel through two register sets: `rdy` holds the tile that is staged next and
+  // `fly` the tile after it, whose loads are still in flight.  Loads are issued TWO tiles ahead
+  // (the memory latency is longer than one tile's scan) and collected one tile later, right
+  // after a barrier, where the shared load/store counter has nothing recent to drain.
+  struct RawTile { Tin u[E], dl[E]; float th[E], rho[E], z[E]; };
+  RawTile rdy, fly;
+  float dsk[E], dbias[E];
   size_t goff[E];
   bool rowok[E];
 #pragma unroll
@@ -81,23 +87,39 @@ __global__ __launch_bounds__(NT) void core_fwd_kernel(const FwdArgs p) {
     goff[k] = ((size_t)b * D + (rowok[k] ? dd : 0)) * L;
     dsk[k] = (p.Dskip && rowok[k]) ? p.Dskip[dd] : 0.f;
     dbias[k] = (VAR == VAR_REAL && p.delta_bias && rowok[k]) ? p.delta_bias[dd] : 0.f;
-    rth[k] = 0.f; rrho[k] = 0.f; rz[k] = 0.f;
+    rdy.th[k] = rdy.rho[k] = rdy.z[k] = 0.f;
+    fly.th[k] = fly.rho[k] = fly.z[k] = 0.f;
+    fly.u[k] = fly.dl[k] = rdy.u[k] = rdy.dl[k] = Tin(0);
   }
 
-  auto load_tile = [&](int l0) {
+  auto load_tile = [&](RawTile& r, int l0) {
 #pragma unroll
     for (int k = 0; k < E; ++k) {
-      const int ll = l0 + col;
-      const bool ok = rowok[k] && ll < L;
-      const size_t o = goff[k] + (ok ? ll : 0);
-      ru[k] = ok ? to_f32(gu[o]) : 0.f;
-      rdl[k] = ok ? to_f32(gdl[o]) : 0.f;
-      if (VAR != VAR_REAL) rth[k] = ok ? p.theta[o] : 0.f;
-      if (VAR == VAR_COMPLEX) rrho[k] = ok ? p.rho[o] : 0.f;
-      if (p.z) rz[k] = ok ? p.z[o] : 0.f;
+      // Unconditional loads from a clamped (always valid) address: nothing may depend on the
+      // loaded value before it is collected, or the wait for it would move up to here.
+      // Out-of-range elements are zeroed when the tile is staged.
+      const int ll = (l0 + col < L) ? l0 + col : L - 1;
+      const size_t o = goff[k] + ll;
+      r.u[k] = gu[o];
+      r.dl[k] = gdl[o];
+      if (VAR != VAR_REAL) r.th[k] = p.theta[o];
+      if (VAR == VAR_COMPLEX) r.rho[k] = p.rho[o];
+      if (p.z) r.z[k] = p.z[o];
     }
   };
-  load_tile(0);
+  // A use of every register of a set: the compiler puts its wait for the loads here.
+  auto collect_tile = [&](RawTile& r) {
+#pragma unroll
+    for (int k = 0; k < E; ++k) {
+      touch_vgpr(r.u[k]); touch_vgpr(r.dl[k]);
+      if (VAR != VAR_REAL) touch_vgpr(r.th[k]);
+      if (VAR == VAR_COMPLEX) touch_vgpr(r.rho[k]);
+      if (p.z) touch_vgpr(r.z[k]);
+    }
+  };
+  load_tile(rdy, 0);
+  collect_tile(rdy);
+  if (T < L) load_tile(fly, T);
 
   // The scan consumes every B_t/C_t line exactly once, so each of its scalar loads would miss
   // the scalar cache and pay the full memory latency.  Instead the lines of the NEXT tile are
@@ -118,8 +140,9 @@ __global__ __launch_bounds__(NT) void core_fwd_kernel(const FwdArgs p) {
     float yin[E], gate[E];
 #pragma unroll
     for (int k = 0; k < E; ++k) {
-      const float uu = ru[k];
-      float dl = rdl[k];
+      const bool ok = rowok[k] && l0 + col < L;
+      const float uu = ok ? to_f32(rdy.u[k]) : 0.f;
+      float dl = ok ? to_f32(rdy.dl[k]) : 0.f;
       float4 rec;
       if (VAR == VAR_REAL) {
         dl += dbias[k];
@@ -127,17 +150,16 @@ __global__ __launch_bounds__(NT) void core_fwd_kernel(const FwdArgs p) {
         rec = make_float4(dl, dl * uu, 0.f, 0.f);
       } else {
         float sn, cs;
-        fast_sincosf(rth[k], &sn, &cs);
-        if (VAR == VAR_COMPLEX) { const float r = expf(rrho[k]); cs *= r; sn *= r; }
+        fast_sincosf(ok ? rdy.th[k] : 0.f, &sn, &cs);
+        if (VAR == VAR_COMPLEX) { const float r = expf(ok ? rdy.rho[k] : 0.f); cs *= r; sn *= r; }
         rec = make_float4(cs, sn, dl * uu, 0.f);
       }
       s_in[col * TS + row0 + k * RSTEP] = rec;
       yin[k] = dsk[k] * uu;
-      gate[k] = rz[k];
+      gate[k] = rdy.z[k];
     }
     if (warm_next) warm.retire();
     __syncthreads();
-    if (l0 + T < L) load_tile(l0 + T);           // next tile's loads fly during the scan
 
     // ---- scan: lane == channel, sequential over the tile's timesteps
     const int tmax = (L - l0 < T) ? (L - l0) : T;
@@ -272,17 +294,33 @@ __global__ __launch_bounds__(NT) void core_fwd_kernel(const FwdArgs p) {
     }
     __syncthreads();
 
+    // ---- the tile's vector-memory traffic, in ONE burst.  Loads, stores and atomics share one
+    // in-order completion counter and the compiler can only wait for "everything": so the wait
+    // comes first, when every outstanding operation (the loads of tile l0+T and the stores of
+    // the previous tile) is a whole tile old, then the new loads, then this tile's stores.
+    if (l0 + T < L) { collect_tile(fly); rdy = fly; }      // tile l0+T has arrived
+    sched_fence();
+    if (l0 + 2 * T < L) load_tile(fly, l0 + 2 * T);        // request tile l0+2T
+    sched_fence();
+
     // ---- epilogue: add the wavefronts' partial read-outs, skip term and gate; coalesced store
     if (p.y) {
+      // all partial sums are fetched before the first add, so their LDS latencies overlap
+      float pv[E][NWV];
+#pragma unroll
+      for (int k = 0; k < E; ++k)
+#pragma unroll
+        for (int w = 0; w < NWV; ++w)
+          pv[k][w] = (w < nwa) ? s_part[(w * T + col) * TS + row0 + k * RSTEP] : 0.f;
+      sched_fence();
 #pragma unroll
       for (int k = 0; k < E; ++k) {
         const int ll = l0 + col;
-        if (rowok[k] && ll < L) {
-          float acc = yin[k];
-          for (int w = 0; w < nwa; ++w) acc += s_part[(w * T + col) * TS + row0 + k * RSTEP];
-          if (p.z) acc *= siluf_(gate[k]);
-          p.y[goff[k] + ll] = acc;
-        }
+        float acc = yin[k];
+#pragma unroll
+        for (int w = 0; w < NWV; ++w) acc += pv[k][w];
+        if (p.z) acc *= siluf_(gate[k]);
+        if (rowok[k] && ll < L) p.y[goff[k] + ll] = acc;
       }
     }
     // ---- checkpoint at the end of every ck-step block (and at the end of the sequence)
