@@ -29,7 +29,9 @@ _SIGNATURES = {
     "aussm_unitary_fwd": [_P] * 11 + [_I] * 6 + [_P],
     "aussm_unitary_bwd": [_P] * 16 + [_I] * 6 + [_P],
     "aussm_complex_fwd": [_P] * 12 + [_I] * 6 + [_P],
+    "aussm_complex_bwd": [_P] * 19 + [_I] * 6 + [_P],
     "aussm_real_fwd": [_P] * 8 + [_I] + [_P] * 4 + [_I] * 6 + [_P],
+    "aussm_real_bwd": [_P] * 9 + [_I] + [_P] * 9 + [_I] * 6 + [_P],
 }
 
 EXPORTED = tuple(_SIGNATURES) + ("aussm_error_string",)

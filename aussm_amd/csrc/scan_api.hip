@@ -6,6 +6,7 @@
 #include <stdio.h>
 #include <stdlib.h>
 
+#include "scan_bwd_recompute.h"
 #include "scan_bwd_unitary.h"
 #include "scan_common.h"
 #include "scan_fwd.h"
@@ -38,10 +39,15 @@ inline int check_common(int B, int D, int N, int L, int ck, int in_dtype) {
   if (B < 1 || D < 1 || N < 1 || L < 1) return AUSSM_E_SHAPE;
   if (N > AUSSM_MAX_STATE) return AUSSM_E_SHAPE;
   if ((long long)B * ((D + CH - 1) / CH) > 0x7fffffffLL) return AUSSM_E_SHAPE;
-  if (ck < AUSSM_TILE || ck % AUSSM_TILE != 0) return AUSSM_E_CK;
+  if (ck != AUSSM_TILE / 2 && (ck < AUSSM_TILE || ck % AUSSM_TILE != 0)) return AUSSM_E_CK;
   if (in_dtype != AUSSM_F32 && in_dtype != AUSSM_BF16) return AUSSM_E_DTYPE;
   return AUSSM_OK;
 }
+
+// The recomputing backward kernels (complex, real) keep a tile of states in registers: four
+// wavefronts of at most four states each.
+constexpr int REC_MAX_STATE = 16;
+constexpr int REC_CK = AUSSM_TILE / 2;
 
 inline bool misaligned(const void* p, size_t a) { return p && (reinterpret_cast<uintptr_t>(p) % a) != 0; }
 
@@ -90,6 +96,25 @@ int launch_unitary_bwd_t(const UniBwdArgs& a, hipStream_t s) {
   return AUSSM_E_SHAPE;
 }
 
+#define AUSSM_RBWD_CASE(NW_)                                                                         \
+  if (nw == NW_) {                                                                                   \
+    hipLaunchKernelGGL((recompute_bwd_kernel<VAR, NW_, 256, Tin>), grid, dim3(256), 0, s, a);        \
+    return launch_status();                                                                          \
+  }
+
+template <int VAR, typename Tin>
+int launch_rec_bwd_t(const RecBwdArgs& a, hipStream_t s) {
+  const dim3 grid((unsigned)(a.B * a.ncg));
+  const int nw = a.N <= 4 ? 1 : (a.N <= 8 ? 2 : 4);
+  AUSSM_RBWD_CASE(1) AUSSM_RBWD_CASE(2) AUSSM_RBWD_CASE(4)
+  return AUSSM_E_SHAPE;
+}
+
+template <int VAR>
+int launch_rec_bwd(const RecBwdArgs& a, int in_dtype, hipStream_t s) {
+  return in_dtype == AUSSM_BF16 ? launch_rec_bwd_t<VAR, bf16_t>(a, s) : launch_rec_bwd_t<VAR, float>(a, s);
+}
+
 }  // namespace
 
 extern "C" {
@@ -110,7 +135,7 @@ const char* aussm_error_string(int code) {
 
 int aussm_num_checkpoints(int L, int ck) { return (L < 1 || ck < 1) ? 0 : (L + ck - 1) / ck; }
 
-int aussm_bwd_checkpoint_interval(int variant) { return variant == VAR_UNITARY ? 0 : AUSSM_TILE; }
+int aussm_bwd_checkpoint_interval(int variant) { return variant == VAR_UNITARY ? 0 : REC_CK; }
 
 int aussm_unitary_fwd(const void* u, const void* delta, const float* theta, const void* Bc, const void* Cc,
                       const float* Dskip, const float* z, const float* h0, float* y, float* hL, float* hck,
@@ -169,6 +194,45 @@ int aussm_unitary_bwd(const float* dy, const float* dhL, const void* u, const vo
   a.hck = hck; a.du = du; a.ddelta = ddelta; a.dtheta = dtheta; a.dB = dB; a.dC = dC; a.dD = dD; a.dh0 = dh0;
   a.B = B; a.D = D; a.N = N; a.L = L; a.ck = ck; a.nck = (L + ck - 1) / ck; a.ncg = (D + CH - 1) / CH;
   return in_dtype == AUSSM_BF16 ? launch_unitary_bwd_t<bf16_t>(a, s) : launch_unitary_bwd_t<float>(a, s);
+}
+
+int aussm_complex_bwd(const float* dy, const float* dhL, const void* u, const void* delta, const float* rho,
+                      const float* theta, const void* Bc, const void* Cc, const float* Dskip,
+                      const float* h0, const float* hck,
+                      float* du, float* ddelta, float* drho, float* dtheta, float* dB, float* dC,
+                      float* dD, float* dh0,
+                      int B, int D, int N, int L, int ck, int in_dtype, void* stream) {
+  if (int e = check_common(B, D, N, L, ck, in_dtype)) return e;
+  if (ck != REC_CK) return AUSSM_E_CK;
+  if (N > REC_MAX_STATE) return AUSSM_E_SHAPE;
+  if (!dy || !u || !delta || !rho || !theta || !Bc || !Cc || !hck || !du || !ddelta || !drho || !dtheta ||
+      !dB || !dC)
+    return AUSSM_E_NULL;
+  const size_t ca = in_dtype == AUSSM_BF16 ? 4 : 8;
+  if (misaligned(Bc, ca) || misaligned(Cc, ca)) return AUSSM_E_ALIGN;
+  RecBwdArgs a{};
+  a.dy = dy; a.dhL = dhL; a.u = u; a.delta = delta; a.theta = theta; a.rho = rho; a.Bm = Bc; a.Cm = Cc;
+  a.Dskip = Dskip; a.h0 = h0; a.hck = hck;
+  a.du = du; a.ddelta = ddelta; a.dtheta = dtheta; a.drho = drho; a.dB = dB; a.dC = dC; a.dD = dD; a.dh0 = dh0;
+  a.B = B; a.D = D; a.N = N; a.L = L; a.nck = (L + ck - 1) / ck; a.ncg = (D + CH - 1) / CH;
+  return launch_rec_bwd<VAR_COMPLEX>(a, in_dtype, (hipStream_t)stream);
+}
+
+int aussm_real_bwd(const float* dy, const float* dhL, const void* u, const void* delta, const float* A,
+                   const void* Bm, const void* Cm, const float* Dskip, const float* delta_bias,
+                   int delta_softplus, const float* h0, const float* hck,
+                   float* du, float* ddelta, float* dA, float* dB, float* dC, float* dD, float* dh0,
+                   int B, int D, int N, int L, int ck, int in_dtype, void* stream) {
+  if (int e = check_common(B, D, N, L, ck, in_dtype)) return e;
+  if (ck != REC_CK) return AUSSM_E_CK;
+  if (N > REC_MAX_STATE) return AUSSM_E_SHAPE;
+  if (!dy || !u || !delta || !A || !Bm || !Cm || !hck || !du || !ddelta || !dB || !dC) return AUSSM_E_NULL;
+  RecBwdArgs a{};
+  a.dy = dy; a.dhL = dhL; a.u = u; a.delta = delta; a.A = A; a.Bm = Bm; a.Cm = Cm; a.Dskip = Dskip;
+  a.delta_bias = delta_bias; a.delta_softplus = delta_softplus; a.h0 = h0; a.hck = hck;
+  a.du = du; a.ddelta = ddelta; a.dA = dA; a.dB = dB; a.dC = dC; a.dD = dD; a.dh0 = dh0;
+  a.B = B; a.D = D; a.N = N; a.L = L; a.nck = (L + ck - 1) / ck; a.ncg = (D + CH - 1) / CH;
+  return launch_rec_bwd<VAR_REAL>(a, in_dtype, (hipStream_t)stream);
 }
 
 }  // extern "C"

@@ -168,6 +168,9 @@ __global__ __launch_bounds__(NT) void core_fwd_kernel(const FwdArgs p) {
     // so that the 8-element scalar load is 4-byte aligned.)
     const bool fast = tmax == T && n0 + NW <= N &&
                       !(VAR == VAR_REAL && sizeof(Tin) == 2 && (L & 1));
+    float mr[NW], mi[NW];                        // state after the first half of the tile
+#pragma unroll
+    for (int k = 0; k < NW; ++k) { mr[k] = 0.f; mi[k] = 0.f; }
     if (active && fast) {
       // The tile is walked in groups of TG timesteps; inside a group the wavefront's states take
       // turns.  One turn = one state row x TG timesteps: its B_t and C_t values are ONE scalar
@@ -220,6 +223,10 @@ __global__ __launch_bounds__(NT) void core_fwd_kernel(const FwdArgs p) {
             s_part[(wave * T + g * TG + t) * TS + lane] = yacc[t];
             if (g + 1 < T / TG) { rx[t] = nx[t]; ry[t] = ny[t]; }
           }
+          if (g == T / 2 / TG - 1) {
+#pragma unroll
+            for (int k = 0; k < NW; ++k) mr[k] = hr[k];
+          }
         }
       } else {
         f32x16 bn = ld_c8(gB, brow), cn = ld_c8(gC, brow);
@@ -263,6 +270,10 @@ __global__ __launch_bounds__(NT) void core_fwd_kernel(const FwdArgs p) {
             s_part[(wave * T + g * TG + t) * TS + lane] = yacc[t];
             if (g + 1 < T / TG) { rx[t] = nx[t]; ry[t] = ny[t]; rz[t] = nz[t]; }
           }
+          if (g == T / 2 / TG - 1) {
+#pragma unroll
+            for (int k = 0; k < NW; ++k) { mr[k] = hr[k]; mi[k] = hi[k]; }
+          }
         }
       }
     } else if (active) {
@@ -290,6 +301,10 @@ __global__ __launch_bounds__(NT) void core_fwd_kernel(const FwdArgs p) {
           }
         }
         s_part[(wave * T + t) * TS + lane] = yacc;
+        if (t == T / 2 - 1) {
+#pragma unroll
+          for (int k = 0; k < NW; ++k) { mr[k] = hr[k]; mi[k] = hi[k]; }
+        }
       }
     }
     __syncthreads();
@@ -323,17 +338,26 @@ __global__ __launch_bounds__(NT) void core_fwd_kernel(const FwdArgs p) {
         if (rowok[k] && ll < L) p.y[goff[k] + ll] = acc;
       }
     }
-    // ---- checkpoint at the end of every ck-step block (and at the end of the sequence)
-    if (p.hck && active && dok && (((l0 + T) % p.ck) == 0 || l0 + T >= L)) {
-      const int kb = l0 / p.ck;
+    // ---- checkpoint at the end of every ck-step block (and at the end of the sequence).
+    // ck is a multiple of the tile, or half a tile (then the mid-tile state saved by the scan
+    // is written as well).
+    if (p.hck && active && dok) {
+      auto put = [&](int kb, const float (&xr)[NW], const float (&xi)[NW]) {
 #pragma unroll
-      for (int k = 0; k < NW; ++k) {
-        const int n = n0 + k;
-        if (n < N) {
-          const size_t o = ((((size_t)b * p.nck + kb) * N + n) * C) * D + d;
-          p.hck[o] = hr[k];
-          if (C == 2) p.hck[o + D] = hi[k];
+        for (int k = 0; k < NW; ++k) {
+          const int n = n0 + k;
+          if (n < N) {
+            const size_t o = ((((size_t)b * p.nck + kb) * N + n) * C) * D + d;
+            p.hck[o] = xr[k];
+            if (C == 2) p.hck[o + D] = xi[k];
+          }
         }
+      };
+      if (p.ck == T / 2) {
+        if (tmax > T / 2) put(l0 / (T / 2), mr, mi);
+        put((l0 + tmax - 1) / (T / 2), hr, hi);
+      } else if (((l0 + T) % p.ck) == 0 || l0 + T >= L) {
+        put(l0 / p.ck, hr, hi);
       }
     }
     // No third barrier: the next stage only writes s_in (all scan reads of it are behind the

@@ -184,3 +184,197 @@ def unitary_scan(u: Tensor, delta: Tensor, theta: Tensor, Bc: Tensor, Cc: Tensor
     if return_last_state:
         return y, torch.view_as_complex(hL)
     return y
+
+
+# --------------------------------------------------------------------------------------------
+# complex scan
+# --------------------------------------------------------------------------------------------
+
+REC_CK = 16          # checkpoint interval the recomputing backward kernels (complex, real) need
+REC_MAX_STATE = 16   # largest state size those kernels take
+
+
+def complex_fwd_raw(u, delta, rho, theta, Bri, Cri, D=None, z=None, h0=None, want_state=False, ck=0):
+    lib = _lib.load()
+    b, d, l = u.shape
+    n = Bri.shape[1]
+    y = torch.empty((b, d, l), device=u.device, dtype=torch.float32)
+    hL = torch.empty((b, d, n, 2), device=u.device, dtype=torch.float32) if want_state else None
+    hck = torch.empty((b, num_checkpoints(l, ck), n, 2, d), device=u.device, dtype=torch.float32) if ck else None
+    check(lib.aussm_complex_fwd(ptr(u), ptr(delta), ptr(rho), ptr(theta), ptr(Bri), ptr(Cri), ptr(D), ptr(z),
+                                ptr(h0), ptr(y), ptr(hL), ptr(hck), b, d, n, l, ck or _lib.TILE, _in_dtype(u),
+                                _stream()), "aussm_complex_fwd")
+    return y, hL, hck
+
+
+def complex_bwd_raw(dy, dhL, u, delta, rho, theta, Bri, Cri, D, h0, hck, want_dD=True, want_dh0=False):
+    lib = _lib.load()
+    b, d, l = u.shape
+    n = Bri.shape[1]
+    f32 = dict(device=u.device, dtype=torch.float32)
+    du, ddelta, drho, dtheta = (torch.empty((b, d, l), **f32) for _ in range(4))
+    dB = torch.zeros((b, n, l, 2), **f32)
+    dC = torch.zeros((b, n, l, 2), **f32)
+    dD = torch.zeros((d,), **f32) if (want_dD and D is not None) else None
+    dh0 = torch.empty((b, d, n, 2), **f32) if want_dh0 else None
+    check(lib.aussm_complex_bwd(ptr(dy), ptr(dhL), ptr(u), ptr(delta), ptr(rho), ptr(theta), ptr(Bri), ptr(Cri),
+                                ptr(D), ptr(h0), ptr(hck), ptr(du), ptr(ddelta), ptr(drho), ptr(dtheta), ptr(dB),
+                                ptr(dC), ptr(dD), ptr(dh0), b, d, n, l, REC_CK, _in_dtype(u), _stream()),
+          "aussm_complex_bwd")
+    return du, ddelta, drho, dtheta, dB, dC, dD, dh0
+
+
+class _ComplexScanFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, u, delta, rho, theta, Bri, Cri, D, h0):
+        y, hL, hck = complex_fwd_raw(u, delta, rho, theta, Bri, Cri, D, None, h0, want_state=True, ck=REC_CK)
+        ctx.save_for_backward(u, delta, rho, theta, Bri, Cri, D, h0, hck)
+        return y, hL
+
+    @staticmethod
+    def backward(ctx, dy, dhL):
+        u, delta, rho, theta, Bri, Cri, D, h0, hck = ctx.saved_tensors
+        dhL = None if dhL is None else dhL.contiguous()
+        du, ddelta, drho, dtheta, dB, dC, dD, dh0 = complex_bwd_raw(
+            dy.contiguous(), dhL, u, delta, rho, theta, Bri, Cri, D, h0, hck,
+            want_dD=D is not None and ctx.needs_input_grad[6], want_dh0=h0 is not None and ctx.needs_input_grad[7])
+        return (du.to(u.dtype), ddelta.to(delta.dtype), drho, dtheta, dB.to(Bri.dtype), dC.to(Cri.dtype), dD, dh0)
+
+
+def complex_scan(u: Tensor, delta: Tensor, rho: Tensor, theta: Tensor, Bc: Tensor, Cc: Tensor,
+                 D: Optional[Tensor] = None, z: Optional[Tensor] = None, h0: Optional[Tensor] = None,
+                 return_last_state: bool = False):
+    """Complex scan, a_l = exp(rho_l + i theta_l).  Shapes as unitary_scan plus rho (b, d, l)."""
+    b, d, l = _check_bdl(u, delta)
+    u = u.contiguous()
+    delta = delta.contiguous()
+    rho = _f32(rho, "rho", (b, d, l))
+    theta = _f32(theta, "theta", (b, d, l))
+    Bri = _complex_as_real(Bc, "B", b, l, u.dtype)
+    Cri = _complex_as_real(Cc, "C", b, l, u.dtype)
+    n = Bri.shape[1]
+    if Cri.shape[1] != n:
+        raise RuntimeError("B and C must have the same state size")
+    D = _f32(D, "D", (d,))
+    z = _f32(z, "z", (b, d, l))
+    h0r = None
+    if h0 is not None:
+        if h0.dtype != torch.complex64 or tuple(h0.shape) != (b, d, n):
+            raise RuntimeError(f"expected h0 complex64 of shape {(b, d, n)}")
+        h0r = torch.view_as_real(h0).contiguous()
+    needs_grad = torch.is_grad_enabled() and any(
+        t is not None and t.requires_grad for t in (u, delta, rho, theta, Bri, Cri, D, z, h0r))
+    if needs_grad:
+        if n > REC_MAX_STATE:
+            raise RuntimeError(f"the complex backward pass supports at most {REC_MAX_STATE} states per channel")
+        y, hL = _ComplexScanFn.apply(u, delta, rho, theta, Bri, Cri, D, h0r)
+        if z is not None:
+            y = y * F.silu(z)
+    else:
+        y, hL, _ = complex_fwd_raw(u, delta, rho, theta, Bri, Cri, D, z, h0r, want_state=return_last_state)
+    if return_last_state:
+        return y, torch.view_as_complex(hL)
+    return y
+
+
+# --------------------------------------------------------------------------------------------
+# real (Mamba S6) selective scan
+# --------------------------------------------------------------------------------------------
+
+def real_fwd_raw(u, delta, A, Bm, Cm, D=None, z=None, delta_bias=None, delta_softplus=False, h0=None,
+                 want_state=False, ck=0):
+    lib = _lib.load()
+    b, d, l = u.shape
+    n = A.shape[1]
+    y = torch.empty((b, d, l), device=u.device, dtype=torch.float32)
+    hL = torch.empty((b, d, n), device=u.device, dtype=torch.float32) if want_state else None
+    hck = torch.empty((b, num_checkpoints(l, ck), n, 1, d), device=u.device, dtype=torch.float32) if ck else None
+    check(lib.aussm_real_fwd(ptr(u), ptr(delta), ptr(A), ptr(Bm), ptr(Cm), ptr(D), ptr(z), ptr(delta_bias),
+                             int(bool(delta_softplus)), ptr(h0), ptr(y), ptr(hL), ptr(hck), b, d, n, l,
+                             ck or _lib.TILE, _in_dtype(u), _stream()), "aussm_real_fwd")
+    return y, hL, hck
+
+
+def real_bwd_raw(dy, dhL, u, delta, A, Bm, Cm, D, delta_bias, delta_softplus, h0, hck, want_dD=True,
+                 want_dh0=False):
+    lib = _lib.load()
+    b, d, l = u.shape
+    n = A.shape[1]
+    f32 = dict(device=u.device, dtype=torch.float32)
+    du, ddelta = torch.empty((b, d, l), **f32), torch.empty((b, d, l), **f32)
+    dA = torch.zeros((d, n), **f32)
+    dB = torch.zeros((b, n, l), **f32)
+    dC = torch.zeros((b, n, l), **f32)
+    dD = torch.zeros((d,), **f32) if (want_dD and D is not None) else None
+    dh0 = torch.empty((b, d, n), **f32) if want_dh0 else None
+    check(lib.aussm_real_bwd(ptr(dy), ptr(dhL), ptr(u), ptr(delta), ptr(A), ptr(Bm), ptr(Cm), ptr(D),
+                             ptr(delta_bias), int(bool(delta_softplus)), ptr(h0), ptr(hck), ptr(du), ptr(ddelta),
+                             ptr(dA), ptr(dB), ptr(dC), ptr(dD), ptr(dh0), b, d, n, l, REC_CK, _in_dtype(u),
+                             _stream()), "aussm_real_bwd")
+    return du, ddelta, dA, dB, dC, dD, dh0
+
+
+class _RealScanFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, u, delta, A, Bm, Cm, D, delta_bias, h0, delta_softplus):
+        y, hL, hck = real_fwd_raw(u, delta, A, Bm, Cm, D, None, delta_bias, delta_softplus, h0,
+                                  want_state=True, ck=REC_CK)
+        ctx.save_for_backward(u, delta, A, Bm, Cm, D, delta_bias, h0, hck)
+        ctx.delta_softplus = delta_softplus
+        return y, hL
+
+    @staticmethod
+    def backward(ctx, dy, dhL):
+        u, delta, A, Bm, Cm, D, delta_bias, h0, hck = ctx.saved_tensors
+        dhL = None if dhL is None else dhL.contiguous()
+        du, ddelta, dA, dB, dC, dD, dh0 = real_bwd_raw(
+            dy.contiguous(), dhL, u, delta, A, Bm, Cm, D, delta_bias, ctx.delta_softplus, h0, hck,
+            want_dD=D is not None and ctx.needs_input_grad[5], want_dh0=h0 is not None and ctx.needs_input_grad[7])
+        dbias = ddelta.sum(dim=(0, 2)) if (delta_bias is not None and ctx.needs_input_grad[6]) else None
+        return (du.to(u.dtype), ddelta.to(delta.dtype), dA, dB.to(Bm.dtype), dC.to(Cm.dtype), dD, dbias, dh0, None)
+
+
+def selective_scan_fn(u: Tensor, delta: Tensor, A: Tensor, B: Tensor, C: Tensor, D: Optional[Tensor] = None,
+                      z: Optional[Tensor] = None, delta_bias: Optional[Tensor] = None,
+                      delta_softplus: bool = False, return_last_state: bool = False,
+                      h0: Optional[Tensor] = None):
+    """Mamba S6 selective scan with the argument names and meaning of the reference's call
+    (ai-modules/wavesAI/model/aussm.py:791-802):
+
+        u, delta, z: (b, d, l); A: (d, n) float32; B, C: (b, n, l); D, delta_bias: (d,) float32.
+        delta <- softplus(delta + delta_bias) if delta_softplus (bias alone if not);
+        h_l = exp(delta_l A) h_{l-1} + delta_l B_l u_l;  y_l = C_l . h_l + D u_l;  y *= silu(z).
+
+    Returns y (b, d, l) float32, plus the last state (b, d, n) if return_last_state.
+    `h0` (b, d, n), a start state, is an extension over the reference's signature."""
+    b, d, l = _check_bdl(u, delta)
+    u = u.contiguous()
+    delta = delta.contiguous()
+    A = _f32(A, "A")
+    if A.dim() != 2 or A.shape[0] != d:
+        raise RuntimeError(f"expected A of shape (d, n) with d = {d}, got {tuple(A.shape)}")
+    n = A.shape[1]
+    for name, t in (("B", B), ("C", C)):
+        if tuple(t.shape) != (b, n, l):
+            raise RuntimeError(f"expected {name} of shape {(b, n, l)}, got {tuple(t.shape)}")
+        if t.dtype != u.dtype:
+            raise RuntimeError(f"{name} must have the dtype of u ({u.dtype}), got {t.dtype}")
+    Bm, Cm = B.contiguous(), C.contiguous()
+    D = _f32(D, "D", (d,))
+    z = _f32(z, "z", (b, d, l))
+    delta_bias = _f32(delta_bias, "delta_bias", (d,))
+    h0 = _f32(h0, "h0", (b, d, n))
+    needs_grad = torch.is_grad_enabled() and any(
+        t is not None and t.requires_grad for t in (u, delta, A, Bm, Cm, D, z, delta_bias, h0))
+    if needs_grad:
+        if n > REC_MAX_STATE:
+            raise RuntimeError(f"the S6 backward pass supports at most {REC_MAX_STATE} states per channel")
+        y, hL = _RealScanFn.apply(u, delta, A, Bm, Cm, D, delta_bias, h0, bool(delta_softplus))
+        if z is not None:
+            y = y * F.silu(z)
+    else:
+        y, hL, _ = real_fwd_raw(u, delta, A, Bm, Cm, D, z, delta_bias, delta_softplus, h0,
+                                want_state=return_last_state)
+    if return_last_state:
+        return y, hL
+    return y
