@@ -1,0 +1,262 @@
+"""The callers of the scan operators: counterparts of the reference's blocks in
+ai-modules/wavesAI/model/aussm.py, with the scans running on the HIP kernels.
+
+    ModelArgsSSMau (:35-62)   ModelArgsMamba (:64-91)   ModelBlockArgs (:94-97)
+    SSMauBlock (:808-902)     MambaBlock (:717-805)     ResidualBlock (:681-714)
+    RMSNorm (:905-916)        SSMTS (:100-227)
+
+The modules keep the reference's parameter names, shapes, creation order and initialisers, so a
+given torch.manual_seed produces the same initial weights and a reference state_dict loads
+unchanged.  Behaviour kept on purpose: the dt_proj bias is added twice in SSMauBlock (:878-880)
+and is passed again as delta_bias in MambaBlock (:789-802); the xA_proj weight is reshaped
+"(n d1) d -> d1 n d" and scaled by 1/sqrt(d_model) (:882-891); conv1d output is trimmed to the
+input length (:863).
+
+Every block takes an optional `scan_impl` callable.  The default is the HIP operator; tests
+pass a CPU implementation with the same signature to check the plumbing around the scan.
+"""
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass
+from typing import Callable, List, Optional, Union
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from . import ops, scan
+
+
+@dataclass
+class ModelArgsSSMau:
+    d_model: int
+    d_state: int
+    dt_rank: Union[int, str] = "auto"
+    d_conv: int = 4
+    conv_bias: bool = True
+    bias: bool = False
+    verbose: bool = False
+    conv_1d: bool = True
+    cuda: bool = True
+
+    def __post_init__(self):
+        self.block = SSMauBlock
+        if self.dt_rank == "auto":
+            self.dt_rank = self.d_state
+
+
+@dataclass
+class ModelArgsMamba:
+    d_model: int
+    d_state: int = 16
+    expand: int = 2
+    dt_rank: Union[int, str] = "auto"
+    d_conv: int = 4
+    conv_bias: bool = True
+    bias: bool = False
+    verbose: bool = False
+
+    def __post_init__(self):
+        self.block = MambaBlock
+        self.d_inner = int(self.expand * self.d_model)
+        if self.dt_rank == "auto":
+            self.dt_rank = math.ceil(self.d_model / 16)
+
+
+@dataclass
+class ModelBlockArgs:
+    layers: List[Union[ModelArgsSSMau, ModelArgsMamba]]
+    d_model: int
+
+
+class RMSNorm(nn.Module):
+    def __init__(self, d_model: int, eps: float = 1e-5):
+        super().__init__()
+        self.eps = eps
+        self.weight = nn.Parameter(torch.ones(d_model))
+
+    def forward(self, x):
+        return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + self.eps) * self.weight
+
+
+class MambaBlock(nn.Module):
+    """A Mamba (S6) block; the scan is selective_scan_fn on the HIP real-scan kernels."""
+
+    def __init__(self, args: ModelArgsMamba, scan_impl: Optional[Callable] = None):
+        super().__init__()
+        self.args = args
+        self.in_proj = nn.Linear(args.d_model, args.d_inner * 2, bias=args.bias)
+        self.conv1d = nn.Conv1d(in_channels=args.d_inner, out_channels=args.d_inner, bias=args.conv_bias,
+                                kernel_size=args.d_conv, groups=args.d_inner, padding=args.d_conv - 1)
+        self.out_proj = nn.Linear(args.d_inner, args.d_model, bias=args.bias)
+        self.x_proj = nn.Linear(args.d_inner, args.dt_rank + args.d_state * 2, bias=False)
+        self.dt_proj = nn.Linear(args.dt_rank, args.d_inner, bias=True)
+        self.D = nn.Parameter(torch.ones(args.d_inner))
+        A = torch.arange(1, args.d_state + 1, dtype=torch.float32).repeat(args.d_inner, 1)
+        self.A_log = nn.Parameter(torch.log(A))
+        self.A_log._no_weight_decay = True
+        self.scan_impl = scan_impl or scan.selective_scan_fn
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        (b, l, d) = x.shape
+        x_and_z = self.in_proj(x)
+        (x, z) = x_and_z.split(split_size=[self.args.d_inner, self.args.d_inner], dim=-1)
+        x = self.conv1d(x.transpose(1, 2))[:, :, :l].transpose(1, 2)
+        y = self.ssm_mamba(x, z)
+        return self.out_proj(y)
+
+    def ssm_mamba(self, x, z):
+        (b, l, d_in) = x.shape
+        x_proj = self.x_proj(x)
+        dt, B, C = x_proj.split([self.args.dt_rank, self.args.d_state, self.args.d_state], dim=-1)
+        dt = self.dt_proj(dt)
+        x = F.silu(x)
+        A = -torch.exp(self.A_log.float())
+        y = self.scan_impl(
+            x.transpose(1, 2).contiguous(),
+            dt.transpose(1, 2).contiguous(),
+            A.contiguous(),
+            B.transpose(1, 2).contiguous(),
+            C.transpose(1, 2).contiguous(),
+            self.D.float().contiguous(),
+            z=z.transpose(1, 2).contiguous(),
+            delta_bias=self.dt_proj.bias.float(),
+            delta_softplus=True,
+            return_last_state=False,
+        )
+        return y.transpose(1, 2)
+
+
+class SSMauBlock(nn.Module):
+    """A single AUSSM block; the scan is ssm_adaptive_interface on the HIP unitary-scan kernels."""
+
+    def __init__(self, args: ModelArgsSSMau, scan_impl: Optional[Callable] = None):
+        super().__init__()
+        self.args = args
+        self.in_proj = nn.Linear(args.d_model, args.d_model * 2, bias=args.bias)
+        self.conv1d = nn.Conv1d(in_channels=args.d_model, out_channels=args.d_model, bias=args.conv_bias,
+                                kernel_size=args.d_conv, groups=args.d_model, padding=args.d_conv - 1)
+        self.out_proj = nn.Linear(args.d_model, args.d_model, bias=args.bias)
+        self.x_proj = nn.Linear(args.d_model, args.dt_rank, bias=False)
+        self.dt_proj = nn.Linear(args.dt_rank, args.d_model, bias=True)
+        self.D = nn.Parameter(torch.ones(args.d_model))
+        self.C = nn.Parameter(torch.randn(args.d_state, dtype=torch.complex64), requires_grad=True)
+        self.B = nn.Parameter(torch.randn(args.d_state, dtype=torch.complex64), requires_grad=True)
+        self.xA_proj = nn.Linear(args.d_model, args.d_model * args.d_state, bias=True)
+        self.xA_proj.bias.data.uniform_(-torch.pi, torch.pi)
+        if scan_impl is not None:
+            self.optimized_SSMa_function = scan_impl
+        elif args.cuda:
+            self.optimized_SSMa_function = lambda **kw: ops.ssm_adaptive_interface(**kw, unitary=True)
+        else:
+            raise NotImplementedError(
+                "cuda=False selects the reference's pure-PyTorch scan, which this package does not ship; "
+                "pass scan_impl=... to use another implementation")
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        (b, l, d) = x.shape
+        x_and_z = self.in_proj(x)
+        (x, z) = x_and_z.split(split_size=[self.args.d_model, self.args.d_model], dim=-1)
+        if self.args.conv_1d:
+            x = self.conv1d(x.transpose(1, 2))[:, :, :l].transpose(1, 2)
+        y = self.ssm_au(x, z)
+        return self.out_proj(y)
+
+    def ssm_au(self, x, z):
+        b, l, d_in = x.shape
+        n = self.args.d_state
+        dt = self.dt_proj(self.x_proj(x))
+        dt = dt + self.dt_proj.bias.float()
+        dt = F.softplus(dt)
+        # "(n dstate1) dstate -> dstate1 n dstate"
+        x_param = self.xA_proj.weight.view(n, d_in, d_in).permute(1, 0, 2)
+        x_bias = self.xA_proj.bias.view(n, d_in).t()
+        self.ssm_args = {
+            "u": x.transpose(1, 2).contiguous(),
+            "dt": dt.transpose(1, 2).contiguous(),
+            "x": x_param.contiguous() * (1 / math.sqrt(self.args.d_model)),
+            "x_bias": x_bias.contiguous(),
+            "B": self.B.contiguous(),
+            "C": self.C.contiguous(),
+            "D": self.D.float().contiguous(),
+            "z": z.transpose(1, 2).contiguous(),
+        }
+        y = self.optimized_SSMa_function(**self.ssm_args)
+        return y.transpose(1, 2)
+
+
+class ResidualBlock(nn.Module):
+    """Norm -> mixer -> add."""
+
+    def __init__(self, args: Union[ModelArgsSSMau, ModelArgsMamba], scan_impl: Optional[Callable] = None):
+        super().__init__()
+        self.args = args
+        self.mixer = args.block(args, scan_impl=scan_impl)
+        self.norm = RMSNorm(args.d_model)
+
+    def forward(self, x):
+        return self.mixer(self.norm(x)) + x
+
+
+class SSMTS(nn.Module):
+    """Time-series model: Linear embedding -> residual AUSSM ('a') / Mamba ('m') blocks given by a
+    layer string such as "a|m|a|m" -> RMSNorm -> Linear read-out."""
+
+    def __init__(self, d_model: int, input_dim: int, output_dim: int, layers: Optional[str] = None,
+                 d_state: int = 16, mamba_expand: int = 2, dt_rank: Union[int, str] = "auto", d_conv: int = 4,
+                 conv_bias: bool = True, bias: bool = False, ssmau_cuda: bool = True, ssmau_conv_1d: bool = True,
+                 embedding_decay: bool = True, verbose: bool = False,
+                 ssmau_scan_impl: Optional[Callable] = None, mamba_scan_impl: Optional[Callable] = None):
+        super().__init__()
+        if layers is None:
+            layers = "m|a"
+        self.n_layers = len(layers.split("|"))
+        self.output_dim = output_dim
+        self.d_model = d_model
+        self.d_state = d_state
+        self.dt_rank = dt_rank
+        self.d_conv = d_conv
+        self.input_dim = input_dim
+        self.mamba_expand = mamba_expand
+        self.conv_bias = conv_bias
+        self.verbose = verbose
+        self.bias = bias
+        self.ssmau_conv_1d = ssmau_conv_1d
+        self.embedding_decay = embedding_decay
+        self.ssmau_cuda = ssmau_cuda
+
+        self.args = ModelBlockArgs(self.parse_layer_string(layers), self.d_model)
+        self.embedding = nn.Linear(self.input_dim, self.d_model)
+        self.layers = nn.ModuleList([
+            ResidualBlock(a, scan_impl=ssmau_scan_impl if isinstance(a, ModelArgsSSMau) else mamba_scan_impl)
+            for a in self.args.layers])
+        self.norm_f = RMSNorm(self.d_model)
+        self.output = nn.Linear(self.d_model, self.output_dim, bias=False)
+
+    def parse_layer_string(self, layer_string: str):
+        layer_args = []
+        for layer in layer_string.replace(" ", "").split("|"):
+            if layer == "a":
+                layer_args.append(ModelArgsSSMau(self.d_model, self.d_state, self.dt_rank, self.d_conv,
+                                                 self.conv_bias, self.bias, self.verbose,
+                                                 conv_1d=self.ssmau_conv_1d, cuda=self.ssmau_cuda))
+            elif layer == "m":
+                layer_args.append(ModelArgsMamba(self.d_model, self.d_state, self.mamba_expand, self.dt_rank,
+                                                 self.d_conv, self.conv_bias, self.bias, self.verbose))
+            else:
+                raise NotImplementedError(f"Layer type \"{layer}\" not recognized")
+        return layer_args
+
+    def get_parameter_groups_for_optimizer(self):
+        emb = {"params": self.embedding.parameters()}
+        if self.embedding_decay:
+            emb["weight_decay"] = 0.0
+        return [emb, {"params": self.layers.parameters()}, {"params": self.norm_f.parameters()},
+                {"params": self.output.parameters()}]
+
+    def forward(self, input_ids, **kwargs):
+        x = self.embedding(input_ids)
+        for layer in self.layers:
+            x = layer(x)
+        return self.output(self.norm_f(x))
