@@ -1,0 +1,74 @@
+"""The C-ABI library: it loads without a GPU and exports every symbol include/aussm_hip.h declares;
+argument checks that need no device run here too (they return before any launch)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "aussm_hip.h")
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(aussm_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_entry_points():
+    names = declared_symbols()
+    for must in ("aussm_unitary_fwd", "aussm_unitary_bwd", "aussm_complex_fwd", "aussm_complex_bwd",
+                 "aussm_real_fwd", "aussm_real_bwd", "aussm_version", "aussm_error_string"):
+        assert must in names
+
+
+def test_library_exports_every_declared_symbol():
+    from aussm_amd import _lib
+    if not os.path.exists(_lib.LIB_PATH):
+        pytest.skip("library not built (python -m aussm_amd.build)")
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    for name in declared_symbols():
+        assert hasattr(lib, name), f"{name} is declared in the header but not exported"
+    for name in _lib.EXPORTED:
+        assert name in declared_symbols(), f"{name} is bound in Python but not declared in the header"
+
+
+def test_argument_checks_without_a_device():
+    from aussm_amd import _lib
+    if not os.path.exists(_lib.LIB_PATH):
+        pytest.skip("library not built")
+    lib = _lib.load()
+    assert lib.aussm_version() >= 100
+    assert lib.aussm_num_checkpoints(2048, 256) == 8 and lib.aussm_num_checkpoints(33, 32) == 2
+    assert lib.aussm_bwd_checkpoint_interval(0) == 0 and lib.aussm_bwd_checkpoint_interval(2) == 16
+    one = ctypes.c_void_p(256)      # never dereferenced: every call below is rejected before launch
+    null = None
+    # NULL required pointer
+    rc = lib.aussm_unitary_fwd(null, one, one, one, one, null, null, null, one, null, null, 1, 1, 1, 32, 32, 0, null)
+    assert rc == -1 and b"NULL" in lib.aussm_error_string(rc)
+    # state size out of range
+    rc = lib.aussm_unitary_fwd(one, one, one, one, one, null, null, null, one, null, null, 1, 1, 65, 32, 32, 0, null)
+    assert rc == -2
+    # checkpoint interval not a multiple of the tile
+    rc = lib.aussm_unitary_fwd(one, one, one, one, one, null, null, null, one, null, null, 1, 1, 1, 32, 48, 0, null)
+    assert rc == -3
+    # unknown dtype
+    rc = lib.aussm_unitary_fwd(one, one, one, one, one, null, null, null, one, null, null, 1, 1, 1, 32, 32, 7, null)
+    assert rc == -4
+    # misaligned complex tensor
+    rc = lib.aussm_unitary_fwd(one, one, one, ctypes.c_void_p(260), one, null, null, null, one, null, null,
+                               1, 1, 1, 32, 32, 0, null)
+    assert rc == -5
+    # the recomputing backward kernels insist on their checkpoint interval and state limit
+    args = [one] * 9 + [0] + [one] * 9
+    assert lib.aussm_real_bwd(*args, 1, 1, 1, 32, 32, 0, null) == -3
+    assert lib.aussm_real_bwd(*args, 1, 1, 17, 32, 16, 0, null) == -2
+
+
+def test_python_layer_fails_loudly_without_library(monkeypatch, tmp_path):
+    from aussm_amd import _lib
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "missing.so"))
+    with pytest.raises(_lib.AussmError):
+        _lib.load()

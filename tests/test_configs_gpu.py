@@ -1,0 +1,174 @@
+"""The benchmark configurations and bfloat16 inputs.
+
+Configuration 1 (forward, B=16 D=128 N=16 L=1024) and the long-sequence configuration 2
+(B=4 D=256 N=16 L=16384) are compared with the oracle directly where it finishes in seconds;
+gradients at L=16384 are compared on a slice of the channels, and the full sizes are covered by
+size-independent properties: splitting the sequence with a carried state, linearity in the
+input, independence of batch elements, and the adjoint identity <dy, J v> = <J^T dy, v>.
+float32 tolerance: atol = rtol = 1e-4; bfloat16 inputs: 2e-2."""
+import pytest
+import torch
+
+from oracle import scan_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _close(got, want, what, tol=1e-4):
+    scale = max(1.0, float(want.abs().max()))
+    torch.testing.assert_close(got.cpu().float() / scale, want.float() / scale, atol=tol, rtol=tol,
+                               msg=lambda m: f"{what}: {m}")
+
+
+def _dev(p):
+    return {k: v.cuda() for k, v in p.items()}
+
+
+def test_config1_forward():
+    from aussm_amd import scan
+    B, D, N, L = 16, 128, 16, 1024
+    p = O.make_core_inputs(B, D, N, L, seed=1)
+    print("case config1 fwd", flush=True)
+    want, _ = O.unitary_core_loop(p["u"], p["delta"], p["theta"], p["Bc"], p["Cc"], p["Dskip"])
+    q = _dev(p)
+    y = scan.unitary_scan(q["u"], q["delta"], q["theta"], q["Bc"], q["Cc"], q["Dskip"])
+    _close(y, want, "y")
+
+
+def test_config2_long_sequence_forward_and_split():
+    from aussm_amd import scan
+    B, D, N, L = 4, 256, 16, 16384
+    p = O.make_core_inputs(B, D, N, L, seed=2)
+    print("case config2 fwd", flush=True)
+    want, want_h = O.unitary_core_loop(p["u"], p["delta"], p["theta"], p["Bc"], p["Cc"], p["Dskip"])
+    q = _dev(p)
+    y, hL = scan.unitary_scan(q["u"], q["delta"], q["theta"], q["Bc"], q["Cc"], q["Dskip"], return_last_state=True)
+    _close(y, want, "y")
+    _close(torch.view_as_real(hL), torch.view_as_real(want_h), "hL")
+    # split at an odd position with the state carried over == one scan
+    cut = 5001
+    sl = lambda t, a, b: t[..., a:b].contiguous()
+    y1, h1 = scan.unitary_scan(sl(q["u"], 0, cut), sl(q["delta"], 0, cut), sl(q["theta"], 0, cut),
+                               sl(q["Bc"], 0, cut), sl(q["Cc"], 0, cut), q["Dskip"], return_last_state=True)
+    y2, h2 = scan.unitary_scan(sl(q["u"], cut, L), sl(q["delta"], cut, L), sl(q["theta"], cut, L),
+                               sl(q["Bc"], cut, L), sl(q["Cc"], cut, L), q["Dskip"], h0=h1, return_last_state=True)
+    _close(torch.cat([y1, y2], -1), y.cpu(), "split y")
+    _close(torch.view_as_real(h2), torch.view_as_real(hL).cpu(), "split hL")
+
+
+def test_config2_long_sequence_gradients_on_a_channel_slice():
+    from aussm_amd import scan
+    B, D, N, L = 1, 64, 16, 16384
+    p = O.make_core_inputs(B, D, N, L, seed=3)
+    names = ("u", "delta", "theta", "Bc", "Cc", "Dskip")
+    print("case config2 bwd slice", flush=True)
+
+    def run(fn, dev):
+        lv = [p[k].clone().to(dev).requires_grad_(True) for k in names]
+        (fn(*lv) * p["dy"].to(dev)).sum().backward()
+        return [t.grad for t in lv]
+
+    want = run(lambda *a: O.unitary_core_loop(*a)[0], "cpu")
+    got = run(scan.unitary_scan, "cuda")
+    for k, w, g in zip(names, want, got):
+        if w.is_complex():
+            w, g = torch.view_as_real(w), torch.view_as_real(g)
+        _close(g, w, f"d{k}", tol=2e-4)
+
+
+def test_config2_full_size_adjoint_identity():
+    """<dy, J v> == <J^T dy, v> with J the Jacobian w.r.t. u.  The scan is linear in u, so J v is
+    simply the scan of v; no oracle is needed at this size."""
+    from aussm_amd import scan
+    B, D, N, L = 4, 256, 16, 16384
+    q = _dev(O.make_core_inputs(B, D, N, L, seed=4))
+    v = torch.randn_like(q["u"])
+    print("case config2 adjoint", flush=True)
+    u = q["u"].clone().requires_grad_(True)
+    y = scan.unitary_scan(u, q["delta"], q["theta"], q["Bc"], q["Cc"], q["Dskip"])
+    (du,) = torch.autograd.grad(y, u, q["dy"])
+    Jv = scan.unitary_scan(v, q["delta"], q["theta"], q["Bc"], q["Cc"], q["Dskip"])
+    lhs = (q["dy"].double() * Jv.double()).sum()
+    rhs = (du.double() * v.double()).sum()
+    mass = float((q["dy"].double() * Jv.double()).abs().sum())      # sum of magnitudes, not of signed terms
+    assert abs(float(lhs - rhs)) <= 1e-5 * mass, (float(lhs), float(rhs), mass)
+    # linearity in u
+    y2 = scan.unitary_scan(2.0 * q["u"] - 3.0 * v, q["delta"], q["theta"], q["Bc"], q["Cc"], q["Dskip"])
+    _close(y2, (2.0 * y.detach() - 3.0 * Jv).cpu(), "linearity")
+
+
+def test_headline_shape_batch_slice_and_independence():
+    """Configuration 3 (B=32 D=512 N=16 L=2048): two batch elements against the oracle (outputs and
+    gradients), then the full batch against runs of its own slices."""
+    from aussm_amd import scan
+    B, D, N, L = 32, 512, 16, 2048
+    p = O.make_core_inputs(B, D, N, L, seed=5)
+    names = ("u", "delta", "theta", "Bc", "Cc")
+    print("case headline slice", flush=True)
+
+    def run(fn, dev, sl):
+        lv = [p[k][sl].clone().to(dev).requires_grad_(True) for k in names]
+        Dk = p["Dskip"].clone().to(dev).requires_grad_(True)
+        y = fn(*lv, Dk)
+        (y * p["dy"][sl].to(dev)).sum().backward()
+        return y.detach(), [t.grad for t in lv] + [Dk.grad]
+
+    y_ref, g_ref = run(lambda *a: O.unitary_core_loop(*a)[0], "cpu", slice(0, 2))
+    y_dev, g_dev = run(scan.unitary_scan, "cuda", slice(0, 2))
+    _close(y_dev, y_ref, "y[0:2]")
+    for k, w, g in zip(names + ("Dskip",), g_ref, g_dev):
+        if w.is_complex():
+            w, g = torch.view_as_real(w), torch.view_as_real(g)
+        _close(g, w, f"d{k}[0:2]")
+    print("case headline full batch", flush=True)
+    y_all, g_all = run(scan.unitary_scan, "cuda", slice(0, B))
+    assert torch.equal(y_all[0:2], y_dev), "forward output must not depend on the other batch elements"
+    y_tail, g_tail = run(scan.unitary_scan, "cuda", slice(B - 3, B))
+    assert torch.equal(y_all[B - 3:], y_tail)
+    for k, ga, gs in zip(names, g_all, g_dev):
+        a, s = ga[0:2], gs
+        if a.is_complex():
+            a, s = torch.view_as_real(a), torch.view_as_real(s)
+        _close(a, s.cpu(), f"d{k} full batch vs slice", tol=1e-5)
+
+
+@pytest.mark.parametrize("variant", ["unitary", "complex", "real"])
+def test_bf16_inputs(variant):
+    """bfloat16 u / delta / B / C with float32 state: compared with the oracle evaluated in float32
+    on the same (already rounded) values, at the 2e-2 tolerance of the benchmark contract."""
+    from aussm_amd import scan
+    B, D, N, L = 2, 96, 16, 200
+    p = O.make_core_inputs(B, D, N, L, seed=6, variant=variant)
+    bf = lambda t: t.to(torch.bfloat16)
+    print(f"case bf16 {variant}", flush=True)
+    if variant == "real":
+        lo = {k: bf(p[k]) for k in ("u", "delta", "Bm", "Cm")}
+        ref_in = [lo["u"].float(), lo["delta"].float(), p["A"], lo["Bm"].float(), lo["Cm"].float(), p["Dskip"]]
+        dev_in = [lo["u"].cuda(), lo["delta"].cuda(), p["A"].cuda(), lo["Bm"].cuda(), lo["Cm"].cuda(), p["Dskip"].cuda()]
+        ref_fn = lambda *a: O.real_core_loop(*a)[0]
+        dev_fn = scan.selective_scan_fn
+    else:
+        lo = {"u": bf(p["u"]), "delta": bf(p["delta"]),
+              "B": bf(torch.view_as_real(p["Bc"])), "C": bf(torch.view_as_real(p["Cc"]))}
+        cplx = lambda t: torch.view_as_complex(t.float().contiguous())
+        mid = [p["theta"]] if variant == "unitary" else [p["rho"], p["theta"]]
+        ref_in = [lo["u"].float(), lo["delta"].float()] + mid + [cplx(lo["B"]), cplx(lo["C"]), p["Dskip"]]
+        dev_in = [lo["u"].cuda(), lo["delta"].cuda()] + [m.cuda() for m in mid] + [lo["B"].cuda(), lo["C"].cuda(),
+                                                                                   p["Dskip"].cuda()]
+        ref_fn = (lambda *a: O.unitary_core_loop(*a)[0]) if variant == "unitary" else (lambda *a: O.complex_core_loop(*a)[0])
+        dev_fn = scan.unitary_scan if variant == "unitary" else scan.complex_scan
+
+    def run(fn, ins, dy):
+        lv = [t.clone().requires_grad_(True) for t in ins]
+        y = fn(*lv)
+        (y.float() * dy).sum().backward()
+        return y.detach(), [t.grad for t in lv]
+
+    y_ref, g_ref = run(ref_fn, ref_in, p["dy"])
+    y_dev, g_dev = run(dev_fn, dev_in, p["dy"].cuda())
+    _close(y_dev, y_ref, "y", tol=2e-2)
+    for i, (w, g) in enumerate(zip(g_ref, g_dev)):
+        assert g.dtype == dev_in[i].dtype
+        if w.is_complex():
+            w = torch.view_as_real(w)
+        _close(g, w, f"grad of input {i}", tol=2e-2)
