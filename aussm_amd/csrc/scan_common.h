@@ -178,6 +178,58 @@ struct TileWarm {
   }
 };
 
+// ---- staging geometry: a thread owns runs of FOUR consecutive timesteps of one channel row, so a
+// tile row of TT timesteps is covered by TT/4 neighbouring lanes with 16-byte accesses.
+template <int NT, int TT>
+struct StageGeom {
+  static constexpr int TPR = TT / 4;                        // threads per channel row
+  static constexpr int RW = 64 / TPR;                       // channel rows covered by one wavefront
+  static constexpr int RP = NT / TPR;                       // channel rows covered per pass
+  static constexpr int PASS = (CH + RP - 1) / RP;           // passes over the tile (1 if RP >= CH)
+};
+
+// Four consecutive raw input elements, kept exactly as loaded (no arithmetic may touch a loaded
+// register before the tile is collected, or the wait for the load moves up to the load).
+template <typename Tin> struct Quad;
+template <> struct Quad<float> {
+  float4 v;
+  __device__ __forceinline__ float get(int i) const { return i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w; }
+  __device__ __forceinline__ void touch() const { touch_vgpr(v.x); touch_vgpr(v.y); touch_vgpr(v.z); touch_vgpr(v.w); }
+  __device__ __forceinline__ void zero() { v = make_float4(0.f, 0.f, 0.f, 0.f); }
+  // vec: one 16-byte load at element offset o (caller guarantees alignment and range);
+  // otherwise four element loads at o + idx[i].
+  __device__ __forceinline__ void load(const float* __restrict__ p, size_t o, bool vec, const int (&idx)[4]) {
+    if (vec) v = *reinterpret_cast<const float4*>(p + o);
+    else v = make_float4(p[o + idx[0]], p[o + idx[1]], p[o + idx[2]], p[o + idx[3]]);
+  }
+};
+template <> struct Quad<bf16_t> {
+  uint2 v;
+  __device__ __forceinline__ float get(int i) const {
+    const uint32_t w = (i < 2) ? v.x : v.y;
+    return __uint_as_float((i & 1) ? (w & 0xffff0000u) : (w << 16));
+  }
+  __device__ __forceinline__ void touch() const { touch_vgpr(__uint_as_float(v.x)); touch_vgpr(__uint_as_float(v.y)); }
+  __device__ __forceinline__ void zero() { v = make_uint2(0u, 0u); }
+  __device__ __forceinline__ void load(const bf16_t* __restrict__ p, size_t o, bool vec, const int (&idx)[4]) {
+    if (vec) v = *reinterpret_cast<const uint2*>(p + o);
+    else v = make_uint2((uint32_t)p[o + idx[0]] | ((uint32_t)p[o + idx[1]] << 16),
+                        (uint32_t)p[o + idx[2]] | ((uint32_t)p[o + idx[3]] << 16));
+  }
+};
+
+// Four consecutive float32 outputs at element offset o: one 16-byte store when `vec`, else
+// element stores for the timesteps < nvalid.
+__device__ __forceinline__ void store4(float* __restrict__ p, size_t o, const float (&x)[4], bool vec, int nvalid) {
+  if (vec && nvalid >= 4) {
+    *reinterpret_cast<float4*>(p + o) = make_float4(x[0], x[1], x[2], x[3]);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (i < nvalid) p[o + i] = x[i];
+  }
+}
+
 // Sum `v` over the lanes of each aligned group of 32 lanes; result valid in every lane.
 __device__ __forceinline__ float half_wave_sum(float v) {
 #pragma unroll

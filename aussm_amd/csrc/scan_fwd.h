@@ -31,12 +31,13 @@ template <int VAR, int NW, int NT, typename Tin>
 __global__ __launch_bounds__(NT) void core_fwd_kernel(const FwdArgs p) {
   constexpr int C = (VAR == VAR_REAL) ? 1 : 2;   // floats per state
   constexpr int NWV = NT / 64;                   // wavefronts per workgroup
-  constexpr int E = CH * T / NT;                 // tile elements per thread in the staging phases
-  constexpr int RSTEP = NT / T;                  // channel-row step between a thread's elements
+  using SG = StageGeom<NT, T>;                   // staging: runs of 4 timesteps per thread
+  constexpr int PASS = SG::PASS;
 
   __shared__ float4 s_in[T * TS];                // per (t, channel): unitary/complex (Re a, Im a, delta*u, -)
                                                  //                   real            (delta, delta*u, -, -)
-  __shared__ float s_part[NWV * T * TS];         // per wavefront partial read-outs  sum_n Re(C h)
+  constexpr int TSP = CH + 2;                    // row stride of the partial slabs (conflict-free both ways)
+  __shared__ float s_part[NWV * T * TSP];        // per wavefront partial read-outs  sum_n Re(C h)
 
   const int tid = threadIdx.x, lane = tid & 63, wave = wave_index();
   const int wg = xcd_remap(blockIdx.x, gridDim.x);
@@ -69,52 +70,64 @@ __global__ __launch_bounds__(NT) void core_fwd_kernel(const FwdArgs p) {
     }
   }
 
-  // ---- staging-side mapping (lanes run along time)
-  const int col = tid % T, row0 = tid / T;
+  // ---- staging-side mapping: a thread owns 4 consecutive timesteps (t0..t0+3) of PASS channel rows
+  // (inside a wavefront the row index runs fastest: the 64 lanes cover RW rows x TPR runs, which
+  // is the same set of 128-byte row segments for the memory system and conflict-free in LDS)
+  const int t0 = 4 * (lane / SG::RW), row0 = wave * SG::RW + lane % SG::RW;
   // Raw inputs travel through two register sets: `rdy` holds the tile that is staged next and
   // `fly` the tile after it, whose loads are still in flight.  Loads are issued TWO tiles ahead
   // (the memory latency is longer than one tile's scan) and collected one tile later, right
   // after a barrier, where the shared load/store counter has nothing recent to drain.
-  struct RawTile { Tin u[E], dl[E]; float th[E], rho[E], z[E]; };
+  struct RawTile { Quad<Tin> u[PASS], dl[PASS]; Quad<float> th[PASS], rho[PASS], z[PASS]; };
   RawTile rdy, fly;
-  float dsk[E], dbias[E];
-  size_t goff[E];
-  bool rowok[E];
+  float dsk[PASS], dbias[PASS];
+  size_t goff[PASS];
+  int srow[PASS];
+  bool rowok[PASS], inrow[PASS];
 #pragma unroll
-  for (int k = 0; k < E; ++k) {
-    const int dd = d0 + row0 + k * RSTEP;
-    rowok[k] = dd < D;
+  for (int k = 0; k < PASS; ++k) {
+    srow[k] = row0 + k * SG::RP;
+    inrow[k] = srow[k] < CH;                     // this thread has a row in this pass
+    const int dd = d0 + srow[k];
+    rowok[k] = inrow[k] && dd < D;
     goff[k] = ((size_t)b * D + (rowok[k] ? dd : 0)) * L;
     dsk[k] = (p.Dskip && rowok[k]) ? p.Dskip[dd] : 0.f;
     dbias[k] = (VAR == VAR_REAL && p.delta_bias && rowok[k]) ? p.delta_bias[dd] : 0.f;
-    rdy.th[k] = rdy.rho[k] = rdy.z[k] = 0.f;
-    fly.th[k] = fly.rho[k] = fly.z[k] = 0.f;
-    fly.u[k] = fly.dl[k] = rdy.u[k] = rdy.dl[k] = Tin(0);
+    rdy.u[k].zero(); rdy.dl[k].zero(); rdy.th[k].zero(); rdy.rho[k].zero(); rdy.z[k].zero();
+    fly.u[k].zero(); fly.dl[k].zero(); fly.th[k].zero(); fly.rho[k].zero(); fly.z[k].zero();
   }
+  // 16-byte accesses need every row start (L % 4 == 0) and every tensor base aligned
+  auto al = [](const void* q, size_t a) { return q == nullptr || (reinterpret_cast<uintptr_t>(q) % a) == 0; };
+  const bool vec = (L % 4 == 0) && al(p.u, 4 * sizeof(Tin)) && al(p.delta, 4 * sizeof(Tin)) && al(p.theta, 16) &&
+                   al(p.rho, 16) && al(p.z, 16) && al(p.y, 16);
 
   auto load_tile = [&](RawTile& r, int l0) {
 #pragma unroll
-    for (int k = 0; k < E; ++k) {
-      // Unconditional loads from a clamped (always valid) address: nothing may depend on the
+    for (int k = 0; k < PASS; ++k) {
+      if (!inrow[k]) continue;
+      // Unconditional loads from clamped (always valid) addresses: nothing may depend on the
       // loaded value before it is collected, or the wait for it would move up to here.
       // Out-of-range elements are zeroed when the tile is staged.
-      const int ll = (l0 + col < L) ? l0 + col : L - 1;
-      const size_t o = goff[k] + ll;
-      r.u[k] = gu[o];
-      r.dl[k] = gdl[o];
-      if (VAR != VAR_REAL) r.th[k] = p.theta[o];
-      if (VAR == VAR_COMPLEX) r.rho[k] = p.rho[o];
-      if (p.z) r.z[k] = p.z[o];
+      const int ll = l0 + t0;
+      int idx[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) idx[i] = (ll + i < L) ? ll + i : L - 1;
+      const size_t o = goff[k] + (vec ? ((ll < L) ? ll : L - 4) : 0);
+      r.u[k].load(gu, o, vec, idx);
+      r.dl[k].load(gdl, o, vec, idx);
+      if (VAR != VAR_REAL) r.th[k].load(p.theta, o, vec, idx);
+      if (VAR == VAR_COMPLEX) r.rho[k].load(p.rho, o, vec, idx);
+      if (p.z) r.z[k].load(p.z, o, vec, idx);
     }
   };
   // A use of every register of a set: the compiler puts its wait for the loads here.
   auto collect_tile = [&](RawTile& r) {
 #pragma unroll
-    for (int k = 0; k < E; ++k) {
-      touch_vgpr(r.u[k]); touch_vgpr(r.dl[k]);
-      if (VAR != VAR_REAL) touch_vgpr(r.th[k]);
-      if (VAR == VAR_COMPLEX) touch_vgpr(r.rho[k]);
-      if (p.z) touch_vgpr(r.z[k]);
+    for (int k = 0; k < PASS; ++k) {
+      r.u[k].touch(); r.dl[k].touch();
+      if (VAR != VAR_REAL) r.th[k].touch();
+      if (VAR == VAR_COMPLEX) r.rho[k].touch();
+      if (p.z) r.z[k].touch();
     }
   };
   load_tile(rdy, 0);
@@ -137,26 +150,29 @@ __global__ __launch_bounds__(NT) void core_fwd_kernel(const FwdArgs p) {
     const bool warm_next = WARM && full_group && l0 + 2 * T <= L;
     if (warm_next) warm.issue(gB, gC, ((size_t)b * N + n0) * L + l0 + T, L);
     // ---- stage: convert this tile once per (channel, t) and transpose into LDS
-    float yin[E], gate[E];
+    float yin[PASS][4], gate[PASS][4];
 #pragma unroll
-    for (int k = 0; k < E; ++k) {
-      const bool ok = rowok[k] && l0 + col < L;
-      const float uu = ok ? to_f32(rdy.u[k]) : 0.f;
-      float dl = ok ? to_f32(rdy.dl[k]) : 0.f;
-      float4 rec;
-      if (VAR == VAR_REAL) {
-        dl += dbias[k];
-        if (p.delta_softplus) dl = softplusf_(dl);
-        rec = make_float4(dl, dl * uu, 0.f, 0.f);
-      } else {
-        float sn, cs;
-        fast_sincosf(ok ? rdy.th[k] : 0.f, &sn, &cs);
-        if (VAR == VAR_COMPLEX) { const float r = expf(ok ? rdy.rho[k] : 0.f); cs *= r; sn *= r; }
-        rec = make_float4(cs, sn, dl * uu, 0.f);
+    for (int k = 0; k < PASS; ++k) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const bool ok = rowok[k] && l0 + t0 + i < L;
+        const float uu = ok ? rdy.u[k].get(i) : 0.f;
+        float dl = ok ? rdy.dl[k].get(i) : 0.f;
+        float4 rec;
+        if (VAR == VAR_REAL) {
+          dl += dbias[k];
+          if (p.delta_softplus) dl = softplusf_(dl);
+          rec = make_float4(dl, dl * uu, 0.f, 0.f);
+        } else {
+          float sn, cs;
+          fast_sincosf(ok ? rdy.th[k].get(i) : 0.f, &sn, &cs);
+          if (VAR == VAR_COMPLEX) { const float r = expf(ok ? rdy.rho[k].get(i) : 0.f); cs *= r; sn *= r; }
+          rec = make_float4(cs, sn, dl * uu, 0.f);
+        }
+        if (inrow[k]) s_in[(t0 + i) * TS + srow[k]] = rec;
+        yin[k][i] = dsk[k] * uu;
+        gate[k][i] = rdy.z[k].get(i);
       }
-      s_in[col * TS + row0 + k * RSTEP] = rec;
-      yin[k] = dsk[k] * uu;
-      gate[k] = rdy.z[k];
     }
     if (warm_next) warm.retire();
     __syncthreads();
@@ -220,7 +236,7 @@ __global__ __launch_bounds__(NT) void core_fwd_kernel(const FwdArgs p) {
           }
 #pragma unroll
           for (int t = 0; t < TG; ++t) {
-            s_part[(wave * T + g * TG + t) * TS + lane] = yacc[t];
+            s_part[(wave * T + g * TG + t) * TSP + lane] = yacc[t];
             if (g + 1 < T / TG) { rx[t] = nx[t]; ry[t] = ny[t]; }
           }
           if (g == T / 2 / TG - 1) {
@@ -267,7 +283,7 @@ __global__ __launch_bounds__(NT) void core_fwd_kernel(const FwdArgs p) {
           }
 #pragma unroll
           for (int t = 0; t < TG; ++t) {
-            s_part[(wave * T + g * TG + t) * TS + lane] = yacc[t];
+            s_part[(wave * T + g * TG + t) * TSP + lane] = yacc[t];
             if (g + 1 < T / TG) { rx[t] = nx[t]; ry[t] = ny[t]; rz[t] = nz[t]; }
           }
           if (g == T / 2 / TG - 1) {
@@ -300,7 +316,7 @@ __global__ __launch_bounds__(NT) void core_fwd_kernel(const FwdArgs p) {
             }
           }
         }
-        s_part[(wave * T + t) * TS + lane] = yacc;
+        s_part[(wave * T + t) * TSP + lane] = yacc;
         if (t == T / 2 - 1) {
 #pragma unroll
           for (int k = 0; k < NW; ++k) { mr[k] = hr[k]; mi[k] = hi[k]; }
@@ -321,21 +337,27 @@ __global__ __launch_bounds__(NT) void core_fwd_kernel(const FwdArgs p) {
     // ---- epilogue: add the wavefronts' partial read-outs, skip term and gate; coalesced store
     if (p.y) {
       // all partial sums are fetched before the first add, so their LDS latencies overlap
-      float pv[E][NWV];
+      float pv[PASS][4][NWV];
 #pragma unroll
-      for (int k = 0; k < E; ++k)
+      for (int k = 0; k < PASS; ++k)
 #pragma unroll
-        for (int w = 0; w < NWV; ++w)
-          pv[k][w] = (w < nwa) ? s_part[(w * T + col) * TS + row0 + k * RSTEP] : 0.f;
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+          for (int w = 0; w < NWV; ++w)
+            pv[k][i][w] = (w < nwa && inrow[k]) ? s_part[(w * T + t0 + i) * TSP + srow[k]] : 0.f;
       sched_fence();
 #pragma unroll
-      for (int k = 0; k < E; ++k) {
-        const int ll = l0 + col;
-        float acc = yin[k];
+      for (int k = 0; k < PASS; ++k) {
+        float acc[4];
 #pragma unroll
-        for (int w = 0; w < NWV; ++w) acc += pv[k][w];
-        if (p.z) acc *= siluf_(gate[k]);
-        if (rowok[k] && ll < L) p.y[goff[k] + ll] = acc;
+        for (int i = 0; i < 4; ++i) {
+          acc[i] = yin[k][i];
+#pragma unroll
+          for (int w = 0; w < NWV; ++w) acc[i] += pv[k][i][w];
+          if (p.z) acc[i] *= siluf_(gate[k][i]);
+        }
+        const int nvalid = L - (l0 + t0);
+        if (rowok[k] && nvalid > 0) store4(p.y, goff[k] + l0 + t0, acc, vec, nvalid);
       }
     }
     // ---- checkpoint at the end of every ck-step block (and at the end of the sequence).
