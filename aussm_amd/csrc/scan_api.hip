@@ -10,6 +10,7 @@
 #include "scan_bwd_unitary.h"
 #include "scan_common.h"
 #include "scan_fwd.h"
+#include "scan_fwd_mfma.h"
 
 using namespace aussm;
 
@@ -72,8 +73,23 @@ int launch_fwd_t(const FwdArgs& a, hipStream_t s) {
   return AUSSM_E_SHAPE;
 }
 
+// The matrix-core forward kernel covers the common unitary case; everything else takes the
+// generic kernel.  AUSSM_MFMA=0 (environment) forces the generic kernel for comparisons.
+inline bool mfma_fwd_ok(const FwdArgs& a, int in_dtype) {
+  static const bool enabled = [] { const char* e = getenv("AUSSM_MFMA"); return !(e && e[0] == '0'); }();
+  if (!enabled || in_dtype != AUSSM_F32 || a.N > MN || a.L % 4 != 0 || a.ck % MT != 0) return false;
+  return !(misaligned(a.u, 16) || misaligned(a.delta, 16) || misaligned(a.theta, 16) || misaligned(a.z, 16) ||
+           misaligned(a.y, 16) || misaligned(a.Bm, 16) || misaligned(a.Cm, 16));
+}
+
 template <int VAR>
 int launch_fwd(const FwdArgs& a, int in_dtype, hipStream_t s) {
+  if (VAR == VAR_UNITARY && mfma_fwd_ok(a, in_dtype)) {
+    const dim3 grid((unsigned)(a.B * a.ncg));
+    if (a.z) hipLaunchKernelGGL(unitary_fwd_mfma_kernel<true>, grid, dim3(256), 0, s, a);
+    else hipLaunchKernelGGL(unitary_fwd_mfma_kernel<false>, grid, dim3(256), 0, s, a);
+    return launch_status();
+  }
   return in_dtype == AUSSM_BF16 ? launch_fwd_t<VAR, bf16_t>(a, s) : launch_fwd_t<VAR, float>(a, s);
 }
 

@@ -1,0 +1,410 @@
+// Unitary forward scan in chunked matrix form on the fp32 matrix cores (N <= 16).
+//
+// Inside a chunk of MT = 32 timesteps starting from the state H (h at the end of the previous
+// chunk), with Theta_t the running sum of theta over the chunk, P_t = exp(i Theta_t),
+// w_s = delta_s u_s and V_s = conj(P_s) w_s (per channel):
+//     h_t[n]  = P_t ( H[n] + sum_{s<=t} B_s[n] V_s )
+//     y_t     = Re( P_t S_t ) + D u_t,     S_t = sum_{s<=t} G[t,s] V_s + sum_n C_t[n] H[n],
+//     G[t,s]  = sum_n C_t[n] B_s[n]        (channel independent, masked to s <= t)
+//     H'[n]   = P_last ( H[n] + sum_s B_s[n] V_s ).
+// Every sum is a small complex GEMM whose free dimension is the channel, so the per-(channel,
+// timestep) vector work is one sincos and a handful of products, independent of N; the recurrence
+// over states runs on v_mfma_f32_16x16x4_f32 (plain fp32, no reduced precision).
+//
+// Work split: a workgroup owns (batch b, 64 channels) and runs the chunks in order; each of its
+// four wavefronts owns 16 channels end to end (no exchange of channel data between wavefronts).
+// Lane l = (dl = l % 16, g = l / 16) of a wavefront is channel dl and owns the eight timesteps
+// 16*st + 4*g + i (st = 0,1; i = 0..3) of every chunk: that is at once the B-operand layout of
+// V (contraction index s = (st, i) per instruction, g across lane groups) and the C/D layout of
+// S (rows 4*g + i of tile st), so u/delta/theta go from global memory to matrix operands and the
+// result rows go back to global memory as 16-byte vectors without passing through LDS.
+// B_t and C_t of the chunk are staged once per workgroup in LDS in the two operand orders, and G
+// is produced co-operatively (three 16x16 tiles, one per wavefront) one chunk ahead.
+#pragma once
+#include "scan_common.h"
+#include "scan_fwd.h"
+
+namespace aussm {
+
+typedef float f4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ f4 mfma4(float a, float b, f4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
+}
+
+#ifndef AUSSM_VALU_PER_MFMA
+#define AUSSM_VALU_PER_MFMA 3
+#endif
+constexpr int MT = 32;       // timesteps per chunk
+constexpr int MN = 16;       // state rows of the matrix tiles (N is zero-padded up to it)
+constexpr int M_RS = 20;     // row stride (floats) of the [t][n] planes
+constexpr int M_RT = 36;     // row stride (floats) of the [n][t] planes and of G
+
+// B_t / C_t of one chunk.  c*/b*: [t][n] (rows of the A operand of C.H and of both operands of
+// G = C B^T); bt*: [n][t] (rows of the A operand of B^T V).
+struct MfmaBC {
+  float cr[MT * M_RS], ci[MT * M_RS], br[MT * M_RS], bi[MT * M_RS];
+  float btr[MN * M_RT], bti[MN * M_RT];
+};
+struct MfmaG { float re[MT * M_RT], im[MT * M_RT]; };
+
+__device__ __forceinline__ f4 lds4(const float* p) { return *reinterpret_cast<const f4*>(p); }
+__device__ __forceinline__ f4 ldg4(const float* p) { return *reinterpret_cast<const f4*>(p); }
+
+// sin and cos without the large-argument branch: the caller keeps |x| below ~150.
+__device__ __forceinline__ void sincos_small(float x, float* sn, float* cs) {
+  const float kf = rintf(x * 0.636619772367581343f);
+  float r = fmaf(-kf, 1.57079637050628662109375f, x);
+  r = fmaf(-kf, -4.37113900018624283e-8f, r);
+  const float r2 = r * r;
+  float ps = fmaf(-1.9515295891e-4f, r2, 8.3321608736e-3f);
+  ps = fmaf(ps, r2, -1.6666654611e-1f);
+  const float s = fmaf(r * r2, ps, r);
+  float pc = fmaf(2.443315711809948e-5f, r2, -1.388731625493765e-3f);
+  pc = fmaf(pc, r2, 4.166664568298827e-2f);
+  const float c = fmaf(r2 * r2, pc, fmaf(-0.5f, r2, 1.0f));
+  const int q = (int)kf;
+  const float s1 = (q & 1) ? c : s;
+  const float c1 = (q & 1) ? s : c;
+  *sn = (q & 2) ? -s1 : s1;
+  *cs = ((q + 1) & 2) ? -c1 : c1;
+}
+
+__device__ __forceinline__ void touch4(const f4& v) { touch_vgpr(v[0]); touch_vgpr(v[1]); touch_vgpr(v[2]); touch_vgpr(v[3]); }
+
+// Requires: N <= 16, L % 4 == 0, u/delta/theta/z/y 16-byte aligned, B/C 16-byte aligned,
+// ck % 32 == 0, float inputs.  The launcher checks these and otherwise takes the generic kernel.
+template <bool GATED>
+__global__ __launch_bounds__(256) void unitary_fwd_mfma_kernel(const FwdArgs p) {
+  __shared__ MfmaBC s_bc[3];
+  __shared__ MfmaG s_g[2];
+
+  const int wg = xcd_remap(blockIdx.x, gridDim.x);
+  const int b = wg / p.ncg, d0 = (wg % p.ncg) * CH;
+  const int tid = threadIdx.x, lane = tid & 63, wave = wave_index();
+  const int dl = lane & 15, g = lane >> 4;
+  const int D = p.D, N = p.N, L = p.L;
+  const int d = d0 + wave * 16 + dl;
+  const bool dok = d < D;
+  const int dc = dok ? d : D - 1;
+  const size_t row = ((size_t)b * D + dc) * L;
+  const float* __restrict__ gu = static_cast<const float*>(p.u) + row;
+  const float* __restrict__ gdl = static_cast<const float*>(p.delta) + row;
+  const float* __restrict__ gth = p.theta + row;
+  const float* __restrict__ gz = GATED ? p.z + row : nullptr;
+  const float* __restrict__ gB = static_cast<const float*>(p.Bm);
+  const float* __restrict__ gC = static_cast<const float*>(p.Cm);
+  const float dsk = (p.Dskip && dok) ? p.Dskip[dc] : 0.0f;
+  const int nchunks = (L + MT - 1) / MT;
+
+  // ---- B/C staging: thread (sn = tid / 16, t = 2 * (tid % 16)) moves two timesteps of row sn
+  const int sn = tid >> 4, stt = (tid & 15) * 2;
+  const bool snok = sn < N;
+  const size_t bc_row = ((size_t)b * N + (snok ? sn : 0)) * L;
+  f4 rawB, rawC;
+  auto bc_load = [&](int c) {
+    const int l = c * MT + stt;
+    const int lc = l < L ? l : 0;
+    rawB = ldg4(gB + (bc_row + lc) * 2);
+    rawC = ldg4(gC + (bc_row + lc) * 2);
+  };
+  auto bc_store = [&](int c, MfmaBC& s) {
+    const bool ok = snok && (c * MT + stt < L);
+    const f4 vb = ok ? rawB : f4{0, 0, 0, 0};
+    const f4 vc = ok ? rawC : f4{0, 0, 0, 0};
+    s.br[stt * M_RS + sn] = vb.x; s.bi[stt * M_RS + sn] = vb.y;
+    s.br[(stt + 1) * M_RS + sn] = vb.z; s.bi[(stt + 1) * M_RS + sn] = vb.w;
+    s.cr[stt * M_RS + sn] = vc.x; s.ci[stt * M_RS + sn] = vc.y;
+    s.cr[(stt + 1) * M_RS + sn] = vc.z; s.ci[(stt + 1) * M_RS + sn] = vc.w;
+    *reinterpret_cast<float2*>(&s.btr[sn * M_RT + stt]) = make_float2(vb.x, vb.z);
+    *reinterpret_cast<float2*>(&s.bti[sn * M_RT + stt]) = make_float2(vb.y, vb.w);
+  };
+
+  // ---- G tile of one wavefront: wave 0 -> (tt 0, st 0), 1 -> (1, 0), 2 and 3 -> (1, 1) (the
+  // same values twice: cheaper than a branch); the tile (0, 1) lies above the diagonal and is
+  // never read.
+  const int gtt = wave >= 1 ? 1 : 0, gst = wave >= 2 ? 1 : 0;
+  auto make_g = [&](const MfmaBC& s, MfmaG& o) {
+    {
+      const f4 cr = lds4(&s.cr[(16 * gtt + dl) * M_RS + 4 * g]);
+      const f4 ci = lds4(&s.ci[(16 * gtt + dl) * M_RS + 4 * g]);
+      const f4 br = lds4(&s.br[(16 * gst + dl) * M_RS + 4 * g]);
+      const f4 bi = lds4(&s.bi[(16 * gst + dl) * M_RS + 4 * g]);
+      f4 gr = {0, 0, 0, 0}, gi = {0, 0, 0, 0};
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        gr = mfma4(cr[k], br[k], gr);
+        gi = mfma4(cr[k], bi[k], gi);
+        gr = mfma4(-ci[k], bi[k], gr);
+        gi = mfma4(ci[k], br[k], gi);
+      }
+      // lane holds column s = dl, rows t = 4 g + i
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int t = 4 * g + i;
+        const bool keep = (gtt != gst) || (dl <= t);
+        o.re[(16 * gtt + t) * M_RT + 16 * gst + dl] = keep ? gr[i] : 0.0f;
+        o.im[(16 * gtt + t) * M_RT + 16 * gst + dl] = keep ? gi[i] : 0.0f;
+      }
+    }
+  };
+
+  // ---- channel data of one chunk: two runs of four timesteps per lane.  Loads are unconditional
+  // from a clamped address; out-of-range runs are zeroed where they are used.
+  struct In { f4 u[2], de[2], th[2], z[2]; };
+  auto in_load = [&](In& r, int c) {
+#pragma unroll
+    for (int st = 0; st < 2; ++st) {
+      const int l = c * MT + 16 * st + 4 * g;
+      const int lc = l < L ? l : 0;
+      r.u[st] = ldg4(gu + lc);
+      r.de[st] = ldg4(gdl + lc);
+      r.th[st] = ldg4(gth + lc);
+      if (GATED) r.z[st] = ldg4(gz + lc);
+    }
+  };
+  auto in_touch = [&](const In& r) {
+#pragma unroll
+    for (int st = 0; st < 2; ++st) {
+      touch4(r.u[st]); touch4(r.de[st]); touch4(r.th[st]);
+      if (GATED) touch4(r.z[st]);
+    }
+  };
+
+  // ---- per-channel vector work of one chunk: phases, rotations, rotated inputs
+  struct Prep {
+    float cs[2][4], sn[2][4], vr[2][4], vi[2][4], nvi[2][4];
+    f4 u[2], z[2];
+    float cT, sT;
+  };
+  // first half: phases of the chunk, reduced to (-pi, pi] when any of them is large so that the
+  // running sums stay small enough for sincos_small and for fp32 sums of 32 terms
+  auto prep_phase = [&](const In& r, int c, float (&th)[2][4]) {
+    bool big = false;
+#pragma unroll
+    for (int st = 0; st < 2; ++st) {
+      const bool ok = c * MT + 16 * st + 4 * g < L;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        th[st][i] = ok ? r.th[st][i] : 0.0f;
+        big |= fabsf(th[st][i]) > 4.0f;
+      }
+    }
+    if (__builtin_expect(__any(big), 0)) {
+#pragma unroll
+      for (int st = 0; st < 2; ++st)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) th[st][i] = (float)remainder((double)th[st][i], 6.283185307179586476925);
+    }
+  };
+  auto prep_rest = [&](const In& r, int c, float (&th)[2][4], Prep& o) {
+    float w[2][4];
+#pragma unroll
+    for (int st = 0; st < 2; ++st) {
+      const bool ok = c * MT + 16 * st + 4 * g < L;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) w[st][i] = ok ? r.de[st][i] * r.u[st][i] : 0.0f;
+      th[st][1] += th[st][0]; th[st][2] += th[st][1]; th[st][3] += th[st][2];
+      o.u[st] = r.u[st];
+      if (GATED) o.z[st] = r.z[st];
+    }
+    // exclusive offsets over the order (st 0: g 0..3), (st 1: g 0..3)
+    float sa = th[0][3], sb = th[1][3];
+    {
+      float ta = __shfl_up(sa, 16), tb = __shfl_up(sb, 16);
+      if (g >= 1) { sa += ta; sb += tb; }
+      ta = __shfl_up(sa, 32); tb = __shfl_up(sb, 32);
+      if (g >= 2) { sa += ta; sb += tb; }
+    }
+    const float tot_a = __shfl(sa, 48 + dl);
+    const float off_a = sa - th[0][3];
+    const float off_b = tot_a + sb - th[1][3];
+#pragma unroll
+    for (int st = 0; st < 2; ++st) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float ph = th[st][i] + (st ? off_b : off_a);
+        sincos_small(ph, &o.sn[st][i], &o.cs[st][i]);
+        o.vr[st][i] = o.cs[st][i] * w[st][i];
+        o.nvi[st][i] = o.sn[st][i] * w[st][i];
+        o.vi[st][i] = -o.nvi[st][i];
+      }
+    }
+    // rotation over the whole chunk: the element (st 1, g 3, i 3) is timestep 31
+    o.cT = __shfl(o.cs[1][3], 48 + dl);
+    o.sT = __shfl(o.sn[1][3], 48 + dl);
+  };
+
+  // ---- state: lane (dl, g) holds H[n = 4 g + i][channel dl]
+  f4 Hr = {0, 0, 0, 0}, Hi = {0, 0, 0, 0};
+  if (p.h0 && dok) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int n = 4 * g + i;
+      if (n < N) {
+        const size_t o = (((size_t)b * D + d) * N + n) * 2;
+        Hr[i] = p.h0[o];
+        Hi[i] = p.h0[o + 1];
+      }
+    }
+  }
+
+  int i0 = 0, i1 = 1, i2 = 2;   // LDS slots of chunks c, c+1, c+2
+  const int ck_chunks = p.ck / MT;
+  int ck_left = ck_chunks, kb = 0;   // chunks to the next checkpoint, its index
+
+  // One chunk.  pc: vector work of chunk c (ready); pn: receives that of chunk c + 1, computed from
+  // in1 in the shadow of the matrix instructions; in2 receives the loads of chunk c + 2.
+  auto step = [&](int c, In& in1, In& in2, Prep& pc, Prep& pn) {
+    const int l0 = c * MT;
+    bc_store(c + 2, s_bc[i2]);
+    bc_load(c + 3);
+    in_load(in2, c + 2);
+    make_g(s_bc[i1], s_g[(c + 1) & 1]);
+    float th[2][4];
+    prep_phase(in1, c + 1, th);
+
+    const MfmaBC& s = s_bc[i0];
+    const MfmaG& G = s_g[c & 1];
+    // ---- S = C.H  (rows t, contraction n = 4 g + k)
+    f4 Sr[2], Si[2];
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt) {
+      const f4 cr = lds4(&s.cr[(16 * tt + dl) * M_RS + 4 * g]);
+      const f4 ci = lds4(&s.ci[(16 * tt + dl) * M_RS + 4 * g]);
+      f4 ar = {0, 0, 0, 0}, ai = {0, 0, 0, 0};
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        ar = mfma4(cr[k], Hr[k], ar);
+        ai = mfma4(cr[k], Hi[k], ai);
+        ar = mfma4(-ci[k], Hi[k], ar);
+        ai = mfma4(ci[k], Hr[k], ai);
+      }
+      Sr[tt] = ar; Si[tt] = ai;
+    }
+    // ---- H += B^T V  (rows n, contraction s), then rotate to the end of the chunk
+#pragma unroll
+    for (int st = 0; st < 2; ++st) {
+      const f4 br = lds4(&s.btr[dl * M_RT + 16 * st + 4 * g]);
+      const f4 bi = lds4(&s.bti[dl * M_RT + 16 * st + 4 * g]);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        Hr = mfma4(br[i], pc.vr[st][i], Hr);
+        Hi = mfma4(br[i], pc.vi[st][i], Hi);
+        Hr = mfma4(bi[i], pc.nvi[st][i], Hr);
+        Hi = mfma4(bi[i], pc.vr[st][i], Hi);
+      }
+    }
+    // ---- S += G.V  (contraction s = 16 st + 4 g + i), lower block triangle only
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt) {
+#pragma unroll
+      for (int st = 0; st <= tt; ++st) {
+        const f4 gr = lds4(&G.re[(16 * tt + dl) * M_RT + 16 * st + 4 * g]);
+        const f4 gi = lds4(&G.im[(16 * tt + dl) * M_RT + 16 * st + 4 * g]);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          Sr[tt] = mfma4(gr[i], pc.vr[st][i], Sr[tt]);
+          Si[tt] = mfma4(gr[i], pc.vi[st][i], Si[tt]);
+          Sr[tt] = mfma4(gi[i], pc.nvi[st][i], Sr[tt]);
+          Si[tt] = mfma4(gi[i], pc.vr[st][i], Si[tt]);
+        }
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float xr = Hr[i], xi = Hi[i];
+      Hr[i] = pc.cT * xr - pc.sT * xi;
+      Hi[i] = fmaf(pc.cT, xi, pc.sT * xr);
+    }
+    // ---- vector work of the next chunk (independent of everything above)
+    prep_rest(in1, c + 1, th, pn);
+
+    // ---- outputs: rows 16 tt + 4 g + i of channel dl are this lane's own timesteps
+    f4 yo[2];
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float v = pc.cs[tt][i] * Sr[tt][i] - pc.sn[tt][i] * Si[tt][i];
+        v = fmaf(dsk, pc.u[tt][i], v);
+        if (GATED) v *= siluf_(pc.z[tt][i]);
+        yo[tt][i] = v;
+      }
+    }
+    // Interleave: one matrix instruction, then vector instructions in its shadow.
+#pragma unroll
+    for (int k = 0; k < 112; ++k) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, AUSSM_VALU_PER_MFMA, 0);
+    }
+    // The loads issued at the top have had a whole chunk to land: collect them here, before the
+    // stores below join the same in-order queue.
+    touch4(rawB); touch4(rawC);
+    in_touch(in2);
+    if (p.y && dok) {
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt) {
+        const int l = l0 + 16 * tt + 4 * g;
+        if (l < L) *reinterpret_cast<f4*>(p.y + row + l) = yo[tt];
+      }
+    }
+    // ---- checkpoint: state at the end of every ck-step block and at the end of the sequence
+    const bool ck_now = l0 < L && (--ck_left == 0 || l0 + MT >= L);
+    if (p.hck && dok && ck_now) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int n = 4 * g + i;
+        if (n < N) {
+          const size_t o = ((((size_t)b * p.nck + kb) * N + n) * 2) * D + d;
+          p.hck[o] = Hr[i];
+          p.hck[o + D] = Hi[i];
+        }
+      }
+    }
+    if (ck_now) { ck_left = ck_chunks; ++kb; }
+    const int tmp = i0; i0 = i1; i1 = i2; i2 = tmp;
+    __syncthreads();
+  };
+
+  // ---- prologue
+  In inA, inB;
+  Prep P0, P1;
+  bc_load(0);
+  in_load(inB, 0);
+  in_load(inA, 1);
+  bc_store(0, s_bc[0]);
+  bc_load(1);
+  bc_store(1, s_bc[1]);
+  bc_load(2);
+  {
+    float th[2][4];
+    prep_phase(inB, 0, th);
+    prep_rest(inB, 0, th, P0);
+  }
+  __syncthreads();
+  make_g(s_bc[0], s_g[0]);
+  __syncthreads();
+
+  // Two chunks per trip so that the register sets alternate without copies.  With an odd number of
+  // chunks the last half-trip runs on an all-padding chunk: zero input, zero phase, no stores, and
+  // the state passes through unchanged.
+  for (int c = 0; c < nchunks; c += 2) {
+    step(c, inA, inB, P0, P1);
+    step(c + 1, inB, inA, P1, P0);
+  }
+
+  if (p.hL && dok) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int n = 4 * g + i;
+      if (n < N) {
+        const size_t o = (((size_t)b * D + d) * N + n) * 2;
+        p.hL[o] = Hr[i];
+        p.hL[o + 1] = Hi[i];
+      }
+    }
+  }
+}
+
+}  // namespace aussm
