@@ -11,6 +11,7 @@
 #include "scan_common.h"
 #include "scan_fwd.h"
 #include "scan_fwd_mfma.h"
+#include "scan_fwd_xdl.h"
 
 using namespace aussm;
 
@@ -74,20 +75,31 @@ int launch_fwd_t(const FwdArgs& a, hipStream_t s) {
 }
 
 // The matrix-core forward kernel covers the common unitary case; everything else takes the
-// generic kernel.  AUSSM_MFMA=0 (environment) forces the generic kernel for comparisons.
-inline bool mfma_fwd_ok(const FwdArgs& a, int in_dtype) {
-  static const bool enabled = [] { const char* e = getenv("AUSSM_MFMA"); return !(e && e[0] == '0'); }();
-  if (!enabled || in_dtype != AUSSM_F32 || a.N > MN || a.L % 4 != 0 || a.ck % MT != 0) return false;
-  return !(misaligned(a.u, 16) || misaligned(a.delta, 16) || misaligned(a.theta, 16) || misaligned(a.z, 16) ||
-           misaligned(a.y, 16) || misaligned(a.Bm, 16) || misaligned(a.Cm, 16));
+// generic kernel.  AUSSM_MFMA (environment) selects for comparisons: 0 generic kernel, 1 fp32
+// matrix instructions, 2 / 3 bf16 matrix instructions on two / three-piece operands (default 3).
+inline int mfma_fwd_mode(const FwdArgs& a, int in_dtype) {
+  static const int mode = [] { const char* e = getenv("AUSSM_MFMA"); return e ? atoi(e) : 3; }();
+  if (mode <= 0 || in_dtype != AUSSM_F32 || a.N > MN || a.L % 4 != 0 || a.ck % MT != 0) return 0;
+  if (misaligned(a.u, 16) || misaligned(a.delta, 16) || misaligned(a.theta, 16) || misaligned(a.z, 16) ||
+      misaligned(a.y, 16) || misaligned(a.Bm, 16) || misaligned(a.Cm, 16))
+    return 0;
+  return mode;
 }
 
 template <int VAR>
 int launch_fwd(const FwdArgs& a, int in_dtype, hipStream_t s) {
-  if (VAR == VAR_UNITARY && mfma_fwd_ok(a, in_dtype)) {
+  if (const int mode = (VAR == VAR_UNITARY) ? mfma_fwd_mode(a, in_dtype) : 0) {
     const dim3 grid((unsigned)(a.B * a.ncg));
-    if (a.z) hipLaunchKernelGGL(unitary_fwd_mfma_kernel<true>, grid, dim3(256), 0, s, a);
-    else hipLaunchKernelGGL(unitary_fwd_mfma_kernel<false>, grid, dim3(256), 0, s, a);
+    if (mode == 1) {
+      if (a.z) hipLaunchKernelGGL(unitary_fwd_mfma_kernel<true>, grid, dim3(256), 0, s, a);
+      else hipLaunchKernelGGL(unitary_fwd_mfma_kernel<false>, grid, dim3(256), 0, s, a);
+    } else if (mode == 2) {
+      if (a.z) hipLaunchKernelGGL((unitary_fwd_xdl_kernel<2, true>), grid, dim3(256), 0, s, a);
+      else hipLaunchKernelGGL((unitary_fwd_xdl_kernel<2, false>), grid, dim3(256), 0, s, a);
+    } else {
+      if (a.z) hipLaunchKernelGGL((unitary_fwd_xdl_kernel<3, true>), grid, dim3(256), 0, s, a);
+      else hipLaunchKernelGGL((unitary_fwd_xdl_kernel<3, false>), grid, dim3(256), 0, s, a);
+    }
     return launch_status();
   }
   return in_dtype == AUSSM_BF16 ? launch_fwd_t<VAR, bf16_t>(a, s) : launch_fwd_t<VAR, float>(a, s);

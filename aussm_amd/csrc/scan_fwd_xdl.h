@@ -1,0 +1,501 @@
+// Unitary forward scan in chunked matrix form on the bf16 matrix cores, fp32-accurate (N <= 16).
+//
+// Inside a chunk of XT = 32 timesteps starting from the state H (h at the end of the previous
+// chunk), with Theta_t the running sum of theta over the chunk, P_t = exp(i Theta_t),
+// w_s = delta_s u_s and V_s = conj(P_s) w_s (per channel):
+//     h_t[n]  = P_t ( H[n] + sum_{s<=t} B_s[n] V_s )
+//     y_t     = Re( P_t S_t ) + D u_t,     S_t = sum_{s<=t} G[t,s] V_s + sum_n C_t[n] H[n],
+//     G[t,s]  = sum_n C_t[n] B_s[n]        (channel independent, masked to s <= t)
+//     H'[n]   = P_last ( H[n] + sum_s B_s[n] V_s ).
+// Every sum is a small complex GEMM whose free dimension is the channel, so the per-(channel,
+// timestep) vector work is one sincos and a handful of products, independent of N.
+//
+// Arithmetic.  The fp32 matrix instructions share the vector ALU, the bf16 ones (XDL) run beside
+// it, so the GEMMs use v_mfma_f32_16x16x32_bf16 on operands split EXACTLY into NP bf16 pieces
+// (x = p1 + p2 + p3, each piece the bf16 rounding of what the previous ones left: three pieces
+// carry 27 significand bits, more than fp32 holds).  A product keeps the partial products
+// p_i q_j with i + j <= NP + 1, accumulated in fp32: with NP = 3 what is dropped is below 2^-26
+// relative, i.e. the GEMMs are fp32-accurate; NP = 2 (2^-17) is there for measurements.
+//
+// Work split: a workgroup owns (batch b, 64 channels) and runs the chunks in order; each of its
+// four wavefronts owns 16 channels end to end.  Lane l = (dl = l % 16, g = l / 16) is channel dl
+// and owns the eight timesteps e = 0..7 -> t(g, e) = 16*(e/4) + 4*g + e%4 of every chunk.  That is
+// the K order of the matrix instruction's B operand (lane group g holds K slots 8g..8g+7) under
+// the permutation slot (g, e) <-> timestep t(g, e), and also the C/D layout of the result tiles
+// (tile e/4, rows 4*g + e%4), so u/delta/theta go from global memory to matrix operands and the
+// results go back to global memory as 16-byte vectors without passing through LDS.
+// The channel-independent A operands (B_t, C_t and G in the orders each product needs, already
+// split into pieces) are staged once per workgroup in LDS as 16-byte records [row][g].
+#pragma once
+#include "scan_common.h"
+#include "scan_fwd.h"
+#include "scan_fwd_mfma.h"
+
+namespace aussm {
+
+typedef float f2v __attribute__((ext_vector_type(2)));
+typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf2v __attribute__((ext_vector_type(2)));
+typedef __bf16 bf8v __attribute__((ext_vector_type(8)));
+
+constexpr int XT = 32;       // timesteps per chunk
+constexpr int XN = 16;       // state rows of the matrix tiles (N is zero-padded up to it)
+
+__device__ __forceinline__ f4 xdl(const u4& a, const u4& b, f4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf8v, a), __builtin_bit_cast(bf8v, b), c, 0, 0, 0);
+}
+// two fp32 -> packed bf16 pair (round to nearest even), low half = a
+__device__ __forceinline__ uint32_t pk_bf16(float a, float b) {
+  const f2v v = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf2v));
+}
+// Split the pair (a, b) into NP packed bf16 pieces.  The residuals are exact in fp32.
+template <int NP>
+__device__ __forceinline__ void split2(float a, float b, uint32_t (&out)[NP]) {
+#pragma unroll
+  for (int p = 0; p < NP; ++p) {
+    out[p] = pk_bf16(a, b);
+    if (p + 1 < NP) {
+      a -= __uint_as_float(out[p] << 16);
+      b -= __uint_as_float(out[p] & 0xffff0000u);
+    }
+  }
+}
+// eight values -> NP operand registers quads (K slots 0..7 of one lane group)
+template <int NP>
+__device__ __forceinline__ void split8(const float (&x)[8], u4 (&out)[NP]) {
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    uint32_t pc[NP];
+    split2<NP>(x[2 * q], x[2 * q + 1], pc);
+#pragma unroll
+    for (int p = 0; p < NP; ++p) out[p][q] = pc[p];
+  }
+}
+// c += a . b over the kept partial products (small terms first)
+template <int NP>
+__device__ __forceinline__ f4 xmm(const u4 (&a)[NP], const u4 (&b)[NP], f4 c) {
+#pragma unroll
+  for (int s = NP - 1; s >= 0; --s)
+#pragma unroll
+    for (int i = 0; i <= s; ++i) c = xdl(a[i], b[s - i], c);
+  return c;
+}
+__device__ __forceinline__ u4 neg_bf16x8(const u4& v) { return v ^ u4{0x80008000u, 0x80008000u, 0x80008000u, 0x80008000u}; }
+
+// LDS records: 8 bf16 (16 bytes) per (row, lane group g), stored [g][row] so that the 16 lanes of a
+// group read consecutive records (no bank conflicts); one plane per piece.
+__device__ __forceinline__ constexpr int xrec(int row, int g, int rows) { return g * rows + row; }
+template <int NP>
+struct XdlBC {
+  u4 cs_r[NP][XT * 4];   // row t: [ Cr[4g..4g+3], -Ci[4g..4g+3] ]   (real part of C.x)
+  u4 cs_i[NP][XT * 4];   // row t: [ Ci[4g..4g+3],  Cr[4g..4g+3] ]   (imaginary part of C.x)
+  u4 bs[NP][XT * 4];     // row s: [ Br[4g..4g+3],  Bi[4g..4g+3] ]
+  u4 bt_r[NP][XN * 4];   // row n: Br[t(g, e)][n], e = 0..7
+  u4 bt_i[NP][XN * 4];   //        Bi
+  u4 bt_ni[NP][XN * 4];  //       -Bi
+};
+template <int NP>
+struct XdlG {
+  u4 re[NP][XT * 4];     // row t: G[t][t(g, e)], e = 0..7 (zero where s > t)
+  u4 im[NP][XT * 4];
+  u4 nim[NP][XT * 4];
+};
+
+// Requires: N <= 16, L % 4 == 0, u/delta/theta/z/y 16-byte aligned, B/C 16-byte aligned,
+// ck % 32 == 0, float inputs.  The launcher checks these and otherwise takes the generic kernel.
+template <int NP, bool GATED>
+__global__ __launch_bounds__(256) void unitary_fwd_xdl_kernel(const FwdArgs p) {
+  __shared__ XdlBC<NP> s_bc[3];
+  __shared__ XdlG<NP> s_g[2];
+
+  const int wg = xcd_remap(blockIdx.x, gridDim.x);
+  const int b = wg / p.ncg, d0 = (wg % p.ncg) * CH;
+  const int tid = threadIdx.x, lane = tid & 63, wave = wave_index();
+  const int dl = lane & 15, g = lane >> 4;
+  const int D = p.D, N = p.N, L = p.L;
+  const int d = d0 + wave * 16 + dl;
+  const bool dok = d < D;
+  const int dc = dok ? d : D - 1;
+  const size_t row = ((size_t)b * D + dc) * L;
+  const float* __restrict__ gu = static_cast<const float*>(p.u) + row;
+  const float* __restrict__ gdl = static_cast<const float*>(p.delta) + row;
+  const float* __restrict__ gth = p.theta + row;
+  const float* __restrict__ gz = GATED ? p.z + row : nullptr;
+  const float* __restrict__ gB = static_cast<const float*>(p.Bm);
+  const float* __restrict__ gC = static_cast<const float*>(p.Cm);
+  const float dsk = (p.Dskip && dok) ? p.Dskip[dc] : 0.0f;
+  const int nchunks = (L + XT - 1) / XT;
+
+  // G tiles above the block diagonal are read (as zeros) but never written
+  for (int i = tid; i < (int)(sizeof(s_g) / 16); i += 256) reinterpret_cast<u4*>(s_g)[i] = u4{0, 0, 0, 0};
+
+  // ---- B/C staging, first mapping: thread (t = tid % 32, g1 = (tid / 32) % 4) of C (tid < 128) or
+  // B (tid >= 128) builds the record [row t][g1] from the four state rows 4 g1 .. 4 g1 + 3.
+  const int m1_t = tid & 31, m1_g = (tid >> 5) & 3;
+  const bool m1_isB = tid >= 128;
+  const float* __restrict__ m1_src = m1_isB ? gB : gC;
+  float2 m1_raw[4];
+  // second mapping: thread (n = tid % 16, g2 = (tid / 16) % 4, half = (tid / 64) % 2) reads the four
+  // timesteps 16 half + 4 g2 .. + 3 of row n of B; tid < 128 writes the Br half-record, the
+  // others the Bi and -Bi half-records.
+  const int m2_n = tid & 15, m2_g = (tid >> 4) & 3, m2_half = (tid >> 6) & 1;
+  const bool m2_im = tid >= 128;
+  f4 m2_raw[2];
+  auto bc_load = [&](int c) {
+    const int l = c * XT + m1_t;
+    const int lc = l < L ? l : 0;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int n = 4 * m1_g + k;
+      const size_t o = (((size_t)b * N + (n < N ? n : 0)) * L + lc) * 2;
+      m1_raw[k] = *reinterpret_cast<const float2*>(m1_src + o);
+    }
+    const int l2 = c * XT + 16 * m2_half + 4 * m2_g;
+    const int l2c = l2 < L ? l2 : 0;
+    const size_t o2 = (((size_t)b * N + (m2_n < N ? m2_n : 0)) * L + l2c) * 2;
+    m2_raw[0] = *reinterpret_cast<const f4*>(gB + o2);
+    m2_raw[1] = *reinterpret_cast<const f4*>(gB + o2 + 4);
+  };
+  auto bc_store = [&](int c, XdlBC<NP>& s) {
+    {
+      const bool tok = c * XT + m1_t < L;
+      float re[4], im[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const bool ok = tok && (4 * m1_g + k < N);
+        re[k] = ok ? m1_raw[k].x : 0.0f;
+        im[k] = ok ? m1_raw[k].y : 0.0f;
+      }
+      const float x[8] = {re[0], re[1], re[2], re[3], im[0], im[1], im[2], im[3]};
+      u4 pc[NP];
+      split8<NP>(x, pc);
+      const int o = xrec(m1_t, m1_g, XT);
+      if (m1_isB) {
+#pragma unroll
+        for (int q = 0; q < NP; ++q) s.bs[q][o] = pc[q];
+      } else {
+#pragma unroll
+        for (int q = 0; q < NP; ++q) {
+          s.cs_r[q][o] = u4{pc[q][0], pc[q][1], pc[q][2] ^ 0x80008000u, pc[q][3] ^ 0x80008000u};
+          s.cs_i[q][o] = u4{pc[q][2], pc[q][3], pc[q][0], pc[q][1]};
+        }
+      }
+    }
+    {
+      const bool ok = (m2_n < N) && (c * XT + 16 * m2_half + 4 * m2_g < L);
+      const int sel = m2_im ? 1 : 0;
+      const float v0 = ok ? m2_raw[0][sel] : 0.0f, v1 = ok ? m2_raw[0][2 + sel] : 0.0f;
+      const float v2 = ok ? m2_raw[1][sel] : 0.0f, v3 = ok ? m2_raw[1][2 + sel] : 0.0f;
+      uint32_t a[NP], c2[NP];
+      split2<NP>(v0, v1, a);
+      split2<NP>(v2, v3, c2);
+      const int o = xrec(m2_n, m2_g, XN) * 2 + m2_half;   // 8-byte half-record index
+#pragma unroll
+      for (int q = 0; q < NP; ++q) {
+        if (!m2_im) {
+          reinterpret_cast<u2*>(s.bt_r[q])[o] = u2{a[q], c2[q]};
+        } else {
+          reinterpret_cast<u2*>(s.bt_i[q])[o] = u2{a[q], c2[q]};
+          reinterpret_cast<u2*>(s.bt_ni[q])[o] = u2{a[q] ^ 0x80008000u, c2[q] ^ 0x80008000u};
+        }
+      }
+    }
+  };
+
+  // ---- G^T tile of one wavefront (rows s of tile st, columns t of tile tt): wave 0 -> (tt 0,
+  // st 0), 1 -> (1, 0), 2 and 3 -> (1, 1) (the same values twice: cheaper than a branch).
+  // A lane ends up with G[t = 16 tt + dl][s = 16 st + 4 g + i], i = 0..3: half a record of row t.
+  const int gtt = wave >= 1 ? 1 : 0, gst = wave >= 2 ? 1 : 0;
+  const int g_lim = (gtt == gst) ? dl : 64;   // diagonal tiles keep s <= t (a per-lane bound: no branch)
+  auto make_g = [&](const XdlBC<NP>& s, XdlG<NP>& o) {
+    u4 a[NP], br[NP], bi[NP];
+#pragma unroll
+    for (int q = 0; q < NP; ++q) {
+      a[q] = s.bs[q][xrec(16 * gst + dl, g, XT)];
+      br[q] = s.cs_r[q][xrec(16 * gtt + dl, g, XT)];
+      bi[q] = s.cs_i[q][xrec(16 * gtt + dl, g, XT)];
+    }
+    f4 gr = xmm<NP>(a, br, f4{0, 0, 0, 0});
+    f4 gi = xmm<NP>(a, bi, f4{0, 0, 0, 0});
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const bool keep = 4 * g + i <= g_lim;
+      gr[i] = keep ? gr[i] : 0.0f;
+      gi[i] = keep ? gi[i] : 0.0f;
+    }
+    uint32_t r0[NP], r1[NP], i0[NP], i1[NP];
+    split2<NP>(gr[0], gr[1], r0);
+    split2<NP>(gr[2], gr[3], r1);
+    split2<NP>(gi[0], gi[1], i0);
+    split2<NP>(gi[2], gi[3], i1);
+    const int h = xrec(16 * gtt + dl, g, XT) * 2 + gst;   // 8-byte half-record index
+#pragma unroll
+    for (int q = 0; q < NP; ++q) {
+      reinterpret_cast<u2*>(o.re[q])[h] = u2{r0[q], r1[q]};
+      reinterpret_cast<u2*>(o.im[q])[h] = u2{i0[q], i1[q]};
+      reinterpret_cast<u2*>(o.nim[q])[h] = u2{i0[q] ^ 0x80008000u, i1[q] ^ 0x80008000u};
+    }
+  };
+
+  // ---- channel data of one chunk: two runs of four timesteps per lane.  Loads are unconditional
+  // from a clamped address; out-of-range runs are zeroed where they are used.
+  struct In { f4 u[2], de[2], th[2], z[2]; };
+  auto in_load = [&](In& r, int c) {
+#pragma unroll
+    for (int st = 0; st < 2; ++st) {
+      const int l = c * XT + 16 * st + 4 * g;
+      const int lc = l < L ? l : 0;
+      r.u[st] = *reinterpret_cast<const f4*>(gu + lc);
+      r.de[st] = *reinterpret_cast<const f4*>(gdl + lc);
+      r.th[st] = *reinterpret_cast<const f4*>(gth + lc);
+      if (GATED) r.z[st] = *reinterpret_cast<const f4*>(gz + lc);
+    }
+  };
+  auto in_touch = [&](const In& r) {
+#pragma unroll
+    for (int st = 0; st < 2; ++st) {
+      touch4(r.u[st]); touch4(r.de[st]); touch4(r.th[st]);
+      if (GATED) touch4(r.z[st]);
+    }
+  };
+
+  // ---- per-channel vector work of one chunk: phases, rotations, rotated inputs (split)
+  struct Prep {
+    float cs[2][4], sn[2][4];
+    u4 vr[NP], vi[NP];
+    f4 u[2], z[2];
+    float cT, sT;
+  };
+  // first half: phases of the chunk, reduced to (-pi, pi] when any of them is large so that the
+  // running sums stay small enough for sincos_small and for fp32 sums of 32 terms
+  auto prep_phase = [&](const In& r, int c, float (&th)[2][4]) {
+    bool big = false;
+#pragma unroll
+    for (int st = 0; st < 2; ++st) {
+      const bool ok = c * XT + 16 * st + 4 * g < L;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        th[st][i] = ok ? r.th[st][i] : 0.0f;
+        big |= fabsf(th[st][i]) > 4.0f;
+      }
+    }
+    if (__builtin_expect(__any(big), 0)) {
+#pragma unroll
+      for (int st = 0; st < 2; ++st)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) th[st][i] = (float)remainder((double)th[st][i], 6.283185307179586476925);
+    }
+  };
+  auto prep_rest = [&](const In& r, int c, float (&th)[2][4], Prep& o) {
+    float w[2][4];
+#pragma unroll
+    for (int st = 0; st < 2; ++st) {
+      const bool ok = c * XT + 16 * st + 4 * g < L;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) w[st][i] = ok ? r.de[st][i] * r.u[st][i] : 0.0f;
+      th[st][1] += th[st][0]; th[st][2] += th[st][1]; th[st][3] += th[st][2];
+      o.u[st] = r.u[st];
+      if (GATED) o.z[st] = r.z[st];
+    }
+    // exclusive offsets over the order (st 0: g 0..3), (st 1: g 0..3)
+    float sa = th[0][3], sb = th[1][3];
+    {
+      float ta = __shfl_up(sa, 16), tb = __shfl_up(sb, 16);
+      if (g >= 1) { sa += ta; sb += tb; }
+      ta = __shfl_up(sa, 32); tb = __shfl_up(sb, 32);
+      if (g >= 2) { sa += ta; sb += tb; }
+    }
+    const float tot_a = __shfl(sa, 48 + dl);
+    const float off_a = sa - th[0][3];
+    const float off_b = tot_a + sb - th[1][3];
+    float vr[8], vi[8];
+#pragma unroll
+    for (int st = 0; st < 2; ++st) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float ph = th[st][i] + (st ? off_b : off_a);
+        sincos_small(ph, &o.sn[st][i], &o.cs[st][i]);
+        vr[4 * st + i] = o.cs[st][i] * w[st][i];
+        vi[4 * st + i] = -o.sn[st][i] * w[st][i];
+      }
+    }
+    split8<NP>(vr, o.vr);
+    split8<NP>(vi, o.vi);
+    // rotation over the whole chunk: the element (st 1, g 3, i 3) is timestep 31
+    o.cT = __shfl(o.cs[1][3], 48 + dl);
+    o.sT = __shfl(o.sn[1][3], 48 + dl);
+  };
+
+  // ---- state: lane (dl, g) holds H[n = 4 g + i][channel dl]
+  f4 Hr = {0, 0, 0, 0}, Hi = {0, 0, 0, 0};
+  if (p.h0 && dok) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int n = 4 * g + i;
+      if (n < N) {
+        const size_t o = (((size_t)b * D + d) * N + n) * 2;
+        Hr[i] = p.h0[o];
+        Hi[i] = p.h0[o + 1];
+      }
+    }
+  }
+
+  int i0 = 0, i1 = 1, i2 = 2;   // LDS slots of chunks c, c+1, c+2
+  const int ck_chunks = p.ck / XT;
+  int ck_left = ck_chunks, kb = 0;   // chunks to the next checkpoint, its index
+
+  // One chunk.  pc: vector work of chunk c (ready); pn: receives that of chunk c + 1, computed from
+  // in1 while the matrix pipe works; in2 receives the loads of chunk c + 2.
+  auto step = [&](int c, In& in1, In& in2, Prep& pc, Prep& pn) {
+    const int l0 = c * XT;
+    float th[2][4];
+    prep_phase(in1, c + 1, th);     // (holds the only branch of the step)
+    bc_store(c + 2, s_bc[i2]);
+    bc_load(c + 3);
+    in_load(in2, c + 2);
+    make_g(s_bc[i1], s_g[(c + 1) & 1]);
+
+    const XdlBC<NP>& s = s_bc[i0];
+    const XdlG<NP>& G = s_g[c & 1];
+    // ---- S = C.H  (rows t; K slot (g, j): j < 4 -> Re H[4g+j], else Im H[4g+j-4])
+    u4 hk[NP];
+    {
+      const float x[8] = {Hr[0], Hr[1], Hr[2], Hr[3], Hi[0], Hi[1], Hi[2], Hi[3]};
+      split8<NP>(x, hk);
+    }
+    f4 Sr[2], Si[2];
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt) {
+      u4 ar[NP], ai[NP];
+#pragma unroll
+      for (int q = 0; q < NP; ++q) {
+        ar[q] = s.cs_r[q][xrec(16 * tt + dl, g, XT)];
+        ai[q] = s.cs_i[q][xrec(16 * tt + dl, g, XT)];
+      }
+      Sr[tt] = xmm<NP>(ar, hk, f4{0, 0, 0, 0});
+      Si[tt] = xmm<NP>(ai, hk, f4{0, 0, 0, 0});
+    }
+    // ---- H += B^T V  (rows n, K slot (g, e) <-> timestep t(g, e))
+    {
+      u4 ar[NP], ai[NP], an[NP];
+#pragma unroll
+      for (int q = 0; q < NP; ++q) {
+        ar[q] = s.bt_r[q][xrec(dl, g, XN)];
+        ai[q] = s.bt_i[q][xrec(dl, g, XN)];
+        an[q] = s.bt_ni[q][xrec(dl, g, XN)];
+      }
+      Hr = xmm<NP>(ar, pc.vr, Hr);
+      Hi = xmm<NP>(ar, pc.vi, Hi);
+      Hr = xmm<NP>(an, pc.vi, Hr);
+      Hi = xmm<NP>(ai, pc.vr, Hi);
+    }
+    // ---- S += G.V
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt) {
+      u4 ar[NP], ai[NP], an[NP];
+#pragma unroll
+      for (int q = 0; q < NP; ++q) {
+        ar[q] = G.re[q][xrec(16 * tt + dl, g, XT)];
+        ai[q] = G.im[q][xrec(16 * tt + dl, g, XT)];
+        an[q] = G.nim[q][xrec(16 * tt + dl, g, XT)];
+      }
+      Sr[tt] = xmm<NP>(ar, pc.vr, Sr[tt]);
+      Si[tt] = xmm<NP>(ar, pc.vi, Si[tt]);
+      Sr[tt] = xmm<NP>(an, pc.vi, Sr[tt]);
+      Si[tt] = xmm<NP>(ai, pc.vr, Si[tt]);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float xr = Hr[i], xi = Hi[i];
+      Hr[i] = pc.cT * xr - pc.sT * xi;
+      Hi[i] = fmaf(pc.cT, xi, pc.sT * xr);
+    }
+    // ---- vector work of the next chunk (independent of everything above)
+    prep_rest(in1, c + 1, th, pn);
+
+    // ---- outputs: rows 16 tt + 4 g + i of channel dl are this lane's own timesteps
+    f4 yo[2];
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float v = pc.cs[tt][i] * Sr[tt][i] - pc.sn[tt][i] * Si[tt][i];
+        v = fmaf(dsk, pc.u[tt][i], v);
+        if (GATED) v *= siluf_(pc.z[tt][i]);
+        yo[tt][i] = v;
+      }
+    }
+    // The loads issued at the top have had a whole chunk to land: collect them here, before the
+    // stores below join the same in-order queue.
+#pragma unroll
+    for (int k = 0; k < 4; ++k) { touch_vgpr(m1_raw[k].x); touch_vgpr(m1_raw[k].y); }
+    touch4(m2_raw[0]); touch4(m2_raw[1]);
+    in_touch(in2);
+    if (p.y && dok) {
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt) {
+        const int l = l0 + 16 * tt + 4 * g;
+        if (l < L) *reinterpret_cast<f4*>(p.y + row + l) = yo[tt];
+      }
+    }
+    // ---- checkpoint: state at the end of every ck-step block and at the end of the sequence
+    const bool ck_now = l0 < L && (--ck_left == 0 || l0 + XT >= L);
+    if (p.hck && dok && ck_now) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int n = 4 * g + i;
+        if (n < N) {
+          const size_t o = ((((size_t)b * p.nck + kb) * N + n) * 2) * D + d;
+          p.hck[o] = Hr[i];
+          p.hck[o + D] = Hi[i];
+        }
+      }
+    }
+    if (ck_now) { ck_left = ck_chunks; ++kb; }
+    const int tmp = i0; i0 = i1; i1 = i2; i2 = tmp;
+    __syncthreads();
+  };
+
+  // ---- prologue
+  In inA, inB;
+  Prep P0, P1;
+  bc_load(0);
+  in_load(inB, 0);
+  in_load(inA, 1);
+  bc_store(0, s_bc[0]);
+  bc_load(1);
+  bc_store(1, s_bc[1]);
+  bc_load(2);
+  {
+    float th[2][4];
+    prep_phase(inB, 0, th);
+    prep_rest(inB, 0, th, P0);
+  }
+  __syncthreads();
+  make_g(s_bc[0], s_g[0]);
+  __syncthreads();
+
+  // Two chunks per trip so that the register sets alternate without copies.  With an odd number of
+  // chunks the last half-trip runs on an all-padding chunk: zero input, zero phase, no stores, and
+  // the state passes through unchanged.
+  for (int c = 0; c < nchunks; c += 2) {
+    step(c, inA, inB, P0, P1);
+    step(c + 1, inB, inA, P1, P0);
+  }
+
+  if (p.hL && dok) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int n = 4 * g + i;
+      if (n < N) {
+        const size_t o = (((size_t)b * D + d) * N + n) * 2;
+        p.hL[o] = Hr[i];
+        p.hL[o + 1] = Hi[i];
+      }
+    }
+  }
+}
+
+}  // namespace aussm
