@@ -8,6 +8,7 @@
 
 #include "scan_bwd_recompute.h"
 #include "scan_bwd_unitary.h"
+#include "scan_bwd_xdl.h"
 #include "scan_common.h"
 #include "scan_fwd.h"
 #include "scan_fwd_mfma.h"
@@ -221,6 +222,17 @@ int aussm_unitary_bwd(const float* dy, const float* dhL, const void* u, const vo
   a.dy = dy; a.dhL = dhL; a.u = u; a.delta = delta; a.theta = theta; a.Bm = Bc; a.Cm = Cc; a.Dskip = Dskip;
   a.hck = hck; a.du = du; a.ddelta = ddelta; a.dtheta = dtheta; a.dB = dB; a.dC = dC; a.dD = dD; a.dh0 = dh0;
   a.B = B; a.D = D; a.N = N; a.L = L; a.ck = ck; a.nck = (L + ck - 1) / ck; a.ncg = (D + CH - 1) / CH;
+  // matrix-core kernel for the common case (AUSSM_MFMA_BWD: 0 generic kernel, 2 / 3 operand pieces)
+  static const int mode = [] { const char* e = getenv("AUSSM_MFMA_BWD"); return e ? atoi(e) : 3; }();
+  if (mode > 0 && in_dtype == AUSSM_F32 && N <= XN && L % 4 == 0 && ck % XT == 0 &&
+      !(misaligned(dy, 16) || misaligned(u, 16) || misaligned(delta, 16) || misaligned(theta, 16) ||
+        misaligned(du, 16) || misaligned(ddelta, 16) || misaligned(dtheta, 16) || misaligned(Bc, 16) ||
+        misaligned(Cc, 16))) {
+    const dim3 grid((unsigned)(a.B * a.ncg));
+    if (mode == 2) hipLaunchKernelGGL(unitary_bwd_xdl_kernel<2>, grid, dim3(256), 0, s, a);
+    else hipLaunchKernelGGL(unitary_bwd_xdl_kernel<3>, grid, dim3(256), 0, s, a);
+    return launch_status();
+  }
   return in_dtype == AUSSM_BF16 ? launch_unitary_bwd_t<bf16_t>(a, s) : launch_unitary_bwd_t<float>(a, s);
 }
 

@@ -30,6 +30,7 @@
 #include "scan_common.h"
 #include "scan_fwd.h"
 #include "scan_fwd_mfma.h"
+#include <type_traits>
 
 namespace aussm {
 
@@ -50,25 +51,38 @@ __device__ __forceinline__ uint32_t pk_bf16(float a, float b) {
   const f2v v = {a, b};
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf2v));
 }
-// Split the pair (a, b) into NP packed bf16 pieces.  The residuals are exact in fp32.
+// Split the pair (a, b) into NP packed bf16 pieces.  The residuals are exact in fp32: they are
+// taken with the bf16 dot instruction, r = x + (-1) * piece (one instruction per value instead of
+// an unpack and a subtract).
+// The multipliers (-1, 0) and (0, -1) are kept in registers the compiler cannot see through: as
+// literal operands of this instruction they do not encode the intended packed pair.
+struct SplitK { uint32_t lo, hi; };
+__device__ __forceinline__ SplitK make_splitk() {
+  SplitK k{0x0000bf80u, 0xbf800000u};
+  asm volatile("" : "+v"(k.lo), "+v"(k.hi));
+  return k;
+}
 template <int NP>
-__device__ __forceinline__ void split2(float a, float b, uint32_t (&out)[NP]) {
+__device__ __forceinline__ void split2(const SplitK& sk, float a, float b, uint32_t (&out)[NP]) {
+  const bf2v m_lo = __builtin_bit_cast(bf2v, sk.lo), m_hi = __builtin_bit_cast(bf2v, sk.hi);
 #pragma unroll
   for (int p = 0; p < NP; ++p) {
-    out[p] = pk_bf16(a, b);
+    const f2v v = {a, b};
+    const bf2v pk = __builtin_convertvector(v, bf2v);
+    out[p] = __builtin_bit_cast(uint32_t, pk);
     if (p + 1 < NP) {
-      a -= __uint_as_float(out[p] << 16);
-      b -= __uint_as_float(out[p] & 0xffff0000u);
+      a = __builtin_amdgcn_fdot2_f32_bf16(pk, m_lo, a, false);
+      b = __builtin_amdgcn_fdot2_f32_bf16(pk, m_hi, b, false);
     }
   }
 }
 // eight values -> NP operand registers quads (K slots 0..7 of one lane group)
 template <int NP>
-__device__ __forceinline__ void split8(const float (&x)[8], u4 (&out)[NP]) {
+__device__ __forceinline__ void split8(const SplitK& sk, const float (&x)[8], u4 (&out)[NP]) {
 #pragma unroll
   for (int q = 0; q < 4; ++q) {
     uint32_t pc[NP];
-    split2<NP>(x[2 * q], x[2 * q + 1], pc);
+    split2<NP>(sk, x[2 * q], x[2 * q + 1], pc);
 #pragma unroll
     for (int p = 0; p < NP; ++p) out[p][q] = pc[p];
   }
@@ -82,6 +96,17 @@ __device__ __forceinline__ f4 xmm(const u4 (&a)[NP], const u4 (&b)[NP], f4 c) {
     for (int i = 0; i <= s; ++i) c = xdl(a[i], b[s - i], c);
   return c;
 }
+// the K-th matrix instruction of xmm (same order)
+template <int NP, int K>
+__device__ __forceinline__ f4 xmm_k(const u4 (&a)[NP], const u4 (&b)[NP], f4 c) {
+  constexpr int s0 = NP - 1;
+  // products are visited with s = NP-1 .. 0 and i = 0 .. s: find (s, i) of index K
+  constexpr int s = (NP == 3) ? (K < 3 ? 2 : (K < 5 ? 1 : 0)) : (NP == 2 ? (K < 2 ? 1 : 0) : 0);
+  constexpr int base = (NP == 3) ? (K < 3 ? 0 : (K < 5 ? 3 : 5)) : (NP == 2 ? (K < 2 ? 0 : 2) : 0);
+  constexpr int i = K - base;
+  static_assert(s <= s0 && i <= s, "bad product index");
+  return xdl(a[i], b[s - i], c);
+}
 __device__ __forceinline__ u4 neg_bf16x8(const u4& v) { return v ^ u4{0x80008000u, 0x80008000u, 0x80008000u, 0x80008000u}; }
 
 // LDS records: 8 bf16 (16 bytes) per (row, lane group g), stored [g][row] so that the 16 lanes of a
@@ -92,15 +117,14 @@ struct XdlBC {
   u4 cs_r[NP][XT * 4];   // row t: [ Cr[4g..4g+3], -Ci[4g..4g+3] ]   (real part of C.x)
   u4 cs_i[NP][XT * 4];   // row t: [ Ci[4g..4g+3],  Cr[4g..4g+3] ]   (imaginary part of C.x)
   u4 bs[NP][XT * 4];     // row s: [ Br[4g..4g+3],  Bi[4g..4g+3] ]
+  u4 bs_c[NP][XT * 4];   // row s: [-Bi[4g..4g+3],  Br[4g..4g+3] ]   (written by the same code path as cs_i)
   u4 bt_r[NP][XN * 4];   // row n: Br[t(g, e)][n], e = 0..7
   u4 bt_i[NP][XN * 4];   //        Bi
-  u4 bt_ni[NP][XN * 4];  //       -Bi
 };
 template <int NP>
 struct XdlG {
   u4 re[NP][XT * 4];     // row t: G[t][t(g, e)], e = 0..7 (zero where s > t)
   u4 im[NP][XT * 4];
-  u4 nim[NP][XT * 4];
 };
 
 // Requires: N <= 16, L % 4 == 0, u/delta/theta/z/y 16-byte aligned, B/C 16-byte aligned,
@@ -127,6 +151,7 @@ __global__ __launch_bounds__(256) void unitary_fwd_xdl_kernel(const FwdArgs p) {
   const float* __restrict__ gC = static_cast<const float*>(p.Cm);
   const float dsk = (p.Dskip && dok) ? p.Dskip[dc] : 0.0f;
   const int nchunks = (L + XT - 1) / XT;
+  const SplitK sk = make_splitk();
 
   // G tiles above the block diagonal are read (as zeros) but never written
   for (int i = tid; i < (int)(sizeof(s_g) / 16); i += 256) reinterpret_cast<u4*>(s_g)[i] = u4{0, 0, 0, 0};
@@ -158,29 +183,28 @@ __global__ __launch_bounds__(256) void unitary_fwd_xdl_kernel(const FwdArgs p) {
     m2_raw[0] = *reinterpret_cast<const f4*>(gB + o2);
     m2_raw[1] = *reinterpret_cast<const f4*>(gB + o2 + 4);
   };
+  // Branch-free: C threads write [re, -im] -> cs_r and [im, re] -> cs_i, B threads [re, im] -> bs and
+  // [-im, re] -> bs_c; real-part threads of the second mapping write bt_r, the others bt_i.
+  const uint32_t m1_s1 = m1_isB ? 0u : 0x80008000u, m1_s2 = m1_isB ? 0x80008000u : 0u;
   auto bc_store = [&](int c, XdlBC<NP>& s) {
     {
       const bool tok = c * XT + m1_t < L;
-      float re[4], im[4];
+      float x[8];
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
         const bool ok = tok && (4 * m1_g + k < N);
-        re[k] = ok ? m1_raw[k].x : 0.0f;
-        im[k] = ok ? m1_raw[k].y : 0.0f;
+        x[k] = ok ? m1_raw[k].x : 0.0f;
+        x[4 + k] = ok ? m1_raw[k].y : 0.0f;
       }
-      const float x[8] = {re[0], re[1], re[2], re[3], im[0], im[1], im[2], im[3]};
       u4 pc[NP];
-      split8<NP>(x, pc);
+      split8<NP>(sk, x, pc);
       const int o = xrec(m1_t, m1_g, XT);
-      if (m1_isB) {
+      u4* d1 = m1_isB ? &s.bs[0][0] : &s.cs_r[0][0];
+      u4* d2 = m1_isB ? &s.bs_c[0][0] : &s.cs_i[0][0];
 #pragma unroll
-        for (int q = 0; q < NP; ++q) s.bs[q][o] = pc[q];
-      } else {
-#pragma unroll
-        for (int q = 0; q < NP; ++q) {
-          s.cs_r[q][o] = u4{pc[q][0], pc[q][1], pc[q][2] ^ 0x80008000u, pc[q][3] ^ 0x80008000u};
-          s.cs_i[q][o] = u4{pc[q][2], pc[q][3], pc[q][0], pc[q][1]};
-        }
+      for (int q = 0; q < NP; ++q) {
+        d1[q * (XT * 4) + o] = u4{pc[q][0], pc[q][1], pc[q][2] ^ m1_s1, pc[q][3] ^ m1_s1};
+        d2[q * (XT * 4) + o] = u4{pc[q][2] ^ m1_s2, pc[q][3] ^ m1_s2, pc[q][0], pc[q][1]};
       }
     }
     {
@@ -189,18 +213,12 @@ __global__ __launch_bounds__(256) void unitary_fwd_xdl_kernel(const FwdArgs p) {
       const float v0 = ok ? m2_raw[0][sel] : 0.0f, v1 = ok ? m2_raw[0][2 + sel] : 0.0f;
       const float v2 = ok ? m2_raw[1][sel] : 0.0f, v3 = ok ? m2_raw[1][2 + sel] : 0.0f;
       uint32_t a[NP], c2[NP];
-      split2<NP>(v0, v1, a);
-      split2<NP>(v2, v3, c2);
+      split2<NP>(sk, v0, v1, a);
+      split2<NP>(sk, v2, v3, c2);
       const int o = xrec(m2_n, m2_g, XN) * 2 + m2_half;   // 8-byte half-record index
+      u2* d1 = reinterpret_cast<u2*>(m2_im ? &s.bt_i[0][0] : &s.bt_r[0][0]);
 #pragma unroll
-      for (int q = 0; q < NP; ++q) {
-        if (!m2_im) {
-          reinterpret_cast<u2*>(s.bt_r[q])[o] = u2{a[q], c2[q]};
-        } else {
-          reinterpret_cast<u2*>(s.bt_i[q])[o] = u2{a[q], c2[q]};
-          reinterpret_cast<u2*>(s.bt_ni[q])[o] = u2{a[q] ^ 0x80008000u, c2[q] ^ 0x80008000u};
-        }
-      }
+      for (int q = 0; q < NP; ++q) d1[q * (XN * 4 * 2) + o] = u2{a[q], c2[q]};
     }
   };
 
@@ -226,16 +244,15 @@ __global__ __launch_bounds__(256) void unitary_fwd_xdl_kernel(const FwdArgs p) {
       gi[i] = keep ? gi[i] : 0.0f;
     }
     uint32_t r0[NP], r1[NP], i0[NP], i1[NP];
-    split2<NP>(gr[0], gr[1], r0);
-    split2<NP>(gr[2], gr[3], r1);
-    split2<NP>(gi[0], gi[1], i0);
-    split2<NP>(gi[2], gi[3], i1);
+    split2<NP>(sk, gr[0], gr[1], r0);
+    split2<NP>(sk, gr[2], gr[3], r1);
+    split2<NP>(sk, gi[0], gi[1], i0);
+    split2<NP>(sk, gi[2], gi[3], i1);
     const int h = xrec(16 * gtt + dl, g, XT) * 2 + gst;   // 8-byte half-record index
 #pragma unroll
     for (int q = 0; q < NP; ++q) {
       reinterpret_cast<u2*>(o.re[q])[h] = u2{r0[q], r1[q]};
       reinterpret_cast<u2*>(o.im[q])[h] = u2{i0[q], i1[q]};
-      reinterpret_cast<u2*>(o.nim[q])[h] = u2{i0[q] ^ 0x80008000u, i1[q] ^ 0x80008000u};
     }
   };
 
@@ -264,7 +281,7 @@ __global__ __launch_bounds__(256) void unitary_fwd_xdl_kernel(const FwdArgs p) {
   // ---- per-channel vector work of one chunk: phases, rotations, rotated inputs (split)
   struct Prep {
     float cs[2][4], sn[2][4];
-    u4 vr[NP], vi[NP];
+    u4 vr[NP], vi[NP], nvi[NP];
     f4 u[2], z[2];
     float cT, sT;
   };
@@ -321,8 +338,10 @@ __global__ __launch_bounds__(256) void unitary_fwd_xdl_kernel(const FwdArgs p) {
         vi[4 * st + i] = -o.sn[st][i] * w[st][i];
       }
     }
-    split8<NP>(vr, o.vr);
-    split8<NP>(vi, o.vi);
+    split8<NP>(sk, vr, o.vr);
+    split8<NP>(sk, vi, o.vi);
+#pragma unroll
+    for (int q = 0; q < NP; ++q) o.nvi[q] = neg_bf16x8(o.vi[q]);
     // rotation over the whole chunk: the element (st 1, g 3, i 3) is timestep 31
     o.cT = __shfl(o.cs[1][3], 48 + dl);
     o.sT = __shfl(o.sn[1][3], 48 + dl);
@@ -348,63 +367,173 @@ __global__ __launch_bounds__(256) void unitary_fwd_xdl_kernel(const FwdArgs p) {
 
   // One chunk.  pc: vector work of chunk c (ready); pn: receives that of chunk c + 1, computed from
   // in1 while the matrix pipe works; in2 receives the loads of chunk c + 2.
+  //
+  // Issue order.  The matrix pipe and the vector ALU run side by side only if their instructions
+  // alternate in the wavefront's (in-order) stream.  The step is therefore cut into regions: each
+  // holds the matrix instructions of one group of products plus independent vector work, and ends
+  // with a scheduling fence.  Inside a region the group barriers ask for one matrix instruction
+  // followed by a few vector ones.  Pure arithmetic is not ordered by a fence, so the inputs of a
+  // region's vector work pass through pin() after the previous fence and its results through
+  // touch_vgpr() before the next one.
+#define XDL_REGION(NMFMA, NVALU)                                  \
+  _Pragma("unroll") for (int k_ = 0; k_ < (NMFMA); ++k_) {        \
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);            \
+    __builtin_amdgcn_sched_group_barrier(0x002, (NVALU), 0);      \
+  }                                                               \
+  __builtin_amdgcn_sched_barrier(0)
+  constexpr int NPP = NP * (NP + 1) / 2;   // matrix instructions per product
+  auto pin = [](float& v) { asm volatile("" : "+v"(v)); };
   auto step = [&](int c, In& in1, In& in2, Prep& pc, Prep& pn) {
     const int l0 = c * XT;
     float th[2][4];
     prep_phase(in1, c + 1, th);     // (holds the only branch of the step)
-    bc_store(c + 2, s_bc[i2]);
-    bc_load(c + 3);
-    in_load(in2, c + 2);
-    make_g(s_bc[i1], s_g[(c + 1) & 1]);
+    __builtin_amdgcn_sched_barrier(0);
 
     const XdlBC<NP>& s = s_bc[i0];
+    const XdlBC<NP>& s1 = s_bc[i1];
     const XdlG<NP>& G = s_g[c & 1];
-    // ---- S = C.H  (rows t; K slot (g, j): j < 4 -> Re H[4g+j], else Im H[4g+j-4])
-    u4 hk[NP];
+    XdlG<NP>& Gn = s_g[(c + 1) & 1];
+    // ---- region 0: operands of the first products, global loads of chunk c + 2
+    u4 hk[NP], ga[NP], gbr[NP], gbi[NP], c_r[2][NP], c_i[2][NP];
     {
       const float x[8] = {Hr[0], Hr[1], Hr[2], Hr[3], Hi[0], Hi[1], Hi[2], Hi[3]};
-      split8<NP>(x, hk);
+      split8<NP>(sk, x, hk);
     }
+#pragma unroll
+    for (int q = 0; q < NP; ++q) {
+      ga[q] = s1.bs[q][xrec(16 * gst + dl, g, XT)];
+      gbr[q] = s1.cs_r[q][xrec(16 * gtt + dl, g, XT)];
+      gbi[q] = s1.cs_i[q][xrec(16 * gtt + dl, g, XT)];
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt) {
+        c_r[tt][q] = s.cs_r[q][xrec(16 * tt + dl, g, XT)];
+        c_i[tt][q] = s.cs_i[q][xrec(16 * tt + dl, g, XT)];
+      }
+    }
+    in_load(in2, c + 2);
+#pragma unroll
+    for (int q = 0; q < NP; ++q)
+#pragma unroll
+      for (int k = 0; k < 4; ++k) touch_vgpr(__uint_as_float(hk[q][k]));
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- region 1: G^T tile of chunk c + 1  |  staging of B/C of chunk c + 2
+#pragma unroll
+    for (int k = 0; k < 4; ++k) { pin(m1_raw[k].x); pin(m1_raw[k].y); }
+#pragma unroll
+    for (int k = 0; k < 2; ++k) asm volatile("" : "+v"(m2_raw[k]));
+    f4 ggr = xmm<NP>(ga, gbr, f4{0, 0, 0, 0});
+    f4 ggi = xmm<NP>(ga, gbi, f4{0, 0, 0, 0});
+    bc_store(c + 2, s_bc[i2]);
+    XDL_REGION(2 * NPP, 12);
+    bc_load(c + 3);
+
+    // ---- region 2: S = C.H  |  G tile to LDS, phases and the first rotations of chunk c + 1
+#pragma unroll
+    for (int st = 0; st < 2; ++st)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) pin(th[st][i]);
     f4 Sr[2], Si[2];
 #pragma unroll
     for (int tt = 0; tt < 2; ++tt) {
-      u4 ar[NP], ai[NP];
-#pragma unroll
-      for (int q = 0; q < NP; ++q) {
-        ar[q] = s.cs_r[q][xrec(16 * tt + dl, g, XT)];
-        ai[q] = s.cs_i[q][xrec(16 * tt + dl, g, XT)];
-      }
-      Sr[tt] = xmm<NP>(ar, hk, f4{0, 0, 0, 0});
-      Si[tt] = xmm<NP>(ai, hk, f4{0, 0, 0, 0});
+      Sr[tt] = xmm<NP>(c_r[tt], hk, f4{0, 0, 0, 0});
+      Si[tt] = xmm<NP>(c_i[tt], hk, f4{0, 0, 0, 0});
     }
-    // ---- H += B^T V  (rows n, K slot (g, e) <-> timestep t(g, e))
     {
-      u4 ar[NP], ai[NP], an[NP];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const bool keep = 4 * g + i <= g_lim;
+        ggr[i] = keep ? ggr[i] : 0.0f;
+        ggi[i] = keep ? ggi[i] : 0.0f;
+      }
+      uint32_t r0[NP], r1[NP], j0[NP], j1[NP];
+      split2<NP>(sk, ggr[0], ggr[1], r0);
+      split2<NP>(sk, ggr[2], ggr[3], r1);
+      split2<NP>(sk, ggi[0], ggi[1], j0);
+      split2<NP>(sk, ggi[2], ggi[3], j1);
+      const int h = xrec(16 * gtt + dl, g, XT) * 2 + gst;   // 8-byte half-record index
 #pragma unroll
       for (int q = 0; q < NP; ++q) {
-        ar[q] = s.bt_r[q][xrec(dl, g, XN)];
-        ai[q] = s.bt_i[q][xrec(dl, g, XN)];
-        an[q] = s.bt_ni[q][xrec(dl, g, XN)];
+        reinterpret_cast<u2*>(Gn.re[q])[h] = u2{r0[q], r1[q]};
+        reinterpret_cast<u2*>(Gn.im[q])[h] = u2{j0[q], j1[q]};
       }
-      Hr = xmm<NP>(ar, pc.vr, Hr);
-      Hi = xmm<NP>(ar, pc.vi, Hi);
-      Hr = xmm<NP>(an, pc.vi, Hr);
-      Hi = xmm<NP>(ai, pc.vr, Hi);
     }
-    // ---- S += G.V
+    float w[8], ph[8];
+    {
+#pragma unroll
+      for (int st = 0; st < 2; ++st) {
+        const bool ok = (c + 1) * XT + 16 * st + 4 * g < L;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) w[4 * st + i] = ok ? in1.de[st][i] * in1.u[st][i] : 0.0f;
+        th[st][1] += th[st][0]; th[st][2] += th[st][1]; th[st][3] += th[st][2];
+        pn.u[st] = in1.u[st];
+        if (GATED) pn.z[st] = in1.z[st];
+      }
+      // exclusive offsets over the order (st 0: g 0..3), (st 1: g 0..3)
+      float sa = th[0][3], sb = th[1][3];
+      float ta = __shfl_up(sa, 16), tb = __shfl_up(sb, 16);
+      if (g >= 1) { sa += ta; sb += tb; }
+      ta = __shfl_up(sa, 32); tb = __shfl_up(sb, 32);
+      if (g >= 2) { sa += ta; sb += tb; }
+      const float tot_a = __shfl(sa, 48 + dl);
+      const float off_a = sa - th[0][3];
+      const float off_b = tot_a + sb - th[1][3];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ph[e] = th[e >> 2][e & 3] + ((e >> 2) ? off_b : off_a);
+    }
+    float* pcs = &pn.cs[0][0];
+    float* psn = &pn.sn[0][0];
+#pragma unroll
+    for (int e = 0; e < 2; ++e) { sincos_small(ph[e], &psn[e], &pcs[e]); touch_vgpr(psn[e]); touch_vgpr(pcs[e]); }
+    u4 b_r[NP], b_i[NP];
+#pragma unroll
+    for (int q = 0; q < NP; ++q) {
+      b_r[q] = s.bt_r[q][xrec(dl, g, XN)];
+      b_i[q] = s.bt_i[q][xrec(dl, g, XN)];
+    }
+    XDL_REGION(4 * NPP, 7);
+
+    // ---- region 3: H += B^T V  |  remaining rotations of chunk c + 1
+#pragma unroll
+    for (int e = 2; e < 8; ++e) pin(ph[e]);
+    {
+      auto quantum = [&](auto ec) {
+        constexpr int e = decltype(ec)::value;          // 2..7
+        constexpr int k = e - 2;                        // product index 0..5 (NP = 3), clipped below
+        sincos_small(ph[e], &psn[e], &pcs[e]);
+        touch_vgpr(psn[e]); touch_vgpr(pcs[e]);
+        if constexpr (k < NPP) {
+          Hr = xmm_k<NP, k>(b_r, pc.vr, Hr);
+          Hi = xmm_k<NP, k>(b_r, pc.vi, Hi);
+          Hr = xmm_k<NP, k>(b_i, pc.nvi, Hr);
+          Hi = xmm_k<NP, k>(b_i, pc.vr, Hi);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      };
+      quantum(std::integral_constant<int, 2>{}); quantum(std::integral_constant<int, 3>{});
+      quantum(std::integral_constant<int, 4>{}); quantum(std::integral_constant<int, 5>{});
+      quantum(std::integral_constant<int, 6>{}); quantum(std::integral_constant<int, 7>{});
+    }
+    u4 g_r[2][NP], g_i[2][NP];
+#pragma unroll
+    for (int q = 0; q < NP; ++q) {
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt) {
+        g_r[tt][q] = G.re[q][xrec(16 * tt + dl, g, XT)];
+        g_i[tt][q] = G.im[q][xrec(16 * tt + dl, g, XT)];
+      }
+    }
+    XDL_REGION(4 * NPP, 6);
+
+    // ---- region 4: S += G.V  |  rotated inputs of chunk c + 1 (split), state rotation
+#pragma unroll
+    for (int e = 0; e < 8; ++e) pin(w[e]);
 #pragma unroll
     for (int tt = 0; tt < 2; ++tt) {
-      u4 ar[NP], ai[NP], an[NP];
-#pragma unroll
-      for (int q = 0; q < NP; ++q) {
-        ar[q] = G.re[q][xrec(16 * tt + dl, g, XT)];
-        ai[q] = G.im[q][xrec(16 * tt + dl, g, XT)];
-        an[q] = G.nim[q][xrec(16 * tt + dl, g, XT)];
-      }
-      Sr[tt] = xmm<NP>(ar, pc.vr, Sr[tt]);
-      Si[tt] = xmm<NP>(ar, pc.vi, Si[tt]);
-      Sr[tt] = xmm<NP>(an, pc.vi, Sr[tt]);
-      Si[tt] = xmm<NP>(ai, pc.vr, Si[tt]);
+      Sr[tt] = xmm<NP>(g_r[tt], pc.vr, Sr[tt]);
+      Si[tt] = xmm<NP>(g_r[tt], pc.vi, Si[tt]);
+      Sr[tt] = xmm<NP>(g_i[tt], pc.nvi, Sr[tt]);
+      Si[tt] = xmm<NP>(g_i[tt], pc.vr, Si[tt]);
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -412,8 +541,26 @@ __global__ __launch_bounds__(256) void unitary_fwd_xdl_kernel(const FwdArgs p) {
       Hr[i] = pc.cT * xr - pc.sT * xi;
       Hi[i] = fmaf(pc.cT, xi, pc.sT * xr);
     }
-    // ---- vector work of the next chunk (independent of everything above)
-    prep_rest(in1, c + 1, th, pn);
+    {
+      float vr[8], vi[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        vr[e] = pcs[e] * w[e];
+        vi[e] = -psn[e] * w[e];
+      }
+      split8<NP>(sk, vr, pn.vr);
+      split8<NP>(sk, vi, pn.vi);
+#pragma unroll
+      for (int q = 0; q < NP; ++q) pn.nvi[q] = neg_bf16x8(pn.vi[q]);
+      // rotation over the whole chunk: the element (st 1, g 3, i 3) is timestep 31
+      pn.cT = __shfl(pcs[7], 48 + dl);
+      pn.sT = __shfl(psn[7], 48 + dl);
+#pragma unroll
+      for (int q = 0; q < NP; ++q)
+#pragma unroll
+        for (int k = 0; k < 4; ++k) { touch_vgpr(__uint_as_float(pn.vr[q][k])); touch_vgpr(__uint_as_float(pn.nvi[q][k])); }
+    }
+    XDL_REGION(8 * NPP, 3);
 
     // ---- outputs: rows 16 tt + 4 g + i of channel dl are this lane's own timesteps
     f4 yo[2];
@@ -427,12 +574,6 @@ __global__ __launch_bounds__(256) void unitary_fwd_xdl_kernel(const FwdArgs p) {
         yo[tt][i] = v;
       }
     }
-    // The loads issued at the top have had a whole chunk to land: collect them here, before the
-    // stores below join the same in-order queue.
-#pragma unroll
-    for (int k = 0; k < 4; ++k) { touch_vgpr(m1_raw[k].x); touch_vgpr(m1_raw[k].y); }
-    touch4(m2_raw[0]); touch4(m2_raw[1]);
-    in_touch(in2);
     if (p.y && dok) {
 #pragma unroll
       for (int tt = 0; tt < 2; ++tt) {
@@ -457,6 +598,7 @@ __global__ __launch_bounds__(256) void unitary_fwd_xdl_kernel(const FwdArgs p) {
     const int tmp = i0; i0 = i1; i1 = i2; i2 = tmp;
     __syncthreads();
   };
+#undef XDL_REGION
 
   // ---- prologue
   In inA, inB;
