@@ -13,6 +13,7 @@
 #include "scan_fwd.h"
 #include "scan_fwd_mfma.h"
 #include "scan_fwd_xdl.h"
+#include "scan_fwd_xdl2.h"
 
 using namespace aussm;
 
@@ -75,11 +76,18 @@ int launch_fwd_t(const FwdArgs& a, hipStream_t s) {
   return AUSSM_E_SHAPE;
 }
 
-// The matrix-core forward kernel covers the common unitary case; everything else takes the
-// generic kernel.  AUSSM_MFMA (environment) selects for comparisons: 0 generic kernel, 1 fp32
-// matrix instructions, 2 / 3 bf16 matrix instructions on two / three-piece operands (default 3).
+// The matrix-core kernels cover the common unitary case (fp32 inputs, N <= 16, L a multiple of 4,
+// 16-byte aligned tensors, checkpoint interval a multiple of 32); everything else takes the
+// generic kernels.  AUSSM_MFMA (environment, read at every call) selects the forward kernel for
+// comparisons: 0 generic, 1 fp32 matrix instructions, 2 / 3 bf16 matrix instructions on two- /
+// three-piece operands with one wavefront per SIMD (3 is the default), 4 three-piece operands with
+// two wavefronts per SIMD.  AUSSM_MFMA_BWD: 0 generic, 2 / 3 pieces (default 3).
+inline int env_mode(const char* name, int dflt) {
+  const char* e = getenv(name);
+  return e ? atoi(e) : dflt;
+}
 inline int mfma_fwd_mode(const FwdArgs& a, int in_dtype) {
-  static const int mode = [] { const char* e = getenv("AUSSM_MFMA"); return e ? atoi(e) : 3; }();
+  const int mode = env_mode("AUSSM_MFMA", 3);
   if (mode <= 0 || in_dtype != AUSSM_F32 || a.N > MN || a.L % 4 != 0 || a.ck % MT != 0) return 0;
   if (misaligned(a.u, 16) || misaligned(a.delta, 16) || misaligned(a.theta, 16) || misaligned(a.z, 16) ||
       misaligned(a.y, 16) || misaligned(a.Bm, 16) || misaligned(a.Cm, 16))
@@ -97,6 +105,9 @@ int launch_fwd(const FwdArgs& a, int in_dtype, hipStream_t s) {
     } else if (mode == 2) {
       if (a.z) hipLaunchKernelGGL((unitary_fwd_xdl_kernel<2, true>), grid, dim3(256), 0, s, a);
       else hipLaunchKernelGGL((unitary_fwd_xdl_kernel<2, false>), grid, dim3(256), 0, s, a);
+    } else if (mode == 4) {
+      if (a.z) hipLaunchKernelGGL((unitary_fwd_xdl2_kernel<3, true>), grid, dim3(512), 0, s, a);
+      else hipLaunchKernelGGL((unitary_fwd_xdl2_kernel<3, false>), grid, dim3(512), 0, s, a);
     } else {
       if (a.z) hipLaunchKernelGGL((unitary_fwd_xdl_kernel<3, true>), grid, dim3(256), 0, s, a);
       else hipLaunchKernelGGL((unitary_fwd_xdl_kernel<3, false>), grid, dim3(256), 0, s, a);
@@ -222,8 +233,7 @@ int aussm_unitary_bwd(const float* dy, const float* dhL, const void* u, const vo
   a.dy = dy; a.dhL = dhL; a.u = u; a.delta = delta; a.theta = theta; a.Bm = Bc; a.Cm = Cc; a.Dskip = Dskip;
   a.hck = hck; a.du = du; a.ddelta = ddelta; a.dtheta = dtheta; a.dB = dB; a.dC = dC; a.dD = dD; a.dh0 = dh0;
   a.B = B; a.D = D; a.N = N; a.L = L; a.ck = ck; a.nck = (L + ck - 1) / ck; a.ncg = (D + CH - 1) / CH;
-  // matrix-core kernel for the common case (AUSSM_MFMA_BWD: 0 generic kernel, 2 / 3 operand pieces)
-  static const int mode = [] { const char* e = getenv("AUSSM_MFMA_BWD"); return e ? atoi(e) : 3; }();
+  const int mode = env_mode("AUSSM_MFMA_BWD", 3);   // matrix-core kernel for the common case
   if (mode > 0 && in_dtype == AUSSM_F32 && N <= XN && L % 4 == 0 && ck % XT == 0 &&
       !(misaligned(dy, 16) || misaligned(u, 16) || misaligned(delta, 16) || misaligned(theta, 16) ||
         misaligned(du, 16) || misaligned(ddelta, 16) || misaligned(dtheta, 16) || misaligned(Bc, 16) ||

@@ -1,0 +1,97 @@
+"""Every unitary kernel of the library against the CPU oracle on the same inputs.
+
+The launcher picks a matrix-core kernel for the common case (float32 inputs, N <= 16, L a multiple
+of 4, aligned tensors) and the generic kernel otherwise; AUSSM_MFMA / AUSSM_MFMA_BWD (environment,
+read at every call) force one of them.  Each mode must meet the float32 tolerance of the benchmark
+contract, atol = rtol = 1e-4 after normalising by the largest magnitude of the expected tensor, on
+shapes that exercise a partial channel group, a partial last chunk, N < 16, a carried-in state, the
+output gate and phases large enough to take the range-reduction path."""
+import os
+
+import pytest
+import torch
+
+from oracle import scan_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+FWD_MODES = ["0", "1", "2", "3", "4"]     # generic, fp32 matrix, bf16 x2 pieces, bf16 x3 pieces, two waves per SIMD
+BWD_MODES = ["0", "2", "3"]               # generic, two pieces, three pieces
+SHAPES = [(2, 80, 16, 200), (1, 64, 5, 36), (2, 128, 16, 512)]
+NAMES = ("u", "delta", "theta", "Bc", "Cc", "Dskip")
+
+
+def _close(got, want, what, tol=1e-4):
+    if want.is_complex():
+        got, want = torch.view_as_real(got), torch.view_as_real(want)
+    scale = max(1.0, float(want.abs().max()))
+    torch.testing.assert_close(got.cpu().float() / scale, want.float() / scale, atol=tol, rtol=tol,
+                               msg=lambda m: f"{what}: {m}")
+
+
+class _Env:
+    def __init__(self, **kv):
+        self.kv = kv
+
+    def __enter__(self):
+        self.old = {k: os.environ.get(k) for k in self.kv}
+        os.environ.update(self.kv)
+
+    def __exit__(self, *a):
+        for k, v in self.old.items():
+            if v is None:
+                os.environ.pop(k, None)
+            else:
+                os.environ[k] = v
+
+
+def _inputs(B, D, N, L, seed, big_theta):
+    p = O.make_core_inputs(B, D, N, L, seed=seed, gate=True)
+    if big_theta:
+        p["theta"] = p["theta"] * 20.0          # |theta| up to ~40 rad: range reduction inside the kernels
+    g = torch.Generator().manual_seed(seed + 1)
+    p["h0"] = torch.complex(torch.randn(B, D, N, generator=g), torch.randn(B, D, N, generator=g))
+    return p
+
+
+@pytest.mark.parametrize("mode", FWD_MODES)
+@pytest.mark.parametrize("B,D,N,L", SHAPES)
+@pytest.mark.parametrize("big_theta", [False, True])
+def test_forward_modes(mode, B, D, N, L, big_theta):
+    from aussm_amd import scan
+    p = _inputs(B, D, N, L, 11 + B + D + L, big_theta)
+    want_y, want_h = O.unitary_core_loop(p["u"], p["delta"], p["theta"], p["Bc"], p["Cc"], p["Dskip"], p["z"], p["h0"])
+    q = {k: v.cuda() for k, v in p.items()}
+    print(f"case fwd mode={mode} B={B} D={D} N={N} L={L} big={big_theta}", flush=True)
+    with _Env(AUSSM_MFMA=mode):
+        y, hL = scan.unitary_scan(q["u"], q["delta"], q["theta"], q["Bc"], q["Cc"], q["Dskip"], q["z"], q["h0"],
+                                  return_last_state=True)
+        torch.cuda.synchronize()
+    _close(y, want_y, "y")
+    _close(hL, want_h, "hL")
+
+
+@pytest.mark.parametrize("mode", BWD_MODES)
+@pytest.mark.parametrize("B,D,N,L", SHAPES)
+@pytest.mark.parametrize("big_theta", [False, True])
+def test_backward_modes(mode, B, D, N, L, big_theta):
+    from aussm_amd import scan
+    p = _inputs(B, D, N, L, 23 + B + D + L, big_theta)
+    g = torch.Generator().manual_seed(5)
+    dh = torch.complex(torch.randn(B, D, N, generator=g), torch.randn(B, D, N, generator=g))
+
+    def run(fn, dev):
+        lv = [p[k].clone().to(dev).requires_grad_(True) for k in NAMES]
+        h0 = p["h0"].clone().to(dev).requires_grad_(True)
+        y, hL = fn(*lv, None, h0)
+        loss = (y * p["dy"].to(dev)).sum() + (torch.view_as_real(hL) * torch.view_as_real(dh.to(dev))).sum()
+        loss.backward()
+        return [t.grad for t in lv] + [h0.grad]
+
+    want = run(lambda *a: O.unitary_core_loop(*a), "cpu")
+    print(f"case bwd mode={mode} B={B} D={D} N={N} L={L} big={big_theta}", flush=True)
+    with _Env(AUSSM_MFMA_BWD=mode):
+        got = run(lambda *a: scan.unitary_scan(*a, return_last_state=True), "cuda")
+        torch.cuda.synchronize()
+    for k, w, gt in zip(NAMES + ("h0",), want, got):
+        _close(gt, w, f"d{k}", tol=2e-4 if big_theta else 1e-4)
