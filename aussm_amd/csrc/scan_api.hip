@@ -81,7 +81,8 @@ int launch_fwd_t(const FwdArgs& a, hipStream_t s) {
 // generic kernels.  AUSSM_MFMA (environment, read at every call) selects the forward kernel for
 // comparisons: 0 generic, 1 fp32 matrix instructions, 2 / 3 bf16 matrix instructions on two- /
 // three-piece operands with one wavefront per SIMD (3 is the default), 4 three-piece operands with
-// two wavefronts per SIMD.  AUSSM_MFMA_BWD: 0 generic, 2 / 3 pieces (default 3).
+// two wavefronts per SIMD.  AUSSM_MFMA_BWD: 0 generic, 2 two pieces everywhere, 3 (default) three
+// pieces along the sequence and two in the sums over the channel (dB, dC), 5 three pieces everywhere.
 inline int env_mode(const char* name, int dflt) {
   const char* e = getenv(name);
   return e ? atoi(e) : dflt;
@@ -239,8 +240,9 @@ int aussm_unitary_bwd(const float* dy, const float* dhL, const void* u, const vo
         misaligned(du, 16) || misaligned(ddelta, 16) || misaligned(dtheta, 16) || misaligned(Bc, 16) ||
         misaligned(Cc, 16))) {
     const dim3 grid((unsigned)(a.B * a.ncg));
-    if (mode == 2) hipLaunchKernelGGL(unitary_bwd_xdl_kernel<2>, grid, dim3(256), 0, s, a);
-    else hipLaunchKernelGGL(unitary_bwd_xdl_kernel<3>, grid, dim3(256), 0, s, a);
+    if (mode == 2) hipLaunchKernelGGL((unitary_bwd_xdl_kernel<2, 2>), grid, dim3(256), 0, s, a);
+    else if (mode == 5) hipLaunchKernelGGL((unitary_bwd_xdl_kernel<3, 3>), grid, dim3(256), 0, s, a);
+    else hipLaunchKernelGGL((unitary_bwd_xdl_kernel<3, 2>), grid, dim3(256), 0, s, a);
     return launch_status();
   }
   return in_dtype == AUSSM_BF16 ? launch_unitary_bwd_t<bf16_t>(a, s) : launch_unitary_bwd_t<float>(a, s);

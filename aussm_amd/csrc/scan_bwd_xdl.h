@@ -85,7 +85,9 @@ __device__ __forceinline__ void ldrec16(const u4 (*plane)[XN * 4], int idx, u4 (
 }
 
 // Requires: N <= 16, L % 4 == 0, 16-byte aligned tensors, ck % 32 == 0, float inputs.
-template <int NP>
+// NP: operand pieces of the products along the sequence (3 = fp32-accurate); NPC: pieces of the
+// products that sum over the channel (M, X1, X2 and the two closing products of dB / dC).
+template <int NP, int NPC>
 __global__ __launch_bounds__(256) void unitary_bwd_xdl_kernel(const UniBwdArgs p) {
   __shared__ XbBC<NP> s_bc;
   __shared__ XbG<NP> s_g;
@@ -276,6 +278,10 @@ __global__ __launch_bounds__(256) void unitary_bwd_xdl_kernel(const UniBwdArgs p
     }
   }
   float accD = 0.0f;
+  // dB / dC output: lane (at_n, at_x) of a closing wavefront adds element (row n = 2 k + at_n,
+  // timestep at_x / 2, part at_x % 2) of its tile, k = 0..7
+  const int at_n = lane >> 5, at_x = lane & 31;
+  const size_t at_off = (((size_t)b * N + at_n) * L + 16 * (wave & 1) + (at_x >> 1)) * 2 + (at_x & 1);
 
   In inA, inB;
   bc_load(nchunks - 1);
@@ -406,34 +412,45 @@ __global__ __launch_bounds__(256) void unitary_bwd_xdl_kernel(const UniBwdArgs p
         thr[o] = Hr[i]; thi[o] = Hi[i]; tjr[o] = Jr[i]; tji[o] = Ji[i];
       }
       __builtin_amdgcn_wave_barrier();
-      auto rec_t = [&](const float* re, const float* im, int tile, u4 (&o)[NP]) {
+      auto rec_t = [&](const float* re, const float* im, int tile, u4 (&o)[NPC]) {
         const f4 a = *reinterpret_cast<const f4*>(re + (g * XB_TS + 16 * tile + dl) * 4);
         const f4 bq = *reinterpret_cast<const f4*>(im + (g * XB_TS + 16 * tile + dl) * 4);
         const float x[8] = {a[0], a[1], a[2], a[3], bq[0], bq[1], bq[2], bq[3]};
-        split8<NP>(sk, x, o);
+        split8<NPC>(sk, x, o);
       };
-      auto rec_n = [&](const float* re, const float* im, u4 (&o)[NP]) {
+      auto rec_n = [&](const float* re, const float* im, u4 (&o)[NPC]) {
         const f4 a = *reinterpret_cast<const f4*>(re + (g * XB_NS + dl) * 4);
         const f4 bq = *reinterpret_cast<const f4*>(im + (g * XB_NS + dl) * 4);
         const float x[8] = {a[0], a[1], a[2], a[3], bq[0], bq[1], bq[2], bq[3]};
-        split8<NP>(sk, x, o);
+        split8<NPC>(sk, x, o);
       };
-      u4 Q0[NP], Q1[NP], V0[NP], V1[NP], V0i[NP], V1i[NP], Hc[NP], Hci[NP], Jc[NP], Jci[NP];
-      rec_t(tqr, tqi, 0, Q0); rec_t(tqr, tqi, 1, Q1);
-      rec_t(tvr, tvi, 0, V0); rec_t(tvr, tvi, 1, V1);
-      rec_n(thr, thi, Hc); rec_n(tjr, tji, Jc);
-      rot_i<NP>(V0, V0i); rot_i<NP>(V1, V1i);    // [-Vi, Vr]
-      rot_i<NP>(Hc, Hci);                        // [-Hi, Hr]
-      rot_mi<NP>(Jc, Jci);                       // [ Ji, -Jr]
+      // Products in an order that keeps few operand records alive at a time.
       const f4 z = {0, 0, 0, 0};
       f4 pj[XB_JOBS];
-      pj[0] = xmm<NP>(Q0, V0, z);  pj[1] = xmm<NP>(Q0, V0i, z);     // M tile (0,0): lane col s, rows t
-      pj[2] = xmm<NP>(Q1, V0, z);  pj[3] = xmm<NP>(Q1, V0i, z);     // M tile (1,0)
-      pj[4] = xmm<NP>(Q1, V1, z);  pj[5] = xmm<NP>(Q1, V1i, z);     // M tile (1,1)
-      pj[6] = xmm<NP>(Q0, Hc, z);  pj[7] = xmm<NP>(Q0, Hci, z);     // X1 tile 0: lane col n, rows t
-      pj[8] = xmm<NP>(Q1, Hc, z);  pj[9] = xmm<NP>(Q1, Hci, z);     // X1 tile 1
-      pj[10] = xmm<NP>(V0, Jc, z); pj[11] = xmm<NP>(V0, Jci, z);    // X2 tile 0: lane col n, rows s
-      pj[12] = xmm<NP>(V1, Jc, z); pj[13] = xmm<NP>(V1, Jci, z);    // X2 tile 1
+      {
+        u4 Q0[NPC], V0[NPC], V0i[NPC], Jc[NPC], Jci[NPC];
+        rec_t(tqr, tqi, 0, Q0);
+        rec_t(tvr, tvi, 0, V0);
+        rot_i<NPC>(V0, V0i);                        // [-Vi, Vr]
+        pj[0] = xmm<NPC>(Q0, V0, z);  pj[1] = xmm<NPC>(Q0, V0i, z);     // M tile (0,0): lane col s, rows t
+        rec_n(tjr, tji, Jc);
+        rot_mi<NPC>(Jc, Jci);                       // [ Ji, -Jr]
+        pj[10] = xmm<NPC>(V0, Jc, z); pj[11] = xmm<NPC>(V0, Jci, z);    // X2 tile 0: lane col n, rows s
+        {
+          u4 Hc[NPC], Hci[NPC], Q1[NPC];
+          rec_n(thr, thi, Hc);
+          rot_i<NPC>(Hc, Hci);                      // [-Hi, Hr]
+          pj[6] = xmm<NPC>(Q0, Hc, z);  pj[7] = xmm<NPC>(Q0, Hci, z);   // X1 tile 0: lane col n, rows t
+          rec_t(tqr, tqi, 1, Q1);
+          pj[8] = xmm<NPC>(Q1, Hc, z);  pj[9] = xmm<NPC>(Q1, Hci, z);   // X1 tile 1
+          pj[2] = xmm<NPC>(Q1, V0, z);  pj[3] = xmm<NPC>(Q1, V0i, z);   // M tile (1,0)
+          u4 V1[NPC], V1i[NPC];
+          rec_t(tvr, tvi, 1, V1);
+          rot_i<NPC>(V1, V1i);
+          pj[4] = xmm<NPC>(Q1, V1, z);  pj[5] = xmm<NPC>(Q1, V1i, z);   // M tile (1,1)
+          pj[12] = xmm<NPC>(V1, Jc, z); pj[13] = xmm<NPC>(V1, Jci, z);  // X2 tile 1
+        }
+      }
       // causal mask of the diagonal M tiles: keep rows t = 4 g + i >= column s = dl
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
@@ -555,34 +572,33 @@ __global__ __launch_bounds__(256) void unitary_bwd_xdl_kernel(const UniBwdArgs p
       }
       const float* mre = s_ms[isC ? 0 : 2] + (16 * tile + dl) * XB_MS;
       const float* mim = s_ms[isC ? 1 : 3] + (16 * tile + dl) * XB_MS;
-      u4 mr[NP], mi[NP], nmr[NP], er[NP], ei[NP];
+      u4 mr[NPC], mi[NPC], nmr[NPC], er[NPC], ei[NPC];
       {
         const f4 a = *reinterpret_cast<const f4*>(mre + 4 * g), a2 = *reinterpret_cast<const f4*>(mre + 16 + 4 * g);
         const f4 c2 = *reinterpret_cast<const f4*>(mim + 4 * g), c3 = *reinterpret_cast<const f4*>(mim + 16 + 4 * g);
         const float x[8] = {a[0], a[1], a[2], a[3], a2[0], a2[1], a2[2], a2[3]};
         const float y[8] = {c2[0], c2[1], c2[2], c2[3], c3[0], c3[1], c3[2], c3[3]};
-        split8<NP>(sk, x, mr);
-        split8<NP>(sk, y, mi);
-        nega<NP>(mr, nmr);
+        split8<NPC>(sk, x, mr);
+        split8<NPC>(sk, y, mi);
+        nega<NPC>(mr, nmr);
       }
-      ldrec16<NP>(isC ? s_bc.bt_r : s_bc.ct_r, xrec(dl, g, XN), er);
-      ldrec16<NP>(isC ? s_bc.bt_i : s_bc.ct_i, xrec(dl, g, XN), ei);
-      xr = xmm<NP>(mr, er, xr);  xr = xmm<NP>(mi, ei, xr);
-      xi = xmm<NP>(mi, er, xi);  xi = xmm<NP>(nmr, ei, xi);
+      ldrec16<NPC>(isC ? s_bc.bt_r : s_bc.ct_r, xrec(dl, g, XN), er);
+      ldrec16<NPC>(isC ? s_bc.bt_i : s_bc.ct_i, xrec(dl, g, XN), ei);
+      xr = xmm<NPC>(mr, er, xr);  xr = xmm<NPC>(mi, ei, xr);
+      xi = xmm<NPC>(mi, er, xi);  xi = xmm<NPC>(nmr, ei, xi);
       // Through a small LDS tile so that one atomic instruction covers two whole rows n of the
       // tile (16 timesteps x (re, im) = one 128-byte line each) instead of sixteen lines.
       float* __restrict__ at = s_at[wave];
       *reinterpret_cast<f4*>(at + dl * XB_AS + 8 * g) = f4{xr[0], xi[0], xr[1], xi[1]};
       *reinterpret_cast<f4*>(at + dl * XB_AS + 8 * g + 4) = f4{xr[2], xi[2], xr[3], xi[3]};
       __builtin_amdgcn_wave_barrier();
-      float* __restrict__ dst = isC ? p.dC : p.dB;
-      const int an = lane >> 5, ax = lane & 31;
-      const int l = l0 + 16 * tile + (ax >> 1);
+      float* __restrict__ dst = (isC ? p.dC : p.dB) + at_off + (size_t)l0 * 2;
+      const bool lok = l0 + 16 * tile + (at_x >> 1) < L;
 #pragma unroll
       for (int k = 0; k < 8; ++k) {
-        const int n = 2 * k + an;
-        const float v = at[n * XB_AS + ax];
-        if (n < N && l < L) atomicAdd(dst + (((size_t)b * N + n) * L + l) * 2 + (ax & 1), v);
+        const int n = 2 * k + at_n;
+        const float v = at[n * XB_AS + at_x];
+        if (n < N && lok) atomicAdd(dst + (size_t)k * 4 * L, v);
       }
     }
     // ---- next chunk: its end state is this chunk's start state (or the stored checkpoint)

@@ -363,7 +363,10 @@ __global__ __launch_bounds__(256) void unitary_fwd_xdl_kernel(const FwdArgs p) {
 
   int i0 = 0, i1 = 1, i2 = 2;   // LDS slots of chunks c, c+1, c+2
   const int ck_chunks = p.ck / XT;
-  int ck_left = ck_chunks, kb = 0;   // chunks to the next checkpoint, its index
+  int ck_left = ck_chunks;           // chunks to the next checkpoint
+  // this lane's rows n = 4 g .. 4 g + 3 of checkpoint 0; one checkpoint further = N * 2 * D floats
+  float* __restrict__ hck_ptr = p.hck ? p.hck + (((size_t)b * p.nck * N + 4 * g) * 2) * D + dc : nullptr;
+  const size_t hck_stride = (size_t)N * 2 * D;
 
   // One chunk.  pc: vector work of chunk c (ready); pn: receives that of chunk c + 1, computed from
   // in1 while the matrix pipe works; in2 receives the loads of chunk c + 2.
@@ -586,15 +589,13 @@ __global__ __launch_bounds__(256) void unitary_fwd_xdl_kernel(const FwdArgs p) {
     if (p.hck && dok && ck_now) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const int n = 4 * g + i;
-        if (n < N) {
-          const size_t o = ((((size_t)b * p.nck + kb) * N + n) * 2) * D + d;
-          p.hck[o] = Hr[i];
-          p.hck[o + D] = Hi[i];
+        if (4 * g + i < N) {
+          hck_ptr[(size_t)i * 2 * D] = Hr[i];
+          hck_ptr[(size_t)i * 2 * D + D] = Hi[i];
         }
       }
     }
-    if (ck_now) { ck_left = ck_chunks; ++kb; }
+    if (ck_now) { ck_left = ck_chunks; hck_ptr += hck_stride; }
     const int tmp = i0; i0 = i1; i1 = i2; i2 = tmp;
     __syncthreads();
   };

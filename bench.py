@@ -11,7 +11,10 @@ resident in HBM.  Prints ONE JSON line.
   value          (b,d,l) samples per second over forward+backward (B*D*L / step time)
   roofline       dominant kernel (the backward scan): algorithmic bytes (28E + 32S + 4D,
                  E = B*D*L, S = B*N*L) / its average launch duration, measured here with HIP
-                 events on the launch stream, against the 8 TB/s HBM peak
+                 events on the launch stream, against the 8 TB/s HBM peak.  "traffic" is the HBM
+                 bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE passes over this same
+                 script (profiles/), scaled by what the counters read for the 256 MiB device copy
+                 that --copy-probe adds to the run; it is a recorded figure, not measured live.
   cpu_baseline   the CPU oracle (sequential-loop PyTorch scan + autograd) timed on this host's
                  cores on a bounded slice of the batch
 """
@@ -28,6 +31,11 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 SHAPE = dict(B=32, D=512, N=16, L=2048)
+# HBM bytes per launch at SHAPE from the counter passes summarised in
+# profiles/unitary_fwd_bwd_B32_D512_N16_L2048_hbm_traffic.md (FETCH_SIZE x 2.00, WRITE_SIZE x 1.00 after
+# calibration on a 256 MiB copy): forward 426 MB read + 151 MB written, backward 576 MB read +
+# 550 MB written (the dB/dC atomics of the eight workgroups of a batch element count as writes).
+TRAFFIC_BYTES = {"unitary_fwd": 577e6, "unitary_bwd": 1126e6}
 
 
 def cpu_baseline(B_sample: int):
@@ -61,6 +69,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-batch", type=int, default=8)
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run one 256 MiB device-to-device copy (calibrates FETCH_SIZE / WRITE_SIZE under rocprofv3)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus must be 1 (no multi-GPU path exists)", file=sys.stderr)
@@ -125,6 +135,12 @@ def main():
         torch.cuda.synchronize()
         return sum(s.elapsed_time(e) for s, e in evs) / reps * 1e3
 
+    if args.copy_probe:
+        src = torch.empty(64 * 1024 * 1024, **f32).normal_()
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     reps = max(10, min(args.steps, 50))
     t_fwd = kernel_us(fwd_only, reps)
     t_bwd = kernel_us(bwd_only, reps)
@@ -152,11 +168,13 @@ def main():
         "fwd_bwd_algorithmic_GBps": (bytes_fwd + bytes_bwd) / ((t_fwd + t_bwd) * 1e-6) / 1e9,
         "fwd_bwd_frac_of_hbm_peak": (bytes_fwd + bytes_bwd) / ((t_fwd + t_bwd) * 1e-6) / 1e9 / HBM_PEAK_GBS,
         "kernels_us": {"unitary_fwd": t_fwd, "unitary_bwd": t_bwd},
-        "roofline": {"bound": "hbm", "kernel": "unitary_bwd_kernel", "achieved": ach, "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": ach / HBM_PEAK_GBS, "traffic": None,
+        "roofline": {"bound": "hbm", "kernel": "unitary_bwd_xdl_kernel<3>", "achieved": ach, "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": ach / HBM_PEAK_GBS, "traffic": TRAFFIC_BYTES["unitary_bwd"],
                      "algorithmic_bytes": bytes_bwd,
-                     "fwd_kernel": {"achieved": bytes_fwd / (t_fwd * 1e-6) / 1e9,
+                     "fwd_kernel": {"kernel": "unitary_fwd_xdl_kernel<3, false>",
+                                    "achieved": bytes_fwd / (t_fwd * 1e-6) / 1e9,
                                     "frac": bytes_fwd / (t_fwd * 1e-6) / 1e9 / HBM_PEAK_GBS,
+                                    "traffic": TRAFFIC_BYTES["unitary_fwd"],
                                     "algorithmic_bytes": bytes_fwd}},
     }
     if not args.no_cpu:
