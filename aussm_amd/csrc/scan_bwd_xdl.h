@@ -283,6 +283,23 @@ __global__ __launch_bounds__(256) void unitary_bwd_xdl_kernel(const UniBwdArgs p
   const int at_n = lane >> 5, at_x = lane & 31;
   const size_t at_off = (((size_t)b * N + at_n) * L + 16 * (wave & 1) + (at_x >> 1)) * 2 + (at_x & 1);
 
+  // dB / dC tile of the chunk starting at l_at, waiting in s_at[wave] (written by this wavefront)
+  auto flush_dbc = [&](int l_at) {
+    const float* __restrict__ at = s_at[wave];
+    float* __restrict__ dst = (wave < 2 ? p.dC : p.dB) + at_off + (size_t)l_at * 2;
+    const bool lok = l_at + 16 * (wave & 1) + (at_x >> 1) < L;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const int n = 2 * k + at_n;
+      const float v = at[n * XB_AS + at_x];
+      if (n < N && lok) atomicAdd(dst + (size_t)k * 4 * L, v);
+    }
+  };
+  // checkpoints: the chunk that starts at a multiple of ck takes its start state from the store
+  const int ck_chunks = p.ck / XT;
+  int ck_left = (nchunks - 1) % ck_chunks + 1;      // chunks down to the next multiple of ck
+  int kb_next = (nchunks - 1) / ck_chunks - 1;      // checkpoint holding the state before that chunk
+
   In inA, inB;
   bc_load(nchunks - 1);
   in_load(inA, nchunks - 1);
@@ -294,6 +311,7 @@ __global__ __launch_bounds__(256) void unitary_bwd_xdl_kernel(const UniBwdArgs p
     bc_store(c);
     bc_load(c - 1);
     in_load(nxt, c - 1);
+    if (c + 1 < nchunks) flush_dbc(l0 + XT);                           // dB / dC of the previous step
     __syncthreads();                                                   // (a) planes of chunk c visible
     make_g();
 
@@ -591,18 +609,10 @@ __global__ __launch_bounds__(256) void unitary_bwd_xdl_kernel(const UniBwdArgs p
       float* __restrict__ at = s_at[wave];
       *reinterpret_cast<f4*>(at + dl * XB_AS + 8 * g) = f4{xr[0], xi[0], xr[1], xi[1]};
       *reinterpret_cast<f4*>(at + dl * XB_AS + 8 * g + 4) = f4{xr[2], xi[2], xr[3], xi[3]};
-      __builtin_amdgcn_wave_barrier();
-      float* __restrict__ dst = (isC ? p.dC : p.dB) + at_off + (size_t)l0 * 2;
-      const bool lok = l0 + 16 * tile + (at_x >> 1) < L;
-#pragma unroll
-      for (int k = 0; k < 8; ++k) {
-        const int n = 2 * k + at_n;
-        const float v = at[n * XB_AS + at_x];
-        if (n < N && lok) atomicAdd(dst + (size_t)k * 4 * L, v);
-      }
+      // (the atomic adds themselves are issued by flush_dbc() in the next step, behind its loads)
     }
     // ---- next chunk: its end state is this chunk's start state (or the stored checkpoint)
-    if (l0 > 0 && (l0 % p.ck) == 0) load_ck(l0 / p.ck - 1);
+    if (--ck_left == 0 && l0 > 0) { load_ck(kb_next); --kb_next; ck_left = ck_chunks; }
     __syncthreads();                                                   // (d) planes, scratch and M free
   };
 
@@ -610,6 +620,7 @@ __global__ __launch_bounds__(256) void unitary_bwd_xdl_kernel(const UniBwdArgs p
     step(c, inA, inB);
     if (c >= 1) step(c - 1, inB, inA);
   }
+  flush_dbc(0);
 
   if (p.dh0 && dok) {
 #pragma unroll

@@ -33,9 +33,9 @@ HBM_PEAK_GBS = 8000.0
 SHAPE = dict(B=32, D=512, N=16, L=2048)
 # HBM bytes per launch at SHAPE from the counter passes summarised in
 # profiles/unitary_fwd_bwd_B32_D512_N16_L2048_hbm_traffic.md (FETCH_SIZE x 2.00, WRITE_SIZE x 1.00 after
-# calibration on a 256 MiB copy): forward 426 MB read + 151 MB written, backward 576 MB read +
-# 550 MB written (the dB/dC atomics of the eight workgroups of a batch element count as writes).
-TRAFFIC_BYTES = {"unitary_fwd": 577e6, "unitary_bwd": 1126e6}
+# calibration on a 256 MiB copy): forward 426 MB read + 151 MB written, backward 574 MB read +
+# 543 MB written (the dB/dC atomics of the eight workgroups of a batch element count as writes).
+TRAFFIC_BYTES = {"unitary_fwd": 577e6, "unitary_bwd": 1116e6}
 
 
 def cpu_baseline(B_sample: int):
@@ -168,7 +168,7 @@ def main():
         "fwd_bwd_algorithmic_GBps": (bytes_fwd + bytes_bwd) / ((t_fwd + t_bwd) * 1e-6) / 1e9,
         "fwd_bwd_frac_of_hbm_peak": (bytes_fwd + bytes_bwd) / ((t_fwd + t_bwd) * 1e-6) / 1e9 / HBM_PEAK_GBS,
         "kernels_us": {"unitary_fwd": t_fwd, "unitary_bwd": t_bwd},
-        "roofline": {"bound": "hbm", "kernel": "unitary_bwd_xdl_kernel<3>", "achieved": ach, "peak": HBM_PEAK_GBS,
+        "roofline": {"bound": "hbm", "kernel": "unitary_bwd_xdl_kernel<3, 2>", "achieved": ach, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": ach / HBM_PEAK_GBS, "traffic": TRAFFIC_BYTES["unitary_bwd"],
                      "algorithmic_bytes": bytes_bwd,
                      "fwd_kernel": {"kernel": "unitary_fwd_xdl_kernel<3, false>",
