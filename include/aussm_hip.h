@@ -46,7 +46,8 @@ extern "C" {
 #define AUSSM_E_DTYPE (-4)     /* unknown in_dtype                                   */
 #define AUSSM_E_ALIGN (-5)     /* a pointer is not aligned to its element size       */
 
-#define AUSSM_TILE 32          /* timesteps per staged tile; ck must be a multiple   */
+#define AUSSM_TILE 32          /* timesteps per staged tile; ck is a multiple of it, */
+                               /* or exactly AUSSM_TILE / 2                          */
 #define AUSSM_MAX_STATE 64     /* largest N accepted                                  */
 
 /* Library version (major*10000 + minor*100 + patch). No reference counterpart. */
@@ -70,6 +71,10 @@ int aussm_bwd_checkpoint_interval(int variant);
  * the device scan of extension-cpp/extension_cpp/csrc/cuda/ssm_adaptive_unitary_forward.cu:113-181
  * for a phase that is given per (b,d,l).
  * Optional (NULL allowed): Dskip, z, h0, y (NULL = states only), hL, hck.
+ * Kernel choice is internal: float32 inputs with N <= 16, L a multiple of 4, 16-byte aligned
+ * tensors and ck a multiple of AUSSM_TILE run on the matrix cores (fp32-accurate, see the
+ * kernel headers); every other accepted call runs on the vector ALU.  Results agree to
+ * rounding.  The environment variables AUSSM_MFMA / AUSSM_MFMA_BWD force one for comparisons.
  * ------------------------------------------------------------------------------------- */
 int aussm_unitary_fwd(const void* u, const void* delta, const float* theta,
                       const void* Bc, const void* Cc, const float* Dskip, const float* z,
