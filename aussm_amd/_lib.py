@@ -28,13 +28,15 @@ _SIGNATURES = {
     "aussm_bwd_checkpoint_interval": [_I],
     "aussm_unitary_fwd": [_P] * 11 + [_I] * 6 + [_P],
     "aussm_unitary_bwd": [_P] * 16 + [_I] * 6 + [_P],
+    "aussm_unitary_fwd_aux": [_P] * 12 + [_I] * 6 + [_P],
+    "aussm_unitary_bwd_aux": [_P] * 17 + [_I] * 6 + [_P],
     "aussm_complex_fwd": [_P] * 12 + [_I] * 6 + [_P],
     "aussm_complex_bwd": [_P] * 19 + [_I] * 6 + [_P],
     "aussm_real_fwd": [_P] * 8 + [_I] + [_P] * 4 + [_I] * 6 + [_P],
     "aussm_real_bwd": [_P] * 9 + [_I] + [_P] * 9 + [_I] * 6 + [_P],
 }
 
-EXPORTED = tuple(_SIGNATURES) + ("aussm_error_string",)
+EXPORTED = tuple(_SIGNATURES) + ("aussm_error_string", "aussm_unitary_aux_floats")
 
 
 class AussmError(RuntimeError):
@@ -59,6 +61,8 @@ def load() -> ctypes.CDLL:
         fn = getattr(lib, name)
         fn.argtypes = argtypes
         fn.restype = c_int
+    lib.aussm_unitary_aux_floats.argtypes = [_I, _I, _I]
+    lib.aussm_unitary_aux_floats.restype = ctypes.c_size_t
     lib.aussm_error_string.argtypes = [c_int]
     lib.aussm_error_string.restype = c_char_p
     _lib = lib

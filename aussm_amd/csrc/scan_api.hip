@@ -83,6 +83,9 @@ int launch_fwd_t(const FwdArgs& a, hipStream_t s) {
 // three-piece operands with one wavefront per SIMD (3 is the default), 4 three-piece operands with
 // two wavefronts per SIMD.  AUSSM_MFMA_BWD: 0 generic, 2 two pieces everywhere, 3 (default) three
 // pieces along the sequence and two in the sums over the channel (dB, dC), 5 three pieces everywhere.
+// marks an auxiliary buffer as NOT filled (a forward kernel that does not fill it ran)
+__global__ void aux_invalidate_kernel(float* tag) { *tag = 0.0f; }
+
 inline int env_mode(const char* name, int dflt) {
   const char* e = getenv(name);
   return e ? atoi(e) : dflt;
@@ -98,7 +101,10 @@ inline int mfma_fwd_mode(const FwdArgs& a, int in_dtype) {
 
 template <int VAR>
 int launch_fwd(const FwdArgs& a, int in_dtype, hipStream_t s) {
-  if (const int mode = (VAR == VAR_UNITARY) ? mfma_fwd_mode(a, in_dtype) : 0) {
+  const int mode = (VAR == VAR_UNITARY) ? mfma_fwd_mode(a, in_dtype) : 0;
+  if (a.aux && mode <= 1)   // this call will not fill the auxiliary buffer
+    hipLaunchKernelGGL(aux_invalidate_kernel, dim3(1), dim3(1), 0, s, a.aux + (size_t)a.B * a.D * a.L);
+  if (mode) {
     const dim3 grid((unsigned)(a.B * a.ncg));
     if (mode == 1) {
       if (a.z) hipLaunchKernelGGL(unitary_fwd_mfma_kernel<true>, grid, dim3(256), 0, s, a);
@@ -178,16 +184,28 @@ int aussm_num_checkpoints(int L, int ck) { return (L < 1 || ck < 1) ? 0 : (L + c
 
 int aussm_bwd_checkpoint_interval(int variant) { return variant == VAR_UNITARY ? 0 : REC_CK; }
 
+size_t aussm_unitary_aux_floats(int B, int D, int L) {
+  return (B < 1 || D < 1 || L < 1) ? 0 : (size_t)B * D * L + AUX_PAD;
+}
+
 int aussm_unitary_fwd(const void* u, const void* delta, const float* theta, const void* Bc, const void* Cc,
                       const float* Dskip, const float* z, const float* h0, float* y, float* hL, float* hck,
                       int B, int D, int N, int L, int ck, int in_dtype, void* stream) {
+  return aussm_unitary_fwd_aux(u, delta, theta, Bc, Cc, Dskip, z, h0, y, hL, hck, nullptr, B, D, N, L, ck, in_dtype,
+                               stream);
+}
+
+int aussm_unitary_fwd_aux(const void* u, const void* delta, const float* theta, const void* Bc, const void* Cc,
+                          const float* Dskip, const float* z, const float* h0, float* y, float* hL, float* hck,
+                          float* aux, int B, int D, int N, int L, int ck, int in_dtype, void* stream) {
   if (int e = check_common(B, D, N, L, ck, in_dtype)) return e;
+  if (misaligned(aux, 16)) return AUSSM_E_ALIGN;
   if (!u || !delta || !theta || !Bc || !Cc) return AUSSM_E_NULL;
   const size_t ca = in_dtype == AUSSM_BF16 ? 4 : 8;
   if (misaligned(Bc, ca) || misaligned(Cc, ca)) return AUSSM_E_ALIGN;
   FwdArgs a{};
   a.u = u; a.delta = delta; a.theta = theta; a.Bm = Bc; a.Cm = Cc; a.Dskip = Dskip; a.z = z;
-  a.h0 = h0; a.y = y; a.hL = hL; a.hck = hck;
+  a.h0 = h0; a.y = y; a.hL = hL; a.hck = hck; a.aux = aux;
   a.B = B; a.D = D; a.N = N; a.L = L; a.ck = ck; a.nck = (L + ck - 1) / ck; a.ncg = (D + CH - 1) / CH;
   return launch_fwd<VAR_UNITARY>(a, in_dtype, (hipStream_t)stream);
 }
@@ -224,7 +242,16 @@ int aussm_unitary_bwd(const float* dy, const float* dhL, const void* u, const vo
                       const void* Bc, const void* Cc, const float* Dskip, const float* hck,
                       float* du, float* ddelta, float* dtheta, float* dB, float* dC, float* dD, float* dh0,
                       int B, int D, int N, int L, int ck, int in_dtype, void* stream) {
+  return aussm_unitary_bwd_aux(dy, dhL, u, delta, theta, Bc, Cc, Dskip, hck, nullptr, du, ddelta, dtheta, dB, dC, dD,
+                               dh0, B, D, N, L, ck, in_dtype, stream);
+}
+
+int aussm_unitary_bwd_aux(const float* dy, const float* dhL, const void* u, const void* delta, const float* theta,
+                          const void* Bc, const void* Cc, const float* Dskip, const float* hck, const float* aux,
+                          float* du, float* ddelta, float* dtheta, float* dB, float* dC, float* dD, float* dh0,
+                          int B, int D, int N, int L, int ck, int in_dtype, void* stream) {
   if (int e = check_common(B, D, N, L, ck, in_dtype)) return e;
+  if (misaligned(aux, 16)) return AUSSM_E_ALIGN;
   if (!dy || !u || !delta || !theta || !Bc || !Cc || !hck || !du || !ddelta || !dtheta || !dB || !dC)
     return AUSSM_E_NULL;
   const size_t ca = in_dtype == AUSSM_BF16 ? 4 : 8;
@@ -232,7 +259,7 @@ int aussm_unitary_bwd(const float* dy, const float* dhL, const void* u, const vo
   hipStream_t s = (hipStream_t)stream;
   UniBwdArgs a{};
   a.dy = dy; a.dhL = dhL; a.u = u; a.delta = delta; a.theta = theta; a.Bm = Bc; a.Cm = Cc; a.Dskip = Dskip;
-  a.hck = hck; a.du = du; a.ddelta = ddelta; a.dtheta = dtheta; a.dB = dB; a.dC = dC; a.dD = dD; a.dh0 = dh0;
+  a.hck = hck; a.aux = aux; a.du = du; a.ddelta = ddelta; a.dtheta = dtheta; a.dB = dB; a.dC = dC; a.dD = dD; a.dh0 = dh0;
   a.B = B; a.D = D; a.N = N; a.L = L; a.ck = ck; a.nck = (L + ck - 1) / ck; a.ncg = (D + CH - 1) / CH;
   const int mode = env_mode("AUSSM_MFMA_BWD", 3);   // matrix-core kernel for the common case
   if (mode > 0 && in_dtype == AUSSM_F32 && N <= XN && L % 4 == 0 && ck % XT == 0 &&

@@ -32,6 +32,7 @@ struct UniBwdArgs {
   const void* Cm;       // [B,N,L,2] Tin
   const float* Dskip;   // [D] or null
   const float* hck;     // [B,nck,N,2,D]
+  const float* aux;     // optional: what the forward call left in its aux buffer
   float *du, *ddelta, *dtheta;   // [B,D,L]
   float *dB, *dC;       // [B,N,L,2]  accumulated into with atomics (caller zero-fills)
   float* dD;            // [D] or null, accumulated into

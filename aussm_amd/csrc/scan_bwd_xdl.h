@@ -113,6 +113,10 @@ __global__ __launch_bounds__(256) void unitary_bwd_xdl_kernel(const UniBwdArgs p
   const float dsk = (p.Dskip && dok) ? p.Dskip[dc] : 0.0f;
   const int nchunks = (L + XT - 1) / XT;
   const SplitK sk = make_splitk();
+  // Im(P_t S_t) left by the forward kernel (if it filled the buffer): saves recomputing S here
+  const bool use_phi = p.aux != nullptr &&
+      __builtin_amdgcn_readfirstlane(__float_as_uint(p.aux[(size_t)p.B * D * L])) == AUX_TAG;
+  const float* __restrict__ gph = use_phi ? p.aux + row : nullptr;
   float* __restrict__ ws = s_ws[wave];
 
   // zero what is read but never written: G tiles off the causal side, the same tile of MS / MT
@@ -220,22 +224,28 @@ __global__ __launch_bounds__(256) void unitary_bwd_xdl_kernel(const UniBwdArgs p
     ldrec<NP>(s_bc.bs, xrec(16 * gst + dl, g, XT), a);
     ldrec<NP>(s_bc.cs_r, xrec(16 * gtt + dl, g, XT), cr);
     ldrec<NP>(s_bc.cs_i, xrec(16 * gtt + dl, g, XT), ci);
-    // rows s, columns t  ->  lane: G[t = dl][s = 4 g + i]
-    f4 xr = xmm<NP>(a, cr, f4{0, 0, 0, 0}), xi = xmm<NP>(a, ci, f4{0, 0, 0, 0});
     // rows t, columns s  ->  lane: G[t = 4 g + i][s = dl]
     f4 yr = xmm<NP>(cr, a, f4{0, 0, 0, 0}), yi = xmm<NP>(ci, a, f4{0, 0, 0, 0});
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const bool k1 = 4 * g + i <= g_lim, k2 = 4 * g + i >= g_low;
-      xr[i] = k1 ? xr[i] : 0.0f; xi[i] = k1 ? xi[i] : 0.0f;
+      const bool k2 = 4 * g + i >= g_low;
       yr[i] = k2 ? yr[i] : 0.0f; yi[i] = k2 ? yi[i] : 0.0f;
     }
-    put_half(s_g.gt_r, s_g.gt_i, xrec(16 * gtt + dl, g, XT) * 2 + gst, xr, xi);
     put_half(s_g.g_r, s_g.g_i, xrec(16 * gst + dl, g, XT) * 2 + gtt, yr, yi);
+    if (!use_phi) {
+      // rows s, columns t  ->  lane: G[t = dl][s = 4 g + i]   (only the S recomputation reads it)
+      f4 xr = xmm<NP>(a, cr, f4{0, 0, 0, 0}), xi = xmm<NP>(a, ci, f4{0, 0, 0, 0});
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const bool k1 = 4 * g + i <= g_lim;
+        xr[i] = k1 ? xr[i] : 0.0f; xi[i] = k1 ? xi[i] : 0.0f;
+      }
+      put_half(s_g.gt_r, s_g.gt_i, xrec(16 * gtt + dl, g, XT) * 2 + gst, xr, xi);
+    }
   };
 
   // ---- channel data of one chunk
-  struct In { f4 u[2], de[2], th[2], dy[2]; };
+  struct In { f4 u[2], de[2], th[2], dy[2], ph[2]; };
   auto in_load = [&](In& r, int c) {
     const int cc = c < 0 ? 0 : c;
 #pragma unroll
@@ -246,6 +256,7 @@ __global__ __launch_bounds__(256) void unitary_bwd_xdl_kernel(const UniBwdArgs p
       r.de[st] = *reinterpret_cast<const f4*>(gdl + lc);
       r.th[st] = *reinterpret_cast<const f4*>(gth + lc);
       r.dy[st] = *reinterpret_cast<const f4*>(gdy + lc);
+      if (use_phi) r.ph[st] = *reinterpret_cast<const f4*>(gph + lc);
     }
   };
   auto in_touch = [&](const In& r) {
@@ -309,8 +320,6 @@ __global__ __launch_bounds__(256) void unitary_bwd_xdl_kernel(const UniBwdArgs p
     const int l0 = c * XT;
     // ================= phase 1: stage B/C, everything that does not need G
     bc_store(c);
-    bc_load(c - 1);
-    in_load(nxt, c - 1);
     if (c + 1 < nchunks) flush_dbc(l0 + XT);                           // dB / dC of the previous step
     __syncthreads();                                                   // (a) planes of chunk c visible
     make_g();
@@ -483,9 +492,12 @@ __global__ __launch_bounds__(256) void unitary_bwd_xdl_kernel(const UniBwdArgs p
     __syncthreads();                                                   // (b) G planes and partial sums visible
 
     // ================= phase 2
-    // ---- S = C.H + G.V  (only Im(P S) is needed)
-    f4 Sr[2], Si[2];
-    {
+    // ---- Im(P_t S_t): read back from the forward pass, or recomputed (S = C.H + G.V)
+    float phi[8];
+    if (use_phi) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) phi[e] = cur.ph[e >> 2][e & 3];
+    } else {
       const float x[8] = {Hr[0], Hr[1], Hr[2], Hr[3], Hi[0], Hi[1], Hi[2], Hi[3]};
       u4 hk[NP];
       split8<NP>(sk, x, hk);
@@ -496,10 +508,12 @@ __global__ __launch_bounds__(256) void unitary_bwd_xdl_kernel(const UniBwdArgs p
         ldrec<NP>(s_bc.cs_i, xrec(16 * tt + dl, g, XT), ai);
         ldrec<NP>(s_g.gt_r, xrec(16 * tt + dl, g, XT), gr);
         ldrec<NP>(s_g.gt_i, xrec(16 * tt + dl, g, XT), gi);
-        Sr[tt] = xmm<NP>(ar, hk, f4{0, 0, 0, 0});
-        Si[tt] = xmm<NP>(ai, hk, f4{0, 0, 0, 0});
-        Sr[tt] = xmm<NP>(gr, Vr, Sr[tt]);  Sr[tt] = xmm<NP>(gi, nVi, Sr[tt]);
-        Si[tt] = xmm<NP>(gr, Vi, Si[tt]);  Si[tt] = xmm<NP>(gi, Vr, Si[tt]);
+        f4 Sr = xmm<NP>(ar, hk, f4{0, 0, 0, 0});
+        f4 Si = xmm<NP>(ai, hk, f4{0, 0, 0, 0});
+        Sr = xmm<NP>(gr, Vr, Sr);  Sr = xmm<NP>(gi, nVi, Sr);
+        Si = xmm<NP>(gr, Vi, Si);  Si = xmm<NP>(gi, Vr, Si);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) phi[4 * tt + i] = cs[4 * tt + i] * Si[i] + sn[4 * tt + i] * Sr[i];
       }
     }
     // ---- gV, second term: sum_{t>=s} conj(G[t,s]) Q_t
@@ -516,9 +530,8 @@ __global__ __launch_bounds__(256) void unitary_bwd_xdl_kernel(const UniBwdArgs p
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       const float gr = gVr[e >> 2][e & 3], gi = gVi[e >> 2][e & 3];
-      const float phi = cs[e] * Si[e >> 2][e & 3] + sn[e] * Sr[e >> 2][e & 3];
       dw[e] = gr * cs[e] - gi * sn[e];
-      gth[e] = gr * vi[e] - gi * vr[e] - dy[e] * phi;
+      gth[e] = gr * vi[e] - gi * vr[e] - dy[e] * phi[e];
     }
     gth[7] += (g == 3) ? tq : 0.0f;
     // suffix sums over the chunk: runs (st 1: g 3..0) then (st 0: g 3..0) in reverse time
@@ -558,11 +571,10 @@ __global__ __launch_bounds__(256) void unitary_bwd_xdl_kernel(const UniBwdArgs p
         for (int i = 0; i < 4; ++i) s_ms[im][(t + i) * XB_MS + s] = sum[i];
       }
     }
-    // collect the prefetched loads before the stores below join the same in-order queue
-#pragma unroll
-    for (int k = 0; k < 4; ++k) { touch_vgpr(m1_raw[k].x); touch_vgpr(m1_raw[k].y); }
-    touch4(m2_raw[0]); touch4(m2_raw[1]);
-    in_touch(nxt);
+    // Loads of the next chunk go into the (single, in-order) vector-memory queue AHEAD of this
+    // chunk's stores; they are first needed a barrier and the closing products later.
+    bc_load(c - 1);
+    in_load(nxt, c - 1);
     if (dok) {
 #pragma unroll
       for (int st = 0; st < 2; ++st) {

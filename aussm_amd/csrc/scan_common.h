@@ -23,6 +23,11 @@ constexpr int NXCD = 8;       // accelerator complex dies, each with a private L
 
 enum { VAR_UNITARY = 0, VAR_COMPLEX = 1, VAR_REAL = 2 };
 
+// The optional auxiliary buffer of the unitary scan holds B*D*L floats followed by AUX_PAD floats;
+// the first of those is AUX_TAG when a forward kernel has filled the buffer, anything else if not.
+constexpr uint32_t AUX_TAG = 0x4f484950u;
+constexpr int AUX_PAD = 64;
+
 constexpr float LOG2E = 1.4426950408889634f;
 
 typedef uint16_t bf16_t;

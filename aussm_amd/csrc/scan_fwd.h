@@ -23,6 +23,7 @@ struct FwdArgs {
   float* y;                 // [B,D,L] or null
   float* hL;                // [B,D,N,C] or null
   float* hck;               // [B,nck,N,C,D] or null
+  float* aux;               // unitary, optional: Im(P_t S_t) [B,D,L] followed by a validity tag
   int B, D, N, L, ck, nck, ncg, delta_softplus;
 };
 

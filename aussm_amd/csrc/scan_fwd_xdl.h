@@ -584,6 +584,19 @@ __global__ __launch_bounds__(256) void unitary_fwd_xdl_kernel(const FwdArgs p) {
         if (l < L) *reinterpret_cast<f4*>(p.y + row + l) = yo[tt];
       }
     }
+    // optional: Im(P_t S_t), which the backward pass would otherwise recompute
+    if (p.aux && dok) {
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt) {
+        const int l = l0 + 16 * tt + 4 * g;
+        if (l < L) {
+          f4 ph;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) ph[i] = pc.cs[tt][i] * Si[tt][i] + pc.sn[tt][i] * Sr[tt][i];
+          *reinterpret_cast<f4*>(p.aux + row + l) = ph;
+        }
+      }
+    }
     // ---- checkpoint: state at the end of every ck-step block and at the end of the sequence
     const bool ck_now = l0 < L && (--ck_left == 0 || l0 + XT >= L);
     if (p.hck && dok && ck_now) {
@@ -628,6 +641,7 @@ __global__ __launch_bounds__(256) void unitary_fwd_xdl_kernel(const FwdArgs p) {
     step(c + 1, inB, inA, P1, P0);
   }
 
+  if (p.aux && blockIdx.x == 0 && tid == 0) p.aux[(size_t)p.B * D * L] = __uint_as_float(AUX_TAG);
   if (p.hL && dok) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {

@@ -318,6 +318,16 @@ __global__ __launch_bounds__(512) void unitary_fwd_xdl2_kernel(const FwdArgs p) 
         *reinterpret_cast<f4*>(p.y + row + l) = yo;
       }
     }
+    // optional: Im(P_t S_t), which the backward pass would otherwise recompute
+    if (p.aux && dok) {
+      const int l = l0 + 16 * hf + 4 * g;
+      if (l < L) {
+        f4 ph;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) ph[i] = pc.cs[i] * Si[i] + pc.sn[i] * Sr[i];
+        *reinterpret_cast<f4*>(p.aux + row + l) = ph;
+      }
+    }
     // ---- checkpoint: state at the end of every ck-step block and at the end of the sequence
     const bool ck_now = l0 < L && (--ck_left == 0 || l0 + XT >= L);
     if (p.hck && dok && ck_now && hf == 0) {
@@ -359,6 +369,7 @@ __global__ __launch_bounds__(512) void unitary_fwd_xdl2_kernel(const FwdArgs p) 
     step(c + 1, inB, inA, P1, P0);
   }
 
+  if (p.aux && blockIdx.x == 0 && tid == 0) p.aux[(size_t)p.B * D * L] = __uint_as_float(AUX_TAG);
   if (p.hL && dok && hf == 0) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {

@@ -92,8 +92,16 @@ def num_checkpoints(L: int, ck: int) -> int:
 # raw launches (no autograd)
 # --------------------------------------------------------------------------------------------
 
-def unitary_fwd_raw(u, delta, theta, Bri, Cri, D=None, z=None, h0=None, want_state=False, ck=0):
-    """Launch aussm_unitary_fwd.  Bri/Cri are real views (b, n, l, 2).  Returns (y, hL, hck);
+def unitary_aux(u) -> Tensor:
+    """The optional auxiliary buffer of the unitary scan for inputs shaped like u (b, d, l): the
+    forward call may leave intermediate results in it that spare the backward call a recomputation."""
+    lib = _lib.load()
+    b, d, l = u.shape
+    return torch.empty((lib.aussm_unitary_aux_floats(b, d, l),), device=u.device, dtype=torch.float32)
+
+
+def unitary_fwd_raw(u, delta, theta, Bri, Cri, D=None, z=None, h0=None, want_state=False, ck=0, aux=None):
+    """Launch aussm_unitary_fwd(_aux).  Bri/Cri are real views (b, n, l, 2).  Returns (y, hL, hck);
     hL is (b, d, n, 2) or None, hck is the checkpoint tensor when ck > 0."""
     lib = _lib.load()
     b, d, l = u.shape
@@ -103,13 +111,14 @@ def unitary_fwd_raw(u, delta, theta, Bri, Cri, D=None, z=None, h0=None, want_sta
     hck = None
     if ck:
         hck = torch.empty((b, num_checkpoints(l, ck), n, 2, d), device=u.device, dtype=torch.float32)
-    check(lib.aussm_unitary_fwd(ptr(u), ptr(delta), ptr(theta), ptr(Bri), ptr(Cri), ptr(D), ptr(z), ptr(h0),
-                                ptr(y), ptr(hL), ptr(hck), b, d, n, l, ck or _lib.TILE, _in_dtype(u), _stream()),
-          "aussm_unitary_fwd")
+    check(lib.aussm_unitary_fwd_aux(ptr(u), ptr(delta), ptr(theta), ptr(Bri), ptr(Cri), ptr(D), ptr(z), ptr(h0),
+                                    ptr(y), ptr(hL), ptr(hck), ptr(aux), b, d, n, l, ck or _lib.TILE, _in_dtype(u),
+                                    _stream()),
+          "aussm_unitary_fwd_aux")
     return y, hL, hck
 
 
-def unitary_bwd_raw(dy, dhL, u, delta, theta, Bri, Cri, D, hck, ck, want_dD=True, want_dh0=False):
+def unitary_bwd_raw(dy, dhL, u, delta, theta, Bri, Cri, D, hck, ck, want_dD=True, want_dh0=False, aux=None):
     lib = _lib.load()
     b, d, l = u.shape
     n = Bri.shape[1]
@@ -120,10 +129,10 @@ def unitary_bwd_raw(dy, dhL, u, delta, theta, Bri, Cri, D, hck, ck, want_dD=True
     dC = torch.zeros((b, n, l, 2), **f32)
     dD = torch.zeros((d,), **f32) if (want_dD and D is not None) else None
     dh0 = torch.empty((b, d, n, 2), **f32) if want_dh0 else None
-    check(lib.aussm_unitary_bwd(ptr(dy), ptr(dhL), ptr(u), ptr(delta), ptr(theta), ptr(Bri), ptr(Cri), ptr(D),
-                                ptr(hck), ptr(du), ptr(ddelta), ptr(dtheta), ptr(dB), ptr(dC), ptr(dD), ptr(dh0),
-                                b, d, n, l, ck, _in_dtype(u), _stream()),
-          "aussm_unitary_bwd")
+    check(lib.aussm_unitary_bwd_aux(ptr(dy), ptr(dhL), ptr(u), ptr(delta), ptr(theta), ptr(Bri), ptr(Cri), ptr(D),
+                                    ptr(hck), ptr(aux), ptr(du), ptr(ddelta), ptr(dtheta), ptr(dB), ptr(dC), ptr(dD),
+                                    ptr(dh0), b, d, n, l, ck, _in_dtype(u), _stream()),
+          "aussm_unitary_bwd_aux")
     return du, ddelta, dtheta, dB, dC, dD, dh0
 
 
@@ -136,19 +145,21 @@ class _UnitaryScanFn(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, u, delta, theta, Bri, Cri, D, h0):
-        y, hL, hck = unitary_fwd_raw(u, delta, theta, Bri, Cri, D, None, h0, want_state=True, ck=UNITARY_CK)
-        ctx.save_for_backward(u, delta, theta, Bri, Cri, D, hck)
+        aux = unitary_aux(u)
+        y, hL, hck = unitary_fwd_raw(u, delta, theta, Bri, Cri, D, None, h0, want_state=True, ck=UNITARY_CK, aux=aux)
+        ctx.save_for_backward(u, delta, theta, Bri, Cri, D, hck, aux)
         ctx.has_h0 = h0 is not None
         return y, hL
 
     @staticmethod
     def backward(ctx, dy, dhL):
-        u, delta, theta, Bri, Cri, D, hck = ctx.saved_tensors
+        u, delta, theta, Bri, Cri, D, hck, aux = ctx.saved_tensors
         dy = dy.contiguous()
         dhL = None if dhL is None else dhL.contiguous()
         du, ddelta, dtheta, dB, dC, dD, dh0 = unitary_bwd_raw(
             dy, dhL, u, delta, theta, Bri, Cri, D, hck, UNITARY_CK,
-            want_dD=D is not None and ctx.needs_input_grad[5], want_dh0=ctx.has_h0 and ctx.needs_input_grad[6])
+            want_dD=D is not None and ctx.needs_input_grad[5], want_dh0=ctx.has_h0 and ctx.needs_input_grad[6],
+            aux=aux)
         return (du.to(u.dtype), ddelta.to(delta.dtype), dtheta, dB.to(Bri.dtype), dC.to(Cri.dtype), dD, dh0)
 
 

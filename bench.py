@@ -91,10 +91,13 @@ def main():
     Cri = torch.view_as_real(p["Cc"]).contiguous()
     ck = scan.UNITARY_CK
 
+    aux = scan.unitary_aux(p["u"])      # what the autograd wrapper hands from forward to backward
+
     def step():
         y, _, hck = scan.unitary_fwd_raw(p["u"], p["delta"], p["theta"], Bri, Cri, p["Dskip"], None, None,
-                                         want_state=False, ck=ck)
-        return scan.unitary_bwd_raw(p["dy"], None, p["u"], p["delta"], p["theta"], Bri, Cri, p["Dskip"], hck, ck)
+                                         want_state=False, ck=ck, aux=aux)
+        return scan.unitary_bwd_raw(p["dy"], None, p["u"], p["delta"], p["theta"], Bri, Cri, p["Dskip"], hck, ck,
+                                    aux=aux)
 
     for _ in range(args.warmup):
         step()
@@ -115,14 +118,14 @@ def main():
     dB, dC, dD = torch.zeros((B, N, L, 2), **f32), torch.zeros((B, N, L, 2), **f32), torch.zeros((D,), **f32)
 
     def fwd_only():
-        scan.check(lib.aussm_unitary_fwd(ptr(p["u"]), ptr(p["delta"]), ptr(p["theta"]), ptr(Bri), ptr(Cri),
-                                         ptr(p["Dskip"]), None, None, ptr(y), None, ptr(hck),
-                                         B, D, N, L, ck, 0, stream), "fwd")
+        scan.check(lib.aussm_unitary_fwd_aux(ptr(p["u"]), ptr(p["delta"]), ptr(p["theta"]), ptr(Bri), ptr(Cri),
+                                             ptr(p["Dskip"]), None, None, ptr(y), None, ptr(hck), ptr(aux),
+                                             B, D, N, L, ck, 0, stream), "fwd")
 
     def bwd_only():
-        scan.check(lib.aussm_unitary_bwd(ptr(p["dy"]), None, ptr(p["u"]), ptr(p["delta"]), ptr(p["theta"]), ptr(Bri),
-                                         ptr(Cri), ptr(p["Dskip"]), ptr(hck), ptr(du), ptr(ddl), ptr(dth),
-                                         ptr(dB), ptr(dC), ptr(dD), None, B, D, N, L, ck, 0, stream), "bwd")
+        scan.check(lib.aussm_unitary_bwd_aux(ptr(p["dy"]), None, ptr(p["u"]), ptr(p["delta"]), ptr(p["theta"]), ptr(Bri),
+                                             ptr(Cri), ptr(p["Dskip"]), ptr(hck), ptr(aux), ptr(du), ptr(ddl), ptr(dth),
+                                             ptr(dB), ptr(dC), ptr(dD), None, B, D, N, L, ck, 0, stream), "bwd")
 
     def kernel_us(fn, reps):
         evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]

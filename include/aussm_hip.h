@@ -98,6 +98,29 @@ int aussm_unitary_bwd(const float* dy, const float* dhL,
                       float* dD, float* dh0,
                       int B, int D, int N, int L, int ck, int in_dtype, void* stream);
 
+/* Variants of the two calls above with an optional auxiliary buffer (NULL allowed; then they are
+ * the calls above).  `aux` holds aussm_unitary_aux_floats(B, D, L) floats, 16-byte aligned.  The
+ * forward call may leave per-(b,d,l) intermediate results in it (Im(P_t S_t), the term of the phase
+ * gradient that needs the forward states) together with a validity tag; the backward call given
+ * the same buffer then skips recomputing them.  A forward kernel that does not fill the buffer
+ * clears the tag, so a backward call never consumes stale contents: handing over `aux` is always
+ * safe and only ever a speed-up.  No counterpart in the reference (its backward kernel recomputes,
+ * ssm_adaptive_unitary_backward.cu:113-181). */
+size_t aussm_unitary_aux_floats(int B, int D, int L);
+
+int aussm_unitary_fwd_aux(const void* u, const void* delta, const float* theta,
+                          const void* Bc, const void* Cc, const float* Dskip, const float* z,
+                          const float* h0, float* y, float* hL, float* hck, float* aux,
+                          int B, int D, int N, int L, int ck, int in_dtype, void* stream);
+
+int aussm_unitary_bwd_aux(const float* dy, const float* dhL,
+                          const void* u, const void* delta, const float* theta,
+                          const void* Bc, const void* Cc, const float* Dskip, const float* hck,
+                          const float* aux,
+                          float* du, float* ddelta, float* dtheta, float* dB, float* dC,
+                          float* dD, float* dh0,
+                          int B, int D, int N, int L, int ck, int in_dtype, void* stream);
+
 /* ---------------------------------------------------------------------------------------
  * Complex scan:  a_l = exp(rho_l[b,d] + i*theta_l[b,d]), otherwise as the unitary scan.
  * Replaces extension-cpp/extension_cpp/ops.py:270-291 (loop) and the semantics of

@@ -95,3 +95,35 @@ def test_backward_modes(mode, B, D, N, L, big_theta):
         torch.cuda.synchronize()
     for k, w, gt in zip(NAMES + ("h0",), want, got):
         _close(gt, w, f"d{k}", tol=2e-4 if big_theta else 1e-4)
+
+
+def test_auxiliary_buffer_is_never_consumed_stale():
+    """The forward call may leave Im(P_t S_t) in the auxiliary buffer for the backward call.  A
+    forward kernel that does not fill it must clear its tag: run a filling forward + backward, then
+    (same shape, so the allocator hands back the same memory) a non-filling forward followed by the
+    matrix-core backward on DIFFERENT inputs, through the raw C-ABI wrappers with one shared buffer."""
+    from aussm_amd import scan
+    B, D, N, L = 2, 64, 16, 256
+    aux = None
+    for seed, fwd_mode in ((1, "3"), (2, "0"), (3, "4"), (4, "1")):
+        p = O.make_core_inputs(B, D, N, L, seed=seed)
+        leaves = [p[k].clone().requires_grad_(True) for k in NAMES]
+        y, _ = O.unitary_core_loop(*leaves)
+        (y * p["dy"]).sum().backward()
+        want = [t.grad for t in leaves]
+        q = {k: v.cuda() for k, v in p.items()}
+        Bri = torch.view_as_real(q["Bc"]).contiguous()
+        Cri = torch.view_as_real(q["Cc"]).contiguous()
+        if aux is None:
+            aux = scan.unitary_aux(q["u"])
+        print(f"case aux seed={seed} fwd_mode={fwd_mode}", flush=True)
+        with _Env(AUSSM_MFMA=fwd_mode):
+            yk, _, hck = scan.unitary_fwd_raw(q["u"], q["delta"], q["theta"], Bri, Cri, q["Dskip"], None, None,
+                                              want_state=False, ck=scan.UNITARY_CK, aux=aux)
+        got = scan.unitary_bwd_raw(q["dy"], None, q["u"], q["delta"], q["theta"], Bri, Cri, q["Dskip"], hck,
+                                   scan.UNITARY_CK, aux=aux)
+        torch.cuda.synchronize()
+        _close(yk, y.detach(), "y")
+        du, ddelta, dtheta, dB, dC, dD, _ = got
+        for k, w, gt in zip(NAMES, want, (du, ddelta, dtheta, torch.view_as_complex(dB), torch.view_as_complex(dC), dD)):
+            _close(gt, w, f"d{k} (forward mode {fwd_mode})")
