@@ -299,11 +299,14 @@ __global__ __launch_bounds__(256) void unitary_bwd_xdl_kernel(const UniBwdArgs p
     const float* __restrict__ at = s_at[wave];
     float* __restrict__ dst = (wave < 2 ? p.dC : p.dB) + at_off + (size_t)l_at * 2;
     const bool lok = l_at + 16 * (wave & 1) + (at_x >> 1) < L;
+    float v[8];
 #pragma unroll
-    for (int k = 0; k < 8; ++k) {
-      const int n = 2 * k + at_n;
-      const float v = at[n * XB_AS + at_x];
-      if (n < N && lok) atomicAdd(dst + (size_t)k * 4 * L, v);
+    for (int k = 0; k < 8; ++k) v[k] = at[(2 * k + at_n) * XB_AS + at_x];   // all reads, then one wait
+    sched_fence();
+    if (lok) {
+#pragma unroll
+      for (int k = 0; k < 8; ++k)
+        if (2 * k + at_n < N) atomicAdd(dst + (size_t)k * 4 * L, v[k]);
     }
   };
   // checkpoints: the chunk that starts at a multiple of ck takes its start state from the store
@@ -320,6 +323,8 @@ __global__ __launch_bounds__(256) void unitary_bwd_xdl_kernel(const UniBwdArgs p
     const int l0 = c * XT;
     // ================= phase 1: stage B/C, everything that does not need G
     bc_store(c);
+    bc_load(c - 1);
+    in_load(nxt, c - 1);
     if (c + 1 < nchunks) flush_dbc(l0 + XT);                           // dB / dC of the previous step
     __syncthreads();                                                   // (a) planes of chunk c visible
     make_g();
@@ -571,10 +576,6 @@ __global__ __launch_bounds__(256) void unitary_bwd_xdl_kernel(const UniBwdArgs p
         for (int i = 0; i < 4; ++i) s_ms[im][(t + i) * XB_MS + s] = sum[i];
       }
     }
-    // Loads of the next chunk go into the (single, in-order) vector-memory queue AHEAD of this
-    // chunk's stores; they are first needed a barrier and the closing products later.
-    bc_load(c - 1);
-    in_load(nxt, c - 1);
     if (dok) {
 #pragma unroll
       for (int st = 0; st < 2; ++st) {
