@@ -84,6 +84,20 @@ __device__ __forceinline__ void ldrec16(const u4 (*plane)[XN * 4], int idx, u4 (
   for (int q = 0; q < NP; ++q) o[q] = plane[q][idx];
 }
 
+// Prefetch loads whose results must sit untouched for a whole step.  The register file of this
+// kernel is full (arch + accumulation registers); left to the compiler such a load lands in an
+// arch register and is copied to an accumulation register a few instructions later, which makes
+// the wavefront wait for the full memory latency at once.  These helpers load straight into
+// accumulation registers; the compiler does not know the data is still in flight, so every value
+// loaded this way passes through landed() (a wait for all vector-memory operations that also pins
+// the values) before its first use.
+__device__ __forceinline__ void ldg_acc(f4& dst, const float* p) {
+  asm volatile("global_load_dwordx4 %0, %1, off" : "=a"(dst) : "v"(p) : "memory");
+}
+__device__ __forceinline__ void ldg_acc(float2& dst, const float* p) {
+  asm volatile("global_load_dwordx2 %0, %1, off" : "=a"(dst) : "v"(p) : "memory");
+}
+
 // Requires: N <= 16, L % 4 == 0, 16-byte aligned tensors, ck % 32 == 0, float inputs.
 // NP: operand pieces of the products along the sequence (3 = fp32-accurate); NPC: pieces of the
 // products that sum over the channel (M, X1, X2 and the two closing products of dB / dC).
@@ -116,7 +130,8 @@ __global__ __launch_bounds__(256) void unitary_bwd_xdl_kernel(const UniBwdArgs p
   // Im(P_t S_t) left by the forward kernel (if it filled the buffer): saves recomputing S here
   const bool use_phi = p.aux != nullptr &&
       __builtin_amdgcn_readfirstlane(__float_as_uint(p.aux[(size_t)p.B * D * L])) == AUX_TAG;
-  const float* __restrict__ gph = use_phi ? p.aux + row : nullptr;
+  // (always a valid address: the load below is unconditional, its result unused without the tag)
+  const float* __restrict__ gph = use_phi ? p.aux + row : gth;
   float* __restrict__ ws = s_ws[wave];
 
   // zero what is read but never written: G tiles off the causal side, the same tile of MS / MT
@@ -143,13 +158,13 @@ __global__ __launch_bounds__(256) void unitary_bwd_xdl_kernel(const UniBwdArgs p
     for (int k = 0; k < 4; ++k) {
       const int n = 4 * m1_g + k;
       const size_t o = (((size_t)b * N + (n < N ? n : 0)) * L + lc) * 2;
-      m1_raw[k] = *reinterpret_cast<const float2*>(m1_src + o);
+      ldg_acc(m1_raw[k], m1_src + o);
     }
     const int l2 = cc * XT + 16 * m2_half + 4 * m2_g;
     const int l2c = l2 < L ? l2 : 0;
     const size_t o2 = (((size_t)b * N + (m2_n < N ? m2_n : 0)) * L + l2c) * 2;
-    m2_raw[0] = *reinterpret_cast<const f4*>(m2_src + o2);
-    m2_raw[1] = *reinterpret_cast<const f4*>(m2_src + o2 + 4);
+    ldg_acc(m2_raw[0], m2_src + o2);
+    ldg_acc(m2_raw[1], m2_src + o2 + 4);
   };
   auto bc_store = [&](int c) {
     {
@@ -252,31 +267,42 @@ __global__ __launch_bounds__(256) void unitary_bwd_xdl_kernel(const UniBwdArgs p
     for (int st = 0; st < 2; ++st) {
       const int l = cc * XT + 16 * st + 4 * g;
       const int lc = l < L ? l : 0;
-      r.u[st] = *reinterpret_cast<const f4*>(gu + lc);
-      r.de[st] = *reinterpret_cast<const f4*>(gdl + lc);
-      r.th[st] = *reinterpret_cast<const f4*>(gth + lc);
-      r.dy[st] = *reinterpret_cast<const f4*>(gdy + lc);
-      if (use_phi) r.ph[st] = *reinterpret_cast<const f4*>(gph + lc);
+      ldg_acc(r.u[st], gu + lc);
+      ldg_acc(r.de[st], gdl + lc);
+      ldg_acc(r.th[st], gth + lc);
+      ldg_acc(r.dy[st], gdy + lc);
+      ldg_acc(r.ph[st], gph + lc);   // unconditional: a value defined on one path only would be copied at the join, before it has landed
     }
   };
-  auto in_touch = [&](const In& r) {
-#pragma unroll
-    for (int st = 0; st < 2; ++st) { touch4(r.u[st]); touch4(r.de[st]); touch4(r.th[st]); touch4(r.dy[st]); }
+  // everything ldg_acc has requested (B/C staging data and one chunk of channel data) has landed
+  auto landed = [&](In& r) {
+    asm volatile("s_waitcnt vmcnt(0)"
+                 : "+a"(r.u[0]), "+a"(r.u[1]), "+a"(r.de[0]), "+a"(r.de[1]), "+a"(r.th[0]), "+a"(r.th[1]),
+                   "+a"(r.dy[0]), "+a"(r.dy[1]), "+a"(r.ph[0]), "+a"(r.ph[1]),
+                   "+a"(m1_raw[0]), "+a"(m1_raw[1]), "+a"(m1_raw[2]), "+a"(m1_raw[3]),
+                   "+a"(m2_raw[0]), "+a"(m2_raw[1])
+                 :
+                 : "memory");
   };
 
   // ---- state at the end of the current chunk and its adjoint: lane (dl, g) holds n = 4 g + i
   f4 Hr = {0, 0, 0, 0}, Hi = {0, 0, 0, 0}, Ar = {0, 0, 0, 0}, Ai = {0, 0, 0, 0};
-  auto load_ck = [&](int kb) {
+  // checkpoint kb: fetched early into temporaries (eight loads in flight at once), applied later
+  // rows of checkpoint 0 for this lane (clamped to valid rows; rows >= N are zeroed on use)
+  const float* __restrict__ ck_row[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int n = 4 * g + i;
-      const size_t o = ((((size_t)b * p.nck + kb) * N + (n < N ? n : 0)) * 2) * D + dc;
-      const float vr = p.hck[o], vi = p.hck[o + D];
-      Hr[i] = n < N ? vr : 0.0f;
-      Hi[i] = n < N ? vi : 0.0f;
-    }
-  };
-  load_ck(p.nck - 1);
+  for (int i = 0; i < 4; ++i) {
+    const int n = 4 * g + i;
+    ck_row[i] = p.hck + ((((size_t)b * p.nck) * N + (n < N ? n : 0)) * 2) * D + dc;
+  }
+  const size_t ck_stride = (size_t)N * 2 * D;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {                      // the state at the end of the sequence
+    const size_t o = (size_t)(p.nck - 1) * ck_stride;
+    const float vr = ck_row[i][o], vi = ck_row[i][o + D];
+    Hr[i] = 4 * g + i < N ? vr : 0.0f;
+    Hi[i] = 4 * g + i < N ? vi : 0.0f;
+  }
   if (p.dhL && dok) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -317,6 +343,7 @@ __global__ __launch_bounds__(256) void unitary_bwd_xdl_kernel(const UniBwdArgs p
   In inA, inB;
   bc_load(nchunks - 1);
   in_load(inA, nchunks - 1);
+  landed(inA);
   __syncthreads();
 
   auto step = [&](int c, In& cur, In& nxt) {
@@ -325,6 +352,13 @@ __global__ __launch_bounds__(256) void unitary_bwd_xdl_kernel(const UniBwdArgs p
     bc_store(c);
     bc_load(c - 1);
     in_load(nxt, c - 1);
+    const bool ck_here = (ck_left == 1) && l0 > 0;   // this chunk starts a checkpoint block
+    float tr[4] = {0, 0, 0, 0}, ti[4] = {0, 0, 0, 0};
+    if (ck_here) {                                   // its start state comes from the store: request it now
+      const size_t o = (size_t)kb_next * ck_stride;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) { tr[i] = ck_row[i][o]; ti[i] = ck_row[i][o + D]; }
+    }
     if (c + 1 < nchunks) flush_dbc(l0 + XT);                           // dB / dC of the previous step
     __syncthreads();                                                   // (a) planes of chunk c visible
     make_g();
@@ -576,6 +610,11 @@ __global__ __launch_bounds__(256) void unitary_bwd_xdl_kernel(const UniBwdArgs p
         for (int i = 0; i < 4; ++i) s_ms[im][(t + i) * XB_MS + s] = sum[i];
       }
     }
+    // collect the loads issued at the top (long landed) before the stores join the in-order queue:
+    // otherwise the next step's first use would have to wait for "everything", stores included
+    landed(nxt);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { touch_vgpr(tr[i]); touch_vgpr(ti[i]); }
     if (dok) {
 #pragma unroll
       for (int st = 0; st < 2; ++st) {
@@ -625,7 +664,12 @@ __global__ __launch_bounds__(256) void unitary_bwd_xdl_kernel(const UniBwdArgs p
       // (the atomic adds themselves are issued by flush_dbc() in the next step, behind its loads)
     }
     // ---- next chunk: its end state is this chunk's start state (or the stored checkpoint)
-    if (--ck_left == 0 && l0 > 0) { load_ck(kb_next); --kb_next; ck_left = ck_chunks; }
+    if (ck_here) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) { Hr[i] = 4 * g + i < N ? tr[i] : 0.0f; Hi[i] = 4 * g + i < N ? ti[i] : 0.0f; }
+      --kb_next;
+    }
+    if (--ck_left == 0) ck_left = ck_chunks;
     __syncthreads();                                                   // (d) planes, scratch and M free
   };
 
