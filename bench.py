@@ -33,9 +33,10 @@ HBM_PEAK_GBS = 8000.0
 SHAPE = dict(B=32, D=512, N=16, L=2048)
 # HBM bytes per launch at SHAPE from the counter passes summarised in
 # profiles/unitary_fwd_bwd_B32_D512_N16_L2048_hbm_traffic.md (FETCH_SIZE x 2.00, WRITE_SIZE x 1.00 after
-# calibration on a 256 MiB copy): forward 426 MB read + 151 MB written, backward 574 MB read +
-# 543 MB written (the dB/dC atomics of the eight workgroups of a batch element count as writes).
-TRAFFIC_BYTES = {"unitary_fwd": 577e6, "unitary_bwd": 1116e6}
+# calibration on a 256 MiB copy): forward 427 MB read + 286 MB written, backward 808 MB read +
+# 544 MB written.  Both include the auxiliary buffer (134 MB written forward, read backward) and the
+# checkpoints; the dB/dC atomics of the eight workgroups of a batch element count as writes.
+TRAFFIC_BYTES = {"unitary_fwd": 713e6, "unitary_bwd": 1353e6}
 
 
 def cpu_baseline(B_sample: int):
