@@ -76,7 +76,7 @@ int launch_fwd_t(const FwdArgs& a, hipStream_t s) {
   return AUSSM_E_SHAPE;
 }
 
-// The matrix-core kernels cover the common unitary case (fp32 inputs, N <= 16, L a multiple of 4,
+// The matrix-core kernels cover the common unitary case (fp32 inputs, 6 <= N <= 16, L a multiple of 4,
 // 16-byte aligned tensors, checkpoint interval a multiple of 32); everything else takes the
 // generic kernels.  AUSSM_MFMA (environment, read at every call) selects the forward kernel for
 // comparisons: 0 generic, 1 fp32 matrix instructions, 2 / 3 bf16 matrix instructions on two- /
@@ -86,12 +86,16 @@ int launch_fwd_t(const FwdArgs& a, hipStream_t s) {
 // marks an auxiliary buffer as NOT filled (a forward kernel that does not fill it ran)
 __global__ void aux_invalidate_kernel(float* tag) { *tag = 0.0f; }
 
-inline int env_mode(const char* name, int dflt) {
+// The matrix-core kernels cost the same for every N <= 16 while the generic ones scale with N:
+// measured, the crossover is between N = 4 (generic 15 % faster) and N = 8 (matrix 30 % faster).
+constexpr int MATRIX_MIN_STATE = 6;
+inline int env_mode(const char* name, int dflt, int N) {
   const char* e = getenv(name);
-  return e ? atoi(e) : dflt;
+  if (e) return atoi(e);                       // an explicit choice is honoured for every N <= 16
+  return N >= MATRIX_MIN_STATE ? dflt : 0;
 }
 inline int mfma_fwd_mode(const FwdArgs& a, int in_dtype) {
-  const int mode = env_mode("AUSSM_MFMA", 3);
+  const int mode = env_mode("AUSSM_MFMA", 3, a.N);
   if (mode <= 0 || in_dtype != AUSSM_F32 || a.N > MN || a.L % 4 != 0 || a.ck % MT != 0) return 0;
   if (misaligned(a.u, 16) || misaligned(a.delta, 16) || misaligned(a.theta, 16) || misaligned(a.z, 16) ||
       misaligned(a.y, 16) || misaligned(a.Bm, 16) || misaligned(a.Cm, 16))
@@ -261,7 +265,7 @@ int aussm_unitary_bwd_aux(const float* dy, const float* dhL, const void* u, cons
   a.dy = dy; a.dhL = dhL; a.u = u; a.delta = delta; a.theta = theta; a.Bm = Bc; a.Cm = Cc; a.Dskip = Dskip;
   a.hck = hck; a.aux = aux; a.du = du; a.ddelta = ddelta; a.dtheta = dtheta; a.dB = dB; a.dC = dC; a.dD = dD; a.dh0 = dh0;
   a.B = B; a.D = D; a.N = N; a.L = L; a.ck = ck; a.nck = (L + ck - 1) / ck; a.ncg = (D + CH - 1) / CH;
-  const int mode = env_mode("AUSSM_MFMA_BWD", 3);   // matrix-core kernel for the common case
+  const int mode = env_mode("AUSSM_MFMA_BWD", 3, N);   // matrix-core kernel for the common case
   if (mode > 0 && in_dtype == AUSSM_F32 && N <= XN && L % 4 == 0 && ck % XT == 0 &&
       !(misaligned(dy, 16) || misaligned(u, 16) || misaligned(delta, 16) || misaligned(theta, 16) ||
         misaligned(du, 16) || misaligned(ddelta, 16) || misaligned(dtheta, 16) || misaligned(Bc, 16) ||
