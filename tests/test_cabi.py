@@ -19,7 +19,8 @@ def declared_symbols():
 def test_header_declares_the_expected_entry_points():
     names = declared_symbols()
     for must in ("aussm_unitary_fwd", "aussm_unitary_bwd", "aussm_complex_fwd", "aussm_complex_bwd",
-                 "aussm_real_fwd", "aussm_real_bwd", "aussm_version", "aussm_error_string"):
+                 "aussm_real_fwd", "aussm_real_bwd", "aussm_version", "aussm_error_string",
+                 "aussm_unitary_fwd_aux", "aussm_unitary_bwd_aux", "aussm_unitary_aux_floats"):
         assert must in names
 
 
@@ -60,6 +61,15 @@ def test_argument_checks_without_a_device():
     rc = lib.aussm_unitary_fwd(one, one, one, ctypes.c_void_p(260), one, null, null, null, one, null, null,
                                1, 1, 1, 32, 32, 0, null)
     assert rc == -5
+    # the auxiliary buffer: size query, alignment check, NULL accepted like the plain entry points
+    assert lib.aussm_unitary_aux_floats(32, 512, 2048) == 32 * 512 * 2048 + 64
+    assert lib.aussm_unitary_aux_floats(0, 1, 1) == 0
+    rc = lib.aussm_unitary_fwd_aux(one, one, one, one, one, null, null, null, one, null, null, ctypes.c_void_p(260),
+                                   1, 1, 1, 32, 32, 0, null)
+    assert rc == -5
+    rc = lib.aussm_unitary_fwd_aux(null, one, one, one, one, null, null, null, one, null, null, null,
+                                   1, 1, 1, 32, 32, 0, null)
+    assert rc == -1
     # the recomputing backward kernels insist on their checkpoint interval and state limit
     args = [one] * 9 + [0] + [one] * 9
     assert lib.aussm_real_bwd(*args, 1, 1, 1, 32, 32, 0, null) == -3
