@@ -17,7 +17,7 @@ pytestmark = pytest.mark.gpu
 
 FWD_MODES = ["0", "1", "2", "3", "4"]     # generic, fp32 matrix, bf16 x2 pieces, bf16 x3 pieces, two waves per SIMD
 BWD_MODES = ["0", "2", "3", "5"]          # generic, two pieces, default (3 along the sequence, 2 over the channel), three pieces
-SHAPES = [(2, 80, 16, 200), (1, 64, 5, 36), (2, 128, 16, 512)]
+SHAPES = [(2, 80, 16, 200), (1, 64, 5, 36), (2, 128, 16, 512), (1, 5, 6, 8)]
 NAMES = ("u", "delta", "theta", "Bc", "Cc", "Dskip")
 
 
