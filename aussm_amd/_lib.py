@@ -61,7 +61,7 @@ def load() -> ctypes.CDLL:
         fn = getattr(lib, name)
         fn.argtypes = argtypes
         fn.restype = c_int
-    lib.aussm_unitary_aux_floats.argtypes = [_I, _I, _I]
+    lib.aussm_unitary_aux_floats.argtypes = [_I, _I, _I, _I, _I]
     lib.aussm_unitary_aux_floats.restype = ctypes.c_size_t
     lib.aussm_error_string.argtypes = [c_int]
     lib.aussm_error_string.restype = c_char_p

@@ -14,6 +14,7 @@
 #include "scan_fwd_mfma.h"
 #include "scan_fwd_xdl.h"
 #include "scan_fwd_xdl2.h"
+#include "scan_seg_xdl.h"
 
 using namespace aussm;
 
@@ -94,6 +95,34 @@ inline int env_mode(const char* name, int dflt, int N) {
   if (e) return atoi(e);                       // an explicit choice is honoured for every N <= 16
   return N >= MATRIX_MIN_STATE ? dflt : 0;
 }
+// Splitting the sequence (scan_seg_xdl.h): with few (batch, channel group) pairs the launch would
+// leave most of the chip idle, so the sequence is cut into ns segments of whole checkpoint blocks
+// until about one workgroup per compute unit exists.  Only the matrix-core kernels take part,
+// and only the *_aux entry points (the segment states live behind the auxiliary buffer).
+// AUSSM_SPLIT (environment): 0 or 1 switches it off, a power of two caps ns.
+constexpr int SPLIT_MIN_WGS = 128;     // launches of at least this many workgroups are left alone
+constexpr int SPLIT_TARGET_WGS = 256;
+constexpr int SPLIT_MAX = 32;
+constexpr int SPLIT_MIN_LEN = 128;
+inline int seg_capacity(int B, int D, int N, int L, int ck) {
+  if (N < MATRIX_MIN_STATE || N > XN || L % 4 != 0 || ck < XT || ck % XT != 0 || L % ck != 0) return 1;
+  const long long wgs = (long long)B * ((D + CH - 1) / CH);
+  if (wgs >= SPLIT_MIN_WGS) return 1;
+  const int nblk = L / ck, target = (int)(SPLIT_TARGET_WGS / wgs);
+  int ns = 1;
+  while (ns * 2 <= target && ns * 2 <= SPLIT_MAX && nblk % (ns * 2) == 0 && L / (ns * 2) >= SPLIT_MIN_LEN) ns *= 2;
+  return ns;
+}
+inline int seg_count(int B, int D, int N, int L, int ck) {
+  int ns = seg_capacity(B, D, N, L, ck);
+  if (const char* e = getenv("AUSSM_SPLIT")) {
+    const int cap = atoi(e);
+    while (ns > 1 && ns > cap) ns /= 2;
+  }
+  return ns;
+}
+inline size_t seg_floats(int B, int D, int N, int ns) { return ns > 1 ? (size_t)B * ns * D * (2 * N + 2) : 0; }
+
 inline int mfma_fwd_mode(const FwdArgs& a, int in_dtype) {
   const int mode = env_mode("AUSSM_MFMA", 3, a.N);
   if (mode <= 0 || in_dtype != AUSSM_F32 || a.N > MN || a.L % 4 != 0 || a.ck % MT != 0) return 0;
@@ -104,11 +133,28 @@ inline int mfma_fwd_mode(const FwdArgs& a, int in_dtype) {
 }
 
 template <int VAR>
-int launch_fwd(const FwdArgs& a, int in_dtype, hipStream_t s) {
+int launch_fwd(FwdArgs a, int in_dtype, hipStream_t s) {
   const int mode = (VAR == VAR_UNITARY) ? mfma_fwd_mode(a, in_dtype) : 0;
   if (a.aux && mode <= 1)   // this call will not fill the auxiliary buffer
     hipLaunchKernelGGL(aux_invalidate_kernel, dim3(1), dim3(1), 0, s, a.aux + (size_t)a.B * a.D * a.L);
   if (mode) {
+    if ((mode == 2 || mode == 3) && a.aux && a.hck) {
+      const int ns = seg_count(a.B, a.D, a.N, a.L, a.ck);
+      if (ns > 1) {
+        // 1. end state of every segment from a zero start and its rotation; 2. chain them;
+        // 3. the scan proper over (batch, segment) pairs, each from its true incoming state
+        const int B = a.B, L = a.L, Ls = a.L / ns;
+        float* seg = a.aux + (size_t)B * a.D * L + AUX_PAD;
+        float* ptot = seg + (size_t)B * ns * a.D * a.N * 2;
+        SegArgs sa{static_cast<const float*>(a.delta), static_cast<const float*>(a.u), a.theta,
+                   static_cast<const float*>(a.Bm), seg, ptot, a.D, a.N, Ls, L, ns, a.ncg};
+        hipLaunchKernelGGL((unitary_seg_state_kernel<3, false>), dim3((unsigned)(B * ns * a.ncg)), dim3(256), 0, s, sa);
+        const size_t nst = (size_t)B * a.D * a.N;
+        hipLaunchKernelGGL(seg_carry_fwd_kernel, dim3((unsigned)((nst + 255) / 256)), dim3(256), 0, s, seg, ptot, a.h0,
+                           a.hL, B, a.D, a.N, ns);
+        a.B = B * ns; a.L = Ls; a.ns = ns; a.nck = Ls / a.ck; a.h0 = seg; a.hL = nullptr;
+      }
+    }
     const dim3 grid((unsigned)(a.B * a.ncg));
     if (mode == 1) {
       if (a.z) hipLaunchKernelGGL(unitary_fwd_mfma_kernel<true>, grid, dim3(256), 0, s, a);
@@ -188,8 +234,9 @@ int aussm_num_checkpoints(int L, int ck) { return (L < 1 || ck < 1) ? 0 : (L + c
 
 int aussm_bwd_checkpoint_interval(int variant) { return variant == VAR_UNITARY ? 0 : REC_CK; }
 
-size_t aussm_unitary_aux_floats(int B, int D, int L) {
-  return (B < 1 || D < 1 || L < 1) ? 0 : (size_t)B * D * L + AUX_PAD;
+size_t aussm_unitary_aux_floats(int B, int D, int N, int L, int ck) {
+  if (B < 1 || D < 1 || N < 1 || L < 1) return 0;
+  return (size_t)B * D * L + AUX_PAD + seg_floats(B, D, N, seg_capacity(B, D, N, L, ck));
 }
 
 int aussm_unitary_fwd(const void* u, const void* delta, const float* theta, const void* Bc, const void* Cc,
@@ -211,6 +258,7 @@ int aussm_unitary_fwd_aux(const void* u, const void* delta, const float* theta, 
   a.u = u; a.delta = delta; a.theta = theta; a.Bm = Bc; a.Cm = Cc; a.Dskip = Dskip; a.z = z;
   a.h0 = h0; a.y = y; a.hL = hL; a.hck = hck; a.aux = aux;
   a.B = B; a.D = D; a.N = N; a.L = L; a.ck = ck; a.nck = (L + ck - 1) / ck; a.ncg = (D + CH - 1) / CH;
+  a.ld = L; a.ns = 1;
   return launch_fwd<VAR_UNITARY>(a, in_dtype, (hipStream_t)stream);
 }
 
@@ -225,6 +273,7 @@ int aussm_complex_fwd(const void* u, const void* delta, const float* rho, const 
   a.u = u; a.delta = delta; a.rho = rho; a.theta = theta; a.Bm = Bc; a.Cm = Cc; a.Dskip = Dskip; a.z = z;
   a.h0 = h0; a.y = y; a.hL = hL; a.hck = hck;
   a.B = B; a.D = D; a.N = N; a.L = L; a.ck = ck; a.nck = (L + ck - 1) / ck; a.ncg = (D + CH - 1) / CH;
+  a.ld = L; a.ns = 1;
   return launch_fwd<VAR_COMPLEX>(a, in_dtype, (hipStream_t)stream);
 }
 
@@ -239,6 +288,7 @@ int aussm_real_fwd(const void* u, const void* delta, const float* A, const void*
   a.delta_bias = delta_bias; a.delta_softplus = delta_softplus;
   a.h0 = h0; a.y = y; a.hL = hL; a.hck = hck;
   a.B = B; a.D = D; a.N = N; a.L = L; a.ck = ck; a.nck = (L + ck - 1) / ck; a.ncg = (D + CH - 1) / CH;
+  a.ld = L; a.ns = 1;
   return launch_fwd<VAR_REAL>(a, in_dtype, (hipStream_t)stream);
 }
 
@@ -251,7 +301,7 @@ int aussm_unitary_bwd(const float* dy, const float* dhL, const void* u, const vo
 }
 
 int aussm_unitary_bwd_aux(const float* dy, const float* dhL, const void* u, const void* delta, const float* theta,
-                          const void* Bc, const void* Cc, const float* Dskip, const float* hck, const float* aux,
+                          const void* Bc, const void* Cc, const float* Dskip, const float* hck, float* aux,
                           float* du, float* ddelta, float* dtheta, float* dB, float* dC, float* dD, float* dh0,
                           int B, int D, int N, int L, int ck, int in_dtype, void* stream) {
   if (int e = check_common(B, D, N, L, ck, in_dtype)) return e;
@@ -265,11 +315,25 @@ int aussm_unitary_bwd_aux(const float* dy, const float* dhL, const void* u, cons
   a.dy = dy; a.dhL = dhL; a.u = u; a.delta = delta; a.theta = theta; a.Bm = Bc; a.Cm = Cc; a.Dskip = Dskip;
   a.hck = hck; a.aux = aux; a.du = du; a.ddelta = ddelta; a.dtheta = dtheta; a.dB = dB; a.dC = dC; a.dD = dD; a.dh0 = dh0;
   a.B = B; a.D = D; a.N = N; a.L = L; a.ck = ck; a.nck = (L + ck - 1) / ck; a.ncg = (D + CH - 1) / CH;
+  a.ld = L; a.ns = 1;
   const int mode = env_mode("AUSSM_MFMA_BWD", 3, N);   // matrix-core kernel for the common case
   if (mode > 0 && in_dtype == AUSSM_F32 && N <= XN && L % 4 == 0 && ck % XT == 0 &&
       !(misaligned(dy, 16) || misaligned(u, 16) || misaligned(delta, 16) || misaligned(theta, 16) ||
         misaligned(du, 16) || misaligned(ddelta, 16) || misaligned(dtheta, 16) || misaligned(Bc, 16) ||
         misaligned(Cc, 16))) {
+    const int ns = aux ? seg_count(B, D, N, L, ck) : 1;
+    if (ns > 1) {
+      // adjoint at the start of every segment from a zero adjoint at its end, chained last to first
+      const int Ls = L / ns;
+      float* seg = aux + (size_t)B * D * L + AUX_PAD;
+      float* ptot = seg + (size_t)B * ns * D * N * 2;
+      SegArgs sa{dy, nullptr, theta, static_cast<const float*>(Cc), seg, ptot, D, N, Ls, L, ns, a.ncg};
+      hipLaunchKernelGGL((unitary_seg_state_kernel<3, true>), dim3((unsigned)(B * ns * a.ncg)), dim3(256), 0, s, sa);
+      const size_t nst = (size_t)B * D * N;
+      hipLaunchKernelGGL(seg_carry_bwd_kernel, dim3((unsigned)((nst + 255) / 256)), dim3(256), 0, s, seg, ptot, dhL, dh0,
+                         B, D, N, ns);
+      a.B = B * ns; a.L = Ls; a.ns = ns; a.nck = Ls / ck; a.dhL = seg; a.dh0 = nullptr;
+    }
     const dim3 grid((unsigned)(a.B * a.ncg));
     if (mode == 2) hipLaunchKernelGGL((unitary_bwd_xdl_kernel<2, 2>), grid, dim3(256), 0, s, a);
     else if (mode == 5) hipLaunchKernelGGL((unitary_bwd_xdl_kernel<3, 3>), grid, dim3(256), 0, s, a);

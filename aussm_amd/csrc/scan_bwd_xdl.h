@@ -117,7 +117,11 @@ __global__ __launch_bounds__(256) void unitary_bwd_xdl_kernel(const UniBwdArgs p
   const int d = d0 + wave * 16 + dl;
   const bool dok = d < D;
   const int dc = dok ? d : D - 1;
-  const size_t row = ((size_t)b * D + dc) * L;
+  // b counts (batch element, segment of L steps) pairs when the launcher has split the sequence:
+  // states and checkpoints are indexed by b, the [.., ld] tensors by (bb, segment offset so)
+  const int bb = b / p.ns;
+  const size_t so = (size_t)(b - bb * p.ns) * L;
+  const size_t row = ((size_t)bb * D + dc) * p.ld + so;
   const float* __restrict__ gu = static_cast<const float*>(p.u) + row;
   const float* __restrict__ gdl = static_cast<const float*>(p.delta) + row;
   const float* __restrict__ gth = p.theta + row;
@@ -157,12 +161,12 @@ __global__ __launch_bounds__(256) void unitary_bwd_xdl_kernel(const UniBwdArgs p
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
       const int n = 4 * m1_g + k;
-      const size_t o = (((size_t)b * N + (n < N ? n : 0)) * L + lc) * 2;
+      const size_t o = (((size_t)bb * N + (n < N ? n : 0)) * p.ld + so + lc) * 2;
       ldg_acc(m1_raw[k], m1_src + o);
     }
     const int l2 = cc * XT + 16 * m2_half + 4 * m2_g;
     const int l2c = l2 < L ? l2 : 0;
-    const size_t o2 = (((size_t)b * N + (m2_n < N ? m2_n : 0)) * L + l2c) * 2;
+    const size_t o2 = (((size_t)bb * N + (m2_n < N ? m2_n : 0)) * p.ld + so + l2c) * 2;
     ldg_acc(m2_raw[0], m2_src + o2);
     ldg_acc(m2_raw[1], m2_src + o2 + 4);
   };
@@ -318,7 +322,7 @@ __global__ __launch_bounds__(256) void unitary_bwd_xdl_kernel(const UniBwdArgs p
   // dB / dC output: lane (at_n, at_x) of a closing wavefront adds element (row n = 2 k + at_n,
   // timestep at_x / 2, part at_x % 2) of its tile, k = 0..7
   const int at_n = lane >> 5, at_x = lane & 31;
-  const size_t at_off = (((size_t)b * N + at_n) * L + 16 * (wave & 1) + (at_x >> 1)) * 2 + (at_x & 1);
+  const size_t at_off = (((size_t)bb * N + at_n) * p.ld + so + 16 * (wave & 1) + (at_x >> 1)) * 2 + (at_x & 1);
 
   // dB / dC tile of the chunk starting at l_at, waiting in s_at[wave] (written by this wavefront)
   auto flush_dbc = [&](int l_at) {
@@ -332,7 +336,7 @@ __global__ __launch_bounds__(256) void unitary_bwd_xdl_kernel(const UniBwdArgs p
     if (lok) {
 #pragma unroll
       for (int k = 0; k < 8; ++k)
-        if (2 * k + at_n < N) atomicAdd(dst + (size_t)k * 4 * L, v[k]);
+        if (2 * k + at_n < N) atomicAdd(dst + (size_t)k * 4 * p.ld, v[k]);
     }
   };
   // checkpoints: the chunk that starts at a multiple of ck takes its start state from the store

@@ -25,6 +25,8 @@ struct FwdArgs {
   float* hck;               // [B,nck,N,C,D] or null
   float* aux;               // unitary, optional: Im(P_t S_t) [B,D,L] followed by a validity tag
   int B, D, N, L, ck, nck, ncg, delta_softplus;
+  int ld, ns;                // matrix-core unitary kernels: row stride of the [.., L] tensors and segments per
+                             // sequence (B then counts batch x segment pairs and L is the segment length)
 };
 
 // VAR: variant.  NW: states per wavefront.  NT: threads per workgroup.  Tin: float or bf16_t.

@@ -142,7 +142,11 @@ __global__ __launch_bounds__(256) void unitary_fwd_xdl_kernel(const FwdArgs p) {
   const int d = d0 + wave * 16 + dl;
   const bool dok = d < D;
   const int dc = dok ? d : D - 1;
-  const size_t row = ((size_t)b * D + dc) * L;
+  // b counts (batch element, segment of L steps) pairs when the launcher has split the sequence:
+  // states and checkpoints are indexed by b, the [.., ld] tensors by (bb, segment offset so)
+  const int bb = b / p.ns;
+  const size_t so = (size_t)(b - bb * p.ns) * L;
+  const size_t row = ((size_t)bb * D + dc) * p.ld + so;
   const float* __restrict__ gu = static_cast<const float*>(p.u) + row;
   const float* __restrict__ gdl = static_cast<const float*>(p.delta) + row;
   const float* __restrict__ gth = p.theta + row;
@@ -174,12 +178,12 @@ __global__ __launch_bounds__(256) void unitary_fwd_xdl_kernel(const FwdArgs p) {
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
       const int n = 4 * m1_g + k;
-      const size_t o = (((size_t)b * N + (n < N ? n : 0)) * L + lc) * 2;
+      const size_t o = (((size_t)bb * N + (n < N ? n : 0)) * p.ld + so + lc) * 2;
       m1_raw[k] = *reinterpret_cast<const float2*>(m1_src + o);
     }
     const int l2 = c * XT + 16 * m2_half + 4 * m2_g;
     const int l2c = l2 < L ? l2 : 0;
-    const size_t o2 = (((size_t)b * N + (m2_n < N ? m2_n : 0)) * L + l2c) * 2;
+    const size_t o2 = (((size_t)bb * N + (m2_n < N ? m2_n : 0)) * p.ld + so + l2c) * 2;
     m2_raw[0] = *reinterpret_cast<const f4*>(gB + o2);
     m2_raw[1] = *reinterpret_cast<const f4*>(gB + o2 + 4);
   };

@@ -1,0 +1,253 @@
+// Splitting the sequence of a unitary scan over workgroups (few (batch, channel) pairs, long L).
+//
+// The recurrence is linear in the state, so a segment [l0, l0 + Ls) of the sequence acts on the
+// state that enters it as  H_out = P H_in + Z  with P = exp(i sum theta) the segment's rotation
+// and Z its end state from a zero start; the adjoint runs the other way, A_in = conj(P) A_out + Y
+// with Y the adjoint at the segment start from a zero adjoint at its end.  The launcher therefore
+//   1. computes (P, Z) or (P, Y) of every segment with unitary_seg_state_kernel (all segments in
+//      parallel; only the sums  Z = P sum_s conj(P_s) delta_s u_s B_s,  Y = sum_t conj(P_t) dy_t conj(C_t)
+//      are formed: per chunk one product with the channel as free index, on the matrix cores in
+//      the layout of the scan kernels),
+//   2. chains the segments of each (batch, channel, state) with seg_carry_*_kernel (ns steps),
+//   3. runs the scan kernel proper with (batch, segment) pairs as its batch index, every segment
+//      starting from its true incoming state or adjoint.
+#pragma once
+#include "scan_fwd_xdl.h"
+
+namespace aussm {
+
+struct SegArgs {
+  const float* x1;      // forward: delta, adjoint: dy        [B, D, ld]
+  const float* x2;      // forward: u, adjoint: unused        [B, D, ld]
+  const float* theta;   //                                    [B, D, ld]
+  const float* M;       // forward: B_t, adjoint: C_t         [B, N, ld, 2]
+  float* out;           // Z or Y                             [B * ns, D, N, 2]
+  float* ptot;          // rotation of the segment            [B * ns, D, 2]
+  int D, N, L, ld, ns, ncg;   // L: segment length
+};
+
+// ADJ = false: Z of each segment, chunks in forward order,  H <- P_T (H + B^T V).
+// ADJ = true:  Y of each segment, chunks in reverse order,  A <- conj(P_T) A + conj(C)^T Q.
+// Requires N <= 16, L % 4 == 0, 16-byte aligned tensors, float inputs.
+template <int NP, bool ADJ>
+__global__ __launch_bounds__(256) void unitary_seg_state_kernel(const SegArgs p) {
+  // row n: M[t(g, e)][n], real and imaginary parts (the imaginary part negated for ADJ: conj(C))
+  __shared__ u4 s_mr[2][NP][XN * 4];
+  __shared__ u4 s_mi[2][NP][XN * 4];
+
+  const int wg = xcd_remap(blockIdx.x, gridDim.x);
+  const int vb = wg / p.ncg, d0 = (wg % p.ncg) * CH;
+  const int tid = threadIdx.x, lane = tid & 63, wave = wave_index();
+  const int dl = lane & 15, g = lane >> 4;
+  const int D = p.D, N = p.N, L = p.L;
+  const int d = d0 + wave * 16 + dl;
+  const bool dok = d < D;
+  const int dc = dok ? d : D - 1;
+  const int bb = vb / p.ns;
+  const size_t so = (size_t)(vb - bb * p.ns) * L;
+  const size_t row = ((size_t)bb * D + dc) * p.ld + so;
+  const float* __restrict__ gx1 = p.x1 + row;
+  const float* __restrict__ gx2 = ADJ ? p.x1 + row : p.x2 + row;
+  const float* __restrict__ gth = p.theta + row;
+  const int nchunks = (L + XT - 1) / XT;
+  const SplitK sk = make_splitk();
+
+  // staging: thread (n = tid % 16, g2 = (tid / 16) % 4, half = (tid / 64) % 2) reads the four
+  // timesteps 16 half + 4 g2 .. + 3 of row n; tid < 128 writes the real half-record, the others
+  // the imaginary one
+  const int m2_n = tid & 15, m2_g = (tid >> 4) & 3, m2_half = (tid >> 6) & 1;
+  const bool m2_im = tid >= 128;
+  f4 m2_raw[2];
+  auto m_load = [&](int c) {
+    const int cc = c < 0 ? 0 : (c >= nchunks ? nchunks - 1 : c);
+    const int l2 = cc * XT + 16 * m2_half + 4 * m2_g;
+    const int l2c = l2 < L ? l2 : 0;
+    const size_t o2 = (((size_t)bb * N + (m2_n < N ? m2_n : 0)) * p.ld + so + l2c) * 2;
+    m2_raw[0] = *reinterpret_cast<const f4*>(p.M + o2);
+    m2_raw[1] = *reinterpret_cast<const f4*>(p.M + o2 + 4);
+  };
+  auto m_store = [&](int c, int slot) {
+    const bool ok = (m2_n < N) && (c * XT + 16 * m2_half + 4 * m2_g < L);
+    const float sg = (ADJ && m2_im) ? -1.0f : 1.0f;
+    float v0 = m2_im ? m2_raw[0][1] : m2_raw[0][0], v1 = m2_im ? m2_raw[0][3] : m2_raw[0][2];
+    float v2 = m2_im ? m2_raw[1][1] : m2_raw[1][0], v3 = m2_im ? m2_raw[1][3] : m2_raw[1][2];
+    v0 = ok ? sg * v0 : 0.0f; v1 = ok ? sg * v1 : 0.0f; v2 = ok ? sg * v2 : 0.0f; v3 = ok ? sg * v3 : 0.0f;
+    uint32_t a0[NP], a1[NP];
+    split2<NP>(sk, v0, v1, a0);
+    split2<NP>(sk, v2, v3, a1);
+    const int o = xrec(m2_n, m2_g, XN) * 2 + m2_half;   // 8-byte half-record index
+    u4 (*dst)[XN * 4] = m2_im ? s_mi[slot] : s_mr[slot];
+#pragma unroll
+    for (int q = 0; q < NP; ++q) reinterpret_cast<u2*>(dst[q])[o] = u2{a0[q], a1[q]};
+  };
+
+  struct In { f4 th[2], a[2], b[2]; };
+  auto in_load = [&](In& r, int c) {
+    const int cc = c < 0 ? 0 : (c >= nchunks ? nchunks - 1 : c);
+#pragma unroll
+    for (int st = 0; st < 2; ++st) {
+      const int l = cc * XT + 16 * st + 4 * g;
+      const int lc = l < L ? l : 0;
+      r.th[st] = *reinterpret_cast<const f4*>(gth + lc);
+      r.a[st] = *reinterpret_cast<const f4*>(gx1 + lc);
+      if (!ADJ) r.b[st] = *reinterpret_cast<const f4*>(gx2 + lc);
+    }
+  };
+
+  // lane (dl, g) holds the state (or adjoint) rows n = 4 g + i of channel dl
+  f4 Sr = {0, 0, 0, 0}, Si = {0, 0, 0, 0};
+  float pr = 1.0f, pi = 0.0f;   // rotation of the chunks done so far
+
+  In cur;
+  const int c_first = ADJ ? nchunks - 1 : 0, c_step = ADJ ? -1 : 1;
+  m_load(c_first);
+  in_load(cur, c_first);
+
+  for (int k = 0; k < nchunks; ++k) {
+    const int c = c_first + k * c_step;
+    const int slot = k & 1;
+    const int l0 = c * XT;
+    m_store(c, slot);
+    In nxt;
+    m_load(c + c_step);
+    in_load(nxt, c + c_step);
+    __syncthreads();   // planes of this chunk visible; the other slot was last read one barrier ago
+
+    float th[2][4], x[8];
+    bool big = false;
+#pragma unroll
+    for (int st = 0; st < 2; ++st) {
+      const bool ok = dok && (l0 + 16 * st + 4 * g < L);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        th[st][i] = ok ? cur.th[st][i] : 0.0f;
+        big |= fabsf(th[st][i]) > 4.0f;
+        const float v = ADJ ? cur.a[st][i] : cur.a[st][i] * cur.b[st][i];
+        x[4 * st + i] = ok ? v : 0.0f;
+      }
+    }
+    if (__builtin_expect(__any(big), 0)) {
+#pragma unroll
+      for (int st = 0; st < 2; ++st)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) th[st][i] = (float)remainder((double)th[st][i], 6.283185307179586476925);
+    }
+    // running phase inside the chunk: the lane's two runs of four steps, then across the lane groups
+#pragma unroll
+    for (int st = 0; st < 2; ++st) { th[st][1] += th[st][0]; th[st][2] += th[st][1]; th[st][3] += th[st][2]; }
+    float sa = th[0][3], sb = th[1][3];
+    {
+      float ta = __shfl_up(sa, 16), tb = __shfl_up(sb, 16);
+      if (g >= 1) { sa += ta; sb += tb; }
+      ta = __shfl_up(sa, 32); tb = __shfl_up(sb, 32);
+      if (g >= 2) { sa += ta; sb += tb; }
+    }
+    const float tot_a = __shfl(sa, 48 + dl);
+    const float off_a = sa - th[0][3];
+    const float off_b = tot_a + sb - th[1][3];
+    float xr[8], xi[8], c7 = 0.0f, s7 = 0.0f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float ph = th[e >> 2][e & 3] + ((e >> 2) ? off_b : off_a);
+      float sn, cs;
+      sincos_small(ph, &sn, &cs);
+      xr[e] = cs * x[e];        // x conj(P)
+      xi[e] = -sn * x[e];
+      if (e == 7) { c7 = cs; s7 = sn; }
+    }
+    const float cT = __shfl(c7, 48 + dl), sT = __shfl(s7, 48 + dl);   // rotation of the whole chunk
+    u4 Xr[NP], Xi[NP], nXi[NP];
+    split8<NP>(sk, xr, Xr);
+    split8<NP>(sk, xi, Xi);
+#pragma unroll
+    for (int q = 0; q < NP; ++q) nXi[q] = neg_bf16x8(Xi[q]);
+    u4 mr[NP], mi[NP];
+#pragma unroll
+    for (int q = 0; q < NP; ++q) { mr[q] = s_mr[slot][q][xrec(dl, g, XN)]; mi[q] = s_mi[slot][q][xrec(dl, g, XN)]; }
+    if (ADJ) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float ar = Sr[i], ai = Si[i];
+        Sr[i] = cT * ar + sT * ai;
+        Si[i] = cT * ai - sT * ar;
+      }
+    }
+    Sr = xmm<NP>(mr, Xr, Sr);  Sr = xmm<NP>(mi, nXi, Sr);
+    Si = xmm<NP>(mr, Xi, Si);  Si = xmm<NP>(mi, Xr, Si);
+    if (!ADJ) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float hr = Sr[i], hi = Si[i];
+        Sr[i] = cT * hr - sT * hi;
+        Si[i] = cT * hi + sT * hr;
+      }
+    }
+    {
+      const float nr = pr * cT - pi * sT, ni = pr * sT + pi * cT;
+      pr = nr; pi = ni;
+    }
+    cur = nxt;
+  }
+
+  if (dok) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int n = 4 * g + i;
+      if (n < N) {
+        const size_t o = (((size_t)vb * D + d) * N + n) * 2;
+        p.out[o] = Sr[i];
+        p.out[o + 1] = Si[i];
+      }
+    }
+    if (g == 0) {
+      p.ptot[((size_t)vb * D + d) * 2] = pr;
+      p.ptot[((size_t)vb * D + d) * 2 + 1] = pi;
+    }
+  }
+}
+
+// Chains the segments of one (batch, channel, state): on entry seg[k] holds Z_k, on return the
+// state that enters segment k; the state after the last segment goes to hL (if wanted).
+__global__ void seg_carry_fwd_kernel(float* __restrict__ seg, const float* __restrict__ ptot,
+                                     const float* __restrict__ h0, float* __restrict__ hL,
+                                     int B, int D, int N, int ns) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (size_t)B * D * N) return;
+  const int n = (int)(idx % N);
+  const int d = (int)((idx / N) % D);
+  const int b = (int)(idx / ((size_t)N * D));
+  float hr = h0 ? h0[idx * 2] : 0.0f, hi = h0 ? h0[idx * 2 + 1] : 0.0f;
+  for (int k = 0; k < ns; ++k) {
+    const size_t v = ((size_t)b * ns + k) * D + d;
+    const size_t o = (v * N + n) * 2;
+    const float zr = seg[o], zi = seg[o + 1], pr = ptot[v * 2], pi = ptot[v * 2 + 1];
+    seg[o] = hr; seg[o + 1] = hi;
+    const float nr = pr * hr - pi * hi + zr, ni = pr * hi + pi * hr + zi;
+    hr = nr; hi = ni;
+  }
+  if (hL) { hL[idx * 2] = hr; hL[idx * 2 + 1] = hi; }
+}
+
+// The same for the adjoint, last segment first: on entry seg[k] holds Y_k, on return the adjoint
+// that enters segment k at its end; the adjoint of the initial state goes to dh0 (if wanted).
+__global__ void seg_carry_bwd_kernel(float* __restrict__ seg, const float* __restrict__ ptot,
+                                     const float* __restrict__ dhL, float* __restrict__ dh0,
+                                     int B, int D, int N, int ns) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (size_t)B * D * N) return;
+  const int n = (int)(idx % N);
+  const int d = (int)((idx / N) % D);
+  const int b = (int)(idx / ((size_t)N * D));
+  float ar = dhL ? dhL[idx * 2] : 0.0f, ai = dhL ? dhL[idx * 2 + 1] : 0.0f;
+  for (int k = ns - 1; k >= 0; --k) {
+    const size_t v = ((size_t)b * ns + k) * D + d;
+    const size_t o = (v * N + n) * 2;
+    const float yr = seg[o], yi = seg[o + 1], pr = ptot[v * 2], pi = ptot[v * 2 + 1];
+    seg[o] = ar; seg[o + 1] = ai;
+    const float nr = pr * ar + pi * ai + yr, ni = pr * ai - pi * ar + yi;
+    ar = nr; ai = ni;
+  }
+  if (dh0) { dh0[idx * 2] = ar; dh0[idx * 2 + 1] = ai; }
+}
+
+}  // namespace aussm

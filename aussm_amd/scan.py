@@ -92,12 +92,15 @@ def num_checkpoints(L: int, ck: int) -> int:
 # raw launches (no autograd)
 # --------------------------------------------------------------------------------------------
 
-def unitary_aux(u) -> Tensor:
-    """The optional auxiliary buffer of the unitary scan for inputs shaped like u (b, d, l): the
-    forward call may leave intermediate results in it that spare the backward call a recomputation."""
+def unitary_aux(u, n: int, ck: int) -> Tensor:
+    """The optional auxiliary buffer of the unitary scan for inputs shaped like u (b, d, l) with n
+    states and checkpoint interval ck: the forward call may leave intermediate results in it that
+    spare the backward call a recomputation, and a call that splits a long sequence over more
+    workgroups keeps its segment states there."""
     lib = _lib.load()
     b, d, l = u.shape
-    return torch.empty((lib.aussm_unitary_aux_floats(b, d, l),), device=u.device, dtype=torch.float32)
+    return torch.empty((lib.aussm_unitary_aux_floats(b, d, n, l, ck or _lib.TILE),), device=u.device,
+                       dtype=torch.float32)
 
 
 def unitary_fwd_raw(u, delta, theta, Bri, Cri, D=None, z=None, h0=None, want_state=False, ck=0, aux=None):
@@ -145,7 +148,7 @@ class _UnitaryScanFn(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, u, delta, theta, Bri, Cri, D, h0):
-        aux = unitary_aux(u)
+        aux = unitary_aux(u, Bri.shape[1], UNITARY_CK)
         y, hL, hck = unitary_fwd_raw(u, delta, theta, Bri, Cri, D, None, h0, want_state=True, ck=UNITARY_CK, aux=aux)
         ctx.save_for_backward(u, delta, theta, Bri, Cri, D, hck, aux)
         ctx.has_h0 = h0 is not None

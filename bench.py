@@ -92,7 +92,7 @@ def main():
     Cri = torch.view_as_real(p["Cc"]).contiguous()
     ck = scan.UNITARY_CK
 
-    aux = scan.unitary_aux(p["u"])      # what the autograd wrapper hands from forward to backward
+    aux = scan.unitary_aux(p["u"], N, scan.UNITARY_CK)      # what the autograd wrapper hands from forward to backward
 
     def step():
         y, _, hck = scan.unitary_fwd_raw(p["u"], p["delta"], p["theta"], Bri, Cri, p["Dskip"], None, None,

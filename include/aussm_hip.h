@@ -99,14 +99,22 @@ int aussm_unitary_bwd(const float* dy, const float* dhL,
                       int B, int D, int N, int L, int ck, int in_dtype, void* stream);
 
 /* Variants of the two calls above with an optional auxiliary buffer (NULL allowed; then they are
- * the calls above).  `aux` holds aussm_unitary_aux_floats(B, D, L) floats, 16-byte aligned.  The
- * forward call may leave per-(b,d,l) intermediate results in it (Im(P_t S_t), the term of the phase
- * gradient that needs the forward states) together with a validity tag; the backward call given
- * the same buffer then skips recomputing them.  A forward kernel that does not fill the buffer
- * clears the tag, so a backward call never consumes stale contents: handing over `aux` is always
- * safe and only ever a speed-up.  No counterpart in the reference (its backward kernel recomputes,
- * ssm_adaptive_unitary_backward.cu:113-181). */
-size_t aussm_unitary_aux_floats(int B, int D, int L);
+ * the calls above).  `aux` holds aussm_unitary_aux_floats(B, D, N, L, ck) floats, 16-byte aligned,
+ * sized with the arguments of the calls it is passed to.  Two uses, both internal:
+ *  - the forward call may leave per-(b,d,l) intermediate results in it (Im(P_t S_t), the term of
+ *    the phase gradient that needs the forward states) together with a validity tag; the backward
+ *    call given the same buffer then skips recomputing them.  A forward kernel that does not fill
+ *    the buffer clears the tag, so a backward call never consumes stale contents: handing over
+ *    `aux` is always safe and only ever a speed-up;
+ *  - a launch with few (batch, channel) pairs and a long sequence is split along L over more
+ *    workgroups (per-segment end states from a zero start, a short chain over the segments, then
+ *    the scan of every segment from its true incoming state - the two-level scan of
+ *    ssm_adaptive_unitary_forward.cu:122-162 one level up); the segment states live behind the
+ *    per-(b,d,l) part of the buffer, during the call only.  Each call writes there: two calls
+ *    that share one buffer must not overlap.  AUSSM_SPLIT=0 (environment) switches the split off.
+ * No counterpart in the reference (its backward kernel recomputes,
+ * ssm_adaptive_unitary_backward.cu:113-181, and its launches cover at most 2048 steps). */
+size_t aussm_unitary_aux_floats(int B, int D, int N, int L, int ck);
 
 int aussm_unitary_fwd_aux(const void* u, const void* delta, const float* theta,
                           const void* Bc, const void* Cc, const float* Dskip, const float* z,
@@ -116,7 +124,7 @@ int aussm_unitary_fwd_aux(const void* u, const void* delta, const float* theta,
 int aussm_unitary_bwd_aux(const float* dy, const float* dhL,
                           const void* u, const void* delta, const float* theta,
                           const void* Bc, const void* Cc, const float* Dskip, const float* hck,
-                          const float* aux,
+                          float* aux,
                           float* du, float* ddelta, float* dtheta, float* dB, float* dC,
                           float* dD, float* dh0,
                           int B, int D, int N, int L, int ck, int in_dtype, void* stream);

@@ -6,6 +6,8 @@ gradients at L=16384 are compared on a slice of the channels, and the full sizes
 size-independent properties: splitting the sequence with a carried state, linearity in the
 input, independence of batch elements, and the adjoint identity <dy, J v> = <J^T dy, v>.
 float32 tolerance: atol = rtol = 1e-4; bfloat16 inputs: 2e-2."""
+import os
+
 import pytest
 import torch
 
@@ -122,8 +124,15 @@ def test_headline_shape_batch_slice_and_independence():
         _close(g, w, f"d{k}[0:2]")
     print("case headline full batch", flush=True)
     y_all, g_all = run(scan.unitary_scan, "cuda", slice(0, B))
-    assert torch.equal(y_all[0:2], y_dev), "forward output must not depend on the other batch elements"
-    y_tail, g_tail = run(scan.unitary_scan, "cuda", slice(B - 3, B))
+    _close(y_all[0:2], y_dev.cpu(), "y full batch vs slice", tol=1e-5)
+    # bit for bit when the same kernels run: small batches are otherwise split along the sequence
+    os.environ["AUSSM_SPLIT"] = "0"
+    try:
+        y_head, _ = run(scan.unitary_scan, "cuda", slice(0, 2))
+        y_tail, _ = run(scan.unitary_scan, "cuda", slice(B - 3, B))
+    finally:
+        del os.environ["AUSSM_SPLIT"]
+    assert torch.equal(y_all[0:2], y_head), "forward output must not depend on the other batch elements"
     assert torch.equal(y_all[B - 3:], y_tail)
     for k, ga, gs in zip(names, g_all, g_dev):
         a, s = ga[0:2], gs

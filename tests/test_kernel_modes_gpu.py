@@ -115,7 +115,7 @@ def test_auxiliary_buffer_is_never_consumed_stale():
         Bri = torch.view_as_real(q["Bc"]).contiguous()
         Cri = torch.view_as_real(q["Cc"]).contiguous()
         if aux is None:
-            aux = scan.unitary_aux(q["u"])
+            aux = scan.unitary_aux(q["u"], N, scan.UNITARY_CK)
         print(f"case aux seed={seed} fwd_mode={fwd_mode}", flush=True)
         with _Env(AUSSM_MFMA=fwd_mode):
             yk, _, hck = scan.unitary_fwd_raw(q["u"], q["delta"], q["theta"], Bri, Cri, q["Dskip"], None, None,
@@ -127,3 +127,41 @@ def test_auxiliary_buffer_is_never_consumed_stale():
         du, ddelta, dtheta, dB, dC, dD, _ = got
         for k, w, gt in zip(NAMES, want, (du, ddelta, dtheta, torch.view_as_complex(dB), torch.view_as_complex(dC), dD)):
             _close(gt, w, f"d{k} (forward mode {fwd_mode})")
+
+
+@pytest.mark.parametrize("B,D,N,L,cap", [(1, 64, 16, 1024, None), (1, 64, 16, 1024, "2"), (2, 80, 8, 512, None),
+                                         (1, 40, 16, 2048, None)])
+def test_sequence_split_over_workgroups(B, D, N, L, cap):
+    """With few (batch, channel) pairs the launcher cuts the sequence into segments that run in
+    parallel (segment end states from a zero start, a chain over the segments, then every segment
+    from its true incoming state; the adjoint likewise in reverse).  Outputs, the final state and
+    every gradient, with a carried-in state and an upstream gradient of the final state, against
+    the CPU oracle and against the same call with the split switched off."""
+    from aussm_amd import scan, _lib
+    lib = _lib.load()
+    # the shapes are chosen so that the split happens: its states need room behind the per-(b,d,l) part
+    assert lib.aussm_unitary_aux_floats(B, D, N, L, scan.UNITARY_CK) > B * D * L + 64
+    p = _inputs(B, D, N, L, 3 + L + D, big_theta=(D == 80))
+    g = torch.Generator().manual_seed(9)
+    dh = torch.complex(torch.randn(B, D, N, generator=g), torch.randn(B, D, N, generator=g))
+
+    def run(fn, dev):
+        lv = [p[k].clone().to(dev).requires_grad_(True) for k in NAMES]
+        h0 = p["h0"].clone().to(dev).requires_grad_(True)
+        y, hL = fn(*lv, None, h0)
+        loss = (y * p["dy"].to(dev)).sum() + (torch.view_as_real(hL) * torch.view_as_real(dh.to(dev))).sum()
+        loss.backward()
+        return [y.detach(), hL.detach()] + [t.grad for t in lv] + [h0.grad]
+
+    names = ("y", "hL") + tuple("d" + k for k in NAMES) + ("dh0",)
+    want = run(lambda *a: O.unitary_core_loop(*a), "cpu")
+    print(f"case split B={B} D={D} N={N} L={L} cap={cap}", flush=True)
+    with _Env(**({"AUSSM_SPLIT": cap} if cap else {})):
+        got = run(lambda *a: scan.unitary_scan(*a, return_last_state=True), "cuda")
+        torch.cuda.synchronize()
+    with _Env(AUSSM_SPLIT="0"):
+        whole = run(lambda *a: scan.unitary_scan(*a, return_last_state=True), "cuda")
+        torch.cuda.synchronize()
+    for k, w, gt, wh in zip(names, want, got, whole):
+        _close(gt, w, k, tol=2e-4 if D == 80 else 1e-4)
+        _close(gt, wh.cpu(), k + " (split vs whole)", tol=2e-5)
