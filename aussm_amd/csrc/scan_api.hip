@@ -121,7 +121,18 @@ inline int seg_count(int B, int D, int N, int L, int ck) {
   }
   return ns;
 }
-inline size_t seg_floats(int B, int D, int N, int ns) { return ns > 1 ? (size_t)B * ns * D * (2 * N + 2) : 0; }
+// The segment states are computed on finer segments than the scan proper uses (the kernel that
+// forms them is light: several workgroups per compute unit hide its latencies); the scan takes
+// every SPLIT_FINE-th of them.
+inline int seg_fine(int L, int ns) {
+  const int Ls = L / ns;
+  for (int r = 4; r > 1; r /= 2)
+    if (Ls % (r * XT) == 0 && Ls / r >= SPLIT_MIN_LEN) return r;
+  return 1;
+}
+inline size_t seg_floats(int B, int D, int N, int L, int ns) {
+  return ns > 1 ? (size_t)B * ns * seg_fine(L, ns) * D * (2 * N + 2) : 0;
+}
 
 inline int mfma_fwd_mode(const FwdArgs& a, int in_dtype) {
   const int mode = env_mode("AUSSM_MFMA", 3, a.N);
@@ -143,16 +154,16 @@ int launch_fwd(FwdArgs a, int in_dtype, hipStream_t s) {
       if (ns > 1) {
         // 1. end state of every segment from a zero start and its rotation; 2. chain them;
         // 3. the scan proper over (batch, segment) pairs, each from its true incoming state
-        const int B = a.B, L = a.L, Ls = a.L / ns;
+        const int B = a.B, L = a.L, Ls = a.L / ns, r = seg_fine(L, ns), nf = ns * r;
         float* seg = a.aux + (size_t)B * a.D * L + AUX_PAD;
-        float* ptot = seg + (size_t)B * ns * a.D * a.N * 2;
+        float* ptot = seg + (size_t)B * nf * a.D * a.N * 2;
         SegArgs sa{static_cast<const float*>(a.delta), static_cast<const float*>(a.u), a.theta,
-                   static_cast<const float*>(a.Bm), seg, ptot, a.D, a.N, Ls, L, ns, a.ncg};
-        hipLaunchKernelGGL((unitary_seg_state_kernel<3, false>), dim3((unsigned)(B * ns * a.ncg)), dim3(256), 0, s, sa);
+                   static_cast<const float*>(a.Bm), seg, ptot, a.D, a.N, Ls / r, L, nf, a.ncg};
+        hipLaunchKernelGGL((unitary_seg_state_kernel<3, false>), dim3((unsigned)(B * nf * a.ncg)), dim3(256), 0, s, sa);
         const size_t nst = (size_t)B * a.D * a.N;
         hipLaunchKernelGGL(seg_carry_fwd_kernel, dim3((unsigned)((nst + 255) / 256)), dim3(256), 0, s, seg, ptot, a.h0,
-                           a.hL, B, a.D, a.N, ns);
-        a.B = B * ns; a.L = Ls; a.ns = ns; a.nck = Ls / a.ck; a.h0 = seg; a.hL = nullptr;
+                           a.hL, B, a.D, a.N, nf);
+        a.B = B * ns; a.L = Ls; a.ns = ns; a.nck = Ls / a.ck; a.h0 = seg; a.hL = nullptr; a.hs = r; a.ho = 0;
       }
     }
     const dim3 grid((unsigned)(a.B * a.ncg));
@@ -236,7 +247,7 @@ int aussm_bwd_checkpoint_interval(int variant) { return variant == VAR_UNITARY ?
 
 size_t aussm_unitary_aux_floats(int B, int D, int N, int L, int ck) {
   if (B < 1 || D < 1 || N < 1 || L < 1) return 0;
-  return (size_t)B * D * L + AUX_PAD + seg_floats(B, D, N, seg_capacity(B, D, N, L, ck));
+  return (size_t)B * D * L + AUX_PAD + seg_floats(B, D, N, L, seg_capacity(B, D, N, L, ck));
 }
 
 int aussm_unitary_fwd(const void* u, const void* delta, const float* theta, const void* Bc, const void* Cc,
@@ -258,7 +269,7 @@ int aussm_unitary_fwd_aux(const void* u, const void* delta, const float* theta, 
   a.u = u; a.delta = delta; a.theta = theta; a.Bm = Bc; a.Cm = Cc; a.Dskip = Dskip; a.z = z;
   a.h0 = h0; a.y = y; a.hL = hL; a.hck = hck; a.aux = aux;
   a.B = B; a.D = D; a.N = N; a.L = L; a.ck = ck; a.nck = (L + ck - 1) / ck; a.ncg = (D + CH - 1) / CH;
-  a.ld = L; a.ns = 1;
+  a.ld = L; a.ns = 1; a.hs = 1; a.ho = 0;
   return launch_fwd<VAR_UNITARY>(a, in_dtype, (hipStream_t)stream);
 }
 
@@ -273,7 +284,7 @@ int aussm_complex_fwd(const void* u, const void* delta, const float* rho, const 
   a.u = u; a.delta = delta; a.rho = rho; a.theta = theta; a.Bm = Bc; a.Cm = Cc; a.Dskip = Dskip; a.z = z;
   a.h0 = h0; a.y = y; a.hL = hL; a.hck = hck;
   a.B = B; a.D = D; a.N = N; a.L = L; a.ck = ck; a.nck = (L + ck - 1) / ck; a.ncg = (D + CH - 1) / CH;
-  a.ld = L; a.ns = 1;
+  a.ld = L; a.ns = 1; a.hs = 1; a.ho = 0;
   return launch_fwd<VAR_COMPLEX>(a, in_dtype, (hipStream_t)stream);
 }
 
@@ -288,7 +299,7 @@ int aussm_real_fwd(const void* u, const void* delta, const float* A, const void*
   a.delta_bias = delta_bias; a.delta_softplus = delta_softplus;
   a.h0 = h0; a.y = y; a.hL = hL; a.hck = hck;
   a.B = B; a.D = D; a.N = N; a.L = L; a.ck = ck; a.nck = (L + ck - 1) / ck; a.ncg = (D + CH - 1) / CH;
-  a.ld = L; a.ns = 1;
+  a.ld = L; a.ns = 1; a.hs = 1; a.ho = 0;
   return launch_fwd<VAR_REAL>(a, in_dtype, (hipStream_t)stream);
 }
 
@@ -315,7 +326,7 @@ int aussm_unitary_bwd_aux(const float* dy, const float* dhL, const void* u, cons
   a.dy = dy; a.dhL = dhL; a.u = u; a.delta = delta; a.theta = theta; a.Bm = Bc; a.Cm = Cc; a.Dskip = Dskip;
   a.hck = hck; a.aux = aux; a.du = du; a.ddelta = ddelta; a.dtheta = dtheta; a.dB = dB; a.dC = dC; a.dD = dD; a.dh0 = dh0;
   a.B = B; a.D = D; a.N = N; a.L = L; a.ck = ck; a.nck = (L + ck - 1) / ck; a.ncg = (D + CH - 1) / CH;
-  a.ld = L; a.ns = 1;
+  a.ld = L; a.ns = 1; a.hs = 1; a.ho = 0;
   const int mode = env_mode("AUSSM_MFMA_BWD", 3, N);   // matrix-core kernel for the common case
   if (mode > 0 && in_dtype == AUSSM_F32 && N <= XN && L % 4 == 0 && ck % XT == 0 &&
       !(misaligned(dy, 16) || misaligned(u, 16) || misaligned(delta, 16) || misaligned(theta, 16) ||
@@ -324,15 +335,16 @@ int aussm_unitary_bwd_aux(const float* dy, const float* dhL, const void* u, cons
     const int ns = aux ? seg_count(B, D, N, L, ck) : 1;
     if (ns > 1) {
       // adjoint at the start of every segment from a zero adjoint at its end, chained last to first
-      const int Ls = L / ns;
+      const int Ls = L / ns, r = seg_fine(L, ns), nf = ns * r;
       float* seg = aux + (size_t)B * D * L + AUX_PAD;
-      float* ptot = seg + (size_t)B * ns * D * N * 2;
-      SegArgs sa{dy, nullptr, theta, static_cast<const float*>(Cc), seg, ptot, D, N, Ls, L, ns, a.ncg};
-      hipLaunchKernelGGL((unitary_seg_state_kernel<3, true>), dim3((unsigned)(B * ns * a.ncg)), dim3(256), 0, s, sa);
+      float* ptot = seg + (size_t)B * nf * D * N * 2;
+      SegArgs sa{dy, nullptr, theta, static_cast<const float*>(Cc), seg, ptot, D, N, Ls / r, L, nf, a.ncg};
+      hipLaunchKernelGGL((unitary_seg_state_kernel<3, true>), dim3((unsigned)(B * nf * a.ncg)), dim3(256), 0, s, sa);
       const size_t nst = (size_t)B * D * N;
       hipLaunchKernelGGL(seg_carry_bwd_kernel, dim3((unsigned)((nst + 255) / 256)), dim3(256), 0, s, seg, ptot, dhL, dh0,
-                         B, D, N, ns);
-      a.B = B * ns; a.L = Ls; a.ns = ns; a.nck = Ls / ck; a.dhL = seg; a.dh0 = nullptr;
+                         B, D, N, nf);
+      // a segment of the scan ends where its last fine segment ends
+      a.B = B * ns; a.L = Ls; a.ns = ns; a.nck = Ls / ck; a.dhL = seg; a.dh0 = nullptr; a.hs = r; a.ho = r - 1;
     }
     const dim3 grid((unsigned)(a.B * a.ncg));
     if (mode == 2) hipLaunchKernelGGL((unitary_bwd_xdl_kernel<2, 2>), grid, dim3(256), 0, s, a);

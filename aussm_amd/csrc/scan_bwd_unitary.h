@@ -39,6 +39,7 @@ struct UniBwdArgs {
   float* dh0;           // [B,D,N,2] or null
   int B, D, N, L, ck, nck, ncg;
   int ld, ns;           // matrix-core kernel: row stride of the [.., L] tensors, segments per sequence
+  int hs, ho;           // ... and dhL of (batch, segment) pair b is entry b * hs + ho of the adjoint array
 };
 
 constexpr int RED_COLS = 4 * TG;        // products per lane per turn: TG x (dB re, dB im) then TG x (dC re, dC im)

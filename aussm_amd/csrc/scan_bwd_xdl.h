@@ -312,7 +312,7 @@ __global__ __launch_bounds__(256) void unitary_bwd_xdl_kernel(const UniBwdArgs p
     for (int i = 0; i < 4; ++i) {
       const int n = 4 * g + i;
       if (n < N) {
-        const size_t o = (((size_t)b * D + d) * N + n) * 2;
+        const size_t o = ((((size_t)b * p.hs + p.ho) * D + d) * N + n) * 2;
         Ar[i] = p.dhL[o];
         Ai[i] = p.dhL[o + 1];
       }

@@ -27,6 +27,7 @@ struct FwdArgs {
   int B, D, N, L, ck, nck, ncg, delta_softplus;
   int ld, ns;                // matrix-core unitary kernels: row stride of the [.., L] tensors and segments per
                              // sequence (B then counts batch x segment pairs and L is the segment length)
+  int hs, ho;                // ... and h0 of pair b is entry b * hs + ho of the state array
 };
 
 // VAR: variant.  NW: states per wavefront.  NT: threads per workgroup.  Tin: float or bf16_t.

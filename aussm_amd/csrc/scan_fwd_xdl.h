@@ -358,7 +358,7 @@ __global__ __launch_bounds__(256) void unitary_fwd_xdl_kernel(const FwdArgs p) {
     for (int i = 0; i < 4; ++i) {
       const int n = 4 * g + i;
       if (n < N) {
-        const size_t o = (((size_t)b * D + d) * N + n) * 2;
+        const size_t o = ((((size_t)b * p.hs + p.ho) * D + d) * N + n) * 2;
         Hr[i] = p.h0[o];
         Hi[i] = p.h0[o + 1];
       }

@@ -206,6 +206,8 @@ __global__ __launch_bounds__(256) void unitary_seg_state_kernel(const SegArgs p)
   }
 }
 
+constexpr int SEG_BATCH = 16;
+
 // Chains the segments of one (batch, channel, state): on entry seg[k] holds Z_k, on return the
 // state that enters segment k; the state after the last segment goes to hL (if wanted).
 __global__ void seg_carry_fwd_kernel(float* __restrict__ seg, const float* __restrict__ ptot,
@@ -217,13 +219,25 @@ __global__ void seg_carry_fwd_kernel(float* __restrict__ seg, const float* __res
   const int d = (int)((idx / N) % D);
   const int b = (int)(idx / ((size_t)N * D));
   float hr = h0 ? h0[idx * 2] : 0.0f, hi = h0 ? h0[idx * 2 + 1] : 0.0f;
-  for (int k = 0; k < ns; ++k) {
-    const size_t v = ((size_t)b * ns + k) * D + d;
-    const size_t o = (v * N + n) * 2;
-    const float zr = seg[o], zi = seg[o + 1], pr = ptot[v * 2], pi = ptot[v * 2 + 1];
-    seg[o] = hr; seg[o + 1] = hi;
-    const float nr = pr * hr - pi * hi + zr, ni = pr * hi + pi * hr + zi;
-    hr = nr; hi = ni;
+  // batches of SEG_BATCH segments: all loads of a batch first (independent of the chain), then the chain
+  for (int k0 = 0; k0 < ns; k0 += SEG_BATCH) {
+    float2 z[SEG_BATCH], q[SEG_BATCH];
+#pragma unroll
+    for (int j = 0; j < SEG_BATCH; ++j) {
+      const int k = k0 + j < ns ? k0 + j : ns - 1;
+      const size_t v = ((size_t)b * ns + k) * D + d;
+      z[j] = *reinterpret_cast<const float2*>(seg + (v * N + n) * 2);
+      q[j] = *reinterpret_cast<const float2*>(ptot + v * 2);
+    }
+#pragma unroll
+    for (int j = 0; j < SEG_BATCH; ++j) {
+      if (k0 + j < ns) {
+        const size_t v = ((size_t)b * ns + k0 + j) * D + d;
+        *reinterpret_cast<float2*>(seg + (v * N + n) * 2) = make_float2(hr, hi);
+        const float nr = q[j].x * hr - q[j].y * hi + z[j].x, ni = q[j].x * hi + q[j].y * hr + z[j].y;
+        hr = nr; hi = ni;
+      }
+    }
   }
   if (hL) { hL[idx * 2] = hr; hL[idx * 2 + 1] = hi; }
 }
@@ -239,13 +253,24 @@ __global__ void seg_carry_bwd_kernel(float* __restrict__ seg, const float* __res
   const int d = (int)((idx / N) % D);
   const int b = (int)(idx / ((size_t)N * D));
   float ar = dhL ? dhL[idx * 2] : 0.0f, ai = dhL ? dhL[idx * 2 + 1] : 0.0f;
-  for (int k = ns - 1; k >= 0; --k) {
-    const size_t v = ((size_t)b * ns + k) * D + d;
-    const size_t o = (v * N + n) * 2;
-    const float yr = seg[o], yi = seg[o + 1], pr = ptot[v * 2], pi = ptot[v * 2 + 1];
-    seg[o] = ar; seg[o + 1] = ai;
-    const float nr = pr * ar + pi * ai + yr, ni = pr * ai - pi * ar + yi;
-    ar = nr; ai = ni;
+  for (int k0 = ns - 1; k0 >= 0; k0 -= SEG_BATCH) {
+    float2 y[SEG_BATCH], q[SEG_BATCH];
+#pragma unroll
+    for (int j = 0; j < SEG_BATCH; ++j) {
+      const int k = k0 - j >= 0 ? k0 - j : 0;
+      const size_t v = ((size_t)b * ns + k) * D + d;
+      y[j] = *reinterpret_cast<const float2*>(seg + (v * N + n) * 2);
+      q[j] = *reinterpret_cast<const float2*>(ptot + v * 2);
+    }
+#pragma unroll
+    for (int j = 0; j < SEG_BATCH; ++j) {
+      if (k0 - j >= 0) {
+        const size_t v = ((size_t)b * ns + k0 - j) * D + d;
+        *reinterpret_cast<float2*>(seg + (v * N + n) * 2) = make_float2(ar, ai);
+        const float nr = q[j].x * ar + q[j].y * ai + y[j].x, ni = q[j].x * ai - q[j].y * ar + y[j].y;
+        ar = nr; ai = ni;
+      }
+    }
   }
   if (dh0) { dh0[idx * 2] = ar; dh0[idx * 2 + 1] = ai; }
 }

@@ -64,8 +64,8 @@ def test_argument_checks_without_a_device():
     # the auxiliary buffer: size query, alignment check, NULL accepted like the plain entry points
     assert lib.aussm_unitary_aux_floats(32, 512, 16, 2048, 256) == 32 * 512 * 2048 + 64
     assert lib.aussm_unitary_aux_floats(0, 1, 1, 1, 32) == 0
-    # few (batch, channel) pairs and a long sequence: room for the states of 16 segments of 1024 steps
-    assert lib.aussm_unitary_aux_floats(4, 256, 16, 16384, 256) == 4 * 256 * 16384 + 64 + 4 * 16 * 256 * (2 * 16 + 2)
+    # few (batch, channel) pairs and a long sequence: room for the states of 64 segments of 256 steps
+    assert lib.aussm_unitary_aux_floats(4, 256, 16, 16384, 256) == 4 * 256 * 16384 + 64 + 4 * 64 * 256 * (2 * 16 + 2)
     # ... which needs whole checkpoint blocks per segment, and states the matrix-core kernels serve
     assert lib.aussm_unitary_aux_floats(4, 256, 16, 16384 + 4, 256) == 4 * 256 * (16384 + 4) + 64
     assert lib.aussm_unitary_aux_floats(4, 256, 4, 16384, 256) == 4 * 256 * 16384 + 64
