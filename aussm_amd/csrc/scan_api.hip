@@ -100,7 +100,7 @@ inline int env_mode(const char* name, int dflt, int N) {
 // until about one workgroup per compute unit exists.  Only the matrix-core kernels take part,
 // and only the *_aux entry points (the segment states live behind the auxiliary buffer).
 // AUSSM_SPLIT (environment): 0 or 1 switches it off, a power of two caps ns.
-constexpr int SPLIT_MIN_WGS = 128;     // launches of at least this many workgroups are left alone
+constexpr int SPLIT_MIN_WGS = 129;     // launches of at least this many workgroups are left alone
 constexpr int SPLIT_TARGET_WGS = 256;
 constexpr int SPLIT_MAX = 32;
 constexpr int SPLIT_MIN_LEN = 128;

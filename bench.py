@@ -2,7 +2,10 @@
 """Headline benchmark: adaptive-unitary core scan, forward + backward, fp32,
 B=32 D=512 N=16 L=2048, on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--shape B,D,N,L]
+
+(--shape runs the same step at another shape, e.g. 4,256,16,16384, the long-sequence case whose
+launches are split along L; the default and the contract line are the headline shape.)
 
 One "step" = one forward launch (y, checkpoints) + zero-fill of the accumulated gradients +
 one backward launch (du, ddelta, dtheta, dB, dC, dD) on synthetic inputs that are already
@@ -72,7 +75,11 @@ def main():
     ap.add_argument("--cpu-batch", type=int, default=8)
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one 256 MiB device-to-device copy (calibrates FETCH_SIZE / WRITE_SIZE under rocprofv3)")
+    ap.add_argument("--shape", default=None, help="B,D,N,L instead of the headline shape (no recorded traffic figure then)")
     args = ap.parse_args()
+    headline = args.shape is None
+    if not headline:
+        SHAPE.update(zip("BDNL", (int(v) for v in args.shape.split(","))))
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus must be 1 (no multi-GPU path exists)", file=sys.stderr)
         sys.exit(2)
@@ -154,7 +161,7 @@ def main():
     ach = bytes_bwd / (t_bwd * 1e-6) / 1e9
 
     out = {
-        "metric": "unitary scan fwd+bwd elements/s + achieved HBM GB/s (% peak), B32 D512 N16 L2048",
+        "metric": f"unitary scan fwd+bwd elements/s + achieved HBM GB/s (% peak), B{B} D{D} N{N} L{L}",
         "value": B * D * L / dt,
         "unit": "(b,d,l) samples/s",
         "n_gpus": 1,
@@ -166,23 +173,24 @@ def main():
         "vs_baseline": None,
         "dtype": "f32",
         "data": "synthetic",
-        "config": {"workload": "unitary core scan fwd+bwd, B=32 D=512 N=16 L=2048, fp32 (BASELINE configs[3], unitary, fp32)",
+        "config": {"workload": (f"unitary core scan fwd+bwd, B={B} D={D} N={N} L={L}, fp32"
+                                + (" (BASELINE configs[3], unitary, fp32)" if headline else "")),
                    "B": B, "D": D, "N": N, "L": L, "checkpoint_interval": ck},
         "state_updates_per_s": B * D * N * L / dt,
         "fwd_bwd_algorithmic_GBps": (bytes_fwd + bytes_bwd) / ((t_fwd + t_bwd) * 1e-6) / 1e9,
         "fwd_bwd_frac_of_hbm_peak": (bytes_fwd + bytes_bwd) / ((t_fwd + t_bwd) * 1e-6) / 1e9 / HBM_PEAK_GBS,
         "kernels_us": {"unitary_fwd": t_fwd, "unitary_bwd": t_bwd},
         "roofline": {"bound": "hbm", "kernel": "unitary_bwd_xdl_kernel<3, 2>", "achieved": ach, "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": ach / HBM_PEAK_GBS, "traffic": TRAFFIC_BYTES["unitary_bwd"],
+                     "unit": "GB/s", "frac": ach / HBM_PEAK_GBS, "traffic": TRAFFIC_BYTES["unitary_bwd"] if headline else None,
                      "algorithmic_bytes": bytes_bwd,
                      "fwd_kernel": {"kernel": "unitary_fwd_xdl_kernel<3, false>",
                                     "achieved": bytes_fwd / (t_fwd * 1e-6) / 1e9,
                                     "frac": bytes_fwd / (t_fwd * 1e-6) / 1e9 / HBM_PEAK_GBS,
-                                    "traffic": TRAFFIC_BYTES["unitary_fwd"],
+                                    "traffic": TRAFFIC_BYTES["unitary_fwd"] if headline else None,
                                     "algorithmic_bytes": bytes_fwd}},
     }
     if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline(args.cpu_batch)
+        out["cpu_baseline"] = cpu_baseline(min(args.cpu_batch, B))
     print(json.dumps(out))
 
 
