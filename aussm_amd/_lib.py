@@ -20,6 +20,7 @@ _lib = None
 
 _P = c_void_p
 _I = c_int
+_LL = ctypes.c_longlong
 
 # name -> argtypes; every entry point returns int
 _SIGNATURES = {
@@ -34,6 +35,8 @@ _SIGNATURES = {
     "aussm_complex_bwd": [_P] * 19 + [_I] * 6 + [_P],
     "aussm_real_fwd": [_P] * 8 + [_I] + [_P] * 4 + [_I] * 6 + [_P],
     "aussm_real_bwd": [_P] * 9 + [_I] + [_P] * 9 + [_I] * 6 + [_P],
+    "aussm_causal_conv1d_fwd": [_P] * 4 + [_I] * 4 + [_LL] * 2 + [_P],
+    "aussm_causal_conv1d_bwd": [_P] * 6 + [_I] * 4 + [_LL] * 2 + [_P],
 }
 
 EXPORTED = tuple(_SIGNATURES) + ("aussm_error_string", "aussm_unitary_aux_floats")

@@ -25,7 +25,17 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from . import ops, scan
+from . import conv, ops, scan
+
+
+def _causal_conv(conv1d: nn.Conv1d, x: torch.Tensor, l: int) -> torch.Tensor:
+    """`conv1d(x^T)[:, :, :l]^T` of ai-modules/wavesAI/model/aussm.py:762 / :863 for x (b, l, d).
+    On the GPU the HIP kernel reads x where it lies; tensors on the CPU (the blocks are also used
+    there, with an injected scan) go through nn.Conv1d itself."""
+    k = conv1d.kernel_size[0]
+    if x.is_cuda and conv1d.groups == conv1d.in_channels == conv1d.out_channels and conv1d.padding[0] == k - 1:
+        return conv.causal_conv1d(x, conv1d.weight, conv1d.bias)
+    return conv1d(x.transpose(1, 2))[:, :, :l].transpose(1, 2)
 
 
 @dataclass
@@ -102,7 +112,7 @@ class MambaBlock(nn.Module):
         (b, l, d) = x.shape
         x_and_z = self.in_proj(x)
         (x, z) = x_and_z.split(split_size=[self.args.d_inner, self.args.d_inner], dim=-1)
-        x = self.conv1d(x.transpose(1, 2))[:, :, :l].transpose(1, 2)
+        x = _causal_conv(self.conv1d, x, l)
         y = self.ssm_mamba(x, z)
         return self.out_proj(y)
 
@@ -159,7 +169,7 @@ class SSMauBlock(nn.Module):
         x_and_z = self.in_proj(x)
         (x, z) = x_and_z.split(split_size=[self.args.d_model, self.args.d_model], dim=-1)
         if self.args.conv_1d:
-            x = self.conv1d(x.transpose(1, 2))[:, :, :l].transpose(1, 2)
+            x = _causal_conv(self.conv1d, x, l)
         y = self.ssm_au(x, z)
         return self.out_proj(y)
 

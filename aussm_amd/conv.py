@@ -1,0 +1,74 @@
+"""Depthwise causal convolution along the sequence on channels-last tensors, the step the blocks
+apply to the scan's input (`self.conv1d(x)[:, :, :l]`, ai-modules/wavesAI/model/aussm.py:762 and
+:863), as HIP kernels behind the C ABI (aussm_causal_conv1d_fwd / _bwd).
+
+    y[b, l, d] = bias[d] + sum_k weight[d, 0, k] * x[b, l - (K - 1) + k, d]
+
+The blocks hold x as (b, l, d); the reference transposes to (b, d, l) for nn.Conv1d and back.
+Here the kernels read the (b, l, d) data in place (a column slice of a wider tensor included).
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+from torch import Tensor
+
+from . import _lib
+from ._lib import check, ptr
+
+__all__ = ["causal_conv1d"]
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _rows(x: Tensor):
+    """x usable in place: float32, channel stride 1, rows that do not overlap."""
+    b, l, d = x.shape
+    if x.dtype != torch.float32 or x.stride(2) != 1 or x.stride(1) < d or x.stride(0) < (l - 1) * x.stride(1) + d:
+        x = x.float().contiguous()
+    return x
+
+
+class _CausalConv1dFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, weight, bias):
+        lib = _lib.load()
+        b, l, d = x.shape
+        k = weight.shape[-1]
+        xr = _rows(x)
+        w = weight.reshape(d, k).float().contiguous()
+        bs = None if bias is None else bias.float().contiguous()
+        y = torch.empty((b, l, d), device=x.device, dtype=torch.float32)
+        check(lib.aussm_causal_conv1d_fwd(ptr(xr), ptr(w), ptr(bs), ptr(y), b, l, d, k, xr.stride(0), xr.stride(1),
+                                          _stream()), "aussm_causal_conv1d_fwd")
+        ctx.save_for_backward(xr, w)
+        ctx.has_bias = bias is not None
+        ctx.wshape = weight.shape
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        lib = _lib.load()
+        xr, w = ctx.saved_tensors
+        b, l, d = xr.shape
+        k = w.shape[1]
+        dy = dy.float().contiguous()
+        dx = torch.empty((b, l, d), device=dy.device, dtype=torch.float32)
+        dw = torch.zeros((d, k), device=dy.device, dtype=torch.float32)     # accumulated into by the kernel
+        db = torch.zeros((d,), device=dy.device, dtype=torch.float32) if ctx.has_bias else None
+        check(lib.aussm_causal_conv1d_bwd(ptr(dy), ptr(xr), ptr(w), ptr(dx), ptr(dw), ptr(db), b, l, d, k,
+                                          xr.stride(0), xr.stride(1), _stream()), "aussm_causal_conv1d_bwd")
+        return dx, dw.reshape(ctx.wshape), db
+
+
+def causal_conv1d(x: Tensor, weight: Tensor, bias: Optional[Tensor] = None) -> Tensor:
+    """x (b, l, d) on the GPU; weight (d, 1, k) or (d, k) as nn.Conv1d(d, d, k, groups=d) holds it;
+    bias (d,) or None.  Returns (b, l, d) float32."""
+    if x.dim() != 3 or not x.is_cuda:
+        raise ValueError("causal_conv1d expects a (b, l, d) tensor on the GPU")
+    if weight.shape[0] != x.shape[2] or weight.numel() != x.shape[2] * weight.shape[-1]:
+        raise ValueError(f"weight {tuple(weight.shape)} does not fit {x.shape[2]} channels")
+    return _CausalConv1dFn.apply(x, weight, bias)

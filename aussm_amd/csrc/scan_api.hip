@@ -6,6 +6,7 @@
 #include <stdio.h>
 #include <stdlib.h>
 
+#include "conv1d.h"
 #include "scan_bwd_recompute.h"
 #include "scan_bwd_unitary.h"
 #include "scan_bwd_xdl.h"
@@ -392,6 +393,36 @@ int aussm_real_bwd(const float* dy, const float* dhL, const void* u, const void*
   a.du = du; a.ddelta = ddelta; a.dA = dA; a.dB = dB; a.dC = dC; a.dD = dD; a.dh0 = dh0;
   a.B = B; a.D = D; a.N = N; a.L = L; a.nck = (L + ck - 1) / ck; a.ncg = (D + CH - 1) / CH;
   return launch_rec_bwd<VAR_REAL>(a, in_dtype, (hipStream_t)stream);
+}
+
+int aussm_causal_conv1d_fwd(const float* x, const float* w, const float* bias, float* y,
+                            int B, int L, int D, int K, long long xs_b, long long xs_l, void* stream) {
+  if (B < 1 || L < 1 || D < 1 || K < 1 || K > CONV_MAX_K || xs_l < D || xs_b < (long long)L * xs_l - (xs_l - D))
+    return AUSSM_E_SHAPE;
+  if (!x || !w || !y) return AUSSM_E_NULL;
+  ConvArgs a{};
+  a.x = x; a.w = w; a.bias = bias; a.y = y; a.xs_b = xs_b; a.xs_l = xs_l; a.B = B; a.L = L; a.D = D; a.K = K;
+  const size_t total = (size_t)B * L * D;
+  if ((total + 255) / 256 > 0x7fffffffULL) return AUSSM_E_SHAPE;
+  hipLaunchKernelGGL(causal_conv1d_fwd_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, (hipStream_t)stream, a);
+  return launch_status();
+}
+
+int aussm_causal_conv1d_bwd(const float* dy, const float* x, const float* w, float* dx, float* dw, float* dbias,
+                            int B, int L, int D, int K, long long xs_b, long long xs_l, void* stream) {
+  if (B < 1 || L < 1 || D < 1 || K < 1 || K > CONV_MAX_K || xs_l < D || xs_b < (long long)L * xs_l - (xs_l - D))
+    return AUSSM_E_SHAPE;
+  if (!dy || !x || !w || !dx || !dw) return AUSSM_E_NULL;
+  ConvArgs a{};
+  a.x = x; a.w = w; a.dy = dy; a.dx = dx; a.dw = dw; a.dbias = dbias;
+  a.xs_b = xs_b; a.xs_l = xs_l; a.B = B; a.L = L; a.D = D; a.K = K;
+  const size_t total = (size_t)B * L * D, rows = (size_t)B * L;
+  if ((total + 255) / 256 > 0x7fffffffULL || (rows + CONV_ROWS - 1) / CONV_ROWS > 65535) return AUSSM_E_SHAPE;
+  hipStream_t s = (hipStream_t)stream;
+  hipLaunchKernelGGL(causal_conv1d_bwd_data_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, a);
+  hipLaunchKernelGGL(causal_conv1d_bwd_weight_kernel,
+                     dim3((unsigned)((D + 63) / 64), (unsigned)((rows + CONV_ROWS - 1) / CONV_ROWS)), dim3(256), 0, s, a);
+  return launch_status();
 }
 
 }  // extern "C"

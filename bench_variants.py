@@ -1,0 +1,171 @@
+#!/usr/bin/env python3
+"""The three scan variants at the headline shape (B=32 D=512 N=16 L=2048), forward and backward,
+once with float32 inputs and once with bfloat16 u / delta / B / C (float32 phases, decay, skip,
+states, outputs and gradients): BASELINE configuration 3.
+
+    python bench_variants.py [--reps R] [--shape B,D,N,L] [--model | --only-model]
+
+With --model it also times BASELINE configuration 4: one training step (forward, MSE loss,
+backward) of SSMTS(d_model=256, input_dim=21, output_dim=21, layers="a|m|a|m") on x ~ N(0,1) of
+shape (32, 720, 21), random-init weights, wall clock around synchronised steps.
+
+Prints one JSON line per (variant, input dtype): the duration of the forward and of the backward
+call (HIP events on the launch stream, mean of R launches after a warm-up long enough for the
+clocks to settle) and the algorithmic bytes over that duration against the 8 TB/s HBM peak.
+`bench.py` stays the contract line (unitary, float32); this script is the table beside it.
+
+Algorithmic bytes (E = B*D*L, S = B*N*L, w = bytes of an input element: 4 or 2):
+  unitary  forward  2wE + 8E  + 4wS       backward 2wE + 20E + 4wS + 16S
+  complex  forward  2wE + 12E + 4wS       backward 2wE + 28E + 4wS + 16S
+  real     forward  2wE + 4E  + 2wS       backward 2wE + 12E + 2wS + 8S
+(reads of u, delta in w bytes; theta / rho / dy and all outputs in float32; B, C complex = two
+elements, real = one; gradients of B, C in float32).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+
+def algorithmic_bytes(variant: str, w: int, E: int, S: int):
+    if variant == "unitary":
+        return 2 * w * E + 8 * E + 4 * w * S, 2 * w * E + 20 * E + 4 * w * S + 16 * S
+    if variant == "complex":
+        return 2 * w * E + 12 * E + 4 * w * S, 2 * w * E + 28 * E + 4 * w * S + 16 * S
+    return 2 * w * E + 4 * E + 2 * w * S, 2 * w * E + 12 * E + 2 * w * S + 8 * S
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--reps", type=int, default=30)
+    ap.add_argument("--shape", default="32,512,16,2048")
+    ap.add_argument("--model", action="store_true", help="also time the hybrid SSMTS training step (configuration 4)")
+    ap.add_argument("--only-model", action="store_true", help="time only the SSMTS training step")
+    args = ap.parse_args()
+    B, D, N, L = (int(v) for v in args.shape.split(","))
+
+    import torch
+    from aussm_amd import scan
+
+    if not torch.cuda.is_available():
+        print("bench_variants.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    def timed(fn):
+        for _ in range(40):
+            fn()
+        torch.cuda.synchronize()
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.reps)]
+        for s, e in evs:
+            s.record()
+            fn()
+            e.record()
+        torch.cuda.synchronize()
+        return sum(s.elapsed_time(e) for s, e in evs) / args.reps * 1e3
+
+    def inputs(variant):
+        """BASELINE's value distributions: u ~ N(0,1), delta = softplus(N(0,1)), theta ~ N(0, 0.5),
+        B, C ~ N(0, 1/sqrt(N)) per part, D ~ N(0,1), A = -exp(N(0,1)), rho = -delta exp(N(0,1))[d]."""
+        g = torch.Generator(device=dev).manual_seed(0)
+        rn = lambda *s: torch.randn(*s, generator=g, device=dev)
+        std = N ** -0.5
+        out = {"u": rn(B, D, L), "delta": torch.nn.functional.softplus(rn(B, D, L)), "Dskip": rn(D), "dy": rn(B, D, L)}
+        if variant == "real":
+            out.update(A=-torch.exp(rn(D, N)), Bm=rn(B, N, L) * std, Cm=rn(B, N, L) * std)
+        else:
+            out.update(theta=rn(B, D, L) * 0.5, Bc=torch.complex(rn(B, N, L) * std, rn(B, N, L) * std),
+                       Cc=torch.complex(rn(B, N, L) * std, rn(B, N, L) * std))
+            if variant == "complex":
+                out["rho"] = -out["delta"] * torch.exp(rn(D))[None, :, None]
+        return out
+
+    E, S = B * D * L, B * N * L
+    for variant in (() if args.only_model else ("unitary", "complex", "real")):
+        base = inputs(variant)
+        for name, dt, w in (("f32", torch.float32, 4), ("bf16", torch.bfloat16, 2)):
+            p = dict(base)
+            u, delta = p["u"].to(dt), p["delta"].to(dt)
+            if variant == "real":
+                Bm, Cm = p["Bm"].to(dt).contiguous(), p["Cm"].to(dt).contiguous()
+                ck = scan.REC_CK
+
+                def fwd():
+                    return scan.real_fwd_raw(u, delta, p["A"], Bm, Cm, p["Dskip"], ck=ck)
+
+                hck = fwd()[2]
+
+                def bwd():
+                    return scan.real_bwd_raw(p["dy"], None, u, delta, p["A"], Bm, Cm, p["Dskip"], None, False, None, hck)
+            else:
+                Bri = torch.view_as_real(p["Bc"]).to(dt).contiguous()
+                Cri = torch.view_as_real(p["Cc"]).to(dt).contiguous()
+                if variant == "unitary":
+                    ck = scan.UNITARY_CK
+                    aux = scan.unitary_aux(u, N, ck)
+
+                    def fwd():
+                        return scan.unitary_fwd_raw(u, delta, p["theta"], Bri, Cri, p["Dskip"], ck=ck, aux=aux)
+
+                    hck = fwd()[2]
+
+                    def bwd():
+                        return scan.unitary_bwd_raw(p["dy"], None, u, delta, p["theta"], Bri, Cri, p["Dskip"], hck, ck,
+                                                    aux=aux)
+                else:
+                    ck = scan.REC_CK
+
+                    def fwd():
+                        return scan.complex_fwd_raw(u, delta, p["rho"], p["theta"], Bri, Cri, p["Dskip"], ck=ck)
+
+                    hck = fwd()[2]
+
+                    def bwd():
+                        return scan.complex_bwd_raw(p["dy"], None, u, delta, p["rho"], p["theta"], Bri, Cri, p["Dskip"],
+                                                    None, hck)
+            t_f, t_b = timed(fwd), timed(bwd)
+            b_f, b_b = algorithmic_bytes(variant, w, E, S)
+            print(json.dumps({
+                "variant": variant, "inputs": name, "shape": {"B": B, "D": D, "N": N, "L": L},
+                "fwd_us": round(t_f, 1), "bwd_us": round(t_b, 1),
+                "fwd_GBps": round(b_f / t_f / 1e3, 1), "bwd_GBps": round(b_b / t_b / 1e3, 1),
+                "fwd_bwd_frac_of_hbm_peak": round((b_f + b_b) / (t_f + t_b) / 1e3 / HBM_PEAK_GBS, 4),
+                "samples_per_s": round(E / ((t_f + t_b) * 1e-6), 1),
+                "note": "durations include the output allocation and the zero-fill of the accumulated gradients",
+            }), flush=True)
+
+    if args.model or args.only_model:
+        import time
+        from aussm_amd import blocks
+        torch.manual_seed(0)
+        net = blocks.SSMTS(d_model=256, input_dim=21, output_dim=21, layers="a|m|a|m").to(dev)
+        x = torch.randn(32, 720, 21, device=dev)
+        tgt = torch.randn(32, 720, 21, device=dev)
+
+        def step():
+            net.zero_grad(set_to_none=True)
+            loss = ((net(x) - tgt) ** 2).mean()
+            loss.backward()
+
+        for _ in range(5):
+            step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(20):
+            step()
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / 20
+        print(json.dumps({"model": "SSMTS d_model=256 layers=a|m|a|m, x (32, 720, 21), fp32, forward + MSE + backward",
+                          "ms_per_step": round(dt * 1e3, 2), "sequences_per_s": round(32 / dt, 1)}), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -173,6 +173,23 @@ int aussm_real_bwd(const float* dy, const float* dhL,
                    float* dD, float* dh0,
                    int B, int D, int N, int L, int ck, int in_dtype, void* stream);
 
+/* ---------------------------------------------------------------------------------------
+ * Depthwise causal convolution along the sequence, channels-last (the step both blocks apply to
+ * the scan's input):
+ *     y[b,l,d] = bias[d] + sum_{k<K} w[d,k] * x[b, l-(K-1)+k, d]          (x = 0 before l = 0)
+ * Replaces `self.conv1d(x)[:, :, :l]` of ai-modules/wavesAI/model/aussm.py:762 (MambaBlock) and
+ * :863 (SSMauBlock) - nn.Conv1d(D, D, K, groups=D, padding=K-1), weight (D, 1, K) - without the
+ * two transposes around it: element (b,l,d) of x is x[b*xs_b + l*xs_l + d] (so a column slice of
+ * a wider (b, l, 2D) tensor can be passed as it is), y, dy and dx are contiguous (B, L, D).
+ * K <= 8.  dw (D, K) and dbias (D, may be NULL) are ACCUMULATED into: zero them for a plain gradient.
+ * ------------------------------------------------------------------------------------- */
+int aussm_causal_conv1d_fwd(const float* x, const float* w, const float* bias, float* y,
+                            int B, int L, int D, int K, long long xs_b, long long xs_l, void* stream);
+
+int aussm_causal_conv1d_bwd(const float* dy, const float* x, const float* w,
+                            float* dx, float* dw, float* dbias,
+                            int B, int L, int D, int K, long long xs_b, long long xs_l, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -261,6 +261,17 @@ def reference_unitary_phase_loop(u: Tensor, dt: Tensor, x: Tensor, x_bias: Tenso
 # Seeded input recipes shared by tests, smoke and bench (synthetic data).
 # --------------------------------------------------------------------------
 
+def causal_conv1d_bld(x: Tensor, weight: Tensor, bias: Optional[Tensor]) -> Tensor:
+    """The blocks' depthwise causal convolution on x (b, l, d), exactly as the reference writes it
+    (ai-modules/wavesAI/model/aussm.py:762, :863): nn.Conv1d(d, d, k, groups=d, padding=k-1) on
+    the transposed tensor, output trimmed to l steps.  Pinned by tests/test_oracle.py against the
+    explicit sum  y[b,l,d] = bias[d] + sum_j w[d,j] x[b, l-(k-1)+j, d]  in plain Python loops."""
+    b, l, d = x.shape
+    k = weight.shape[-1]
+    y = F.conv1d(x.transpose(1, 2), weight.reshape(d, 1, k), bias, padding=k - 1, groups=d)
+    return y[:, :, :l].transpose(1, 2)
+
+
 def make_core_inputs(B: int, D: int, N: int, L: int, seed: int = 0, variant: str = "unitary",
                      dtype: torch.dtype = torch.float32, gate: bool = False):
     """Value distributions of the benchmark configurations:

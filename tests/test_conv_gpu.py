@@ -1,0 +1,53 @@
+"""The depthwise causal convolution of the blocks (HIP, channels-last, through the C ABI) against
+the CPU restatement of the reference's nn.Conv1d call: outputs and all three gradients, on a
+contiguous tensor and on a column slice of a wider one (what the blocks pass), float32 tolerance
+atol = rtol = 1e-5 (a handful of fused multiply-adds per output)."""
+import pytest
+import torch
+
+from oracle import scan_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("b,l,d,k,sliced", [(2, 37, 70, 4, False), (3, 16, 64, 4, True), (1, 5, 3, 2, True),
+                                            (2, 9, 130, 8, False), (4, 720, 256, 4, True)])
+def test_causal_conv_matches_reference_conv(b, l, d, k, sliced):
+    from aussm_amd import conv
+    g = torch.Generator().manual_seed(b + l + d)
+    wide = torch.randn(b, l, 2 * d, generator=g)
+    w = torch.randn(d, 1, k, generator=g)
+    bias = torch.randn(d, generator=g)
+    dy = torch.randn(b, l, d, generator=g)
+
+    def run(dev):
+        src = wide.clone().to(dev).requires_grad_(True)
+        x = src[:, :, :d] if sliced else src[:, :, d:].contiguous()
+        wd, bd = w.clone().to(dev).requires_grad_(True), bias.clone().to(dev).requires_grad_(True)
+        y = O.causal_conv1d_bld(x, wd, bd) if dev == "cpu" else conv.causal_conv1d(x, wd, bd)
+        (y * dy.to(dev)).sum().backward()
+        return y.detach(), src.grad, wd.grad, bd.grad
+
+    want = run("cpu")
+    print(f"case conv b={b} l={l} d={d} k={k} sliced={sliced}", flush=True)
+    got = run("cuda")
+    torch.cuda.synchronize()
+    for name, a, e in zip(("y", "dx", "dw", "dbias"), got, want):
+        scale = max(1.0, float(e.abs().max()))
+        torch.testing.assert_close(a.cpu() / scale, e / scale, atol=1e-5, rtol=1e-5, msg=lambda m: f"{name}: {m}")
+
+
+def test_causal_conv_without_bias_and_rejections():
+    from aussm_amd import conv
+    x = torch.randn(2, 8, 6, device="cuda", requires_grad=True)
+    w = torch.randn(6, 1, 4, device="cuda", requires_grad=True)
+    y = conv.causal_conv1d(x, w, None)
+    y.sum().backward()
+    want = O.causal_conv1d_bld(x.detach().cpu(), w.detach().cpu(), None)
+    torch.testing.assert_close(y.detach().cpu(), want, atol=1e-5, rtol=1e-5)
+    with pytest.raises(ValueError):
+        conv.causal_conv1d(x.cpu(), w, None)
+    with pytest.raises(ValueError):
+        conv.causal_conv1d(x, w[:5], None)
+    with pytest.raises(Exception):
+        conv.causal_conv1d(x, torch.randn(6, 1, 9, device="cuda"), None)     # K > 8 is rejected by the library

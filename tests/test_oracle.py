@@ -253,3 +253,24 @@ def test_reference_phase_loop_bruteforce():
                     acc += (cmath.exp(1j * float(Cph[ib, j, t])) * h[j]).real
                 val = (acc + float(u[ib, i, t]) * float(D[i])) * _silu(float(z[ib, i, t]))
                 assert abs(val - float(y[ib, i, t])) < 1e-11
+
+
+def test_causal_conv_bruteforce():
+    """The blocks' convolution against the explicit causal sum in Python loops (a wrong shift,
+    a flipped kernel or a missing trim fails it)."""
+    g = torch.Generator().manual_seed(4)
+    b, l, d, k = 2, 7, 3, 4
+    x = torch.randn(b, l, d, generator=g, dtype=torch.float64)
+    w = torch.randn(d, 1, k, generator=g, dtype=torch.float64)
+    bias = torch.randn(d, generator=g, dtype=torch.float64)
+    got = O.causal_conv1d_bld(x, w, bias)
+    assert got.shape == (b, l, d)
+    for bi in range(b):
+        for li in range(l):
+            for di in range(d):
+                want = float(bias[di])
+                for j in range(k):
+                    ls = li - (k - 1) + j
+                    if ls >= 0:
+                        want += float(w[di, 0, j]) * float(x[bi, ls, di])
+                assert abs(float(got[bi, li, di]) - want) < 1e-12
