@@ -26,37 +26,34 @@ struct ConvArgs {
   int B, L, D, K;
 };
 
+// grid: x = (b, l) row, y = block of 256 channels
 __global__ __launch_bounds__(256) void causal_conv1d_fwd_kernel(const ConvArgs p) {
-  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
-  const size_t total = (size_t)p.B * p.L * p.D;
-  if (idx >= total) return;
-  const int d = (int)(idx % p.D);
-  const int l = (int)((idx / p.D) % p.L);
-  const int b = (int)(idx / ((size_t)p.D * p.L));
+  const int d = blockIdx.y * 256 + threadIdx.x;
+  if (d >= p.D) return;
+  const unsigned r = blockIdx.x;
+  const int b = (int)(r / (unsigned)p.L), l = (int)(r % (unsigned)p.L);
   const float* __restrict__ xr = p.x + (size_t)b * p.xs_b + d;
   float acc = p.bias ? p.bias[d] : 0.0f;
   for (int k = 0; k < p.K; ++k) {
     const int ls = l - (p.K - 1) + k;
     if (ls >= 0) acc = fmaf(p.w[(size_t)d * p.K + k], xr[(size_t)ls * p.xs_l], acc);
   }
-  p.y[idx] = acc;
+  p.y[(size_t)r * p.D + d] = acc;
 }
 
 // dx[b,l,d] = sum_k w[d,k] dy[b, l + (K-1) - k, d]   (terms past the end of the sequence drop out)
 __global__ __launch_bounds__(256) void causal_conv1d_bwd_data_kernel(const ConvArgs p) {
-  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
-  const size_t total = (size_t)p.B * p.L * p.D;
-  if (idx >= total) return;
-  const int d = (int)(idx % p.D);
-  const int l = (int)((idx / p.D) % p.L);
-  const int b = (int)(idx / ((size_t)p.D * p.L));
-  const float* __restrict__ gr = p.dy + (size_t)b * p.L * p.D + d;
+  const int d = blockIdx.y * 256 + threadIdx.x;
+  if (d >= p.D) return;
+  const unsigned r = blockIdx.x;
+  const int l = (int)(r % (unsigned)p.L);
+  const float* __restrict__ gr = p.dy + (size_t)r * p.D + d;      // row (b, l); later rows of b follow
   float acc = 0.0f;
   for (int k = 0; k < p.K; ++k) {
     const int lt = l + (p.K - 1) - k;
-    if (lt < p.L) acc = fmaf(p.w[(size_t)d * p.K + k], gr[(size_t)lt * p.D], acc);
+    if (lt < p.L) acc = fmaf(p.w[(size_t)d * p.K + k], gr[(size_t)(lt - l) * p.D], acc);
   }
-  p.dx[idx] = acc;
+  p.dx[(size_t)r * p.D + d] = acc;
 }
 
 // dw[d,k] += sum_{b,l} dy[b,l,d] x[b, l - (K-1) + k, d],  dbias[d] += sum_{b,l} dy[b,l,d].
@@ -72,10 +69,11 @@ __global__ __launch_bounds__(256) void causal_conv1d_bwd_weight_kernel(const Con
 #pragma unroll
   for (int k = 0; k <= CONV_MAX_K; ++k) acc[k] = 0.0f;
   if (dok) {
-    for (int i = rg; i < CONV_ROWS; i += 4) {
+    int b = (int)((unsigned)(r0 + rg) / (unsigned)p.L), l = (int)((unsigned)(r0 + rg) % (unsigned)p.L);
+    for (int i = rg; i < CONV_ROWS; i += 4, l += 4) {
       const size_t r = r0 + i;
       if (r >= rows) break;
-      const int b = (int)(r / p.L), l = (int)(r % p.L);
+      while (l >= p.L) { l -= p.L; ++b; }
       const float g = p.dy[r * p.D + d];
       const float* __restrict__ xr = p.x + (size_t)b * p.xs_b + d;
 #pragma unroll
