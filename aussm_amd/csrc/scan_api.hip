@@ -136,8 +136,9 @@ inline size_t seg_floats(int B, int D, int N, int L, int ns) {
 }
 
 inline int mfma_fwd_mode(const FwdArgs& a, int in_dtype) {
-  const int mode = env_mode("AUSSM_MFMA", 3, a.N);
-  if (mode <= 0 || in_dtype != AUSSM_F32 || a.N > MN || a.L % 4 != 0 || a.ck % MT != 0) return 0;
+  int mode = env_mode("AUSSM_MFMA", 3, a.N);
+  if (mode <= 0 || a.N > MN || a.L % 4 != 0 || a.ck % MT != 0) return 0;
+  if (in_dtype != AUSSM_F32) mode = 3;       // bf16 inputs: the default matrix-core kernel only
   if (misaligned(a.u, 16) || misaligned(a.delta, 16) || misaligned(a.theta, 16) || misaligned(a.z, 16) ||
       misaligned(a.y, 16) || misaligned(a.Bm, 16) || misaligned(a.Cm, 16))
     return 0;
@@ -150,7 +151,7 @@ int launch_fwd(FwdArgs a, int in_dtype, hipStream_t s) {
   if (a.aux && mode <= 1)   // this call will not fill the auxiliary buffer
     hipLaunchKernelGGL(aux_invalidate_kernel, dim3(1), dim3(1), 0, s, a.aux + (size_t)a.B * a.D * a.L);
   if (mode) {
-    if ((mode == 2 || mode == 3) && a.aux && a.hck) {
+    if ((mode == 2 || mode == 3) && a.aux && a.hck && in_dtype == AUSSM_F32) {
       const int ns = seg_count(a.B, a.D, a.N, a.L, a.ck);
       if (ns > 1) {
         // 1. end state of every segment from a zero start and its rotation; 2. chain them;
@@ -177,6 +178,9 @@ int launch_fwd(FwdArgs a, int in_dtype, hipStream_t s) {
     } else if (mode == 4) {
       if (a.z) hipLaunchKernelGGL((unitary_fwd_xdl2_kernel<3, true>), grid, dim3(512), 0, s, a);
       else hipLaunchKernelGGL((unitary_fwd_xdl2_kernel<3, false>), grid, dim3(512), 0, s, a);
+    } else if (in_dtype == AUSSM_BF16) {
+      if (a.z) hipLaunchKernelGGL((unitary_fwd_xdl_kernel<3, true, bf16_t>), grid, dim3(256), 0, s, a);
+      else hipLaunchKernelGGL((unitary_fwd_xdl_kernel<3, false, bf16_t>), grid, dim3(256), 0, s, a);
     } else {
       if (a.z) hipLaunchKernelGGL((unitary_fwd_xdl_kernel<3, true>), grid, dim3(256), 0, s, a);
       else hipLaunchKernelGGL((unitary_fwd_xdl_kernel<3, false>), grid, dim3(256), 0, s, a);

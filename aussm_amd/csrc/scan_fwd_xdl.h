@@ -127,9 +127,65 @@ struct XdlG {
   u4 im[NP][XT * 4];
 };
 
+// Inputs as they lie in memory, kept raw in registers from the (early) load to the use: float
+// tensors as they are, bf16 tensors as packed words that are widened where they are consumed
+// (a bf16 value is the upper half of the float of the same value).
+__device__ __forceinline__ float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+// four consecutive real inputs of a channel
+template <typename Tin> struct Raw4;
+template <> struct Raw4<float> {
+  f4 v;
+  __device__ __forceinline__ void load(const float* p) { v = *reinterpret_cast<const f4*>(p); }
+  __device__ __forceinline__ float get(int i) const { return v[i]; }
+  __device__ __forceinline__ void touch() const { touch_vgpr(v[0]); touch_vgpr(v[1]); touch_vgpr(v[2]); touch_vgpr(v[3]); }
+};
+template <> struct Raw4<bf16_t> {
+  u2 v;
+  __device__ __forceinline__ void load(const bf16_t* p) { v = *reinterpret_cast<const u2*>(p); }
+  __device__ __forceinline__ float get(int i) const { return (i & 1) ? bf16_hi(v[i >> 1]) : bf16_lo(v[i >> 1]); }
+  __device__ __forceinline__ void touch() const { touch_vgpr(__uint_as_float(v[0])); touch_vgpr(__uint_as_float(v[1])); }
+};
+// one complex input (re, im)
+template <typename Tin> struct RawC;
+template <> struct RawC<float> {
+  float2 v;
+  __device__ __forceinline__ void load(const float* p) { v = *reinterpret_cast<const float2*>(p); }
+  __device__ __forceinline__ float re() const { return v.x; }
+  __device__ __forceinline__ float im() const { return v.y; }
+  __device__ __forceinline__ void pin() { asm volatile("" : "+v"(v.x), "+v"(v.y)); }
+};
+template <> struct RawC<bf16_t> {
+  uint32_t v;
+  __device__ __forceinline__ void load(const bf16_t* p) { v = *reinterpret_cast<const uint32_t*>(p); }
+  __device__ __forceinline__ float re() const { return bf16_lo(v); }
+  __device__ __forceinline__ float im() const { return bf16_hi(v); }
+  __device__ __forceinline__ void pin() { asm volatile("" : "+v"(v)); }
+};
+// four consecutive complex inputs of a state row
+template <typename Tin> struct RawC4;
+template <> struct RawC4<float> {
+  f4 a, b;
+  __device__ __forceinline__ void load(const float* p) {
+    a = *reinterpret_cast<const f4*>(p);
+    b = *reinterpret_cast<const f4*>(p + 4);
+  }
+  __device__ __forceinline__ float re(int j) const { return j < 2 ? a[2 * j] : b[2 * j - 4]; }
+  __device__ __forceinline__ float im(int j) const { return j < 2 ? a[2 * j + 1] : b[2 * j - 3]; }
+  __device__ __forceinline__ void pin() { asm volatile("" : "+v"(a), "+v"(b)); }
+};
+template <> struct RawC4<bf16_t> {
+  u4 a;
+  __device__ __forceinline__ void load(const bf16_t* p) { a = *reinterpret_cast<const u4*>(p); }
+  __device__ __forceinline__ float re(int j) const { return bf16_lo(a[j]); }
+  __device__ __forceinline__ float im(int j) const { return bf16_hi(a[j]); }
+  __device__ __forceinline__ void pin() { asm volatile("" : "+v"(a)); }
+};
+
 // Requires: N <= 16, L % 4 == 0, u/delta/theta/z/y 16-byte aligned, B/C 16-byte aligned,
-// ck % 32 == 0, float inputs.  The launcher checks these and otherwise takes the generic kernel.
-template <int NP, bool GATED>
+// ck % 32 == 0.  Tin: float or bf16_t (u, delta, B, C).  The launcher checks these and otherwise
+// takes the generic kernel.
+template <int NP, bool GATED, typename Tin = float>
 __global__ __launch_bounds__(256) void unitary_fwd_xdl_kernel(const FwdArgs p) {
   __shared__ XdlBC<NP> s_bc[3];
   __shared__ XdlG<NP> s_g[2];
@@ -147,12 +203,12 @@ __global__ __launch_bounds__(256) void unitary_fwd_xdl_kernel(const FwdArgs p) {
   const int bb = b / p.ns;
   const size_t so = (size_t)(b - bb * p.ns) * L;
   const size_t row = ((size_t)bb * D + dc) * p.ld + so;
-  const float* __restrict__ gu = static_cast<const float*>(p.u) + row;
-  const float* __restrict__ gdl = static_cast<const float*>(p.delta) + row;
+  const Tin* __restrict__ gu = static_cast<const Tin*>(p.u) + row;
+  const Tin* __restrict__ gdl = static_cast<const Tin*>(p.delta) + row;
   const float* __restrict__ gth = p.theta + row;
   const float* __restrict__ gz = GATED ? p.z + row : nullptr;
-  const float* __restrict__ gB = static_cast<const float*>(p.Bm);
-  const float* __restrict__ gC = static_cast<const float*>(p.Cm);
+  const Tin* __restrict__ gB = static_cast<const Tin*>(p.Bm);
+  const Tin* __restrict__ gC = static_cast<const Tin*>(p.Cm);
   const float dsk = (p.Dskip && dok) ? p.Dskip[dc] : 0.0f;
   const int nchunks = (L + XT - 1) / XT;
   const SplitK sk = make_splitk();
@@ -164,14 +220,14 @@ __global__ __launch_bounds__(256) void unitary_fwd_xdl_kernel(const FwdArgs p) {
   // B (tid >= 128) builds the record [row t][g1] from the four state rows 4 g1 .. 4 g1 + 3.
   const int m1_t = tid & 31, m1_g = (tid >> 5) & 3;
   const bool m1_isB = tid >= 128;
-  const float* __restrict__ m1_src = m1_isB ? gB : gC;
-  float2 m1_raw[4];
+  const Tin* __restrict__ m1_src = m1_isB ? gB : gC;
+  RawC<Tin> m1_raw[4];
   // second mapping: thread (n = tid % 16, g2 = (tid / 16) % 4, half = (tid / 64) % 2) reads the four
   // timesteps 16 half + 4 g2 .. + 3 of row n of B; tid < 128 writes the Br half-record, the
   // others the Bi and -Bi half-records.
   const int m2_n = tid & 15, m2_g = (tid >> 4) & 3, m2_half = (tid >> 6) & 1;
   const bool m2_im = tid >= 128;
-  f4 m2_raw[2];
+  RawC4<Tin> m2_raw;
   auto bc_load = [&](int c) {
     const int l = c * XT + m1_t;
     const int lc = l < L ? l : 0;
@@ -179,13 +235,12 @@ __global__ __launch_bounds__(256) void unitary_fwd_xdl_kernel(const FwdArgs p) {
     for (int k = 0; k < 4; ++k) {
       const int n = 4 * m1_g + k;
       const size_t o = (((size_t)bb * N + (n < N ? n : 0)) * p.ld + so + lc) * 2;
-      m1_raw[k] = *reinterpret_cast<const float2*>(m1_src + o);
+      m1_raw[k].load(m1_src + o);
     }
     const int l2 = c * XT + 16 * m2_half + 4 * m2_g;
     const int l2c = l2 < L ? l2 : 0;
     const size_t o2 = (((size_t)bb * N + (m2_n < N ? m2_n : 0)) * p.ld + so + l2c) * 2;
-    m2_raw[0] = *reinterpret_cast<const f4*>(gB + o2);
-    m2_raw[1] = *reinterpret_cast<const f4*>(gB + o2 + 4);
+    m2_raw.load(gB + o2);
   };
   // Branch-free: C threads write [re, -im] -> cs_r and [im, re] -> cs_i, B threads [re, im] -> bs and
   // [-im, re] -> bs_c; real-part threads of the second mapping write bt_r, the others bt_i.
@@ -197,8 +252,8 @@ __global__ __launch_bounds__(256) void unitary_fwd_xdl_kernel(const FwdArgs p) {
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
         const bool ok = tok && (4 * m1_g + k < N);
-        x[k] = ok ? m1_raw[k].x : 0.0f;
-        x[4 + k] = ok ? m1_raw[k].y : 0.0f;
+        x[k] = ok ? m1_raw[k].re() : 0.0f;
+        x[4 + k] = ok ? m1_raw[k].im() : 0.0f;
       }
       u4 pc[NP];
       split8<NP>(sk, x, pc);
@@ -213,9 +268,8 @@ __global__ __launch_bounds__(256) void unitary_fwd_xdl_kernel(const FwdArgs p) {
     }
     {
       const bool ok = (m2_n < N) && (c * XT + 16 * m2_half + 4 * m2_g < L);
-      const int sel = m2_im ? 1 : 0;
-      const float v0 = ok ? m2_raw[0][sel] : 0.0f, v1 = ok ? m2_raw[0][2 + sel] : 0.0f;
-      const float v2 = ok ? m2_raw[1][sel] : 0.0f, v3 = ok ? m2_raw[1][2 + sel] : 0.0f;
+      const float v0 = ok ? (m2_im ? m2_raw.im(0) : m2_raw.re(0)) : 0.0f, v1 = ok ? (m2_im ? m2_raw.im(1) : m2_raw.re(1)) : 0.0f;
+      const float v2 = ok ? (m2_im ? m2_raw.im(2) : m2_raw.re(2)) : 0.0f, v3 = ok ? (m2_im ? m2_raw.im(3) : m2_raw.re(3)) : 0.0f;
       uint32_t a[NP], c2[NP];
       split2<NP>(sk, v0, v1, a);
       split2<NP>(sk, v2, v3, c2);
@@ -262,14 +316,14 @@ __global__ __launch_bounds__(256) void unitary_fwd_xdl_kernel(const FwdArgs p) {
 
   // ---- channel data of one chunk: two runs of four timesteps per lane.  Loads are unconditional
   // from a clamped address; out-of-range runs are zeroed where they are used.
-  struct In { f4 u[2], de[2], th[2], z[2]; };
+  struct In { Raw4<Tin> u[2], de[2]; f4 th[2], z[2]; };
   auto in_load = [&](In& r, int c) {
 #pragma unroll
     for (int st = 0; st < 2; ++st) {
       const int l = c * XT + 16 * st + 4 * g;
       const int lc = l < L ? l : 0;
-      r.u[st] = *reinterpret_cast<const f4*>(gu + lc);
-      r.de[st] = *reinterpret_cast<const f4*>(gdl + lc);
+      r.u[st].load(gu + lc);
+      r.de[st].load(gdl + lc);
       r.th[st] = *reinterpret_cast<const f4*>(gth + lc);
       if (GATED) r.z[st] = *reinterpret_cast<const f4*>(gz + lc);
     }
@@ -277,7 +331,7 @@ __global__ __launch_bounds__(256) void unitary_fwd_xdl_kernel(const FwdArgs p) {
   auto in_touch = [&](const In& r) {
 #pragma unroll
     for (int st = 0; st < 2; ++st) {
-      touch4(r.u[st]); touch4(r.de[st]); touch4(r.th[st]);
+      r.u[st].touch(); r.de[st].touch(); touch4(r.th[st]);
       if (GATED) touch4(r.z[st]);
     }
   };
@@ -315,9 +369,8 @@ __global__ __launch_bounds__(256) void unitary_fwd_xdl_kernel(const FwdArgs p) {
     for (int st = 0; st < 2; ++st) {
       const bool ok = c * XT + 16 * st + 4 * g < L;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) w[st][i] = ok ? r.de[st][i] * r.u[st][i] : 0.0f;
+      for (int i = 0; i < 4; ++i) { o.u[st][i] = r.u[st].get(i); w[st][i] = ok ? r.de[st].get(i) * o.u[st][i] : 0.0f; }
       th[st][1] += th[st][0]; th[st][2] += th[st][1]; th[st][3] += th[st][2];
-      o.u[st] = r.u[st];
       if (GATED) o.z[st] = r.z[st];
     }
     // exclusive offsets over the order (st 0: g 0..3), (st 1: g 0..3)
@@ -426,9 +479,8 @@ __global__ __launch_bounds__(256) void unitary_fwd_xdl_kernel(const FwdArgs p) {
 
     // ---- region 1: G^T tile of chunk c + 1  |  staging of B/C of chunk c + 2
 #pragma unroll
-    for (int k = 0; k < 4; ++k) { pin(m1_raw[k].x); pin(m1_raw[k].y); }
-#pragma unroll
-    for (int k = 0; k < 2; ++k) asm volatile("" : "+v"(m2_raw[k]));
+    for (int k = 0; k < 4; ++k) m1_raw[k].pin();
+    m2_raw.pin();
     f4 ggr = xmm<NP>(ga, gbr, f4{0, 0, 0, 0});
     f4 ggi = xmm<NP>(ga, gbi, f4{0, 0, 0, 0});
     bc_store(c + 2, s_bc[i2]);
@@ -471,9 +523,8 @@ __global__ __launch_bounds__(256) void unitary_fwd_xdl_kernel(const FwdArgs p) {
       for (int st = 0; st < 2; ++st) {
         const bool ok = (c + 1) * XT + 16 * st + 4 * g < L;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) w[4 * st + i] = ok ? in1.de[st][i] * in1.u[st][i] : 0.0f;
+        for (int i = 0; i < 4; ++i) { pn.u[st][i] = in1.u[st].get(i); w[4 * st + i] = ok ? in1.de[st].get(i) * pn.u[st][i] : 0.0f; }
         th[st][1] += th[st][0]; th[st][2] += th[st][1]; th[st][3] += th[st][2];
-        pn.u[st] = in1.u[st];
         if (GATED) pn.z[st] = in1.z[st];
       }
       // exclusive offsets over the order (st 0: g 0..3), (st 1: g 0..3)
