@@ -333,11 +333,11 @@ int aussm_unitary_bwd_aux(const float* dy, const float* dhL, const void* u, cons
   a.B = B; a.D = D; a.N = N; a.L = L; a.ck = ck; a.nck = (L + ck - 1) / ck; a.ncg = (D + CH - 1) / CH;
   a.ld = L; a.ns = 1; a.hs = 1; a.ho = 0;
   const int mode = env_mode("AUSSM_MFMA_BWD", 3, N);   // matrix-core kernel for the common case
-  if (mode > 0 && in_dtype == AUSSM_F32 && N <= XN && L % 4 == 0 && ck % XT == 0 &&
+  if (mode > 0 && N <= XN && L % 4 == 0 && ck % XT == 0 &&
       !(misaligned(dy, 16) || misaligned(u, 16) || misaligned(delta, 16) || misaligned(theta, 16) ||
         misaligned(du, 16) || misaligned(ddelta, 16) || misaligned(dtheta, 16) || misaligned(Bc, 16) ||
         misaligned(Cc, 16))) {
-    const int ns = aux ? seg_count(B, D, N, L, ck) : 1;
+    const int ns = (aux && in_dtype == AUSSM_F32) ? seg_count(B, D, N, L, ck) : 1;
     if (ns > 1) {
       // adjoint at the start of every segment from a zero adjoint at its end, chained last to first
       const int Ls = L / ns, r = seg_fine(L, ns), nf = ns * r;
@@ -352,7 +352,8 @@ int aussm_unitary_bwd_aux(const float* dy, const float* dhL, const void* u, cons
       a.B = B * ns; a.L = Ls; a.ns = ns; a.nck = Ls / ck; a.dhL = seg; a.dh0 = nullptr; a.hs = r; a.ho = r - 1;
     }
     const dim3 grid((unsigned)(a.B * a.ncg));
-    if (mode == 2) hipLaunchKernelGGL((unitary_bwd_xdl_kernel<2, 2>), grid, dim3(256), 0, s, a);
+    if (in_dtype == AUSSM_BF16) hipLaunchKernelGGL((unitary_bwd_xdl_kernel<3, 2, bf16_t>), grid, dim3(256), 0, s, a);
+    else if (mode == 2) hipLaunchKernelGGL((unitary_bwd_xdl_kernel<2, 2>), grid, dim3(256), 0, s, a);
     else if (mode == 5) hipLaunchKernelGGL((unitary_bwd_xdl_kernel<3, 3>), grid, dim3(256), 0, s, a);
     else hipLaunchKernelGGL((unitary_bwd_xdl_kernel<3, 2>), grid, dim3(256), 0, s, a);
     return launch_status();

@@ -91,17 +91,62 @@ __device__ __forceinline__ void ldrec16(const u4 (*plane)[XN * 4], int idx, u4 (
 // accumulation registers; the compiler does not know the data is still in flight, so every value
 // loaded this way passes through landed() (a wait for all vector-memory operations that also pins
 // the values) before its first use.
-__device__ __forceinline__ void ldg_acc(f4& dst, const float* p) {
+__device__ __forceinline__ void ldg_acc(f4& dst, const void* p) {
   asm volatile("global_load_dwordx4 %0, %1, off" : "=a"(dst) : "v"(p) : "memory");
 }
-__device__ __forceinline__ void ldg_acc(float2& dst, const float* p) {
+__device__ __forceinline__ void ldg_acc(float2& dst, const void* p) {
   asm volatile("global_load_dwordx2 %0, %1, off" : "=a"(dst) : "v"(p) : "memory");
 }
+__device__ __forceinline__ void ldg_acc(float& dst, const void* p) {
+  asm volatile("global_load_dword %0, %1, off" : "=a"(dst) : "v"(p) : "memory");
+}
+// The raw inputs of scan_fwd_xdl.h (Raw4, RawC, RawC4) loaded this way: float tensors as they are,
+// bf16 tensors as packed words held in float-typed registers and widened where they are used.
+template <typename Tin> struct AccRaw4;
+template <> struct AccRaw4<float> {
+  f4 v;
+  __device__ __forceinline__ void load(const float* p) { ldg_acc(v, p); }
+  __device__ __forceinline__ float get(int i) const { return v[i]; }
+};
+template <> struct AccRaw4<bf16_t> {
+  float2 v;
+  __device__ __forceinline__ void load(const bf16_t* p) { ldg_acc(v, p); }
+  __device__ __forceinline__ float get(int i) const {
+    const uint32_t w = __float_as_uint(i < 2 ? v.x : v.y);
+    return (i & 1) ? bf16_hi(w) : bf16_lo(w);
+  }
+};
+template <typename Tin> struct AccRawC;
+template <> struct AccRawC<float> {
+  float2 v;
+  __device__ __forceinline__ void load(const float* p) { ldg_acc(v, p); }
+  __device__ __forceinline__ float re() const { return v.x; }
+  __device__ __forceinline__ float im() const { return v.y; }
+};
+template <> struct AccRawC<bf16_t> {
+  float v;
+  __device__ __forceinline__ void load(const bf16_t* p) { ldg_acc(v, p); }
+  __device__ __forceinline__ float re() const { return bf16_lo(__float_as_uint(v)); }
+  __device__ __forceinline__ float im() const { return bf16_hi(__float_as_uint(v)); }
+};
+template <typename Tin> struct AccRawC4;
+template <> struct AccRawC4<float> {
+  f4 a, b;
+  __device__ __forceinline__ void load(const float* p) { ldg_acc(a, p); ldg_acc(b, p + 4); }
+  __device__ __forceinline__ float re(int j) const { return j < 2 ? a[2 * j] : b[2 * j - 4]; }
+  __device__ __forceinline__ float im(int j) const { return j < 2 ? a[2 * j + 1] : b[2 * j - 3]; }
+};
+template <> struct AccRawC4<bf16_t> {
+  f4 a;
+  __device__ __forceinline__ void load(const bf16_t* p) { ldg_acc(a, p); }
+  __device__ __forceinline__ float re(int j) const { return bf16_lo(__float_as_uint(a[j])); }
+  __device__ __forceinline__ float im(int j) const { return bf16_hi(__float_as_uint(a[j])); }
+};
 
-// Requires: N <= 16, L % 4 == 0, 16-byte aligned tensors, ck % 32 == 0, float inputs.
+// Requires: N <= 16, L % 4 == 0, 16-byte aligned tensors, ck % 32 == 0.  Tin: float or bf16_t (u, delta, B, C).
 // NP: operand pieces of the products along the sequence (3 = fp32-accurate); NPC: pieces of the
 // products that sum over the channel (M, X1, X2 and the two closing products of dB / dC).
-template <int NP, int NPC>
+template <int NP, int NPC, typename Tin = float>
 __global__ __launch_bounds__(256) void unitary_bwd_xdl_kernel(const UniBwdArgs p) {
   __shared__ XbBC<NP> s_bc;
   __shared__ XbG<NP> s_g;
@@ -122,12 +167,12 @@ __global__ __launch_bounds__(256) void unitary_bwd_xdl_kernel(const UniBwdArgs p
   const int bb = b / p.ns;
   const size_t so = (size_t)(b - bb * p.ns) * L;
   const size_t row = ((size_t)bb * D + dc) * p.ld + so;
-  const float* __restrict__ gu = static_cast<const float*>(p.u) + row;
-  const float* __restrict__ gdl = static_cast<const float*>(p.delta) + row;
+  const Tin* __restrict__ gu = static_cast<const Tin*>(p.u) + row;
+  const Tin* __restrict__ gdl = static_cast<const Tin*>(p.delta) + row;
   const float* __restrict__ gth = p.theta + row;
   const float* __restrict__ gdy = p.dy + row;
-  const float* __restrict__ gB = static_cast<const float*>(p.Bm);
-  const float* __restrict__ gC = static_cast<const float*>(p.Cm);
+  const Tin* __restrict__ gB = static_cast<const Tin*>(p.Bm);
+  const Tin* __restrict__ gC = static_cast<const Tin*>(p.Cm);
   const float dsk = (p.Dskip && dok) ? p.Dskip[dc] : 0.0f;
   const int nchunks = (L + XT - 1) / XT;
   const SplitK sk = make_splitk();
@@ -148,12 +193,12 @@ __global__ __launch_bounds__(256) void unitary_bwd_xdl_kernel(const UniBwdArgs p
   // half-records [row n][g2] from the four timesteps 16 half + 4 g2 .. + 3.
   const int m1_t = tid & 31, m1_g = (tid >> 5) & 3;
   const bool m1_isB = tid >= 128;
-  const float* __restrict__ m1_src = m1_isB ? gB : gC;
+  const Tin* __restrict__ m1_src = m1_isB ? gB : gC;
   const int m2_n = tid & 15, m2_g = (tid >> 4) & 3, m2_half = (tid >> 6) & 1;
   const bool m2_isC = tid >= 128;
-  const float* __restrict__ m2_src = m2_isC ? gC : gB;
-  float2 m1_raw[4];
-  f4 m2_raw[2];
+  const Tin* __restrict__ m2_src = m2_isC ? gC : gB;
+  AccRawC<Tin> m1_raw[4];
+  AccRawC4<Tin> m2_raw;
   auto bc_load = [&](int c) {
     const int cc = c < 0 ? 0 : c;
     const int l = cc * XT + m1_t;
@@ -162,13 +207,12 @@ __global__ __launch_bounds__(256) void unitary_bwd_xdl_kernel(const UniBwdArgs p
     for (int k = 0; k < 4; ++k) {
       const int n = 4 * m1_g + k;
       const size_t o = (((size_t)bb * N + (n < N ? n : 0)) * p.ld + so + lc) * 2;
-      ldg_acc(m1_raw[k], m1_src + o);
+      m1_raw[k].load(m1_src + o);
     }
     const int l2 = cc * XT + 16 * m2_half + 4 * m2_g;
     const int l2c = l2 < L ? l2 : 0;
     const size_t o2 = (((size_t)bb * N + (m2_n < N ? m2_n : 0)) * p.ld + so + l2c) * 2;
-    ldg_acc(m2_raw[0], m2_src + o2);
-    ldg_acc(m2_raw[1], m2_src + o2 + 4);
+    m2_raw.load(m2_src + o2);
   };
   auto bc_store = [&](int c) {
     {
@@ -177,8 +221,8 @@ __global__ __launch_bounds__(256) void unitary_bwd_xdl_kernel(const UniBwdArgs p
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
         const bool ok = tok && (4 * m1_g + k < N);
-        x[k] = ok ? m1_raw[k].x : 0.0f;
-        x[4 + k] = ok ? m1_raw[k].y : 0.0f;
+        x[k] = ok ? m1_raw[k].re() : 0.0f;
+        x[4 + k] = ok ? m1_raw[k].im() : 0.0f;
       }
       u4 pc[NP], pi[NP], pcs[NP];
       split8<NP>(sk, x, pc);                 // [re, im]
@@ -198,10 +242,10 @@ __global__ __launch_bounds__(256) void unitary_bwd_xdl_kernel(const UniBwdArgs p
     }
     {
       const bool ok = (m2_n < N) && (c * XT + 16 * m2_half + 4 * m2_g < L);
-      const float r0 = ok ? m2_raw[0][0] : 0.0f, r1 = ok ? m2_raw[0][2] : 0.0f;
-      const float r2 = ok ? m2_raw[1][0] : 0.0f, r3 = ok ? m2_raw[1][2] : 0.0f;
-      const float j0 = ok ? m2_raw[0][1] : 0.0f, j1 = ok ? m2_raw[0][3] : 0.0f;
-      const float j2 = ok ? m2_raw[1][1] : 0.0f, j3 = ok ? m2_raw[1][3] : 0.0f;
+      const float r0 = ok ? m2_raw.re(0) : 0.0f, r1 = ok ? m2_raw.re(1) : 0.0f;
+      const float r2 = ok ? m2_raw.re(2) : 0.0f, r3 = ok ? m2_raw.re(3) : 0.0f;
+      const float j0 = ok ? m2_raw.im(0) : 0.0f, j1 = ok ? m2_raw.im(1) : 0.0f;
+      const float j2 = ok ? m2_raw.im(2) : 0.0f, j3 = ok ? m2_raw.im(3) : 0.0f;
       uint32_t a0[NP], a1[NP], b0[NP], b1[NP];
       split2<NP>(sk, r0, r1, a0);
       split2<NP>(sk, r2, r3, a1);
@@ -264,15 +308,15 @@ __global__ __launch_bounds__(256) void unitary_bwd_xdl_kernel(const UniBwdArgs p
   };
 
   // ---- channel data of one chunk
-  struct In { f4 u[2], de[2], th[2], dy[2], ph[2]; };
+  struct In { AccRaw4<Tin> u[2], de[2]; f4 th[2], dy[2], ph[2]; };
   auto in_load = [&](In& r, int c) {
     const int cc = c < 0 ? 0 : c;
 #pragma unroll
     for (int st = 0; st < 2; ++st) {
       const int l = cc * XT + 16 * st + 4 * g;
       const int lc = l < L ? l : 0;
-      ldg_acc(r.u[st], gu + lc);
-      ldg_acc(r.de[st], gdl + lc);
+      r.u[st].load(gu + lc);
+      r.de[st].load(gdl + lc);
       ldg_acc(r.th[st], gth + lc);
       ldg_acc(r.dy[st], gdy + lc);
       ldg_acc(r.ph[st], gph + lc);   // unconditional: a value defined on one path only would be copied at the join, before it has landed
@@ -280,13 +324,23 @@ __global__ __launch_bounds__(256) void unitary_bwd_xdl_kernel(const UniBwdArgs p
   };
   // everything ldg_acc has requested (B/C staging data and one chunk of channel data) has landed
   auto landed = [&](In& r) {
-    asm volatile("s_waitcnt vmcnt(0)"
-                 : "+a"(r.u[0]), "+a"(r.u[1]), "+a"(r.de[0]), "+a"(r.de[1]), "+a"(r.th[0]), "+a"(r.th[1]),
-                   "+a"(r.dy[0]), "+a"(r.dy[1]), "+a"(r.ph[0]), "+a"(r.ph[1]),
-                   "+a"(m1_raw[0]), "+a"(m1_raw[1]), "+a"(m1_raw[2]), "+a"(m1_raw[3]),
-                   "+a"(m2_raw[0]), "+a"(m2_raw[1])
-                 :
-                 : "memory");
+    if constexpr (sizeof(Tin) == 4) {
+      asm volatile("s_waitcnt vmcnt(0)"
+                   : "+a"(r.u[0].v), "+a"(r.u[1].v), "+a"(r.de[0].v), "+a"(r.de[1].v), "+a"(r.th[0]), "+a"(r.th[1]),
+                     "+a"(r.dy[0]), "+a"(r.dy[1]), "+a"(r.ph[0]), "+a"(r.ph[1]),
+                     "+a"(m1_raw[0].v), "+a"(m1_raw[1].v), "+a"(m1_raw[2].v), "+a"(m1_raw[3].v),
+                     "+a"(m2_raw.a), "+a"(m2_raw.b)
+                   :
+                   : "memory");
+    } else {
+      asm volatile("s_waitcnt vmcnt(0)"
+                   : "+a"(r.u[0].v), "+a"(r.u[1].v), "+a"(r.de[0].v), "+a"(r.de[1].v), "+a"(r.th[0]), "+a"(r.th[1]),
+                     "+a"(r.dy[0]), "+a"(r.dy[1]), "+a"(r.ph[0]), "+a"(r.ph[1]),
+                     "+a"(m1_raw[0].v), "+a"(m1_raw[1].v), "+a"(m1_raw[2].v), "+a"(m1_raw[3].v),
+                     "+a"(m2_raw.a)
+                   :
+                   : "memory");
+    }
   };
 
   // ---- state at the end of the current chunk and its adjoint: lane (dl, g) holds n = 4 g + i
@@ -377,8 +431,8 @@ __global__ __launch_bounds__(256) void unitary_bwd_xdl_kernel(const UniBwdArgs p
       for (int i = 0; i < 4; ++i) {
         th[st][i] = ok ? cur.th[st][i] : 0.0f;
         big |= fabsf(th[st][i]) > 4.0f;
-        uu[4 * st + i] = ok ? cur.u[st][i] : 0.0f;
-        de[4 * st + i] = ok ? cur.de[st][i] : 0.0f;
+        uu[4 * st + i] = ok ? cur.u[st].get(i) : 0.0f;
+        de[4 * st + i] = ok ? cur.de[st].get(i) : 0.0f;
         dy[4 * st + i] = ok ? cur.dy[st][i] : 0.0f;
         w[4 * st + i] = de[4 * st + i] * uu[4 * st + i];
       }

@@ -165,3 +165,29 @@ def test_sequence_split_over_workgroups(B, D, N, L, cap):
     for k, w, gt, wh in zip(names, want, got, whole):
         _close(gt, w, k, tol=2e-4 if D == 80 else 1e-4)
         _close(gt, wh.cpu(), k + " (split vs whole)", tol=2e-5)
+
+
+@pytest.mark.parametrize("B,D,N,L", [(2, 80, 16, 200), (1, 64, 7, 64)])
+def test_bf16_inputs_equal_the_float_run_on_the_same_values(B, D, N, L):
+    """bfloat16 u / delta / B / C are widened exactly inside the matrix-core kernels: outputs and
+    (float32) gradients must agree with the float32 call on the same, already rounded, values to
+    float32 rounding — far inside the 2e-2 the contract allows for bf16 inputs."""
+    from aussm_amd import scan
+    p = {k: v.cuda() for k, v in O.make_core_inputs(B, D, N, L, seed=17).items()}
+    ck = scan.UNITARY_CK
+    lo = {k: p[k].to(torch.bfloat16) for k in ("u", "delta")}
+    lo["Bri"] = torch.view_as_real(p["Bc"]).to(torch.bfloat16).contiguous()
+    lo["Cri"] = torch.view_as_real(p["Cc"]).to(torch.bfloat16).contiguous()
+    hi = {k: v.float() for k, v in lo.items()}
+    outs = []
+    for q in (lo, hi):
+        aux = scan.unitary_aux(q["u"], N, ck)
+        print(f"case bf16-vs-float dtype={q['u'].dtype} B={B} D={D} N={N} L={L}", flush=True)
+        y, hL, hck = scan.unitary_fwd_raw(q["u"], q["delta"], p["theta"], q["Bri"], q["Cri"], p["Dskip"], None, None,
+                                          want_state=True, ck=ck, aux=aux)
+        g = scan.unitary_bwd_raw(p["dy"], None, q["u"], q["delta"], p["theta"], q["Bri"], q["Cri"], p["Dskip"], hck, ck,
+                                 aux=aux)
+        torch.cuda.synchronize()
+        outs.append((y, hL) + tuple(g[:6]))
+    for name, a, b in zip(("y", "hL", "du", "ddelta", "dtheta", "dB", "dC", "dD"), *outs):
+        _close(a, b.cpu(), name, tol=1e-5)
