@@ -151,7 +151,7 @@ int launch_fwd(FwdArgs a, int in_dtype, hipStream_t s) {
   if (a.aux && mode <= 1)   // this call will not fill the auxiliary buffer
     hipLaunchKernelGGL(aux_invalidate_kernel, dim3(1), dim3(1), 0, s, a.aux + (size_t)a.B * a.D * a.L);
   if (mode) {
-    if ((mode == 2 || mode == 3) && a.aux && a.hck && in_dtype == AUSSM_F32) {
+    if ((mode == 2 || mode == 3) && a.aux && a.hck) {
       const int ns = seg_count(a.B, a.D, a.N, a.L, a.ck);
       if (ns > 1) {
         // 1. end state of every segment from a zero start and its rotation; 2. chain them;
@@ -159,9 +159,10 @@ int launch_fwd(FwdArgs a, int in_dtype, hipStream_t s) {
         const int B = a.B, L = a.L, Ls = a.L / ns, r = seg_fine(L, ns), nf = ns * r;
         float* seg = a.aux + (size_t)B * a.D * L + AUX_PAD;
         float* ptot = seg + (size_t)B * nf * a.D * a.N * 2;
-        SegArgs sa{static_cast<const float*>(a.delta), static_cast<const float*>(a.u), a.theta,
-                   static_cast<const float*>(a.Bm), seg, ptot, a.D, a.N, Ls / r, L, nf, a.ncg};
-        hipLaunchKernelGGL((unitary_seg_state_kernel<3, false>), dim3((unsigned)(B * nf * a.ncg)), dim3(256), 0, s, sa);
+        SegArgs sa{a.delta, a.u, a.theta, a.Bm, seg, ptot, a.D, a.N, Ls / r, L, nf, a.ncg};
+        const dim3 sgrid((unsigned)(B * nf * a.ncg));
+        if (in_dtype == AUSSM_BF16) hipLaunchKernelGGL((unitary_seg_state_kernel<3, false, bf16_t>), sgrid, dim3(256), 0, s, sa);
+        else hipLaunchKernelGGL((unitary_seg_state_kernel<3, false>), sgrid, dim3(256), 0, s, sa);
         const size_t nst = (size_t)B * a.D * a.N;
         hipLaunchKernelGGL(seg_carry_fwd_kernel, dim3((unsigned)((nst + 255) / 256)), dim3(256), 0, s, seg, ptot, a.h0,
                            a.hL, B, a.D, a.N, nf);
@@ -337,14 +338,16 @@ int aussm_unitary_bwd_aux(const float* dy, const float* dhL, const void* u, cons
       !(misaligned(dy, 16) || misaligned(u, 16) || misaligned(delta, 16) || misaligned(theta, 16) ||
         misaligned(du, 16) || misaligned(ddelta, 16) || misaligned(dtheta, 16) || misaligned(Bc, 16) ||
         misaligned(Cc, 16))) {
-    const int ns = (aux && in_dtype == AUSSM_F32) ? seg_count(B, D, N, L, ck) : 1;
+    const int ns = aux ? seg_count(B, D, N, L, ck) : 1;
     if (ns > 1) {
       // adjoint at the start of every segment from a zero adjoint at its end, chained last to first
       const int Ls = L / ns, r = seg_fine(L, ns), nf = ns * r;
       float* seg = aux + (size_t)B * D * L + AUX_PAD;
       float* ptot = seg + (size_t)B * nf * D * N * 2;
-      SegArgs sa{dy, nullptr, theta, static_cast<const float*>(Cc), seg, ptot, D, N, Ls / r, L, nf, a.ncg};
-      hipLaunchKernelGGL((unitary_seg_state_kernel<3, true>), dim3((unsigned)(B * nf * a.ncg)), dim3(256), 0, s, sa);
+      SegArgs sa{dy, nullptr, theta, Cc, seg, ptot, D, N, Ls / r, L, nf, a.ncg};
+      const dim3 sgrid((unsigned)(B * nf * a.ncg));
+      if (in_dtype == AUSSM_BF16) hipLaunchKernelGGL((unitary_seg_state_kernel<3, true, bf16_t>), sgrid, dim3(256), 0, s, sa);
+      else hipLaunchKernelGGL((unitary_seg_state_kernel<3, true>), sgrid, dim3(256), 0, s, sa);
       const size_t nst = (size_t)B * D * N;
       hipLaunchKernelGGL(seg_carry_bwd_kernel, dim3((unsigned)((nst + 255) / 256)), dim3(256), 0, s, seg, ptot, dhL, dh0,
                          B, D, N, nf);

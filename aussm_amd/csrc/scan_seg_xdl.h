@@ -12,15 +12,17 @@
 //   3. runs the scan kernel proper with (batch, segment) pairs as its batch index, every segment
 //      starting from its true incoming state or adjoint.
 #pragma once
+#include <type_traits>
+
 #include "scan_fwd_xdl.h"
 
 namespace aussm {
 
 struct SegArgs {
-  const float* x1;      // forward: delta, adjoint: dy        [B, D, ld]
-  const float* x2;      // forward: u, adjoint: unused        [B, D, ld]
+  const void* x1;       // forward: delta (Tin), adjoint: dy (float)   [B, D, ld]
+  const void* x2;       // forward: u (Tin), adjoint: unused           [B, D, ld]
   const float* theta;   //                                    [B, D, ld]
-  const float* M;       // forward: B_t, adjoint: C_t         [B, N, ld, 2]
+  const void* M;        // forward: B_t, adjoint: C_t (Tin)            [B, N, ld, 2]
   float* out;           // Z or Y                             [B * ns, D, N, 2]
   float* ptot;          // rotation of the segment            [B * ns, D, 2]
   int D, N, L, ld, ns, ncg;   // L: segment length
@@ -28,8 +30,8 @@ struct SegArgs {
 
 // ADJ = false: Z of each segment, chunks in forward order,  H <- P_T (H + B^T V).
 // ADJ = true:  Y of each segment, chunks in reverse order,  A <- conj(P_T) A + conj(C)^T Q.
-// Requires N <= 16, L % 4 == 0, 16-byte aligned tensors, float inputs.
-template <int NP, bool ADJ>
+// Requires N <= 16, L % 4 == 0, 16-byte aligned tensors.  Tin: float or bf16_t (u, delta, B, C).
+template <int NP, bool ADJ, typename Tin = float>
 __global__ __launch_bounds__(256) void unitary_seg_state_kernel(const SegArgs p) {
   // row n: M[t(g, e)][n], real and imaginary parts (the imaginary part negated for ADJ: conj(C))
   __shared__ u4 s_mr[2][NP][XN * 4];
@@ -46,8 +48,10 @@ __global__ __launch_bounds__(256) void unitary_seg_state_kernel(const SegArgs p)
   const int bb = vb / p.ns;
   const size_t so = (size_t)(vb - bb * p.ns) * L;
   const size_t row = ((size_t)bb * D + dc) * p.ld + so;
-  const float* __restrict__ gx1 = p.x1 + row;
-  const float* __restrict__ gx2 = ADJ ? p.x1 + row : p.x2 + row;
+  using TA = typename std::conditional<ADJ, float, Tin>::type;   // dy is always float
+  const TA* __restrict__ gx1 = static_cast<const TA*>(p.x1) + row;
+  const Tin* __restrict__ gx2 = ADJ ? nullptr : static_cast<const Tin*>(p.x2) + row;
+  const Tin* __restrict__ gM = static_cast<const Tin*>(p.M);
   const float* __restrict__ gth = p.theta + row;
   const int nchunks = (L + XT - 1) / XT;
   const SplitK sk = make_splitk();
@@ -57,20 +61,19 @@ __global__ __launch_bounds__(256) void unitary_seg_state_kernel(const SegArgs p)
   // the imaginary one
   const int m2_n = tid & 15, m2_g = (tid >> 4) & 3, m2_half = (tid >> 6) & 1;
   const bool m2_im = tid >= 128;
-  f4 m2_raw[2];
+  RawC4<Tin> m2_raw;
   auto m_load = [&](int c) {
     const int cc = c < 0 ? 0 : (c >= nchunks ? nchunks - 1 : c);
     const int l2 = cc * XT + 16 * m2_half + 4 * m2_g;
     const int l2c = l2 < L ? l2 : 0;
     const size_t o2 = (((size_t)bb * N + (m2_n < N ? m2_n : 0)) * p.ld + so + l2c) * 2;
-    m2_raw[0] = *reinterpret_cast<const f4*>(p.M + o2);
-    m2_raw[1] = *reinterpret_cast<const f4*>(p.M + o2 + 4);
+    m2_raw.load(gM + o2);
   };
   auto m_store = [&](int c, int slot) {
     const bool ok = (m2_n < N) && (c * XT + 16 * m2_half + 4 * m2_g < L);
     const float sg = (ADJ && m2_im) ? -1.0f : 1.0f;
-    float v0 = m2_im ? m2_raw[0][1] : m2_raw[0][0], v1 = m2_im ? m2_raw[0][3] : m2_raw[0][2];
-    float v2 = m2_im ? m2_raw[1][1] : m2_raw[1][0], v3 = m2_im ? m2_raw[1][3] : m2_raw[1][2];
+    float v0 = m2_im ? m2_raw.im(0) : m2_raw.re(0), v1 = m2_im ? m2_raw.im(1) : m2_raw.re(1);
+    float v2 = m2_im ? m2_raw.im(2) : m2_raw.re(2), v3 = m2_im ? m2_raw.im(3) : m2_raw.re(3);
     v0 = ok ? sg * v0 : 0.0f; v1 = ok ? sg * v1 : 0.0f; v2 = ok ? sg * v2 : 0.0f; v3 = ok ? sg * v3 : 0.0f;
     uint32_t a0[NP], a1[NP];
     split2<NP>(sk, v0, v1, a0);
@@ -81,7 +84,7 @@ __global__ __launch_bounds__(256) void unitary_seg_state_kernel(const SegArgs p)
     for (int q = 0; q < NP; ++q) reinterpret_cast<u2*>(dst[q])[o] = u2{a0[q], a1[q]};
   };
 
-  struct In { f4 th[2], a[2], b[2]; };
+  struct In { f4 th[2]; Raw4<TA> a[2]; Raw4<Tin> b[2]; };
   auto in_load = [&](In& r, int c) {
     const int cc = c < 0 ? 0 : (c >= nchunks ? nchunks - 1 : c);
 #pragma unroll
@@ -89,8 +92,8 @@ __global__ __launch_bounds__(256) void unitary_seg_state_kernel(const SegArgs p)
       const int l = cc * XT + 16 * st + 4 * g;
       const int lc = l < L ? l : 0;
       r.th[st] = *reinterpret_cast<const f4*>(gth + lc);
-      r.a[st] = *reinterpret_cast<const f4*>(gx1 + lc);
-      if (!ADJ) r.b[st] = *reinterpret_cast<const f4*>(gx2 + lc);
+      r.a[st].load(gx1 + lc);
+      if (!ADJ) r.b[st].load(gx2 + lc);
     }
   };
 
@@ -122,7 +125,7 @@ __global__ __launch_bounds__(256) void unitary_seg_state_kernel(const SegArgs p)
       for (int i = 0; i < 4; ++i) {
         th[st][i] = ok ? cur.th[st][i] : 0.0f;
         big |= fabsf(th[st][i]) > 4.0f;
-        const float v = ADJ ? cur.a[st][i] : cur.a[st][i] * cur.b[st][i];
+        const float v = ADJ ? cur.a[st].get(i) : cur.a[st].get(i) * cur.b[st].get(i);
         x[4 * st + i] = ok ? v : 0.0f;
       }
     }

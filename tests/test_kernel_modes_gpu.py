@@ -167,7 +167,7 @@ def test_sequence_split_over_workgroups(B, D, N, L, cap):
         _close(gt, wh.cpu(), k + " (split vs whole)", tol=2e-5)
 
 
-@pytest.mark.parametrize("B,D,N,L", [(2, 80, 16, 200), (1, 64, 7, 64)])
+@pytest.mark.parametrize("B,D,N,L", [(2, 80, 16, 200), (1, 64, 7, 64), (1, 64, 16, 1024)])   # the last one is split along L
 def test_bf16_inputs_equal_the_float_run_on_the_same_values(B, D, N, L):
     """bfloat16 u / delta / B / C are widened exactly inside the matrix-core kernels: outputs and
     (float32) gradients must agree with the float32 call on the same, already rounded, values to
