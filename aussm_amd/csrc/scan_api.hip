@@ -78,7 +78,7 @@ int launch_fwd_t(const FwdArgs& a, hipStream_t s) {
   return AUSSM_E_SHAPE;
 }
 
-// The matrix-core kernels cover the common unitary case (fp32 inputs, 6 <= N <= 16, L a multiple of 4,
+// The matrix-core kernels cover the common unitary case (fp32 or bf16 inputs, 6 <= N <= 16, L a multiple of 4,
 // 16-byte aligned tensors, checkpoint interval a multiple of 32); everything else takes the
 // generic kernels.  AUSSM_MFMA (environment, read at every call) selects the forward kernel for
 // comparisons: 0 generic, 1 fp32 matrix instructions, 2 / 3 bf16 matrix instructions on two- /

@@ -71,7 +71,7 @@ int aussm_bwd_checkpoint_interval(int variant);
  * the device scan of extension-cpp/extension_cpp/csrc/cuda/ssm_adaptive_unitary_forward.cu:113-181
  * for a phase that is given per (b,d,l).
  * Optional (NULL allowed): Dskip, z, h0, y (NULL = states only), hL, hck.
- * Kernel choice is internal: float32 inputs with 6 <= N <= 16, L a multiple of 4, 16-byte aligned
+ * Kernel choice is internal: calls with 6 <= N <= 16, L a multiple of 4, 16-byte aligned
  * tensors and ck a multiple of AUSSM_TILE run on the matrix cores (fp32-accurate, see the
  * kernel headers); every other accepted call runs on the vector ALU.  Results agree to
  * rounding.  The environment variables AUSSM_MFMA / AUSSM_MFMA_BWD force one for comparisons.
