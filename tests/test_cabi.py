@@ -80,6 +80,12 @@ def test_argument_checks_without_a_device():
     args = [one] * 9 + [0] + [one] * 9
     assert lib.aussm_real_bwd(*args, 1, 1, 1, 32, 32, 0, null) == -3
     assert lib.aussm_real_bwd(*args, 1, 1, 17, 32, 16, 0, null) == -2
+    # the blocks' causal convolution: kernel length limit, overlapping rows, required pointers
+    assert lib.aussm_causal_conv1d_fwd(one, one, null, one, 1, 8, 4, 9, 32, 4, null) == -2
+    assert lib.aussm_causal_conv1d_fwd(one, one, null, one, 1, 8, 4, 4, 32, 3, null) == -2      # row stride < D
+    assert lib.aussm_causal_conv1d_fwd(one, one, null, one, 2, 8, 4, 4, 16, 4, null) == -2      # batches overlap
+    assert lib.aussm_causal_conv1d_fwd(null, one, null, one, 1, 8, 4, 4, 32, 4, null) == -1
+    assert lib.aussm_causal_conv1d_bwd(one, one, one, one, null, null, 1, 8, 4, 4, 32, 4, null) == -1
 
 
 def test_python_layer_fails_loudly_without_library(monkeypatch, tmp_path):
