@@ -191,3 +191,60 @@ def test_bf16_inputs_equal_the_float_run_on_the_same_values(B, D, N, L):
         outs.append((y, hL) + tuple(g[:6]))
     for name, a, b in zip(("y", "hL", "du", "ddelta", "dtheta", "dB", "dC", "dD"), *outs):
         _close(a, b.cpu(), name, tol=1e-5)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_shapes_inputs_and_checkpoint_intervals(seed):
+    """A seeded sweep over what the launcher has to get right together: partial channel groups and
+    chunks, every N the matrix-core kernels serve, checkpoint intervals 32 / 64 / 256 (which also
+    set the segment length of the split along L), float32 and bfloat16 inputs, output gate, carried
+    state and upstream gradient of the final state.  Forward and backward through the raw wrappers
+    against the CPU oracle on the same (for bf16: already rounded) values."""
+    import random
+    from aussm_amd import scan
+    r = random.Random(1000 + seed)
+    B, D, N = r.randint(1, 3), r.randint(1, 150), r.randint(6, 16)
+    ck = r.choice([32, 64, 256])
+    L = ck * r.randint(1, 6) if r.random() < 0.6 else 4 * r.randint(1, 160)
+    lowp, gate, carried = r.random() < 0.4, r.random() < 0.5, r.random() < 0.5
+    p = O.make_core_inputs(B, D, N, L, seed=seed, gate=gate)
+    g = torch.Generator().manual_seed(seed)
+    h0 = torch.complex(torch.randn(B, D, N, generator=g), torch.randn(B, D, N, generator=g)) if carried else None
+    dh = torch.complex(torch.randn(B, D, N, generator=g), torch.randn(B, D, N, generator=g)) if carried else None
+    if lowp:
+        for k in ("u", "delta", "Bc", "Cc"):
+            t = p[k]
+            p[k] = (torch.view_as_complex(torch.view_as_real(t).bfloat16().float().contiguous()) if t.is_complex()
+                    else t.bfloat16().float())
+    # oracle (gradients of the gated output are only needed for the ungated backward kernel: gate off there)
+    leaves = [p[k].clone().requires_grad_(True) for k in NAMES]
+    h0l = h0.clone().requires_grad_(True) if carried else None
+    y_want, hL_want = O.unitary_core_loop(*leaves, p.get("z"), h0l)
+    y_ng, hL_ng = O.unitary_core_loop(*leaves, None, h0l)
+    loss = (y_ng * p["dy"]).sum()
+    if carried:
+        loss = loss + (torch.view_as_real(hL_ng) * torch.view_as_real(dh)).sum()
+    loss.backward()
+    want = [t.grad for t in leaves]
+
+    dt = torch.bfloat16 if lowp else torch.float32
+    q = {k: v.cuda() for k, v in p.items()}
+    u, de = q["u"].to(dt), q["delta"].to(dt)
+    Bri = torch.view_as_real(q["Bc"]).to(dt).contiguous()
+    Cri = torch.view_as_real(q["Cc"]).to(dt).contiguous()
+    h0d = torch.view_as_real(h0).contiguous().cuda() if carried else None
+    dhd = torch.view_as_real(dh).contiguous().cuda() if carried else None
+    aux = scan.unitary_aux(u, N, ck)
+    print(f"case sweep seed={seed} B={B} D={D} N={N} L={L} ck={ck} bf16={lowp} gate={gate} carried={carried}", flush=True)
+    y, hL, _ = scan.unitary_fwd_raw(u, de, q["theta"], Bri, Cri, q["Dskip"], q.get("z"), h0d, want_state=True, ck=ck, aux=aux)
+    _close(y, y_want.detach(), "y")
+    _close(torch.view_as_complex(hL), hL_want.detach(), "hL")
+    _, _, hck = scan.unitary_fwd_raw(u, de, q["theta"], Bri, Cri, q["Dskip"], None, h0d, want_state=False, ck=ck, aux=aux)
+    du, dde, dth, dB, dC, dD, dh0 = scan.unitary_bwd_raw(q["dy"], dhd, u, de, q["theta"], Bri, Cri, q["Dskip"], hck, ck,
+                                                         want_dh0=carried, aux=aux)
+    torch.cuda.synchronize()
+    got = (du, dde, dth, torch.view_as_complex(dB), torch.view_as_complex(dC), dD)
+    for k, w, gt in zip(NAMES, want, got):
+        _close(gt, w, f"d{k}")
+    if carried:
+        _close(torch.view_as_complex(dh0), h0l.grad, "dh0")
