@@ -36,10 +36,10 @@ HBM_PEAK_GBS = 8000.0
 SHAPE = dict(B=32, D=512, N=16, L=2048)
 # HBM bytes per launch at SHAPE from the counter passes summarised in
 # profiles/unitary_fwd_bwd_B32_D512_N16_L2048_hbm_traffic.md (FETCH_SIZE x 2.00, WRITE_SIZE x 1.00 after
-# calibration on a 256 MiB copy): forward 427 MB read + 286 MB written, backward 808 MB read +
-# 544 MB written.  Both include the auxiliary buffer (134 MB written forward, read backward) and the
+# calibration on a 256 MiB copy): forward 427 MB read + 286 MB written, backward 818 MB read +
+# 547 MB written.  Both include the auxiliary buffer (134 MB written forward, read backward) and the
 # checkpoints; the dB/dC atomics of the eight workgroups of a batch element count as writes.
-TRAFFIC_BYTES = {"unitary_fwd": 713e6, "unitary_bwd": 1353e6}
+TRAFFIC_BYTES = {"unitary_fwd": 713e6, "unitary_bwd": 1366e6}
 
 
 def cpu_baseline(B_sample: int):
@@ -180,10 +180,10 @@ def main():
         "fwd_bwd_algorithmic_GBps": (bytes_fwd + bytes_bwd) / ((t_fwd + t_bwd) * 1e-6) / 1e9,
         "fwd_bwd_frac_of_hbm_peak": (bytes_fwd + bytes_bwd) / ((t_fwd + t_bwd) * 1e-6) / 1e9 / HBM_PEAK_GBS,
         "kernels_us": {"unitary_fwd": t_fwd, "unitary_bwd": t_bwd},
-        "roofline": {"bound": "hbm", "kernel": "unitary_bwd_xdl_kernel<3, 2>", "achieved": ach, "peak": HBM_PEAK_GBS,
+        "roofline": {"bound": "hbm", "kernel": "unitary_bwd_xdl_kernel<3, 2, float>", "achieved": ach, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": ach / HBM_PEAK_GBS, "traffic": TRAFFIC_BYTES["unitary_bwd"] if headline else None,
                      "algorithmic_bytes": bytes_bwd,
-                     "fwd_kernel": {"kernel": "unitary_fwd_xdl_kernel<3, false>",
+                     "fwd_kernel": {"kernel": "unitary_fwd_xdl_kernel<3, false, float>",
                                     "achieved": bytes_fwd / (t_fwd * 1e-6) / 1e9,
                                     "frac": bytes_fwd / (t_fwd * 1e-6) / 1e9 / HBM_PEAK_GBS,
                                     "traffic": TRAFFIC_BYTES["unitary_fwd"] if headline else None,
