@@ -17,6 +17,8 @@
 // gradient structure of extension-cpp/extension_cpp/csrc/cuda/ssm_adaptive_complex.cu:358-660 and
 // ssm_adaptive_real.cu:267-488, selective-scan call at ai-modules/wavesAI/model/aussm.py:791-802.
 #pragma once
+#include <type_traits>
+
 #include "scan_bwd_unitary.h"
 #include "scan_common.h"
 
@@ -69,6 +71,19 @@ __device__ __forceinline__ f32x8 ld_r8_safe(const Tin* p, size_t row, int t0, in
 #pragma unroll
   for (int i = 0; i < TG; ++i) r[i] = ld_r(p, row + ((t0 + i < L) ? t0 + i : L - 1));
   return r;
+}
+
+// FULL: the whole tile lies inside the sequence, wide loads are aligned and the wavefront owns NW
+// existing states, known once per tile: no branch per load or state, so the compiler can issue the scalar loads of a tile ahead of their use.
+template <bool FULL, typename Tin>
+__device__ __forceinline__ f32x16 ld_c8_tile(const Tin* p, size_t row, int t0, int L) {
+  if constexpr (FULL) return ld_c8(p, row + t0);
+  else return ld_c8_safe(p, row, t0, L);
+}
+template <bool FULL, typename Tin>
+__device__ __forceinline__ f32x8 ld_r8_tile(const Tin* p, size_t row, int t0, int L) {
+  if constexpr (FULL) return ld_r8(p, row + t0);
+  else return ld_r8_safe(p, row, t0, L);
 }
 
 template <int VAR, int NW, int NT, typename Tin>
@@ -224,7 +239,8 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
     __syncthreads();
 
     float rres[NRES > 0 ? NRES : 1];
-    if (active) {
+    auto tile_body = [&](auto full_tag) {
+      constexpr bool FULL = decltype(full_tag)::value;
       const size_t brow = row_base + l0;
       // ---- 1. recompute the tile's states from its start state
       float hsr[RT][NW], hsi[RT][NW];
@@ -241,9 +257,9 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
         }
 #pragma unroll
         for (int k = 0; k < NW; ++k) {
-          if (n0 + k < N) {                        // wave-uniform
+          if (FULL || n0 + k < N) {                // wave-uniform; FULL: all NW states of the wavefront exist
             if constexpr (VAR == VAR_REAL) {
-              const f32x8 bc = ld_r8_safe(gB, brow + (size_t)k * L - l0, l0 + g * TG, L);
+              const f32x8 bc = ld_r8_tile<FULL>(gB, brow + (size_t)k * L - l0, l0 + g * TG, L);
 #pragma unroll
               for (int t = 0; t < TG; ++t) {
                 const float a = __builtin_amdgcn_exp2f(rx[t] * a2[k]);
@@ -251,7 +267,7 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
                 hsr[g * TG + t][k] = cr_[k];
               }
             } else {
-              const f32x16 bc = ld_c8_safe(gB, brow + (size_t)k * L - l0, l0 + g * TG, L);
+              const f32x16 bc = ld_c8_tile<FULL>(gB, brow + (size_t)k * L - l0, l0 + g * TG, L);
 #pragma unroll
               for (int t = 0; t < TG; ++t) {
                 const float nr = fmaf(rx[t], cr_[k], fmaf(-ry[t], ci_[k], bc[2 * t] * rz[t]));
@@ -284,10 +300,10 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
         for (int j = 0; j < RED_COLS; ++j) vals[j] = 0.f;
 #pragma unroll
         for (int k = 0; k < NW; ++k) {
-          if (n0 + k < N) {                        // wave-uniform
+          if (FULL || n0 + k < N) {                // wave-uniform; FULL: all NW states of the wavefront exist
             if constexpr (VAR == VAR_REAL) {
-              const f32x8 bc = ld_r8_safe(gB, brow + (size_t)k * L - l0, l0 + g * TG, L);
-              const f32x8 cc = ld_r8_safe(gC, brow + (size_t)k * L - l0, l0 + g * TG, L);
+              const f32x8 bc = ld_r8_tile<FULL>(gB, brow + (size_t)k * L - l0, l0 + g * TG, L);
+              const f32x8 cc = ld_r8_tile<FULL>(gC, brow + (size_t)k * L - l0, l0 + g * TG, L);
               constexpr int VB = 0;                // filled below per row slot
               (void)VB;
               const int slot = (RPT == 2) ? (k & 1) : 0;
@@ -307,8 +323,8 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
                 gr[k] *= a;
               }
             } else {
-              const f32x16 bc = ld_c8_safe(gB, brow + (size_t)k * L - l0, l0 + g * TG, L);
-              const f32x16 cc = ld_c8_safe(gC, brow + (size_t)k * L - l0, l0 + g * TG, L);
+              const f32x16 bc = ld_c8_tile<FULL>(gB, brow + (size_t)k * L - l0, l0 + g * TG, L);
+              const f32x16 cc = ld_c8_tile<FULL>(gC, brow + (size_t)k * L - l0, l0 + g * TG, L);
 #pragma unroll
               for (int t = TG - 1; t >= 0; --t) {
                 const int tt = g * TG + t;
@@ -346,6 +362,12 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
 #pragma unroll
         for (int t = 0; t < TG; ++t) part[(g * TG + t) * TS + lane] = make_float4(kacc[t], xacc[t], zacc[t], 0.f);
       }
+        };
+    if (active) {
+      // (bf16 rows start at even element offsets when L is even: wide loads stay 4-byte aligned)
+      const bool full = (l0 + RT <= L) && (n0 + NW <= N) && (sizeof(Tin) == 4 || (L & 1) == 0);
+      if (full) tile_body(std::true_type{});
+      else tile_body(std::false_type{});
     }
     __syncthreads();
 

@@ -3,7 +3,7 @@
 once with float32 inputs and once with bfloat16 u / delta / B / C (float32 phases, decay, skip,
 states, outputs and gradients): BASELINE configuration 3.
 
-    python bench_variants.py [--reps R] [--shape B,D,N,L] [--model | --only-model]
+    python bench_variants.py [--reps R] [--shape B,D,N,L] [--variants real,...] [--model | --only-model]
 
 With --model it also times BASELINE configuration 4: one training step (forward, MSE loss,
 backward) of SSMTS(d_model=256, input_dim=21, output_dim=21, layers="a|m|a|m") on x ~ N(0,1) of
@@ -48,6 +48,7 @@ def main():
     ap.add_argument("--shape", default="32,512,16,2048")
     ap.add_argument("--model", action="store_true", help="also time the hybrid SSMTS training step (configuration 4)")
     ap.add_argument("--only-model", action="store_true", help="time only the SSMTS training step")
+    ap.add_argument("--variants", default="unitary,complex,real", help="comma-separated subset of the variants")
     args = ap.parse_args()
     B, D, N, L = (int(v) for v in args.shape.split(","))
 
@@ -89,7 +90,7 @@ def main():
         return out
 
     E, S = B * D * L, B * N * L
-    for variant in (() if args.only_model else ("unitary", "complex", "real")):
+    for variant in (() if args.only_model else tuple(args.variants.split(","))):
         base = inputs(variant)
         for name, dt, w in (("f32", torch.float32, 4), ("bf16", torch.bfloat16, 2)):
             p = dict(base)
