@@ -29,8 +29,8 @@ _SIGNATURES = {
     "aussm_bwd_checkpoint_interval": [_I],
     "aussm_unitary_fwd": [_P] * 11 + [_I] * 6 + [_P],
     "aussm_unitary_bwd": [_P] * 16 + [_I] * 6 + [_P],
-    "aussm_unitary_fwd_aux": [_P] * 12 + [_I] * 6 + [_P],
-    "aussm_unitary_bwd_aux": [_P] * 17 + [_I] * 6 + [_P],
+    "aussm_unitary_fwd_aux": [_P] * 12 + [_I] * 7 + [_P],
+    "aussm_unitary_bwd_aux": [_P] * 17 + [_I] * 7 + [_P],
     "aussm_complex_fwd": [_P] * 12 + [_I] * 6 + [_P],
     "aussm_complex_bwd": [_P] * 19 + [_I] * 6 + [_P],
     "aussm_real_fwd": [_P] * 8 + [_I] + [_P] * 4 + [_I] * 6 + [_P],

@@ -137,7 +137,7 @@ inline size_t seg_floats(int B, int D, int N, int L, int ns) {
 
 inline int mfma_fwd_mode(const FwdArgs& a, int in_dtype) {
   int mode = env_mode("AUSSM_MFMA", 3, a.N);
-  if (mode <= 0 || a.N > MN || a.L % 4 != 0 || a.ck % MT != 0) return 0;
+  if (mode <= 0 || a.urep != 1 || a.N > MN || a.L % 4 != 0 || a.ck % MT != 0) return 0;
   if (in_dtype != AUSSM_F32) mode = 3;       // bf16 inputs: the default matrix-core kernel only
   if (misaligned(a.u, 16) || misaligned(a.delta, 16) || misaligned(a.theta, 16) || misaligned(a.z, 16) ||
       misaligned(a.y, 16) || misaligned(a.Bm, 16) || misaligned(a.Cm, 16))
@@ -260,13 +260,14 @@ int aussm_unitary_fwd(const void* u, const void* delta, const float* theta, cons
                       const float* Dskip, const float* z, const float* h0, float* y, float* hL, float* hck,
                       int B, int D, int N, int L, int ck, int in_dtype, void* stream) {
   return aussm_unitary_fwd_aux(u, delta, theta, Bc, Cc, Dskip, z, h0, y, hL, hck, nullptr, B, D, N, L, ck, in_dtype,
-                               stream);
+                               1, stream);
 }
 
 int aussm_unitary_fwd_aux(const void* u, const void* delta, const float* theta, const void* Bc, const void* Cc,
                           const float* Dskip, const float* z, const float* h0, float* y, float* hL, float* hck,
-                          float* aux, int B, int D, int N, int L, int ck, int in_dtype, void* stream) {
+                          float* aux, int B, int D, int N, int L, int ck, int in_dtype, int urep, void* stream) {
   if (int e = check_common(B, D, N, L, ck, in_dtype)) return e;
+  if (urep < 1 || B % urep != 0) return AUSSM_E_SHAPE;
   if (misaligned(aux, 16)) return AUSSM_E_ALIGN;
   if (!u || !delta || !theta || !Bc || !Cc) return AUSSM_E_NULL;
   const size_t ca = in_dtype == AUSSM_BF16 ? 4 : 8;
@@ -275,7 +276,7 @@ int aussm_unitary_fwd_aux(const void* u, const void* delta, const float* theta, 
   a.u = u; a.delta = delta; a.theta = theta; a.Bm = Bc; a.Cm = Cc; a.Dskip = Dskip; a.z = z;
   a.h0 = h0; a.y = y; a.hL = hL; a.hck = hck; a.aux = aux;
   a.B = B; a.D = D; a.N = N; a.L = L; a.ck = ck; a.nck = (L + ck - 1) / ck; a.ncg = (D + CH - 1) / CH;
-  a.ld = L; a.ns = 1; a.hs = 1; a.ho = 0;
+  a.ld = L; a.ns = 1; a.hs = 1; a.ho = 0; a.urep = urep;
   return launch_fwd<VAR_UNITARY>(a, in_dtype, (hipStream_t)stream);
 }
 
@@ -290,7 +291,7 @@ int aussm_complex_fwd(const void* u, const void* delta, const float* rho, const 
   a.u = u; a.delta = delta; a.rho = rho; a.theta = theta; a.Bm = Bc; a.Cm = Cc; a.Dskip = Dskip; a.z = z;
   a.h0 = h0; a.y = y; a.hL = hL; a.hck = hck;
   a.B = B; a.D = D; a.N = N; a.L = L; a.ck = ck; a.nck = (L + ck - 1) / ck; a.ncg = (D + CH - 1) / CH;
-  a.ld = L; a.ns = 1; a.hs = 1; a.ho = 0;
+  a.ld = L; a.ns = 1; a.hs = 1; a.ho = 0; a.urep = 1;
   return launch_fwd<VAR_COMPLEX>(a, in_dtype, (hipStream_t)stream);
 }
 
@@ -305,7 +306,7 @@ int aussm_real_fwd(const void* u, const void* delta, const float* A, const void*
   a.delta_bias = delta_bias; a.delta_softplus = delta_softplus;
   a.h0 = h0; a.y = y; a.hL = hL; a.hck = hck;
   a.B = B; a.D = D; a.N = N; a.L = L; a.ck = ck; a.nck = (L + ck - 1) / ck; a.ncg = (D + CH - 1) / CH;
-  a.ld = L; a.ns = 1; a.hs = 1; a.ho = 0;
+  a.ld = L; a.ns = 1; a.hs = 1; a.ho = 0; a.urep = 1;
   return launch_fwd<VAR_REAL>(a, in_dtype, (hipStream_t)stream);
 }
 
@@ -314,14 +315,15 @@ int aussm_unitary_bwd(const float* dy, const float* dhL, const void* u, const vo
                       float* du, float* ddelta, float* dtheta, float* dB, float* dC, float* dD, float* dh0,
                       int B, int D, int N, int L, int ck, int in_dtype, void* stream) {
   return aussm_unitary_bwd_aux(dy, dhL, u, delta, theta, Bc, Cc, Dskip, hck, nullptr, du, ddelta, dtheta, dB, dC, dD,
-                               dh0, B, D, N, L, ck, in_dtype, stream);
+                               dh0, B, D, N, L, ck, in_dtype, 1, stream);
 }
 
 int aussm_unitary_bwd_aux(const float* dy, const float* dhL, const void* u, const void* delta, const float* theta,
                           const void* Bc, const void* Cc, const float* Dskip, const float* hck, float* aux,
                           float* du, float* ddelta, float* dtheta, float* dB, float* dC, float* dD, float* dh0,
-                          int B, int D, int N, int L, int ck, int in_dtype, void* stream) {
+                          int B, int D, int N, int L, int ck, int in_dtype, int urep, void* stream) {
   if (int e = check_common(B, D, N, L, ck, in_dtype)) return e;
+  if (urep < 1 || B % urep != 0) return AUSSM_E_SHAPE;
   if (misaligned(aux, 16)) return AUSSM_E_ALIGN;
   if (!dy || !u || !delta || !theta || !Bc || !Cc || !hck || !du || !ddelta || !dtheta || !dB || !dC)
     return AUSSM_E_NULL;
@@ -332,9 +334,10 @@ int aussm_unitary_bwd_aux(const float* dy, const float* dhL, const void* u, cons
   a.dy = dy; a.dhL = dhL; a.u = u; a.delta = delta; a.theta = theta; a.Bm = Bc; a.Cm = Cc; a.Dskip = Dskip;
   a.hck = hck; a.aux = aux; a.du = du; a.ddelta = ddelta; a.dtheta = dtheta; a.dB = dB; a.dC = dC; a.dD = dD; a.dh0 = dh0;
   a.B = B; a.D = D; a.N = N; a.L = L; a.ck = ck; a.nck = (L + ck - 1) / ck; a.ncg = (D + CH - 1) / CH;
-  a.ld = L; a.ns = 1; a.hs = 1; a.ho = 0;
+  a.ld = L; a.ns = 1; a.hs = 1; a.ho = 0; a.urep = 1;
   const int mode = env_mode("AUSSM_MFMA_BWD", 3, N);   // matrix-core kernel for the common case
-  if (mode > 0 && N <= XN && L % 4 == 0 && ck % XT == 0 &&
+  a.urep = urep;
+  if (mode > 0 && urep == 1 && N <= XN && L % 4 == 0 && ck % XT == 0 &&
       !(misaligned(dy, 16) || misaligned(u, 16) || misaligned(delta, 16) || misaligned(theta, 16) ||
         misaligned(du, 16) || misaligned(ddelta, 16) || misaligned(dtheta, 16) || misaligned(Bc, 16) ||
         misaligned(Cc, 16))) {

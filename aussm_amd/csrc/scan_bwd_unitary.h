@@ -40,6 +40,7 @@ struct UniBwdArgs {
   int B, D, N, L, ck, nck, ncg;
   int ld, ns;           // matrix-core kernel: row stride of the [.., L] tensors, segments per sequence
   int hs, ho;           // ... and dhL of (batch, segment) pair b is entry b * hs + ho of the adjoint array
+  int urep;             // generic kernel: u and delta are [B / urep, D, L], shared by urep consecutive batch elements
 };
 
 constexpr int RED_COLS = 4 * TG;        // products per lane per turn: TG x (dB re, dB im) then TG x (dC re, dC im)
@@ -99,8 +100,11 @@ __global__ __launch_bounds__(NT) void unitary_bwd_kernel(const UniBwdArgs p) {
   const int d = d0 + lane;
   const bool dok = d < D;
 
-  const Tin* __restrict__ gu = static_cast<const Tin*>(p.u);
-  const Tin* __restrict__ gdl = static_cast<const Tin*>(p.delta);
+  // u and delta may be shared by p.urep consecutive batch elements (tensors [B / urep, D, L]): every
+  // address below is formed for batch element b, so their base steps back by the difference
+  const size_t uback = (size_t)(b - b / p.urep) * p.D * p.L;
+  const Tin* __restrict__ gu = static_cast<const Tin*>(p.u) - uback;
+  const Tin* __restrict__ gdl = static_cast<const Tin*>(p.delta) - uback;
   const Tin* __restrict__ gB = static_cast<const Tin*>(p.Bm);
   const Tin* __restrict__ gC = static_cast<const Tin*>(p.Cm);
   float* red = s_red + wave * 64 * RED_RS;

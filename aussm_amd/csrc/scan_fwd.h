@@ -28,6 +28,7 @@ struct FwdArgs {
   int ld, ns;                // matrix-core unitary kernels: row stride of the [.., L] tensors and segments per
                              // sequence (B then counts batch x segment pairs and L is the segment length)
   int hs, ho;                // ... and h0 of pair b is entry b * hs + ho of the state array
+  int urep;                  // generic kernels: u and delta are [B / urep, D, L], shared by urep consecutive batch elements
 };
 
 // VAR: variant.  NW: states per wavefront.  NT: threads per workgroup.  Tin: float or bf16_t.
@@ -53,8 +54,11 @@ __global__ __launch_bounds__(NT) void core_fwd_kernel(const FwdArgs p) {
   const int d = d0 + lane;
   const bool dok = d < D;
 
-  const Tin* __restrict__ gu = static_cast<const Tin*>(p.u);
-  const Tin* __restrict__ gdl = static_cast<const Tin*>(p.delta);
+  // u and delta may be shared by p.urep consecutive batch elements (tensors [B / urep, D, L]): every
+  // address below is formed for batch element b, so their base steps back by the difference
+  const size_t uback = (size_t)(b - b / p.urep) * p.D * p.L;
+  const Tin* __restrict__ gu = static_cast<const Tin*>(p.u) - uback;
+  const Tin* __restrict__ gdl = static_cast<const Tin*>(p.delta) - uback;
   const Tin* __restrict__ gB = static_cast<const Tin*>(p.Bm);
   const Tin* __restrict__ gC = static_cast<const Tin*>(p.Cm);
 

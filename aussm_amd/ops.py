@@ -74,12 +74,12 @@ def _composite(u, dt, x, x_bias, B_r, B_theta, C_r, C_theta, D, z, h_r, h_i):
     xm = x.permute(1, 0, 2).reshape(n * d, d)                          # (j i) x r
     theta = torch.matmul(xm, u).view(b, n, d, l) + x_bias.t()[None, :, :, None]
     us = F.silu(u)
-    rep = lambda t: t[:, None].expand(b, n, d, l).reshape(b * n, d, l)
     Bt = torch.polar(B_r, B_theta)                                     # (n,)
     Ct = torch.polar(C_r, C_theta)
     row = lambda c: c[None, :, None].expand(b, n, l).reshape(b * n, 1, l)
     h0 = torch.complex(h_r, h_i).permute(0, 2, 1).reshape(b * n, d, 1)
-    y, hL = scan.unitary_scan(rep(us), rep(dt), theta.reshape(b * n, d, l), row(Bt), row(Ct), None, None, h0,
+    # us, dt stay (b, d, l): each of their batch elements serves the n consecutive (batch, state) pairs
+    y, hL = scan.unitary_scan(us, dt.contiguous(), theta.reshape(b * n, d, l), row(Bt), row(Ct), None, None, h0,
                               return_last_state=True)
     y = y.view(b, n, d, l).sum(dim=1)
     y = (y + us * D[None, :, None]) * F.silu(z)

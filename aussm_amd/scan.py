@@ -105,9 +105,12 @@ def unitary_aux(u, n: int, ck: int) -> Tensor:
 
 def unitary_fwd_raw(u, delta, theta, Bri, Cri, D=None, z=None, h0=None, want_state=False, ck=0, aux=None):
     """Launch aussm_unitary_fwd(_aux).  Bri/Cri are real views (b, n, l, 2).  Returns (y, hL, hck);
-    hL is (b, d, n, 2) or None, hck is the checkpoint tensor when ck > 0."""
+    hL is (b, d, n, 2) or None, hck is the checkpoint tensor when ck > 0.  u and delta may have a
+    batch size that divides theta's: each of their batch elements then serves that many
+    consecutive ones of theta."""
     lib = _lib.load()
-    b, d, l = u.shape
+    b, d, l = theta.shape
+    urep = b // u.shape[0]
     n = Bri.shape[1]
     y = torch.empty((b, d, l), device=u.device, dtype=torch.float32)
     hL = torch.empty((b, d, n, 2), device=u.device, dtype=torch.float32) if want_state else None
@@ -116,14 +119,17 @@ def unitary_fwd_raw(u, delta, theta, Bri, Cri, D=None, z=None, h0=None, want_sta
         hck = torch.empty((b, num_checkpoints(l, ck), n, 2, d), device=u.device, dtype=torch.float32)
     check(lib.aussm_unitary_fwd_aux(ptr(u), ptr(delta), ptr(theta), ptr(Bri), ptr(Cri), ptr(D), ptr(z), ptr(h0),
                                     ptr(y), ptr(hL), ptr(hck), ptr(aux), b, d, n, l, ck or _lib.TILE, _in_dtype(u),
-                                    _stream()),
+                                    urep, _stream()),
           "aussm_unitary_fwd_aux")
     return y, hL, hck
 
 
 def unitary_bwd_raw(dy, dhL, u, delta, theta, Bri, Cri, D, hck, ck, want_dD=True, want_dh0=False, aux=None):
+    """Gradients; du and ddelta come back per batch element of theta (b, d, l) also when u and delta
+    are shared by several of them (the caller adds them up)."""
     lib = _lib.load()
-    b, d, l = u.shape
+    b, d, l = theta.shape
+    urep = b // u.shape[0]
     n = Bri.shape[1]
     f32 = dict(device=u.device, dtype=torch.float32)
     du, ddelta, dtheta = (torch.empty((b, d, l), **f32) for _ in range(3))
@@ -134,7 +140,7 @@ def unitary_bwd_raw(dy, dhL, u, delta, theta, Bri, Cri, D, hck, ck, want_dD=True
     dh0 = torch.empty((b, d, n, 2), **f32) if want_dh0 else None
     check(lib.aussm_unitary_bwd_aux(ptr(dy), ptr(dhL), ptr(u), ptr(delta), ptr(theta), ptr(Bri), ptr(Cri), ptr(D),
                                     ptr(hck), ptr(aux), ptr(du), ptr(ddelta), ptr(dtheta), ptr(dB), ptr(dC), ptr(dD),
-                                    ptr(dh0), b, d, n, l, ck, _in_dtype(u), _stream()),
+                                    ptr(dh0), b, d, n, l, ck, _in_dtype(u), urep, _stream()),
           "aussm_unitary_bwd_aux")
     return du, ddelta, dtheta, dB, dC, dD, dh0
 
@@ -148,7 +154,7 @@ class _UnitaryScanFn(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, u, delta, theta, Bri, Cri, D, h0):
-        aux = unitary_aux(u, Bri.shape[1], UNITARY_CK)
+        aux = unitary_aux(theta, Bri.shape[1], UNITARY_CK)
         y, hL, hck = unitary_fwd_raw(u, delta, theta, Bri, Cri, D, None, h0, want_state=True, ck=UNITARY_CK, aux=aux)
         ctx.save_for_backward(u, delta, theta, Bri, Cri, D, hck, aux)
         ctx.has_h0 = h0 is not None
@@ -163,6 +169,9 @@ class _UnitaryScanFn(torch.autograd.Function):
             dy, dhL, u, delta, theta, Bri, Cri, D, hck, UNITARY_CK,
             want_dD=D is not None and ctx.needs_input_grad[5], want_dh0=ctx.has_h0 and ctx.needs_input_grad[6],
             aux=aux)
+        if u.shape[0] != theta.shape[0]:             # u, delta shared by consecutive batch elements
+            du = du.view(u.shape[0], -1, *u.shape[1:]).sum(dim=1)
+            ddelta = ddelta.view(u.shape[0], -1, *u.shape[1:]).sum(dim=1)
         return (du.to(u.dtype), ddelta.to(delta.dtype), dtheta, dB.to(Bri.dtype), dC.to(Cri.dtype), dD, dh0)
 
 
@@ -170,10 +179,15 @@ def unitary_scan(u: Tensor, delta: Tensor, theta: Tensor, Bc: Tensor, Cc: Tensor
                  z: Optional[Tensor] = None, h0: Optional[Tensor] = None, return_last_state: bool = False):
     """Adaptive-unitary scan.  u, delta, theta, z: (b, d, l); Bc, Cc: (b, n, l) complex64 (or
     (b, n, l, 2) real); D: (d,); h0: (b, d, n) complex64.  Returns y (b, d, l) float32, and the final
-    state (b, d, n) complex64 if return_last_state."""
-    b, d, l = _check_bdl(u, delta)
+    state (b, d, n) complex64 if return_last_state.  u and delta may be (b / r, d, l): batch element i
+    of theirs then serves the r consecutive batch elements i r .. i r + r - 1 of everything else
+    (one input, r phase sequences)."""
+    bu, d, l = _check_bdl(u, delta)
     u = u.contiguous()
     delta = delta.contiguous()
+    b = theta.shape[0] if theta.dim() == 3 else bu
+    if b % bu != 0:
+        raise RuntimeError(f"batch size of theta ({b}) must be a multiple of that of u ({bu})")
     theta = _f32(theta, "theta", (b, d, l))
     Bri = _complex_as_real(Bc, "B", b, l, u.dtype)
     Cri = _complex_as_real(Cc, "C", b, l, u.dtype)

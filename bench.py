@@ -128,12 +128,12 @@ def main():
     def fwd_only():
         scan.check(lib.aussm_unitary_fwd_aux(ptr(p["u"]), ptr(p["delta"]), ptr(p["theta"]), ptr(Bri), ptr(Cri),
                                              ptr(p["Dskip"]), None, None, ptr(y), None, ptr(hck), ptr(aux),
-                                             B, D, N, L, ck, 0, stream), "fwd")
+                                             B, D, N, L, ck, 0, 1, stream), "fwd")
 
     def bwd_only():
         scan.check(lib.aussm_unitary_bwd_aux(ptr(p["dy"]), None, ptr(p["u"]), ptr(p["delta"]), ptr(p["theta"]), ptr(Bri),
                                              ptr(Cri), ptr(p["Dskip"]), ptr(hck), ptr(aux), ptr(du), ptr(ddl), ptr(dth),
-                                             ptr(dB), ptr(dC), ptr(dD), None, B, D, N, L, ck, 0, stream), "bwd")
+                                             ptr(dB), ptr(dC), ptr(dD), None, B, D, N, L, ck, 0, 1, stream), "bwd")
 
     def kernel_us(fn, reps):
         evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]

@@ -112,6 +112,11 @@ int aussm_unitary_bwd(const float* dy, const float* dhL,
  *    ssm_adaptive_unitary_forward.cu:122-162 one level up); the segment states live behind the
  *    per-(b,d,l) part of the buffer, during the call only.  Each call writes there: two calls
  *    that share one buffer must not overlap.  AUSSM_SPLIT=0 (environment) switches the split off.
+ * urep (>= 1, divides B): u and delta are [B / urep, D, L] and shared by urep consecutive batch
+ * elements (theta, z, y, dy and every gradient stay [B, D, L]).  This is how the drop-in operator
+ * runs its n states per channel, each with its own phase, as n batch elements of one launch without
+ * replicating its inputs (the reference loops over the state inside one thread block,
+ * ssm_adaptive_unitary_forward.cu:57-181).  urep > 1 takes the vector-ALU kernels.
  * No counterpart in the reference (its backward kernel recomputes,
  * ssm_adaptive_unitary_backward.cu:113-181, and its launches cover at most 2048 steps). */
 size_t aussm_unitary_aux_floats(int B, int D, int N, int L, int ck);
@@ -119,7 +124,7 @@ size_t aussm_unitary_aux_floats(int B, int D, int N, int L, int ck);
 int aussm_unitary_fwd_aux(const void* u, const void* delta, const float* theta,
                           const void* Bc, const void* Cc, const float* Dskip, const float* z,
                           const float* h0, float* y, float* hL, float* hck, float* aux,
-                          int B, int D, int N, int L, int ck, int in_dtype, void* stream);
+                          int B, int D, int N, int L, int ck, int in_dtype, int urep, void* stream);
 
 int aussm_unitary_bwd_aux(const float* dy, const float* dhL,
                           const void* u, const void* delta, const float* theta,
@@ -127,7 +132,7 @@ int aussm_unitary_bwd_aux(const float* dy, const float* dhL,
                           float* aux,
                           float* du, float* ddelta, float* dtheta, float* dB, float* dC,
                           float* dD, float* dh0,
-                          int B, int D, int N, int L, int ck, int in_dtype, void* stream);
+                          int B, int D, int N, int L, int ck, int in_dtype, int urep, void* stream);
 
 /* ---------------------------------------------------------------------------------------
  * Complex scan:  a_l = exp(rho_l[b,d] + i*theta_l[b,d]), otherwise as the unitary scan.

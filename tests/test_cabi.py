@@ -71,11 +71,17 @@ def test_argument_checks_without_a_device():
     assert lib.aussm_unitary_aux_floats(4, 256, 16, 16384 + 4, 256) == 4 * 256 * (16384 + 4) + 64
     assert lib.aussm_unitary_aux_floats(4, 256, 4, 16384, 256) == 4 * 256 * 16384 + 64
     rc = lib.aussm_unitary_fwd_aux(one, one, one, one, one, null, null, null, one, null, null, ctypes.c_void_p(260),
-                                   1, 1, 1, 32, 32, 0, null)
+                                   1, 1, 1, 32, 32, 0, 1, null)
     assert rc == -5
     rc = lib.aussm_unitary_fwd_aux(null, one, one, one, one, null, null, null, one, null, null, null,
-                                   1, 1, 1, 32, 32, 0, null)
+                                   1, 1, 1, 32, 32, 0, 1, null)
     assert rc == -1
+    # u / delta shared by urep consecutive batch elements: urep must divide B
+    rc = lib.aussm_unitary_fwd_aux(one, one, one, one, one, null, null, null, one, null, null, null,
+                                   3, 1, 1, 32, 32, 0, 2, null)
+    assert rc == -2
+    rc = lib.aussm_unitary_bwd_aux(*([one] * 17), 3, 1, 1, 32, 32, 0, 0, null)
+    assert rc == -2
     # the recomputing backward kernels insist on their checkpoint interval and state limit
     args = [one] * 9 + [0] + [one] * 9
     assert lib.aussm_real_bwd(*args, 1, 1, 1, 32, 32, 0, null) == -3

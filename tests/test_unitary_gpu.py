@@ -96,3 +96,32 @@ def test_rejects_bad_arguments():
     big = _dev(O.make_core_inputs(1, 4, 65, 8))
     with pytest.raises(RuntimeError):
         scan.unitary_scan(big["u"], big["delta"], big["theta"], big["Bc"], big["Cc"])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("b,r,d,n,l", [(2, 3, 70, 1, 52), (1, 4, 33, 2, 37), (3, 2, 64, 1, 128)])
+def test_inputs_shared_by_consecutive_batch_elements(b, r, d, n, l):
+    """u and delta of batch size b serve b * r phase sequences (how the drop-in operator runs its
+    states): outputs and gradients equal those of the call with u and delta replicated, and the
+    gradients of u and delta are the sums over the r users."""
+    from aussm_amd import scan
+    p = O.make_core_inputs(b * r, d, n, l, seed=b + r + l)
+    u, delta = p["u"][::r].contiguous(), p["delta"][::r].contiguous()
+    dev = "cuda"
+
+    def run(fn, uu, dd, device):
+        lv = [t.clone().to(device).requires_grad_(True) for t in (uu, dd, p["theta"], p["Bc"], p["Cc"], p["Dskip"])]
+        y = fn(*lv)
+        (y * p["dy"].to(device)).sum().backward()
+        return [y.detach()] + [t.grad for t in lv]
+
+    rep = lambda t: t[:, None].expand(b, r, d, l).reshape(b * r, d, l)
+    want = run(lambda uu, dd, *a: O.unitary_core_loop(rep(uu), rep(dd), *a)[0], u, delta, "cpu")
+    print(f"case shared inputs b={b} r={r} d={d} n={n} l={l}", flush=True)
+    got = run(scan.unitary_scan, u, delta, dev)
+    torch.cuda.synchronize()
+    for name, w, g in zip(("y", "du", "ddelta", "dtheta", "dB", "dC", "dD"), want, got):
+        if w.is_complex():
+            w, g = torch.view_as_real(w), torch.view_as_real(g)
+        scale = max(1.0, float(w.abs().max()))
+        torch.testing.assert_close(g.cpu() / scale, w / scale, atol=1e-4, rtol=1e-4, msg=lambda m: f"{name}: {m}")
