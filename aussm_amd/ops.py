@@ -72,7 +72,9 @@ def _composite(u, dt, x, x_bias, B_r, B_theta, C_r, C_theta, D, z, h_r, h_i):
     b, d, n, l = _check_op_inputs((u, dt, x, x_bias, B_r, B_theta, C_r, C_theta, D, z, h_r, h_i))
     # phase projection: theta[b, j, i, l]  (state index before channel so that (b, j) is a batch)
     xm = x.permute(1, 0, 2).reshape(n * d, d)                          # (j i) x r
-    theta = torch.matmul(xm, u).view(b, n, d, l) + x_bias.t()[None, :, :, None]
+    # one strided-batched GEMM straight into (b, (j i), l); the 2-D x 3-D form of matmul goes through
+    # transposed copies of the whole phase tensor
+    theta = torch.baddbmm(x_bias.t().reshape(1, n * d, 1), xm.unsqueeze(0).expand(b, n * d, d), u).view(b, n, d, l)
     us = F.silu(u)
     Bt = torch.polar(B_r, B_theta)                                     # (n,)
     Ct = torch.polar(C_r, C_theta)
