@@ -37,6 +37,7 @@ _SIGNATURES = {
     "aussm_real_bwd": [_P] * 9 + [_I] + [_P] * 9 + [_I] * 6 + [_P],
     "aussm_causal_conv1d_fwd": [_P] * 4 + [_I] * 4 + [_LL] * 2 + [_P],
     "aussm_causal_conv1d_bwd": [_P] * 6 + [_I] * 4 + [_LL] * 2 + [_P],
+    "aussm_swap_last2": [_P] * 2 + [_I] * 3 + [_LL] * 2 + [_P],
 }
 
 EXPORTED = tuple(_SIGNATURES) + ("aussm_error_string", "aussm_unitary_aux_floats")

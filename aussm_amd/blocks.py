@@ -38,6 +38,14 @@ def _causal_conv(conv1d: nn.Conv1d, x: torch.Tensor, l: int) -> torch.Tensor:
     return conv1d(x.transpose(1, 2))[:, :, :l].transpose(1, 2)
 
 
+def _swap(x: torch.Tensor) -> torch.Tensor:
+    """Contiguous copy with the last two dimensions swapped: (b, l, d) <-> (b, d, l), the
+    `rearrange` calls around the scans (ai-modules/wavesAI/model/aussm.py:760-803, :861-900)."""
+    if x.is_cuda and x.dtype == torch.float32:
+        return conv.swap_last2(x)
+    return x.transpose(1, 2).contiguous()
+
+
 @dataclass
 class ModelArgsSSMau:
     d_model: int
@@ -124,18 +132,18 @@ class MambaBlock(nn.Module):
         x = F.silu(x)
         A = -torch.exp(self.A_log.float())
         y = self.scan_impl(
-            x.transpose(1, 2).contiguous(),
-            dt.transpose(1, 2).contiguous(),
+            _swap(x),
+            _swap(dt),
             A.contiguous(),
-            B.transpose(1, 2).contiguous(),
-            C.transpose(1, 2).contiguous(),
+            _swap(B),
+            _swap(C),
             self.D.float().contiguous(),
-            z=z.transpose(1, 2).contiguous(),
+            z=_swap(z),
             delta_bias=self.dt_proj.bias.float(),
             delta_softplus=True,
             return_last_state=False,
         )
-        return y.transpose(1, 2)
+        return _swap(y)
 
 
 class SSMauBlock(nn.Module):
@@ -183,17 +191,17 @@ class SSMauBlock(nn.Module):
         x_param = self.xA_proj.weight.view(n, d_in, d_in).permute(1, 0, 2)
         x_bias = self.xA_proj.bias.view(n, d_in).t()
         self.ssm_args = {
-            "u": x.transpose(1, 2).contiguous(),
-            "dt": dt.transpose(1, 2).contiguous(),
+            "u": _swap(x),
+            "dt": _swap(dt),
             "x": x_param.contiguous() * (1 / math.sqrt(self.args.d_model)),
             "x_bias": x_bias.contiguous(),
             "B": self.B.contiguous(),
             "C": self.C.contiguous(),
             "D": self.D.float().contiguous(),
-            "z": z.transpose(1, 2).contiguous(),
+            "z": _swap(z),
         }
         y = self.optimized_SSMa_function(**self.ssm_args)
-        return y.transpose(1, 2)
+        return _swap(y)
 
 
 class ResidualBlock(nn.Module):

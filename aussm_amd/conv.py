@@ -17,7 +17,7 @@ from torch import Tensor
 from . import _lib
 from ._lib import check, ptr
 
-__all__ = ["causal_conv1d"]
+__all__ = ["causal_conv1d", "swap_last2"]
 
 
 def _stream() -> int:
@@ -72,3 +72,32 @@ def causal_conv1d(x: Tensor, weight: Tensor, bias: Optional[Tensor] = None) -> T
     if weight.shape[0] != x.shape[2] or weight.numel() != x.shape[2] * weight.shape[-1]:
         raise ValueError(f"weight {tuple(weight.shape)} does not fit {x.shape[2]} channels")
     return _CausalConv1dFn.apply(x, weight, bias)
+
+
+class _SwapLast2Fn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x):
+        return _swap_last2(x)
+
+    @staticmethod
+    def backward(ctx, dy):
+        return _swap_last2(dy)
+
+
+def _swap_last2(x: Tensor) -> Tensor:
+    lib = _lib.load()
+    b, r, c = x.shape
+    xr = _rows(x)
+    y = torch.empty((b, c, r), device=x.device, dtype=torch.float32)
+    check(lib.aussm_swap_last2(ptr(xr), ptr(y), b, r, c, xr.stride(0), xr.stride(1), _stream()), "aussm_swap_last2")
+    return y
+
+
+def swap_last2(x: Tensor) -> Tensor:
+    """Contiguous (b, c, r) copy of x (b, r, c) on the GPU: `x.transpose(1, 2).contiguous()` between
+    the blocks' (b, l, d) activations and the scans' (b, d, l) tensors, through LDS tiles."""
+    if x.dim() != 3 or not x.is_cuda:
+        raise ValueError("swap_last2 expects a (b, r, c) tensor on the GPU")
+    if x.shape[0] > 65535:
+        return x.transpose(1, 2).contiguous()
+    return _SwapLast2Fn.apply(x)

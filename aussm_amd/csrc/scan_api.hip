@@ -7,6 +7,7 @@
 #include <stdlib.h>
 
 #include "conv1d.h"
+#include "layout.h"
 #include "scan_bwd_recompute.h"
 #include "scan_bwd_unitary.h"
 #include "scan_bwd_xdl.h"
@@ -434,6 +435,16 @@ int aussm_causal_conv1d_bwd(const float* dy, const float* x, const float* w, flo
   hipLaunchKernelGGL(causal_conv1d_bwd_data_kernel, dim3((unsigned)rows, (unsigned)((D + 255) / 256)), dim3(256), 0, s, a);
   hipLaunchKernelGGL(causal_conv1d_bwd_weight_kernel,
                      dim3((unsigned)((D + 63) / 64), (unsigned)((rows + CONV_ROWS - 1) / CONV_ROWS)), dim3(256), 0, s, a);
+  return launch_status();
+}
+
+int aussm_swap_last2(const float* x, float* y, int B, int R, int C, long long xs_b, long long xs_r, void* stream) {
+  if (B < 1 || R < 1 || C < 1 || B > 65535 || xs_r < C || xs_b < (long long)R * xs_r - (xs_r - C)) return AUSSM_E_SHAPE;
+  if ((R + 31) / 32 > 65535) return AUSSM_E_SHAPE;
+  if (!x || !y) return AUSSM_E_NULL;
+  SwapArgs a{x, y, xs_b, xs_r, R, C};
+  hipLaunchKernelGGL(swap_last2_kernel, dim3((unsigned)((C + 31) / 32), (unsigned)((R + 31) / 32), (unsigned)B), dim3(256), 0,
+                     (hipStream_t)stream, a);
   return launch_status();
 }
 

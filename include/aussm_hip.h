@@ -195,6 +195,14 @@ int aussm_causal_conv1d_bwd(const float* dy, const float* x, const float* w,
                             float* dx, float* dw, float* dbias,
                             int B, int L, int D, int K, long long xs_b, long long xs_l, void* stream);
 
+/* y[b, c, r] = x[b, r, c]: the layout change between the blocks' channels-last activations
+ * (b, l, d) and the scans' (b, d, l) tensors - `rearrange(x, 'b l d -> b d l')` and its inverse,
+ * ai-modules/wavesAI/model/aussm.py:760-803 and :861-900.  Element (b, r, c) of x is
+ * x[b*xs_b + r*xs_r + c] (a column slice of a wider tensor is fine), y is contiguous (B, C, R).
+ * B <= 65535. */
+int aussm_swap_last2(const float* x, float* y, int B, int R, int C,
+                     long long xs_b, long long xs_r, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -21,7 +21,7 @@ def test_header_declares_the_expected_entry_points():
     for must in ("aussm_unitary_fwd", "aussm_unitary_bwd", "aussm_complex_fwd", "aussm_complex_bwd",
                  "aussm_real_fwd", "aussm_real_bwd", "aussm_version", "aussm_error_string",
                  "aussm_unitary_fwd_aux", "aussm_unitary_bwd_aux", "aussm_unitary_aux_floats",
-                 "aussm_causal_conv1d_fwd", "aussm_causal_conv1d_bwd"):
+                 "aussm_causal_conv1d_fwd", "aussm_causal_conv1d_bwd", "aussm_swap_last2"):
         assert must in names
 
 

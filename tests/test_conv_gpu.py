@@ -51,3 +51,20 @@ def test_causal_conv_without_bias_and_rejections():
         conv.causal_conv1d(x, w[:5], None)
     with pytest.raises(Exception):
         conv.causal_conv1d(x, torch.randn(6, 1, 9, device="cuda"), None)     # K > 8 is rejected by the library
+
+
+@pytest.mark.parametrize("b,r,c,sliced", [(2, 37, 70, False), (3, 720, 256, True), (1, 1, 5, False), (2, 33, 31, True)])
+def test_swap_last2_matches_transpose(b, r, c, sliced):
+    from aussm_amd import conv
+    g = torch.Generator().manual_seed(r + c)
+    wide = torch.randn(b, r, 2 * c, generator=g).cuda().requires_grad_(True)
+    x = wide[:, :, c:] if sliced else wide[:, :, :c].contiguous()
+    print(f"case swap b={b} r={r} c={c} sliced={sliced}", flush=True)
+    y = conv.swap_last2(x)
+    assert y.is_contiguous() and y.shape == (b, c, r)
+    assert torch.equal(y, x.transpose(1, 2))
+    dy = torch.randn(b, c, r, generator=g).cuda()
+    (gx,) = torch.autograd.grad(y, wide, dy)
+    want = torch.zeros_like(wide)
+    (want[:, :, c:] if sliced else want[:, :, :c]).copy_(dy.transpose(1, 2))
+    assert torch.equal(gx, want)
