@@ -166,7 +166,7 @@ def pad_to_multiple_of(tensor: Tensor, multiple_of: int) -> Tensor:
 
 def ssm_adaptive_interface(u: Tensor, dt: Tensor, x: Tensor, x_bias: Tensor, B: Tensor, C: Tensor, D: Tensor,
                            z: Tensor, unitary: bool = True, preal: bool = False,
-                           max_parallel_length: int = 2048, **kwargs) -> Tensor:
+                           max_parallel_length: int = 2048, save_intermediates: bool = True, **kwargs) -> Tensor:
     """Front-end of the adaptive-unitary operator (ops.py:28-93).
 
     u, dt, z: (b, d, l) float32; x: (d, n, d); x_bias: (d, n); B, C: (n,) complex64; D: (d,).
@@ -176,6 +176,11 @@ def ssm_adaptive_interface(u: Tensor, dt: Tensor, x: Tensor, x_bias: Tensor, B: 
     from zero, exactly as the reference does; unknown keyword arguments are ignored as there.
     (The reference zero-pads the sequence to a multiple of 16 for its kernel; this kernel takes
     any length, and the padded steps never influence the returned y.)
+
+    save_intermediates (not in the reference): True keeps the phase tensor (b, n, d, l) and the
+    scan's checkpoints for the backward pass; False goes through the dispatcher operator, whose
+    backward pass keeps only the twelve inputs and recomputes, as the reference's does
+    (ops.py:148-151) - less memory, one more phase projection and forward scan per step.
     """
     assert not (unitary and preal), "Both unitary and preal cannot be used at the same time"
     if not unitary:
@@ -193,8 +198,9 @@ def ssm_adaptive_interface(u: Tensor, dt: Tensor, x: Tensor, x_bias: Tensor, B: 
     outs = []
     for s in range(0, l, max_parallel_length):
         e = min(s + max_parallel_length, l)
-        y, h_r, h_i = ssm_adaptive_unitary(u[:, :, s:e].contiguous(), dt[:, :, s:e].contiguous(), x.contiguous(),
-                                           x_bias.contiguous(), B_r, B_theta, C_r, C_theta, D.contiguous(),
-                                           z[:, :, s:e].contiguous(), h_r, h_i)
+        op = _composite if save_intermediates else ssm_adaptive_unitary
+        y, h_r, h_i = op(u[:, :, s:e].contiguous(), dt[:, :, s:e].contiguous(), x.contiguous(),
+                         x_bias.contiguous(), B_r, B_theta, C_r, C_theta, D.contiguous(),
+                         z[:, :, s:e].contiguous(), h_r, h_i)
         outs.append(y)
     return outs[0] if len(outs) == 1 else torch.cat(outs, dim=-1)

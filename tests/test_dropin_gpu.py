@@ -34,19 +34,20 @@ def test_correctness_unitary(chunk, l):
     torch.testing.assert_close(result.cpu(), O.adaptive_unitary_loop(*args), atol=7e-5, rtol=5e-5)
 
 
+@pytest.mark.parametrize("save", [True, False])     # keep intermediates / recompute in the dispatcher operator
 @pytest.mark.parametrize("chunk", [2048, 5])
-def test_gradients_unitary(chunk):
+def test_gradients_unitary(chunk, save):
     from aussm_amd import ops
     args = O.make_adaptive_inputs()
     g = torch.Generator().manual_seed(11)
     y_random = torch.randn(args[0].shape, generator=g)
-    print(f"case drop-in bwd chunk={chunk}", flush=True)
+    print(f"case drop-in bwd chunk={chunk} save={save}", flush=True)
 
     ref = [a.clone().requires_grad_(True) for a in args]
     torch.mean((O.adaptive_unitary_polar(*ref) - y_random) ** 2).backward()
 
     dev = [a.clone().cuda().requires_grad_(True) for a in args]
-    y = ops.ssm_adaptive_interface(*dev, unitary=True, max_parallel_length=chunk)
+    y = ops.ssm_adaptive_interface(*dev, unitary=True, max_parallel_length=chunk, save_intermediates=save)
     torch.mean((y - y_random.cuda()) ** 2).backward()
 
     for name, r, d in zip(NAMES, ref, dev):
