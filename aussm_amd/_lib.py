@@ -14,6 +14,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "libaussm_hip.so")
 
 F32, BF16 = 0, 1
 TILE = 32
+AUX_PAD = 64          # floats between the per-(b,d,l) part of the auxiliary buffer and the segment states
 MAX_STATE = 64
 
 _lib = None

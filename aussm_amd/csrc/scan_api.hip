@@ -152,7 +152,7 @@ int launch_fwd(FwdArgs a, int in_dtype, hipStream_t s) {
   if (a.aux && mode <= 1)   // this call will not fill the auxiliary buffer
     hipLaunchKernelGGL(aux_invalidate_kernel, dim3(1), dim3(1), 0, s, a.aux + (size_t)a.B * a.D * a.L);
   if (mode) {
-    if ((mode == 2 || mode == 3) && a.aux && a.hck) {
+    if ((mode == 2 || mode == 3) && a.aux) {
       const int ns = seg_count(a.B, a.D, a.N, a.L, a.ck);
       if (ns > 1) {
         // 1. end state of every segment from a zero start and its rotation; 2. chain them;

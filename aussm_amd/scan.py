@@ -208,7 +208,12 @@ def unitary_scan(u: Tensor, delta: Tensor, theta: Tensor, Bc: Tensor, Cc: Tensor
         if z is not None:
             y = y * F.silu(z)
     else:
-        y, hL, _ = unitary_fwd_raw(u, delta, theta, Bri, Cri, D, z, h0r, want_state=return_last_state)
+        # no backward pass: the auxiliary buffer is only worth allocating when the launch would be split along L
+        lib = _lib.load()
+        split = lib.aussm_unitary_aux_floats(b, d, n, l, UNITARY_CK) > b * d * l + _lib.AUX_PAD
+        aux = unitary_aux(theta, n, UNITARY_CK) if (split and u.shape[0] == b) else None
+        y, hL, _ = unitary_fwd_raw(u, delta, theta, Bri, Cri, D, z, h0r, want_state=return_last_state,
+                                   ck=UNITARY_CK if aux is not None else 0, aux=aux)
     if return_last_state:
         return y, torch.view_as_complex(hL)
     return y

@@ -248,3 +248,25 @@ def test_random_shapes_inputs_and_checkpoint_intervals(seed):
         _close(gt, w, f"d{k}")
     if carried:
         _close(torch.view_as_complex(dh0), h0l.grad, "dh0")
+
+
+def test_forward_only_call_takes_the_split_too():
+    """Without a backward pass unitary_scan allocates the auxiliary buffer only when the launch is
+    split along L (BASELINE configuration 1 is such a call): same outputs as with the split off."""
+    from aussm_amd import scan
+    B, D, N, L = 2, 64, 16, 1024
+    p = _inputs(B, D, N, L, 77, big_theta=False)
+    q = {k: v.cuda() for k, v in p.items()}
+    want_y, want_h = O.unitary_core_loop(p["u"], p["delta"], p["theta"], p["Bc"], p["Cc"], p["Dskip"], p["z"], p["h0"])
+    print("case forward-only split", flush=True)
+    with torch.no_grad():
+        y, hL = scan.unitary_scan(q["u"], q["delta"], q["theta"], q["Bc"], q["Cc"], q["Dskip"], q["z"], q["h0"],
+                                  return_last_state=True)
+        with _Env(AUSSM_SPLIT="0"):
+            y0, hL0 = scan.unitary_scan(q["u"], q["delta"], q["theta"], q["Bc"], q["Cc"], q["Dskip"], q["z"], q["h0"],
+                                        return_last_state=True)
+    torch.cuda.synchronize()
+    _close(y, want_y, "y")
+    _close(hL, want_h, "hL")
+    _close(y, y0.cpu(), "y split vs whole", tol=2e-5)
+    assert not torch.equal(y, y0), "the split should have changed the association order"
