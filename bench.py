@@ -86,7 +86,6 @@ def main():
 
     import torch
     from aussm_amd import scan
-    from oracle import scan_oracle as O
 
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
@@ -94,7 +93,14 @@ def main():
     B, D, N, L = SHAPE["B"], SHAPE["D"], SHAPE["N"], SHAPE["L"]
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    p = {k: v.to(dev) for k, v in O.make_core_inputs(B, D, N, L, seed=0).items()}
+    # synthetic inputs with BASELINE's value distributions, generated on the device (the CPU oracle is only
+    # used by the cpu_baseline leg): u ~ N(0,1), delta = softplus(N(0,1)), theta ~ N(0, 0.5), B_t and C_t complex
+    # with parts ~ N(0, 1/sqrt(N)), D ~ N(0,1), dy ~ N(0,1)
+    g = torch.Generator(device=dev).manual_seed(0)
+    rn = lambda *shape: torch.randn(*shape, generator=g, device=dev)
+    p = {"u": rn(B, D, L), "delta": torch.nn.functional.softplus(rn(B, D, L)), "theta": rn(B, D, L) * 0.5,
+         "Bc": torch.complex(rn(B, N, L), rn(B, N, L)) * N ** -0.5, "Cc": torch.complex(rn(B, N, L), rn(B, N, L)) * N ** -0.5,
+         "Dskip": rn(D), "dy": rn(B, D, L)}
     Bri = torch.view_as_real(p["Bc"]).contiguous()
     Cri = torch.view_as_real(p["Cc"]).contiguous()
     ck = scan.UNITARY_CK
