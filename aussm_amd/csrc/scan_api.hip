@@ -416,8 +416,13 @@ int aussm_causal_conv1d_fwd(const float* x, const float* w, const float* bias, f
   a.x = x; a.w = w; a.bias = bias; a.y = y; a.xs_b = xs_b; a.xs_l = xs_l; a.B = B; a.L = L; a.D = D; a.K = K;
   const size_t rows = (size_t)B * L;
   if (rows > 0x7fffffffULL || (D + 255) / 256 > 65535) return AUSSM_E_SHAPE;
-  hipLaunchKernelGGL(causal_conv1d_fwd_kernel, dim3((unsigned)rows, (unsigned)((D + 255) / 256)), dim3(256), 0,
-                     (hipStream_t)stream, a);
+  const size_t runs = (size_t)B * ((L + CONV_RUN - 1) / CONV_RUN);
+  if (K == 4)
+    hipLaunchKernelGGL(causal_conv1d_k4_fwd_kernel, dim3((unsigned)runs, (unsigned)((D + 255) / 256)), dim3(256), 0,
+                       (hipStream_t)stream, a);
+  else
+    hipLaunchKernelGGL(causal_conv1d_fwd_kernel, dim3((unsigned)rows, (unsigned)((D + 255) / 256)), dim3(256), 0,
+                       (hipStream_t)stream, a);
   return launch_status();
 }
 
@@ -432,9 +437,15 @@ int aussm_causal_conv1d_bwd(const float* dy, const float* x, const float* w, flo
   const size_t rows = (size_t)B * L;
   if (rows > 0x7fffffffULL || (D + 255) / 256 > 65535 || (rows + CONV_ROWS - 1) / CONV_ROWS > 65535) return AUSSM_E_SHAPE;
   hipStream_t s = (hipStream_t)stream;
-  hipLaunchKernelGGL(causal_conv1d_bwd_data_kernel, dim3((unsigned)rows, (unsigned)((D + 255) / 256)), dim3(256), 0, s, a);
-  hipLaunchKernelGGL(causal_conv1d_bwd_weight_kernel,
-                     dim3((unsigned)((D + 63) / 64), (unsigned)((rows + CONV_ROWS - 1) / CONV_ROWS)), dim3(256), 0, s, a);
+  const dim3 wgrid((unsigned)((D + 63) / 64), (unsigned)((rows + CONV_ROWS - 1) / CONV_ROWS));
+  if (K == 4) {
+    const size_t runs = (size_t)B * ((L + CONV_RUN - 1) / CONV_RUN);
+    hipLaunchKernelGGL(causal_conv1d_k4_bwd_data_kernel, dim3((unsigned)runs, (unsigned)((D + 255) / 256)), dim3(256), 0, s, a);
+    hipLaunchKernelGGL(causal_conv1d_k4_bwd_weight_kernel, wgrid, dim3(256), 0, s, a);
+  } else {
+    hipLaunchKernelGGL(causal_conv1d_bwd_data_kernel, dim3((unsigned)rows, (unsigned)((D + 255) / 256)), dim3(256), 0, s, a);
+    hipLaunchKernelGGL(causal_conv1d_bwd_weight_kernel, wgrid, dim3(256), 0, s, a);
+  }
   return launch_status();
 }
 
