@@ -95,7 +95,8 @@ class RMSNorm(nn.Module):
         self.weight = nn.Parameter(torch.ones(d_model))
 
     def forward(self, x):
-        return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + self.eps) * self.weight
+        # x * rsqrt(mean(x^2) + eps) * weight (ai-modules/wavesAI/model/aussm.py:905-916) as torch's fused op
+        return F.rms_norm(x, (x.shape[-1],), self.weight, self.eps)
 
 
 class MambaBlock(nn.Module):

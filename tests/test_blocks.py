@@ -143,3 +143,14 @@ def test_ssmts_full_size_step_runs():
 
 def F_mse(a, b):
     return ((a - b) ** 2).mean()
+
+
+def test_rmsnorm_is_the_reference_formula_cpu():
+    """x * rsqrt(mean(x^2, -1) + eps) * weight (ai-modules/wavesAI/model/aussm.py:905-916)."""
+    torch.manual_seed(3)
+    norm = blocks.RMSNorm(24)
+    with torch.no_grad():
+        norm.weight.copy_(torch.randn(24))
+    x = torch.randn(2, 5, 24)
+    want = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + norm.eps) * norm.weight
+    torch.testing.assert_close(norm(x), want, atol=1e-6, rtol=1e-6)
