@@ -252,6 +252,10 @@ int aussm_num_checkpoints(int L, int ck) { return (L < 1 || ck < 1) ? 0 : (L + c
 
 int aussm_bwd_checkpoint_interval(int variant) { return variant == VAR_UNITARY ? 0 : REC_CK; }
 
+int aussm_unitary_split_segments(int B, int D, int N, int L, int ck) {
+  return (B < 1 || D < 1 || N < 1 || L < 1) ? 0 : seg_capacity(B, D, N, L, ck);
+}
+
 size_t aussm_unitary_aux_floats(int B, int D, int N, int L, int ck) {
   if (B < 1 || D < 1 || N < 1 || L < 1) return 0;
   return (size_t)B * D * L + AUX_PAD + seg_floats(B, D, N, L, seg_capacity(B, D, N, L, ck));

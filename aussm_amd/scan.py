@@ -36,6 +36,17 @@ Tensor = torch.Tensor
 # so a long interval is enough; the complex and real backward passes recompute every tile from
 # its checkpoint and need one per tile.
 UNITARY_CK = 256
+
+
+def unitary_ck(b: int, d: int, n: int, l: int) -> int:
+    """Checkpoint interval of the unitary scan for a shape: UNITARY_CK, or half of it where that
+    lets a launch with few (batch, channel) pairs be split into more segments along L (a segment
+    is a whole number of checkpoint blocks)."""
+    lib = _lib.load()
+    half = UNITARY_CK // 2
+    if lib.aussm_unitary_split_segments(b, d, n, l, half) > lib.aussm_unitary_split_segments(b, d, n, l, UNITARY_CK):
+        return half
+    return UNITARY_CK
 TILE_CK = _lib.TILE
 
 
@@ -154,9 +165,11 @@ class _UnitaryScanFn(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, u, delta, theta, Bri, Cri, D, h0):
-        aux = unitary_aux(theta, Bri.shape[1], UNITARY_CK)
-        y, hL, hck = unitary_fwd_raw(u, delta, theta, Bri, Cri, D, None, h0, want_state=True, ck=UNITARY_CK, aux=aux)
+        ck = unitary_ck(theta.shape[0], theta.shape[1], Bri.shape[1], theta.shape[2])
+        aux = unitary_aux(theta, Bri.shape[1], ck)
+        y, hL, hck = unitary_fwd_raw(u, delta, theta, Bri, Cri, D, None, h0, want_state=True, ck=ck, aux=aux)
         ctx.save_for_backward(u, delta, theta, Bri, Cri, D, hck, aux)
+        ctx.ck = ck
         ctx.has_h0 = h0 is not None
         return y, hL
 
@@ -166,7 +179,7 @@ class _UnitaryScanFn(torch.autograd.Function):
         dy = dy.contiguous()
         dhL = None if dhL is None else dhL.contiguous()
         du, ddelta, dtheta, dB, dC, dD, dh0 = unitary_bwd_raw(
-            dy, dhL, u, delta, theta, Bri, Cri, D, hck, UNITARY_CK,
+            dy, dhL, u, delta, theta, Bri, Cri, D, hck, ctx.ck,
             want_dD=D is not None and ctx.needs_input_grad[5], want_dh0=ctx.has_h0 and ctx.needs_input_grad[6],
             aux=aux)
         if u.shape[0] != theta.shape[0]:             # u, delta shared by consecutive batch elements
@@ -210,10 +223,11 @@ def unitary_scan(u: Tensor, delta: Tensor, theta: Tensor, Bc: Tensor, Cc: Tensor
     else:
         # no backward pass: the auxiliary buffer is only worth allocating when the launch would be split along L
         lib = _lib.load()
-        split = lib.aussm_unitary_aux_floats(b, d, n, l, UNITARY_CK) > b * d * l + _lib.AUX_PAD
-        aux = unitary_aux(theta, n, UNITARY_CK) if (split and u.shape[0] == b) else None
+        ck = unitary_ck(b, d, n, l)
+        split = lib.aussm_unitary_aux_floats(b, d, n, l, ck) > b * d * l + _lib.AUX_PAD
+        aux = unitary_aux(theta, n, ck) if (split and u.shape[0] == b) else None
         y, hL, _ = unitary_fwd_raw(u, delta, theta, Bri, Cri, D, z, h0r, want_state=return_last_state,
-                                   ck=UNITARY_CK if aux is not None else 0, aux=aux)
+                                   ck=ck if aux is not None else 0, aux=aux)
     if return_last_state:
         return y, torch.view_as_complex(hL)
     return y

@@ -121,6 +121,10 @@ int aussm_unitary_bwd(const float* dy, const float* dhL,
  * ssm_adaptive_unitary_backward.cu:113-181, and its launches cover at most 2048 steps). */
 size_t aussm_unitary_aux_floats(int B, int D, int N, int L, int ck);
 
+/* Number of segments a call of this shape is split into along L when it is given an auxiliary
+ * buffer (1 = not split); lets a caller choose ck (a segment is a whole number of checkpoint blocks). */
+int aussm_unitary_split_segments(int B, int D, int N, int L, int ck);
+
 int aussm_unitary_fwd_aux(const void* u, const void* delta, const float* theta,
                           const void* Bc, const void* Cc, const float* Dskip, const float* z,
                           const float* h0, float* y, float* hL, float* hck, float* aux,

@@ -21,7 +21,7 @@ def test_header_declares_the_expected_entry_points():
     for must in ("aussm_unitary_fwd", "aussm_unitary_bwd", "aussm_complex_fwd", "aussm_complex_bwd",
                  "aussm_real_fwd", "aussm_real_bwd", "aussm_version", "aussm_error_string",
                  "aussm_unitary_fwd_aux", "aussm_unitary_bwd_aux", "aussm_unitary_aux_floats",
-                 "aussm_causal_conv1d_fwd", "aussm_causal_conv1d_bwd", "aussm_swap_last2"):
+                 "aussm_causal_conv1d_fwd", "aussm_causal_conv1d_bwd", "aussm_swap_last2", "aussm_unitary_split_segments"):
         assert must in names
 
 
@@ -70,6 +70,10 @@ def test_argument_checks_without_a_device():
     # ... which needs whole checkpoint blocks per segment, and states the matrix-core kernels serve
     assert lib.aussm_unitary_aux_floats(4, 256, 16, 16384 + 4, 256) == 4 * 256 * (16384 + 4) + 64
     assert lib.aussm_unitary_aux_floats(4, 256, 4, 16384, 256) == 4 * 256 * 16384 + 64
+    assert lib.aussm_unitary_split_segments(4, 256, 16, 16384, 256) == 16
+    assert lib.aussm_unitary_split_segments(16, 128, 16, 1024, 256) == 4
+    assert lib.aussm_unitary_split_segments(16, 128, 16, 1024, 128) == 8
+    assert lib.aussm_unitary_split_segments(32, 512, 16, 2048, 256) == 1
     rc = lib.aussm_unitary_fwd_aux(one, one, one, one, one, null, null, null, one, null, null, ctypes.c_void_p(260),
                                    1, 1, 1, 32, 32, 0, 1, null)
     assert rc == -5
