@@ -32,6 +32,8 @@ Pinning status (which independent check fixes each function):
   adaptive_unitary_polar same pair                                     pinned
   reference_unitary_phase_loop
                          brute-force scalar loop                       pinned
+  causal_conv1d_bld      torch's conv1d called exactly as the reference's blocks
+                         call it; explicit causal sum in Python loops  pinned
 """
 from __future__ import annotations
 
