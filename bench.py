@@ -93,7 +93,7 @@ def main():
     B, D, N, L = SHAPE["B"], SHAPE["D"], SHAPE["N"], SHAPE["L"]
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    # synthetic inputs with BASELINE's value distributions, generated on the device (the CPU oracle is only
+    # synthetic inputs with the benchmark contract's value distributions, generated on the device (the CPU oracle is only
     # used by the cpu_baseline leg): u ~ N(0,1), delta = softplus(N(0,1)), theta ~ N(0, 0.5), B_t and C_t complex
     # with parts ~ N(0, 1/sqrt(N)), D ~ N(0,1), dy ~ N(0,1)
     g = torch.Generator(device=dev).manual_seed(0)

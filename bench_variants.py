@@ -1,11 +1,11 @@
 #!/usr/bin/env python3
 """The three scan variants at the headline shape (B=32 D=512 N=16 L=2048), forward and backward,
 once with float32 inputs and once with bfloat16 u / delta / B / C (float32 phases, decay, skip,
-states, outputs and gradients): BASELINE configuration 3.
+states, outputs and gradients): configuration 3 of the benchmark contract.
 
     python bench_variants.py [--reps R] [--shape B,D,N,L] [--variants real,...] [--model | --only-model]
 
-With --model it also times BASELINE configuration 4: one training step (forward, MSE loss,
+With --model it also times configuration 4 of the contract: one training step (forward, MSE loss,
 backward) of SSMTS(d_model=256, input_dim=21, output_dim=21, layers="a|m|a|m") on x ~ N(0,1) of
 shape (32, 720, 21), random-init weights, wall clock around synchronised steps.
 
@@ -74,7 +74,7 @@ def main():
         return sum(s.elapsed_time(e) for s, e in evs) / args.reps * 1e3
 
     def inputs(variant):
-        """BASELINE's value distributions: u ~ N(0,1), delta = softplus(N(0,1)), theta ~ N(0, 0.5),
+        """The contract's value distributions: u ~ N(0,1), delta = softplus(N(0,1)), theta ~ N(0, 0.5),
         B, C ~ N(0, 1/sqrt(N)) per part, D ~ N(0,1), A = -exp(N(0,1)), rho = -delta exp(N(0,1))[d]."""
         g = torch.Generator(device=dev).manual_seed(0)
         rn = lambda *s: torch.randn(*s, generator=g, device=dev)

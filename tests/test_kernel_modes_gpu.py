@@ -252,7 +252,7 @@ def test_random_shapes_inputs_and_checkpoint_intervals(seed):
 
 def test_forward_only_call_takes_the_split_too():
     """Without a backward pass unitary_scan allocates the auxiliary buffer only when the launch is
-    split along L (BASELINE configuration 1 is such a call): same outputs as with the split off."""
+    split along L (configuration 1 of the benchmark contract, B=16 D=128 L=1024 forward only, is such a call): same outputs as with the split off."""
     from aussm_amd import scan
     B, D, N, L = 2, 64, 16, 1024
     p = _inputs(B, D, N, L, 77, big_theta=False)
