@@ -96,8 +96,28 @@ __device__ __forceinline__ f4 xmm(const u4 (&a)[NP], const u4 (&b)[NP], f4 c) {
     for (int i = 0; i <= s; ++i) c = xdl(a[i], b[s - i], c);
   return c;
 }
-// the K-th matrix instruction of xmm (same order)
-template <int NP, int K>
+// The same when only the first NPA pieces of a (and, for xmm_pp, of b too) can be non-zero: operands
+// that came from bf16 inputs are a single exact piece, the products with their other pieces vanish.
+template <int NP, int NPA>
+__device__ __forceinline__ f4 xmm_p(const u4 (&a)[NP], const u4 (&b)[NP], f4 c) {
+#pragma unroll
+  for (int s = NP - 1; s >= 0; --s)
+#pragma unroll
+    for (int i = 0; i <= s; ++i)
+      if (i < NPA) c = xdl(a[i], b[s - i], c);
+  return c;
+}
+template <int NP, int NPA>
+__device__ __forceinline__ f4 xmm_pp(const u4 (&a)[NP], const u4 (&b)[NP], f4 c) {
+#pragma unroll
+  for (int s = NP - 1; s >= 0; --s)
+#pragma unroll
+    for (int i = 0; i <= s; ++i)
+      if (i < NPA && s - i < NPA) c = xdl(a[i], b[s - i], c);
+  return c;
+}
+// the K-th matrix instruction of xmm (same order); skipped when it involves a piece >= NPA of a
+template <int NP, int K, int NPA = NP>
 __device__ __forceinline__ f4 xmm_k(const u4 (&a)[NP], const u4 (&b)[NP], f4 c) {
   constexpr int s0 = NP - 1;
   // products are visited with s = NP-1 .. 0 and i = 0 .. s: find (s, i) of index K
@@ -105,7 +125,8 @@ __device__ __forceinline__ f4 xmm_k(const u4 (&a)[NP], const u4 (&b)[NP], f4 c) 
   constexpr int base = (NP == 3) ? (K < 3 ? 0 : (K < 5 ? 3 : 5)) : (NP == 2 ? (K < 2 ? 0 : 2) : 0);
   constexpr int i = K - base;
   static_assert(s <= s0 && i <= s, "bad product index");
-  return xdl(a[i], b[s - i], c);
+  if constexpr (i >= NPA) return c;
+  else return xdl(a[i], b[s - i], c);
 }
 __device__ __forceinline__ u4 neg_bf16x8(const u4& v) { return v ^ u4{0x80008000u, 0x80008000u, 0x80008000u, 0x80008000u}; }
 
@@ -212,6 +233,7 @@ __global__ __launch_bounds__(256) void unitary_fwd_xdl_kernel(const FwdArgs p) {
   const float dsk = (p.Dskip && dok) ? p.Dskip[dc] : 0.0f;
   const int nchunks = (L + XT - 1) / XT;
   const SplitK sk = make_splitk();
+  constexpr int NPA = sizeof(Tin) == 2 ? 1 : NP;   // non-zero pieces of the staged B / C records
 
   // G tiles above the block diagonal are read (as zeros) but never written
   for (int i = tid; i < (int)(sizeof(s_g) / 16); i += 256) reinterpret_cast<u4*>(s_g)[i] = u4{0, 0, 0, 0};
@@ -293,8 +315,8 @@ __global__ __launch_bounds__(256) void unitary_fwd_xdl_kernel(const FwdArgs p) {
       br[q] = s.cs_r[q][xrec(16 * gtt + dl, g, XT)];
       bi[q] = s.cs_i[q][xrec(16 * gtt + dl, g, XT)];
     }
-    f4 gr = xmm<NP>(a, br, f4{0, 0, 0, 0});
-    f4 gi = xmm<NP>(a, bi, f4{0, 0, 0, 0});
+    f4 gr = xmm_pp<NP, NPA>(a, br, f4{0, 0, 0, 0});
+    f4 gi = xmm_pp<NP, NPA>(a, bi, f4{0, 0, 0, 0});
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const bool keep = 4 * g + i <= g_lim;
@@ -481,8 +503,8 @@ __global__ __launch_bounds__(256) void unitary_fwd_xdl_kernel(const FwdArgs p) {
 #pragma unroll
     for (int k = 0; k < 4; ++k) m1_raw[k].pin();
     m2_raw.pin();
-    f4 ggr = xmm<NP>(ga, gbr, f4{0, 0, 0, 0});
-    f4 ggi = xmm<NP>(ga, gbi, f4{0, 0, 0, 0});
+    f4 ggr = xmm_pp<NP, NPA>(ga, gbr, f4{0, 0, 0, 0});
+    f4 ggi = xmm_pp<NP, NPA>(ga, gbi, f4{0, 0, 0, 0});
     bc_store(c + 2, s_bc[i2]);
     XDL_REGION(2 * NPP, 12);
     bc_load(c + 3);
@@ -495,8 +517,8 @@ __global__ __launch_bounds__(256) void unitary_fwd_xdl_kernel(const FwdArgs p) {
     f4 Sr[2], Si[2];
 #pragma unroll
     for (int tt = 0; tt < 2; ++tt) {
-      Sr[tt] = xmm<NP>(c_r[tt], hk, f4{0, 0, 0, 0});
-      Si[tt] = xmm<NP>(c_i[tt], hk, f4{0, 0, 0, 0});
+      Sr[tt] = xmm_p<NP, NPA>(c_r[tt], hk, f4{0, 0, 0, 0});
+      Si[tt] = xmm_p<NP, NPA>(c_i[tt], hk, f4{0, 0, 0, 0});
     }
     {
 #pragma unroll
@@ -561,10 +583,10 @@ __global__ __launch_bounds__(256) void unitary_fwd_xdl_kernel(const FwdArgs p) {
         sincos_small(ph[e], &psn[e], &pcs[e]);
         touch_vgpr(psn[e]); touch_vgpr(pcs[e]);
         if constexpr (k < NPP) {
-          Hr = xmm_k<NP, k>(b_r, pc.vr, Hr);
-          Hi = xmm_k<NP, k>(b_r, pc.vi, Hi);
-          Hr = xmm_k<NP, k>(b_i, pc.nvi, Hr);
-          Hi = xmm_k<NP, k>(b_i, pc.vr, Hi);
+          Hr = xmm_k<NP, k, NPA>(b_r, pc.vr, Hr);
+          Hi = xmm_k<NP, k, NPA>(b_r, pc.vi, Hi);
+          Hr = xmm_k<NP, k, NPA>(b_i, pc.nvi, Hr);
+          Hi = xmm_k<NP, k, NPA>(b_i, pc.vr, Hi);
         }
         __builtin_amdgcn_sched_barrier(0);
       };
