@@ -176,6 +176,8 @@ __global__ __launch_bounds__(256) void unitary_bwd_xdl_kernel(const UniBwdArgs p
   const float dsk = (p.Dskip && dok) ? p.Dskip[dc] : 0.0f;
   const int nchunks = (L + XT - 1) / XT;
   const SplitK sk = make_splitk();
+  // non-zero pieces of the staged B / C records: bf16 inputs are a single exact piece
+  constexpr int NPA = sizeof(Tin) == 2 ? 1 : NP, NPAC = sizeof(Tin) == 2 ? 1 : NPC;
   // Im(P_t S_t) left by the forward kernel (if it filled the buffer): saves recomputing S here
   const bool use_phi = p.aux != nullptr &&
       __builtin_amdgcn_readfirstlane(__float_as_uint(p.aux[(size_t)p.B * D * L])) == AUX_TAG;
@@ -288,7 +290,7 @@ __global__ __launch_bounds__(256) void unitary_bwd_xdl_kernel(const UniBwdArgs p
     ldrec<NP>(s_bc.cs_r, xrec(16 * gtt + dl, g, XT), cr);
     ldrec<NP>(s_bc.cs_i, xrec(16 * gtt + dl, g, XT), ci);
     // rows t, columns s  ->  lane: G[t = 4 g + i][s = dl]
-    f4 yr = xmm<NP>(cr, a, f4{0, 0, 0, 0}), yi = xmm<NP>(ci, a, f4{0, 0, 0, 0});
+    f4 yr = xmm_pp<NP, NPA>(cr, a, f4{0, 0, 0, 0}), yi = xmm_pp<NP, NPA>(ci, a, f4{0, 0, 0, 0});
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const bool k2 = 4 * g + i >= g_low;
@@ -297,7 +299,7 @@ __global__ __launch_bounds__(256) void unitary_bwd_xdl_kernel(const UniBwdArgs p
     put_half(s_g.g_r, s_g.g_i, xrec(16 * gst + dl, g, XT) * 2 + gtt, yr, yi);
     if (!use_phi) {
       // rows s, columns t  ->  lane: G[t = dl][s = 4 g + i]   (only the S recomputation reads it)
-      f4 xr = xmm<NP>(a, cr, f4{0, 0, 0, 0}), xi = xmm<NP>(a, ci, f4{0, 0, 0, 0});
+      f4 xr = xmm_pp<NP, NPA>(a, cr, f4{0, 0, 0, 0}), xi = xmm_pp<NP, NPA>(a, ci, f4{0, 0, 0, 0});
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const bool k1 = 4 * g + i <= g_lim;
@@ -493,10 +495,10 @@ __global__ __launch_bounds__(256) void unitary_bwd_xdl_kernel(const UniBwdArgs p
       ldrec16<NP>(s_bc.bt_i, xrec(dl, g, XN), bi);
       ldrec16<NP>(s_bc.ct_r, xrec(dl, g, XN), cr);
       ldrec16<NP>(s_bc.ct_i, xrec(dl, g, XN), ci);
-      Hr = xmm<NP>(br, nVr, Hr);  Hr = xmm<NP>(bi, Vi, Hr);
-      Hi = xmm<NP>(br, nVi, Hi);  Hi = xmm<NP>(bi, nVr, Hi);
-      Ar = xmm<NP>(cr, Qr, Jr);   Ar = xmm<NP>(ci, Qi, Ar);
-      Ai = xmm<NP>(cr, Qi, Ji);   Ai = xmm<NP>(ci, nQr, Ai);
+      Hr = xmm_p<NP, NPA>(br, nVr, Hr);  Hr = xmm_p<NP, NPA>(bi, Vi, Hr);
+      Hi = xmm_p<NP, NPA>(br, nVi, Hi);  Hi = xmm_p<NP, NPA>(bi, nVr, Hi);
+      Ar = xmm_p<NP, NPA>(cr, Qr, Jr);   Ar = xmm_p<NP, NPA>(ci, Qi, Ar);
+      Ai = xmm_p<NP, NPA>(cr, Qi, Ji);   Ai = xmm_p<NP, NPA>(ci, nQr, Ai);
     }
     // ---- gV, first term: sum_n conj(B_s[n]) J[n]
     f4 gVr[2], gVi[2];
@@ -509,8 +511,8 @@ __global__ __launch_bounds__(256) void unitary_bwd_xdl_kernel(const UniBwdArgs p
         u4 a[NP], ac[NP];
         ldrec<NP>(s_bc.bs, xrec(16 * st + dl, g, XT), a);
         ldrec<NP>(s_bc.bs_c, xrec(16 * st + dl, g, XT), ac);
-        gVr[st] = xmm<NP>(a, jk, f4{0, 0, 0, 0});
-        gVi[st] = xmm<NP>(ac, jk, f4{0, 0, 0, 0});
+        gVr[st] = xmm_p<NP, NPA>(a, jk, f4{0, 0, 0, 0});
+        gVi[st] = xmm_p<NP, NPA>(ac, jk, f4{0, 0, 0, 0});
       }
     }
     // ---- sums over the channel: transpose Q, V, H, J through the private scratch
@@ -605,8 +607,8 @@ __global__ __launch_bounds__(256) void unitary_bwd_xdl_kernel(const UniBwdArgs p
         ldrec<NP>(s_bc.cs_i, xrec(16 * tt + dl, g, XT), ai);
         ldrec<NP>(s_g.gt_r, xrec(16 * tt + dl, g, XT), gr);
         ldrec<NP>(s_g.gt_i, xrec(16 * tt + dl, g, XT), gi);
-        f4 Sr = xmm<NP>(ar, hk, f4{0, 0, 0, 0});
-        f4 Si = xmm<NP>(ai, hk, f4{0, 0, 0, 0});
+        f4 Sr = xmm_p<NP, NPA>(ar, hk, f4{0, 0, 0, 0});
+        f4 Si = xmm_p<NP, NPA>(ai, hk, f4{0, 0, 0, 0});
         Sr = xmm<NP>(gr, Vr, Sr);  Sr = xmm<NP>(gi, nVi, Sr);
         Si = xmm<NP>(gr, Vi, Si);  Si = xmm<NP>(gi, Vr, Si);
 #pragma unroll
@@ -712,8 +714,8 @@ __global__ __launch_bounds__(256) void unitary_bwd_xdl_kernel(const UniBwdArgs p
       }
       ldrec16<NPC>(isC ? s_bc.bt_r : s_bc.ct_r, xrec(dl, g, XN), er);
       ldrec16<NPC>(isC ? s_bc.bt_i : s_bc.ct_i, xrec(dl, g, XN), ei);
-      xr = xmm<NPC>(mr, er, xr);  xr = xmm<NPC>(mi, ei, xr);
-      xi = xmm<NPC>(mi, er, xi);  xi = xmm<NPC>(nmr, ei, xi);
+      xr = xmm_q<NPC, NPAC>(mr, er, xr);  xr = xmm_q<NPC, NPAC>(mi, ei, xr);
+      xi = xmm_q<NPC, NPAC>(mi, er, xi);  xi = xmm_q<NPC, NPAC>(nmr, ei, xi);
       // Through a small LDS tile so that one atomic instruction covers two whole rows n of the
       // tile (16 timesteps x (re, im) = one 128-byte line each) instead of sixteen lines.
       float* __restrict__ at = s_at[wave];

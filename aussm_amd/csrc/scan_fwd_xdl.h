@@ -116,6 +116,16 @@ __device__ __forceinline__ f4 xmm_pp(const u4 (&a)[NP], const u4 (&b)[NP], f4 c)
       if (i < NPA && s - i < NPA) c = xdl(a[i], b[s - i], c);
   return c;
 }
+// ... and when it is the second operand whose pieces >= NPB vanish
+template <int NP, int NPB>
+__device__ __forceinline__ f4 xmm_q(const u4 (&a)[NP], const u4 (&b)[NP], f4 c) {
+#pragma unroll
+  for (int s = NP - 1; s >= 0; --s)
+#pragma unroll
+    for (int i = 0; i <= s; ++i)
+      if (s - i < NPB) c = xdl(a[i], b[s - i], c);
+  return c;
+}
 // the K-th matrix instruction of xmm (same order); skipped when it involves a piece >= NPA of a
 template <int NP, int K, int NPA = NP>
 __device__ __forceinline__ f4 xmm_k(const u4 (&a)[NP], const u4 (&b)[NP], f4 c) {

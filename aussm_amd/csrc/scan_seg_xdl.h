@@ -175,8 +175,9 @@ __global__ __launch_bounds__(256) void unitary_seg_state_kernel(const SegArgs p)
         Si[i] = cT * ai - sT * ar;
       }
     }
-    Sr = xmm<NP>(mr, Xr, Sr);  Sr = xmm<NP>(mi, nXi, Sr);
-    Si = xmm<NP>(mr, Xi, Si);  Si = xmm<NP>(mi, Xr, Si);
+    constexpr int NPA = sizeof(Tin) == 2 ? 1 : NP;   // bf16 B / C: a single exact piece
+    Sr = xmm_p<NP, NPA>(mr, Xr, Sr);  Sr = xmm_p<NP, NPA>(mi, nXi, Sr);
+    Si = xmm_p<NP, NPA>(mr, Xi, Si);  Si = xmm_p<NP, NPA>(mi, Xr, Si);
     if (!ADJ) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
