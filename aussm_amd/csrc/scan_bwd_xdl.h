@@ -216,6 +216,7 @@ __global__ __launch_bounds__(256) void unitary_bwd_xdl_kernel(const UniBwdArgs p
     const size_t o2 = (((size_t)bb * N + (m2_n < N ? m2_n : 0)) * p.ld + so + l2c) * 2;
     m2_raw.load(m2_src + o2);
   };
+  // (only the NPA pieces that can be non-zero are formed and stored; the others are never read)
   auto bc_store = [&](int c) {
     {
       const bool tok = c * XT + m1_t < L;
@@ -226,16 +227,16 @@ __global__ __launch_bounds__(256) void unitary_bwd_xdl_kernel(const UniBwdArgs p
         x[k] = ok ? m1_raw[k].re() : 0.0f;
         x[4 + k] = ok ? m1_raw[k].im() : 0.0f;
       }
-      u4 pc[NP], pi[NP], pcs[NP];
-      split8<NP>(sk, x, pc);                 // [re, im]
-      rot_i<NP>(pc, pi);                 // [-im, re]
+      u4 pc[NPA], pi[NPA], pcs[NPA];
+      split8<NPA>(sk, x, pc);                 // [re, im]
+      rot_i<NPA>(pc, pi);                 // [-im, re]
       const int o = xrec(m1_t, m1_g, XT);
       if (m1_isB) {
 #pragma unroll
-        for (int q = 0; q < NP; ++q) { s_bc.bs[q][o] = pc[q]; s_bc.bs_c[q][o] = pi[q]; }
+        for (int q = 0; q < NPA; ++q) { s_bc.bs[q][o] = pc[q]; s_bc.bs_c[q][o] = pi[q]; }
       } else {
 #pragma unroll
-        for (int q = 0; q < NP; ++q) {
+        for (int q = 0; q < NPA; ++q) {
           pcs[q] = u4{pc[q][0], pc[q][1], pc[q][2] ^ 0x80008000u, pc[q][3] ^ 0x80008000u};   // [re, -im]
           s_bc.cs_r[q][o] = pcs[q];
           s_bc.cs_i[q][o] = u4{pc[q][2], pc[q][3], pc[q][0], pc[q][1]};                        // [im, re]
@@ -248,14 +249,14 @@ __global__ __launch_bounds__(256) void unitary_bwd_xdl_kernel(const UniBwdArgs p
       const float r2 = ok ? m2_raw.re(2) : 0.0f, r3 = ok ? m2_raw.re(3) : 0.0f;
       const float j0 = ok ? m2_raw.im(0) : 0.0f, j1 = ok ? m2_raw.im(1) : 0.0f;
       const float j2 = ok ? m2_raw.im(2) : 0.0f, j3 = ok ? m2_raw.im(3) : 0.0f;
-      uint32_t a0[NP], a1[NP], b0[NP], b1[NP];
-      split2<NP>(sk, r0, r1, a0);
-      split2<NP>(sk, r2, r3, a1);
-      split2<NP>(sk, j0, j1, b0);
-      split2<NP>(sk, j2, j3, b1);
+      uint32_t a0[NPA], a1[NPA], b0[NPA], b1[NPA];
+      split2<NPA>(sk, r0, r1, a0);
+      split2<NPA>(sk, r2, r3, a1);
+      split2<NPA>(sk, j0, j1, b0);
+      split2<NPA>(sk, j2, j3, b1);
       const int o = xrec(m2_n, m2_g, XN) * 2 + m2_half;   // 8-byte half-record index
 #pragma unroll
-      for (int q = 0; q < NP; ++q) {
+      for (int q = 0; q < NPA; ++q) {
         if (m2_isC) {
           reinterpret_cast<u2*>(s_bc.ct_r[q])[o] = u2{a0[q], a1[q]};
           reinterpret_cast<u2*>(s_bc.ct_i[q])[o] = u2{b0[q], b1[q]};

@@ -277,6 +277,7 @@ __global__ __launch_bounds__(256) void unitary_fwd_xdl_kernel(const FwdArgs p) {
   // Branch-free: C threads write [re, -im] -> cs_r and [im, re] -> cs_i, B threads [re, im] -> bs and
   // [-im, re] -> bs_c; real-part threads of the second mapping write bt_r, the others bt_i.
   const uint32_t m1_s1 = m1_isB ? 0u : 0x80008000u, m1_s2 = m1_isB ? 0x80008000u : 0u;
+  // (only the NPA pieces that can be non-zero are formed and stored; the others are never read)
   auto bc_store = [&](int c, XdlBC<NP>& s) {
     {
       const bool tok = c * XT + m1_t < L;
@@ -287,13 +288,13 @@ __global__ __launch_bounds__(256) void unitary_fwd_xdl_kernel(const FwdArgs p) {
         x[k] = ok ? m1_raw[k].re() : 0.0f;
         x[4 + k] = ok ? m1_raw[k].im() : 0.0f;
       }
-      u4 pc[NP];
-      split8<NP>(sk, x, pc);
+      u4 pc[NPA];
+      split8<NPA>(sk, x, pc);
       const int o = xrec(m1_t, m1_g, XT);
       u4* d1 = m1_isB ? &s.bs[0][0] : &s.cs_r[0][0];
       u4* d2 = m1_isB ? &s.bs_c[0][0] : &s.cs_i[0][0];
 #pragma unroll
-      for (int q = 0; q < NP; ++q) {
+      for (int q = 0; q < NPA; ++q) {
         d1[q * (XT * 4) + o] = u4{pc[q][0], pc[q][1], pc[q][2] ^ m1_s1, pc[q][3] ^ m1_s1};
         d2[q * (XT * 4) + o] = u4{pc[q][2] ^ m1_s2, pc[q][3] ^ m1_s2, pc[q][0], pc[q][1]};
       }
@@ -302,13 +303,13 @@ __global__ __launch_bounds__(256) void unitary_fwd_xdl_kernel(const FwdArgs p) {
       const bool ok = (m2_n < N) && (c * XT + 16 * m2_half + 4 * m2_g < L);
       const float v0 = ok ? (m2_im ? m2_raw.im(0) : m2_raw.re(0)) : 0.0f, v1 = ok ? (m2_im ? m2_raw.im(1) : m2_raw.re(1)) : 0.0f;
       const float v2 = ok ? (m2_im ? m2_raw.im(2) : m2_raw.re(2)) : 0.0f, v3 = ok ? (m2_im ? m2_raw.im(3) : m2_raw.re(3)) : 0.0f;
-      uint32_t a[NP], c2[NP];
-      split2<NP>(sk, v0, v1, a);
-      split2<NP>(sk, v2, v3, c2);
+      uint32_t a[NPA], c2[NPA];
+      split2<NPA>(sk, v0, v1, a);
+      split2<NPA>(sk, v2, v3, c2);
       const int o = xrec(m2_n, m2_g, XN) * 2 + m2_half;   // 8-byte half-record index
       u2* d1 = reinterpret_cast<u2*>(m2_im ? &s.bt_i[0][0] : &s.bt_r[0][0]);
 #pragma unroll
-      for (int q = 0; q < NP; ++q) d1[q * (XN * 4 * 2) + o] = u2{a[q], c2[q]};
+      for (int q = 0; q < NPA; ++q) d1[q * (XN * 4 * 2) + o] = u2{a[q], c2[q]};
     }
   };
 

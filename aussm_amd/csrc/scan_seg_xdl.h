@@ -75,13 +75,14 @@ __global__ __launch_bounds__(256) void unitary_seg_state_kernel(const SegArgs p)
     float v0 = m2_im ? m2_raw.im(0) : m2_raw.re(0), v1 = m2_im ? m2_raw.im(1) : m2_raw.re(1);
     float v2 = m2_im ? m2_raw.im(2) : m2_raw.re(2), v3 = m2_im ? m2_raw.im(3) : m2_raw.re(3);
     v0 = ok ? sg * v0 : 0.0f; v1 = ok ? sg * v1 : 0.0f; v2 = ok ? sg * v2 : 0.0f; v3 = ok ? sg * v3 : 0.0f;
-    uint32_t a0[NP], a1[NP];
-    split2<NP>(sk, v0, v1, a0);
-    split2<NP>(sk, v2, v3, a1);
+    constexpr int NPS = sizeof(Tin) == 2 ? 1 : NP;   // bf16 values are a single exact piece
+    uint32_t a0[NPS], a1[NPS];
+    split2<NPS>(sk, v0, v1, a0);
+    split2<NPS>(sk, v2, v3, a1);
     const int o = xrec(m2_n, m2_g, XN) * 2 + m2_half;   // 8-byte half-record index
     u4 (*dst)[XN * 4] = m2_im ? s_mi[slot] : s_mr[slot];
 #pragma unroll
-    for (int q = 0; q < NP; ++q) reinterpret_cast<u2*>(dst[q])[o] = u2{a0[q], a1[q]};
+    for (int q = 0; q < NPS; ++q) reinterpret_cast<u2*>(dst[q])[o] = u2{a0[q], a1[q]};
   };
 
   struct In { f4 th[2]; Raw4<TA> a[2]; Raw4<Tin> b[2]; };
