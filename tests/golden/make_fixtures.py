@@ -38,6 +38,13 @@ def main():
     for k, v in zip(("u", "dt", "x", "x_bias", "B", "C", "D", "z"), args):
         out[f"adaptive_{k}"] = ri(v).astype(np.float32)
     out["adaptive_y"] = O.adaptive_unitary_polar(*args).numpy().astype(np.float32)
+    # the blocks' depthwise causal convolution (ai-modules/wavesAI/model/aussm.py:762, :863) on (b, l, d)
+    g = torch.Generator().manual_seed(21)
+    cx = torch.randn(2, 9, 5, generator=g, dtype=torch.float64)
+    cw = torch.randn(5, 1, 4, generator=g, dtype=torch.float64)
+    cb = torch.randn(5, generator=g, dtype=torch.float64)
+    out["conv_x"], out["conv_w"], out["conv_b"] = (v.numpy().astype(np.float32) for v in (cx, cw, cb))
+    out["conv_y"] = O.causal_conv1d_bld(cx, cw, cb).numpy().astype(np.float32)
     np.savez_compressed(os.path.join(HERE, "scan_fixtures.npz"), **out)
     print("wrote", len(out), "arrays")
 

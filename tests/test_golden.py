@@ -68,3 +68,15 @@ def test_hip_reproduces_adaptive_fixture():
            [t("adaptive_D"), t("adaptive_z")]
     y = ops.ssm_adaptive_interface(*[a.cuda() for a in args], unitary=True)
     torch.testing.assert_close(y.cpu(), t("adaptive_y"), atol=7e-5, rtol=5e-5)
+
+
+def test_oracle_reproduces_conv_fixture():
+    y = O.causal_conv1d_bld(t("conv_x"), t("conv_w"), t("conv_b"))
+    torch.testing.assert_close(y, t("conv_y"), atol=1e-6, rtol=1e-6)
+
+
+@pytest.mark.gpu
+def test_hip_reproduces_conv_fixture():
+    from aussm_amd import conv
+    y = conv.causal_conv1d(t("conv_x").cuda(), t("conv_w").cuda(), t("conv_b").cuda())
+    torch.testing.assert_close(y.cpu(), t("conv_y"), atol=1e-5, rtol=1e-5)
