@@ -26,6 +26,8 @@ _LL = ctypes.c_longlong
 # name -> argtypes; every entry point returns int
 _SIGNATURES = {
     "aussm_version": [],
+    "aussm_set_option": [_I, _I],
+    "aussm_get_option": [_I],
     "aussm_num_checkpoints": [_I, _I],
     "aussm_bwd_checkpoint_interval": [_I],
     "aussm_unitary_split_segments": [_I] * 5,
@@ -43,6 +45,9 @@ _SIGNATURES = {
 }
 
 EXPORTED = tuple(_SIGNATURES) + ("aussm_error_string", "aussm_unitary_aux_floats")
+
+
+OPT_UNITARY_FWD, OPT_UNITARY_BWD, OPT_SPLIT_CAP, OPT_GENERIC_NW, OPT_GENERIC_NT = range(5)
 
 
 class AussmError(RuntimeError):
@@ -84,3 +89,26 @@ def check(code: int, what: str) -> None:
 def ptr(t) -> c_void_p | None:
     """Device pointer of a tensor (None -> NULL)."""
     return None if t is None else c_void_p(t.data_ptr())
+
+
+class options:
+    """Context manager: library options (aussm_set_option) for the duration of a block, e.g.
+    `with options(unitary_fwd=0, split_cap=0): ...`; the previous values come back on exit."""
+    _KEYS = {"unitary_fwd": OPT_UNITARY_FWD, "unitary_bwd": OPT_UNITARY_BWD, "split_cap": OPT_SPLIT_CAP,
+             "generic_nw": OPT_GENERIC_NW, "generic_nt": OPT_GENERIC_NT}
+
+    def __init__(self, **kw):
+        self.kw = {self._KEYS[k]: (-1 if v is None else int(v)) for k, v in kw.items()}
+
+    def __enter__(self):
+        lib = load()
+        self.old = {k: lib.aussm_get_option(k) for k in self.kw}
+        for k, v in self.kw.items():
+            check(lib.aussm_set_option(k, v), "aussm_set_option")
+        return self
+
+    def __exit__(self, *exc):
+        lib = load()
+        for k, v in self.old.items():
+            lib.aussm_set_option(k, v)
+        return False

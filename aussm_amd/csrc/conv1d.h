@@ -8,23 +8,11 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
+#include "scan_args.h"
+
 namespace aussm {
 
-constexpr int CONV_MAX_K = 8;
-constexpr int CONV_ROWS = 128;   // (b, l) rows per workgroup of the weight-gradient kernel
 
-struct ConvArgs {
-  const float* x;      // element (b, l, d) at x[b * xs_b + l * xs_l + d]
-  const float* w;      // [D, K]
-  const float* bias;   // [D] or null
-  const float* dy;     // [B, L, D] contiguous (backward)
-  float* y;            // [B, L, D] contiguous (forward)
-  float* dx;           // [B, L, D] contiguous (backward)
-  float* dw;           // [D, K], accumulated into
-  float* dbias;        // [D] or null, accumulated into
-  long long xs_b, xs_l;
-  int B, L, D, K;
-};
 
 // grid: x = (b, l) row, y = block of 256 channels
 __global__ __launch_bounds__(256) void causal_conv1d_fwd_kernel(const ConvArgs p) {
@@ -99,7 +87,6 @@ __global__ __launch_bounds__(256) void causal_conv1d_bwd_weight_kernel(const Con
 
 // ---- kernel length 4 (the blocks' default d_conv): each thread owns CONV_RUN consecutive steps of
 // one channel and slides a register window over them, one load per step instead of four.
-constexpr int CONV_RUN = 8;
 
 // grid: x = (b, run of CONV_RUN steps), y = block of 256 channels
 __global__ __launch_bounds__(256) void causal_conv1d_k4_fwd_kernel(const ConvArgs p) {

@@ -1,0 +1,113 @@
+// Translation unit of the vector-ALU kernels: the three forward scans, the unitary reverse scan,
+// the recomputing reverse scans (complex, real), the causal convolution and the layout swap.
+#include "conv1d.h"
+#include "launch.h"
+#include "layout.h"
+#include "scan_bwd_recompute.h"
+#include "scan_bwd_unitary.h"
+#include "scan_fwd.h"
+
+namespace aussm {
+
+#define AUSSM_FWD_CASE(NW_, NT_)                                                                     \
+  if (c.nw == NW_ && c.nt == NT_) {                                                                  \
+    hipLaunchKernelGGL((core_fwd_kernel<VAR, NW_, NT_, Tin>), grid, dim3(NT_), 0, s, a);             \
+    return launch_status();                                                                          \
+  }
+
+template <int VAR, typename Tin>
+static int core_fwd_t(const FwdArgs& a, Cfg c, hipStream_t s) {
+  const dim3 grid((unsigned)(a.B * a.ncg));
+  AUSSM_FWD_CASE(1, 256) AUSSM_FWD_CASE(2, 256) AUSSM_FWD_CASE(4, 256) AUSSM_FWD_CASE(8, 256)
+  AUSSM_FWD_CASE(16, 256) AUSSM_FWD_CASE(1, 512) AUSSM_FWD_CASE(2, 512) AUSSM_FWD_CASE(4, 512)
+  AUSSM_FWD_CASE(8, 512)
+  return -2;
+}
+
+template <int VAR>
+static int core_fwd_v(const FwdArgs& a, int in_dtype, Cfg c, hipStream_t s) {
+  return in_dtype == 1 ? core_fwd_t<VAR, bf16_t>(a, c, s) : core_fwd_t<VAR, float>(a, c, s);
+}
+
+int run_core_fwd(int variant, const FwdArgs& a, int in_dtype, Cfg c, hipStream_t s) {
+  if (variant == VAR_UNITARY) return core_fwd_v<VAR_UNITARY>(a, in_dtype, c, s);
+  if (variant == VAR_COMPLEX) return core_fwd_v<VAR_COMPLEX>(a, in_dtype, c, s);
+  return core_fwd_v<VAR_REAL>(a, in_dtype, c, s);
+}
+
+// The backward workgroup keeps a (dw, dtheta) slab per wavefront in LDS: four wavefronts afford
+// 32-step tiles, eight wavefronts 16-step tiles.
+#define AUSSM_UBWD_CASE(NW_, NT_, TT_)                                                               \
+  if (c.nw == NW_ && c.nt == NT_) {                                                                  \
+    hipLaunchKernelGGL((unitary_bwd_kernel<NW_, NT_, TT_, Tin>), grid, dim3(NT_), 0, s, a);          \
+    return launch_status();                                                                          \
+  }
+
+template <typename Tin>
+static int unitary_bwd_t(const UniBwdArgs& a, Cfg c, hipStream_t s) {
+  const dim3 grid((unsigned)(a.B * a.ncg));
+  AUSSM_UBWD_CASE(1, 256, 32) AUSSM_UBWD_CASE(2, 256, 32) AUSSM_UBWD_CASE(4, 256, 32)
+  AUSSM_UBWD_CASE(8, 256, 32) AUSSM_UBWD_CASE(16, 256, 32)
+  AUSSM_UBWD_CASE(1, 512, 16) AUSSM_UBWD_CASE(2, 512, 16) AUSSM_UBWD_CASE(4, 512, 16)
+  AUSSM_UBWD_CASE(8, 512, 16)
+  return -2;
+}
+
+int run_unitary_bwd_generic(const UniBwdArgs& a, int in_dtype, Cfg c, hipStream_t s) {
+  return in_dtype == 1 ? unitary_bwd_t<bf16_t>(a, c, s) : unitary_bwd_t<float>(a, c, s);
+}
+
+#define AUSSM_RBWD_CASE(NW_)                                                                         \
+  if (nw == NW_) {                                                                                   \
+    hipLaunchKernelGGL((recompute_bwd_kernel<VAR, NW_, 256, Tin>), grid, dim3(256), 0, s, a);        \
+    return launch_status();                                                                          \
+  }
+
+template <int VAR, typename Tin>
+static int rec_bwd_t(const RecBwdArgs& a, hipStream_t s) {
+  const dim3 grid((unsigned)(a.B * a.ncg));
+  const int nw = a.N <= 4 ? 1 : (a.N <= 8 ? 2 : 4);
+  AUSSM_RBWD_CASE(1) AUSSM_RBWD_CASE(2) AUSSM_RBWD_CASE(4)
+  return -2;
+}
+
+int run_rec_bwd(int variant, const RecBwdArgs& a, int in_dtype, hipStream_t s) {
+  if (variant == VAR_COMPLEX)
+    return in_dtype == 1 ? rec_bwd_t<VAR_COMPLEX, bf16_t>(a, s) : rec_bwd_t<VAR_COMPLEX, float>(a, s);
+  return in_dtype == 1 ? rec_bwd_t<VAR_REAL, bf16_t>(a, s) : rec_bwd_t<VAR_REAL, float>(a, s);
+}
+
+// marks an auxiliary buffer as NOT filled (a forward kernel that does not fill it ran)
+__global__ void aux_invalidate_kernel(float* tag) { *tag = 0.0f; }
+void run_aux_invalidate(float* tag, hipStream_t s) { hipLaunchKernelGGL(aux_invalidate_kernel, dim3(1), dim3(1), 0, s, tag); }
+
+int run_conv_fwd(const ConvArgs& a, hipStream_t s) {
+  const size_t rows = (size_t)a.B * a.L;
+  const size_t runs = (size_t)a.B * ((a.L + CONV_RUN - 1) / CONV_RUN);
+  if (a.K == 4)
+    hipLaunchKernelGGL(causal_conv1d_k4_fwd_kernel, dim3((unsigned)runs, (unsigned)((a.D + 255) / 256)), dim3(256), 0, s, a);
+  else
+    hipLaunchKernelGGL(causal_conv1d_fwd_kernel, dim3((unsigned)rows, (unsigned)((a.D + 255) / 256)), dim3(256), 0, s, a);
+  return launch_status();
+}
+
+int run_conv_bwd(const ConvArgs& a, hipStream_t s) {
+  const size_t rows = (size_t)a.B * a.L;
+  const dim3 wgrid((unsigned)((a.D + 63) / 64), (unsigned)((rows + CONV_ROWS - 1) / CONV_ROWS));
+  if (a.K == 4) {
+    const size_t runs = (size_t)a.B * ((a.L + CONV_RUN - 1) / CONV_RUN);
+    hipLaunchKernelGGL(causal_conv1d_k4_bwd_data_kernel, dim3((unsigned)runs, (unsigned)((a.D + 255) / 256)), dim3(256), 0, s, a);
+    hipLaunchKernelGGL(causal_conv1d_k4_bwd_weight_kernel, wgrid, dim3(256), 0, s, a);
+  } else {
+    hipLaunchKernelGGL(causal_conv1d_bwd_data_kernel, dim3((unsigned)rows, (unsigned)((a.D + 255) / 256)), dim3(256), 0, s, a);
+    hipLaunchKernelGGL(causal_conv1d_bwd_weight_kernel, wgrid, dim3(256), 0, s, a);
+  }
+  return launch_status();
+}
+
+int run_swap_last2(const SwapArgs& a, int B, hipStream_t s) {
+  hipLaunchKernelGGL(swap_last2_kernel, dim3((unsigned)((a.C + 31) / 32), (unsigned)((a.R + 31) / 32), (unsigned)B), dim3(256), 0, s, a);
+  return launch_status();
+}
+
+}  // namespace aussm

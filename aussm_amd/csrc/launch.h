@@ -1,0 +1,42 @@
+// Launch functions of the library's translation units (one unit per kernel family, so that they
+// compile side by side).  Each enqueues on the given stream and returns AUSSM_OK or the launch's
+// hipError_t; argument checking is done by the callers in scan_api.hip.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include "scan_args.h"
+
+namespace aussm {
+
+inline int launch_status() {
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? 0 : (int)e;
+}
+
+// A workgroup of nt threads (nt / 64 wavefronts) of the vector-ALU kernels owns 64 channels; each
+// wavefront owns nw states.
+struct Cfg { int nw, nt; };
+
+// ---- k_generic.hip: vector-ALU scans, convolution, layout swap
+int run_core_fwd(int variant, const FwdArgs& a, int in_dtype, Cfg c, hipStream_t s);
+int run_unitary_bwd_generic(const UniBwdArgs& a, int in_dtype, Cfg c, hipStream_t s);
+int run_rec_bwd(int variant, const RecBwdArgs& a, int in_dtype, hipStream_t s);
+void run_aux_invalidate(float* tag, hipStream_t s);
+int run_conv_fwd(const ConvArgs& a, hipStream_t s);
+int run_conv_bwd(const ConvArgs& a, hipStream_t s);
+int run_swap_last2(const SwapArgs& a, int B, hipStream_t s);
+
+// ---- k_xdl.hip: matrix-core unitary scans that prepare their operands themselves, and the
+// kernels of the split along L.  mode: operand pieces (2, 3; backward also 5 = three everywhere).
+int run_xdl_fwd(int mode, const FwdArgs& a, int in_dtype, hipStream_t s);
+int run_xdl_bwd(int mode, const UniBwdArgs& a, int in_dtype, hipStream_t s);
+void run_seg_state(bool adjoint, const SegArgs& a, int in_dtype, unsigned grid, hipStream_t s);
+void run_seg_carry_fwd(float* seg, const float* ptot, const float* h0, float* hL, int B, int D, int N, int nf, hipStream_t s);
+void run_seg_carry_bwd(float* seg, const float* ptot, const float* dhL, float* dh0, int B, int D, int N, int nf, hipStream_t s);
+
+// ---- k_px.hip: matrix-core unitary scans on operands prepared by a pre-pass
+void run_px_prep(const PrepArgs& a, int B, int in_dtype, hipStream_t s);
+int run_px_fwd(const FwdArgs& a, const u4* img, int in_dtype, hipStream_t s);
+int run_px_bwd(const UniBwdArgs& a, const u4* img, int in_dtype, hipStream_t s);
+
+}  // namespace aussm

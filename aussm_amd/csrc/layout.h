@@ -6,14 +6,10 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
+#include "scan_args.h"
+
 namespace aussm {
 
-struct SwapArgs {
-  const float* x;      // element (b, r, c) at x[b * xs_b + r * xs_r + c]
-  float* y;            // [B, C, R] contiguous
-  long long xs_b, xs_r;
-  int R, C;
-};
 
 __global__ __launch_bounds__(256) void swap_last2_kernel(const SwapArgs p) {
   __shared__ float tile[32][33];

@@ -3,37 +3,29 @@
 #include "../../include/aussm_hip.h"
 
 #include <hip/hip_runtime.h>
-#include <stdio.h>
-#include <stdlib.h>
+#include <atomic>
 
-#include "conv1d.h"
-#include "layout.h"
-#include "scan_bwd_recompute.h"
-#include "scan_bwd_unitary.h"
-#include "scan_bwd_xdl.h"
-#include "scan_common.h"
-#include "scan_fwd.h"
-#include "scan_fwd_mfma.h"
-#include "scan_fwd_xdl.h"
-#include "scan_fwd_xdl2.h"
-#include "scan_seg_xdl.h"
+#include "launch.h"
+#include "scan_args.h"
 
 using namespace aussm;
 
 namespace {
 
-// ---- kernel configuration -------------------------------------------------------------------
-// A workgroup of NT threads (NT/64 wavefronts) owns 64 channels; each wavefront owns NW states.
+// Process-wide options (aussm_set_option): kernel selection for comparisons and tuning.  They are
+// plain atomics read once per call; -1 means "let the launcher decide".
+std::atomic<int> g_opt[AUSSM_OPT_COUNT] = {{-1}, {-1}, {-1}, {-1}, {-1}};
+inline int opt(int key) { return g_opt[key].load(std::memory_order_relaxed); }
+
+// ---- configuration of the vector-ALU kernels --------------------------------------------------
 // The scalar loads of B_t/C_t are issued one "turn" ahead; with two or more wavefronts per SIMD
 // the turn of another wavefront doubles that distance, so for a given N the configuration with
 // MORE wavefronts (smaller NW) is preferred as long as the launch still fits one workgroup.
-struct Cfg { int nw, nt; };
-
 inline Cfg pick_cfg(int N, int max_waves) {
-  // test/tuning override: AUSSM_CFG="NW,NT" (must be one of the compiled configurations)
-  if (const char* e = getenv("AUSSM_CFG")) {
-    Cfg c{0, 0};
-    if (sscanf(e, "%d,%d", &c.nw, &c.nt) == 2 && c.nw > 0 && c.nw * (c.nt / 64) >= N) return c;
+  // test/tuning override (must be one of the compiled configurations)
+  {
+    const Cfg c{opt(AUSSM_OPT_GENERIC_NW), opt(AUSSM_OPT_GENERIC_NT)};
+    if (c.nw > 0 && c.nt > 0 && c.nw * (c.nt / 64) >= N) return c;
   }
   const Cfg table[] = {{1, 256}, {1, 512}, {2, 512}, {4, 512}, {8, 512},
                        {2, 256}, {4, 256}, {8, 256}, {16, 256}};
@@ -58,56 +50,36 @@ constexpr int REC_CK = AUSSM_TILE / 2;
 
 inline bool misaligned(const void* p, size_t a) { return p && (reinterpret_cast<uintptr_t>(p) % a) != 0; }
 
-inline int launch_status() {
-  hipError_t e = hipGetLastError();
-  return e == hipSuccess ? AUSSM_OK : (int)e;
-}
-
-#define AUSSM_FWD_CASE(NW_, NT_)                                                                     \
-  if (c.nw == NW_ && c.nt == NT_) {                                                                  \
-    hipLaunchKernelGGL((core_fwd_kernel<VAR, NW_, NT_, Tin>), grid, dim3(NT_), 0, s, a);             \
-    return launch_status();                                                                          \
-  }
-
-template <int VAR, typename Tin>
-int launch_fwd_t(const FwdArgs& a, hipStream_t s) {
-  const dim3 grid((unsigned)(a.B * a.ncg));
-  const Cfg c = pick_cfg(a.N, 8);
-  AUSSM_FWD_CASE(1, 256) AUSSM_FWD_CASE(2, 256) AUSSM_FWD_CASE(4, 256) AUSSM_FWD_CASE(8, 256)
-  AUSSM_FWD_CASE(16, 256) AUSSM_FWD_CASE(1, 512) AUSSM_FWD_CASE(2, 512) AUSSM_FWD_CASE(4, 512)
-  AUSSM_FWD_CASE(8, 512)
-  return AUSSM_E_SHAPE;
-}
-
 // The matrix-core kernels cover the common unitary case (fp32 or bf16 inputs, 6 <= N <= 16, L a multiple of 4,
 // 16-byte aligned tensors, checkpoint interval a multiple of 32); everything else takes the
-// generic kernels.  AUSSM_MFMA (environment, read at every call) selects the forward kernel for
-// comparisons: 0 generic, 1 fp32 matrix instructions, 2 / 3 bf16 matrix instructions on two- /
-// three-piece operands with one wavefront per SIMD (3 is the default), 4 three-piece operands with
-// two wavefronts per SIMD.  AUSSM_MFMA_BWD: 0 generic, 2 two pieces everywhere, 3 (default) three
-// pieces along the sequence and two in the sums over the channel (dB, dC), 5 three pieces everywhere.
-// marks an auxiliary buffer as NOT filled (a forward kernel that does not fill it ran)
-__global__ void aux_invalidate_kernel(float* tag) { *tag = 0.0f; }
-
-// The matrix-core kernels cost the same for every N <= 16 while the generic ones scale with N:
-// measured, the crossover is between N = 4 (generic 15 % faster) and N = 8 (matrix 30 % faster).
+// vector-ALU kernels.  aussm_set_option(AUSSM_OPT_UNITARY_FWD, m) selects the forward kernel for
+// comparisons: 0 vector ALU, 2 / 3 bf16 matrix instructions on two- / three-piece operands built
+// inside the scan kernel, 6 three-piece operands prepared by a pre-pass, two wavefronts per SIMD
+// (the default when the call brings the workspace for them, i.e. an auxiliary buffer; builds with
+// AUSSM_EXPERIMENTAL_KERNELS also know 1 = fp32 matrix instructions and 4).
+// AUSSM_OPT_UNITARY_BWD: 0 vector ALU, 2 two pieces everywhere, 3 three pieces along the sequence
+// and two in the sums over the channel (dB, dC), 5 three pieces everywhere, 6 prepared operands.
+//
+// The matrix-core kernels cost the same for every N <= 16 while the vector-ALU ones scale with N:
+// measured, the crossover is between N = 4 (vector ALU 15 % faster) and N = 8 (matrix 30 % faster).
 constexpr int MATRIX_MIN_STATE = 6;
-inline int env_mode(const char* name, int dflt, int N) {
-  const char* e = getenv(name);
-  if (e) return atoi(e);                       // an explicit choice is honoured for every N <= 16
+inline int kernel_mode(int key, int dflt, int N) {
+  const int e = opt(key);
+  if (e >= 0) return e;                        // an explicit choice is honoured for every N <= 16
   return N >= MATRIX_MIN_STATE ? dflt : 0;
 }
 // Splitting the sequence (scan_seg_xdl.h): with few (batch, channel group) pairs the launch would
 // leave most of the chip idle, so the sequence is cut into ns segments of whole checkpoint blocks
 // until about one workgroup per compute unit exists.  Only the matrix-core kernels take part,
 // and only the *_aux entry points (the segment states live behind the auxiliary buffer).
-// AUSSM_SPLIT (environment): 0 or 1 switches it off, a power of two caps ns.
+// aussm_set_option(AUSSM_OPT_SPLIT_CAP, c): 0 or 1 switches it off, a power of two caps ns.
 constexpr int SPLIT_MIN_WGS = 129;     // launches of at least this many workgroups are left alone
 constexpr int SPLIT_TARGET_WGS = 256;
 constexpr int SPLIT_MAX = 32;
 constexpr int SPLIT_MIN_LEN = 128;
+inline bool matrix_shape(int N, int L, int ck) { return N <= XN && L % 4 == 0 && ck >= XT && ck % XT == 0; }
 inline int seg_capacity(int B, int D, int N, int L, int ck) {
-  if (N < MATRIX_MIN_STATE || N > XN || L % 4 != 0 || ck < XT || ck % XT != 0 || L % ck != 0) return 1;
+  if (N < MATRIX_MIN_STATE || !matrix_shape(N, L, ck) || L % ck != 0) return 1;
   const long long wgs = (long long)B * ((D + CH - 1) / CH);
   if (wgs >= SPLIT_MIN_WGS) return 1;
   const int nblk = L / ck, target = (int)(SPLIT_TARGET_WGS / wgs);
@@ -117,10 +89,9 @@ inline int seg_capacity(int B, int D, int N, int L, int ck) {
 }
 inline int seg_count(int B, int D, int N, int L, int ck) {
   int ns = seg_capacity(B, D, N, L, ck);
-  if (const char* e = getenv("AUSSM_SPLIT")) {
-    const int cap = atoi(e);
+  const int cap = opt(AUSSM_OPT_SPLIT_CAP);
+  if (cap >= 0)
     while (ns > 1 && ns > cap) ns /= 2;
-  }
   return ns;
 }
 // The segment states are computed on finer segments than the scan proper uses (the kernel that
@@ -132,102 +103,69 @@ inline int seg_fine(int L, int ns) {
     if (Ls % (r * XT) == 0 && Ls / r >= SPLIT_MIN_LEN) return r;
   return 1;
 }
+inline size_t round64(size_t n) { return (n + 63) & ~(size_t)63; }
 inline size_t seg_floats(int B, int D, int N, int L, int ns) {
-  return ns > 1 ? (size_t)B * ns * seg_fine(L, ns) * D * (2 * N + 2) : 0;
+  return ns > 1 ? round64((size_t)B * ns * seg_fine(L, ns) * D * (2 * N + 2)) : 0;
+}
+// Workspace of the prepared operands: one image per (batch element, chunk), sized for the larger
+// (backward) image; a forward and a backward call each write their own images into it.
+inline size_t img_floats(int B, int N, int L, int ck) {
+  if (!matrix_shape(N, L, ck)) return 0;
+  // (below MATRIX_MIN_STATE only when the prepared-operand kernels have been asked for explicitly)
+  if (N < MATRIX_MIN_STATE && opt(AUSSM_OPT_UNITARY_FWD) != 6 && opt(AUSSM_OPT_UNITARY_BWD) != 6) return 0;
+  return (size_t)B * ((L + XT - 1) / XT) * PXB_REC * 4;
+}
+// Layout of the auxiliary buffer: [B*D*L floats Im(P S)] [AUX_PAD] [segment states] [images]
+struct AuxLayout { float* seg; u4* img; };
+inline AuxLayout aux_layout(float* aux, int B, int D, int N, int L, int ck) {
+  if (!aux) return AuxLayout{nullptr, nullptr};
+  float* seg = aux + (size_t)B * D * L + AUX_PAD;
+  float* img = seg + seg_floats(B, D, N, L, seg_capacity(B, D, N, L, ck));
+  return AuxLayout{seg, img_floats(B, N, L, ck) ? reinterpret_cast<u4*>(img) : nullptr};
 }
 
-inline int mfma_fwd_mode(const FwdArgs& a, int in_dtype) {
-  int mode = env_mode("AUSSM_MFMA", 3, a.N);
-  if (mode <= 0 || a.urep != 1 || a.N > MN || a.L % 4 != 0 || a.ck % MT != 0) return 0;
-  if (in_dtype != AUSSM_F32) mode = 3;       // bf16 inputs: the default matrix-core kernel only
+inline int mfma_fwd_mode(const FwdArgs& a, int in_dtype, bool have_img) {
+  int mode = kernel_mode(AUSSM_OPT_UNITARY_FWD, have_img ? 6 : 3, a.N);
+  if (mode <= 0 || a.urep != 1 || !matrix_shape(a.N, a.L, a.ck)) return 0;
+  if (mode == 6 && !have_img) mode = 3;
+  if (in_dtype != AUSSM_F32 && mode != 6) mode = 3;       // bf16 inputs: three-piece kernels only
   if (misaligned(a.u, 16) || misaligned(a.delta, 16) || misaligned(a.theta, 16) || misaligned(a.z, 16) ||
       misaligned(a.y, 16) || misaligned(a.Bm, 16) || misaligned(a.Cm, 16))
     return 0;
   return mode;
 }
 
-template <int VAR>
-int launch_fwd(FwdArgs a, int in_dtype, hipStream_t s) {
-  const int mode = (VAR == VAR_UNITARY) ? mfma_fwd_mode(a, in_dtype) : 0;
-  if (a.aux && mode <= 1)   // this call will not fill the auxiliary buffer
-    hipLaunchKernelGGL(aux_invalidate_kernel, dim3(1), dim3(1), 0, s, a.aux + (size_t)a.B * a.D * a.L);
-  if (mode) {
-    if ((mode == 2 || mode == 3) && a.aux) {
-      const int ns = seg_count(a.B, a.D, a.N, a.L, a.ck);
-      if (ns > 1) {
-        // 1. end state of every segment from a zero start and its rotation; 2. chain them;
-        // 3. the scan proper over (batch, segment) pairs, each from its true incoming state
-        const int B = a.B, L = a.L, Ls = a.L / ns, r = seg_fine(L, ns), nf = ns * r;
-        float* seg = a.aux + (size_t)B * a.D * L + AUX_PAD;
-        float* ptot = seg + (size_t)B * nf * a.D * a.N * 2;
-        SegArgs sa{a.delta, a.u, a.theta, a.Bm, seg, ptot, a.D, a.N, Ls / r, L, nf, a.ncg};
-        const dim3 sgrid((unsigned)(B * nf * a.ncg));
-        if (in_dtype == AUSSM_BF16) hipLaunchKernelGGL((unitary_seg_state_kernel<3, false, bf16_t>), sgrid, dim3(256), 0, s, sa);
-        else hipLaunchKernelGGL((unitary_seg_state_kernel<3, false>), sgrid, dim3(256), 0, s, sa);
-        const size_t nst = (size_t)B * a.D * a.N;
-        hipLaunchKernelGGL(seg_carry_fwd_kernel, dim3((unsigned)((nst + 255) / 256)), dim3(256), 0, s, seg, ptot, a.h0,
-                           a.hL, B, a.D, a.N, nf);
-        a.B = B * ns; a.L = Ls; a.ns = ns; a.nck = Ls / a.ck; a.h0 = seg; a.hL = nullptr; a.hs = r; a.ho = 0;
-      }
+// ws: workspace of the call (segment states for a launch that is split along L, images of the
+// prepared operands); either part may be null.
+int launch_unitary_fwd(FwdArgs a, int in_dtype, hipStream_t s, AuxLayout ws) {
+  const int mode = mfma_fwd_mode(a, in_dtype, ws.img != nullptr);
+  // Im(P S) is only worth writing when a backward call can follow (it needs the checkpoints too);
+  // a call that does not fill the buffer marks it as not filled
+  const bool fill = a.aux && a.hck && mode >= 2;
+  if (a.aux && !fill) run_aux_invalidate(a.aux + (size_t)a.B * a.D * a.L, s);
+  if (!fill) a.aux = nullptr;
+  if (!mode) return run_core_fwd(VAR_UNITARY, a, in_dtype, pick_cfg(a.N, 8), s);
+  const int B = a.B, L = a.L;
+  if ((mode == 2 || mode == 3 || mode == 6) && ws.seg) {
+    const int ns = seg_count(B, a.D, a.N, L, a.ck);
+    if (ns > 1) {
+      // 1. end state of every segment from a zero start and its rotation; 2. chain them;
+      // 3. the scan proper over (batch, segment) pairs, each from its true incoming state
+      const int Ls = L / ns, r = seg_fine(L, ns), nf = ns * r;
+      float* seg = ws.seg;
+      float* ptot = seg + (size_t)B * nf * a.D * a.N * 2;
+      SegArgs sa{a.delta, a.u, a.theta, a.Bm, seg, ptot, a.D, a.N, Ls / r, L, nf, a.ncg};
+      run_seg_state(false, sa, in_dtype, (unsigned)(B * nf * a.ncg), s);
+      run_seg_carry_fwd(seg, ptot, a.h0, a.hL, B, a.D, a.N, nf, s);
+      a.B = B * ns; a.L = Ls; a.ns = ns; a.nck = Ls / a.ck; a.h0 = seg; a.hL = nullptr; a.hs = r; a.ho = 0;
     }
-    const dim3 grid((unsigned)(a.B * a.ncg));
-    if (mode == 1) {
-      if (a.z) hipLaunchKernelGGL(unitary_fwd_mfma_kernel<true>, grid, dim3(256), 0, s, a);
-      else hipLaunchKernelGGL(unitary_fwd_mfma_kernel<false>, grid, dim3(256), 0, s, a);
-    } else if (mode == 2) {
-      if (a.z) hipLaunchKernelGGL((unitary_fwd_xdl_kernel<2, true>), grid, dim3(256), 0, s, a);
-      else hipLaunchKernelGGL((unitary_fwd_xdl_kernel<2, false>), grid, dim3(256), 0, s, a);
-    } else if (mode == 4) {
-      if (a.z) hipLaunchKernelGGL((unitary_fwd_xdl2_kernel<3, true>), grid, dim3(512), 0, s, a);
-      else hipLaunchKernelGGL((unitary_fwd_xdl2_kernel<3, false>), grid, dim3(512), 0, s, a);
-    } else if (in_dtype == AUSSM_BF16) {
-      if (a.z) hipLaunchKernelGGL((unitary_fwd_xdl_kernel<3, true, bf16_t>), grid, dim3(256), 0, s, a);
-      else hipLaunchKernelGGL((unitary_fwd_xdl_kernel<3, false, bf16_t>), grid, dim3(256), 0, s, a);
-    } else {
-      if (a.z) hipLaunchKernelGGL((unitary_fwd_xdl_kernel<3, true>), grid, dim3(256), 0, s, a);
-      else hipLaunchKernelGGL((unitary_fwd_xdl_kernel<3, false>), grid, dim3(256), 0, s, a);
-    }
-    return launch_status();
   }
-  return in_dtype == AUSSM_BF16 ? launch_fwd_t<VAR, bf16_t>(a, s) : launch_fwd_t<VAR, float>(a, s);
-}
-
-// The backward workgroup keeps a (dw, dtheta) slab per wavefront in LDS: four wavefronts afford
-// 32-step tiles, eight wavefronts 16-step tiles.
-#define AUSSM_UBWD_CASE(NW_, NT_, TT_)                                                               \
-  if (c.nw == NW_ && c.nt == NT_) {                                                                  \
-    hipLaunchKernelGGL((unitary_bwd_kernel<NW_, NT_, TT_, Tin>), grid, dim3(NT_), 0, s, a);          \
-    return launch_status();                                                                          \
+  if (mode == 6) {
+    PrepArgs pa{a.Bm, a.Cm, ws.img, nullptr, a.N, L, (L + XT - 1) / XT};
+    run_px_prep(pa, B, in_dtype, s);
+    return run_px_fwd(a, ws.img, in_dtype, s);
   }
-
-template <typename Tin>
-int launch_unitary_bwd_t(const UniBwdArgs& a, hipStream_t s) {
-  const dim3 grid((unsigned)(a.B * a.ncg));
-  const Cfg c = pick_cfg(a.N, 8);
-  AUSSM_UBWD_CASE(1, 256, 32) AUSSM_UBWD_CASE(2, 256, 32) AUSSM_UBWD_CASE(4, 256, 32)
-  AUSSM_UBWD_CASE(8, 256, 32) AUSSM_UBWD_CASE(16, 256, 32)
-  AUSSM_UBWD_CASE(1, 512, 16) AUSSM_UBWD_CASE(2, 512, 16) AUSSM_UBWD_CASE(4, 512, 16)
-  AUSSM_UBWD_CASE(8, 512, 16)
-  return AUSSM_E_SHAPE;
-}
-
-#define AUSSM_RBWD_CASE(NW_)                                                                         \
-  if (nw == NW_) {                                                                                   \
-    hipLaunchKernelGGL((recompute_bwd_kernel<VAR, NW_, 256, Tin>), grid, dim3(256), 0, s, a);        \
-    return launch_status();                                                                          \
-  }
-
-template <int VAR, typename Tin>
-int launch_rec_bwd_t(const RecBwdArgs& a, hipStream_t s) {
-  const dim3 grid((unsigned)(a.B * a.ncg));
-  const int nw = a.N <= 4 ? 1 : (a.N <= 8 ? 2 : 4);
-  AUSSM_RBWD_CASE(1) AUSSM_RBWD_CASE(2) AUSSM_RBWD_CASE(4)
-  return AUSSM_E_SHAPE;
-}
-
-template <int VAR>
-int launch_rec_bwd(const RecBwdArgs& a, int in_dtype, hipStream_t s) {
-  return in_dtype == AUSSM_BF16 ? launch_rec_bwd_t<VAR, bf16_t>(a, s) : launch_rec_bwd_t<VAR, float>(a, s);
+  return run_xdl_fwd(mode, a, in_dtype, s);
 }
 
 }  // namespace
@@ -248,6 +186,17 @@ const char* aussm_error_string(int code) {
   }
 }
 
+int aussm_set_option(int key, int value) {
+  if (key < 0 || key >= AUSSM_OPT_COUNT) return AUSSM_E_SHAPE;
+  g_opt[key].store(value < 0 ? -1 : value, std::memory_order_relaxed);
+  return AUSSM_OK;
+}
+
+int aussm_get_option(int key) {
+  if (key < 0 || key >= AUSSM_OPT_COUNT) return AUSSM_E_SHAPE;
+  return opt(key);
+}
+
 int aussm_num_checkpoints(int L, int ck) { return (L < 1 || ck < 1) ? 0 : (L + ck - 1) / ck; }
 
 int aussm_bwd_checkpoint_interval(int variant) { return variant == VAR_UNITARY ? 0 : REC_CK; }
@@ -258,7 +207,7 @@ int aussm_unitary_split_segments(int B, int D, int N, int L, int ck) {
 
 size_t aussm_unitary_aux_floats(int B, int D, int N, int L, int ck) {
   if (B < 1 || D < 1 || N < 1 || L < 1) return 0;
-  return (size_t)B * D * L + AUX_PAD + seg_floats(B, D, N, L, seg_capacity(B, D, N, L, ck));
+  return (size_t)B * D * L + AUX_PAD + seg_floats(B, D, N, L, seg_capacity(B, D, N, L, ck)) + img_floats(B, N, L, ck);
 }
 
 int aussm_unitary_fwd(const void* u, const void* delta, const float* theta, const void* Bc, const void* Cc,
@@ -282,7 +231,7 @@ int aussm_unitary_fwd_aux(const void* u, const void* delta, const float* theta, 
   a.h0 = h0; a.y = y; a.hL = hL; a.hck = hck; a.aux = aux;
   a.B = B; a.D = D; a.N = N; a.L = L; a.ck = ck; a.nck = (L + ck - 1) / ck; a.ncg = (D + CH - 1) / CH;
   a.ld = L; a.ns = 1; a.hs = 1; a.ho = 0; a.urep = urep;
-  return launch_fwd<VAR_UNITARY>(a, in_dtype, (hipStream_t)stream);
+  return launch_unitary_fwd(a, in_dtype, (hipStream_t)stream, aux_layout(aux, B, D, N, L, ck));
 }
 
 int aussm_complex_fwd(const void* u, const void* delta, const float* rho, const float* theta, const void* Bc,
@@ -297,7 +246,7 @@ int aussm_complex_fwd(const void* u, const void* delta, const float* rho, const 
   a.h0 = h0; a.y = y; a.hL = hL; a.hck = hck;
   a.B = B; a.D = D; a.N = N; a.L = L; a.ck = ck; a.nck = (L + ck - 1) / ck; a.ncg = (D + CH - 1) / CH;
   a.ld = L; a.ns = 1; a.hs = 1; a.ho = 0; a.urep = 1;
-  return launch_fwd<VAR_COMPLEX>(a, in_dtype, (hipStream_t)stream);
+  return run_core_fwd(VAR_COMPLEX, a, in_dtype, pick_cfg(a.N, 8), (hipStream_t)stream);
 }
 
 int aussm_real_fwd(const void* u, const void* delta, const float* A, const void* Bm, const void* Cm,
@@ -312,7 +261,7 @@ int aussm_real_fwd(const void* u, const void* delta, const float* A, const void*
   a.h0 = h0; a.y = y; a.hL = hL; a.hck = hck;
   a.B = B; a.D = D; a.N = N; a.L = L; a.ck = ck; a.nck = (L + ck - 1) / ck; a.ncg = (D + CH - 1) / CH;
   a.ld = L; a.ns = 1; a.hs = 1; a.ho = 0; a.urep = 1;
-  return launch_fwd<VAR_REAL>(a, in_dtype, (hipStream_t)stream);
+  return run_core_fwd(VAR_REAL, a, in_dtype, pick_cfg(a.N, 8), (hipStream_t)stream);
 }
 
 int aussm_unitary_bwd(const float* dy, const float* dhL, const void* u, const void* delta, const float* theta,
@@ -340,9 +289,11 @@ int aussm_unitary_bwd_aux(const float* dy, const float* dhL, const void* u, cons
   a.hck = hck; a.aux = aux; a.du = du; a.ddelta = ddelta; a.dtheta = dtheta; a.dB = dB; a.dC = dC; a.dD = dD; a.dh0 = dh0;
   a.B = B; a.D = D; a.N = N; a.L = L; a.ck = ck; a.nck = (L + ck - 1) / ck; a.ncg = (D + CH - 1) / CH;
   a.ld = L; a.ns = 1; a.hs = 1; a.ho = 0; a.urep = 1;
-  const int mode = env_mode("AUSSM_MFMA_BWD", 3, N);   // matrix-core kernel for the common case
   a.urep = urep;
-  if (mode > 0 && urep == 1 && N <= XN && L % 4 == 0 && ck % XT == 0 &&
+  const AuxLayout ws = aux_layout(aux, B, D, N, L, ck);
+  int mode = kernel_mode(AUSSM_OPT_UNITARY_BWD, ws.img ? 6 : 3, N);   // matrix-core kernels for the common case
+  if (mode == 6 && !ws.img) mode = 3;
+  if (mode > 0 && urep == 1 && matrix_shape(N, L, ck) &&
       !(misaligned(dy, 16) || misaligned(u, 16) || misaligned(delta, 16) || misaligned(theta, 16) ||
         misaligned(du, 16) || misaligned(ddelta, 16) || misaligned(dtheta, 16) || misaligned(Bc, 16) ||
         misaligned(Cc, 16))) {
@@ -350,26 +301,22 @@ int aussm_unitary_bwd_aux(const float* dy, const float* dhL, const void* u, cons
     if (ns > 1) {
       // adjoint at the start of every segment from a zero adjoint at its end, chained last to first
       const int Ls = L / ns, r = seg_fine(L, ns), nf = ns * r;
-      float* seg = aux + (size_t)B * D * L + AUX_PAD;
+      float* seg = ws.seg;
       float* ptot = seg + (size_t)B * nf * D * N * 2;
       SegArgs sa{dy, nullptr, theta, Cc, seg, ptot, D, N, Ls / r, L, nf, a.ncg};
-      const dim3 sgrid((unsigned)(B * nf * a.ncg));
-      if (in_dtype == AUSSM_BF16) hipLaunchKernelGGL((unitary_seg_state_kernel<3, true, bf16_t>), sgrid, dim3(256), 0, s, sa);
-      else hipLaunchKernelGGL((unitary_seg_state_kernel<3, true>), sgrid, dim3(256), 0, s, sa);
-      const size_t nst = (size_t)B * D * N;
-      hipLaunchKernelGGL(seg_carry_bwd_kernel, dim3((unsigned)((nst + 255) / 256)), dim3(256), 0, s, seg, ptot, dhL, dh0,
-                         B, D, N, nf);
+      run_seg_state(true, sa, in_dtype, (unsigned)(B * nf * a.ncg), s);
+      run_seg_carry_bwd(seg, ptot, dhL, dh0, B, D, N, nf, s);
       // a segment of the scan ends where its last fine segment ends
       a.B = B * ns; a.L = Ls; a.ns = ns; a.nck = Ls / ck; a.dhL = seg; a.dh0 = nullptr; a.hs = r; a.ho = r - 1;
     }
-    const dim3 grid((unsigned)(a.B * a.ncg));
-    if (in_dtype == AUSSM_BF16) hipLaunchKernelGGL((unitary_bwd_xdl_kernel<3, 2, bf16_t>), grid, dim3(256), 0, s, a);
-    else if (mode == 2) hipLaunchKernelGGL((unitary_bwd_xdl_kernel<2, 2>), grid, dim3(256), 0, s, a);
-    else if (mode == 5) hipLaunchKernelGGL((unitary_bwd_xdl_kernel<3, 3>), grid, dim3(256), 0, s, a);
-    else hipLaunchKernelGGL((unitary_bwd_xdl_kernel<3, 2>), grid, dim3(256), 0, s, a);
-    return launch_status();
+    if (mode == 6) {
+      PrepArgs pa{Bc, Cc, nullptr, ws.img, N, L, (L + XT - 1) / XT};
+      run_px_prep(pa, B, in_dtype, s);
+      return run_px_bwd(a, ws.img, in_dtype, s);
+    }
+    return run_xdl_bwd(mode, a, in_dtype, s);
   }
-  return in_dtype == AUSSM_BF16 ? launch_unitary_bwd_t<bf16_t>(a, s) : launch_unitary_bwd_t<float>(a, s);
+  return run_unitary_bwd_generic(a, in_dtype, pick_cfg(a.N, 8), s);
 }
 
 int aussm_complex_bwd(const float* dy, const float* dhL, const void* u, const void* delta, const float* rho,
@@ -391,7 +338,7 @@ int aussm_complex_bwd(const float* dy, const float* dhL, const void* u, const vo
   a.Dskip = Dskip; a.h0 = h0; a.hck = hck;
   a.du = du; a.ddelta = ddelta; a.dtheta = dtheta; a.drho = drho; a.dB = dB; a.dC = dC; a.dD = dD; a.dh0 = dh0;
   a.B = B; a.D = D; a.N = N; a.L = L; a.nck = (L + ck - 1) / ck; a.ncg = (D + CH - 1) / CH;
-  return launch_rec_bwd<VAR_COMPLEX>(a, in_dtype, (hipStream_t)stream);
+  return run_rec_bwd(VAR_COMPLEX, a, in_dtype, (hipStream_t)stream);
 }
 
 int aussm_real_bwd(const float* dy, const float* dhL, const void* u, const void* delta, const float* A,
@@ -408,7 +355,7 @@ int aussm_real_bwd(const float* dy, const float* dhL, const void* u, const void*
   a.delta_bias = delta_bias; a.delta_softplus = delta_softplus; a.h0 = h0; a.hck = hck;
   a.du = du; a.ddelta = ddelta; a.dA = dA; a.dB = dB; a.dC = dC; a.dD = dD; a.dh0 = dh0;
   a.B = B; a.D = D; a.N = N; a.L = L; a.nck = (L + ck - 1) / ck; a.ncg = (D + CH - 1) / CH;
-  return launch_rec_bwd<VAR_REAL>(a, in_dtype, (hipStream_t)stream);
+  return run_rec_bwd(VAR_REAL, a, in_dtype, (hipStream_t)stream);
 }
 
 int aussm_causal_conv1d_fwd(const float* x, const float* w, const float* bias, float* y,
@@ -420,14 +367,7 @@ int aussm_causal_conv1d_fwd(const float* x, const float* w, const float* bias, f
   a.x = x; a.w = w; a.bias = bias; a.y = y; a.xs_b = xs_b; a.xs_l = xs_l; a.B = B; a.L = L; a.D = D; a.K = K;
   const size_t rows = (size_t)B * L;
   if (rows > 0x7fffffffULL || (D + 255) / 256 > 65535) return AUSSM_E_SHAPE;
-  const size_t runs = (size_t)B * ((L + CONV_RUN - 1) / CONV_RUN);
-  if (K == 4)
-    hipLaunchKernelGGL(causal_conv1d_k4_fwd_kernel, dim3((unsigned)runs, (unsigned)((D + 255) / 256)), dim3(256), 0,
-                       (hipStream_t)stream, a);
-  else
-    hipLaunchKernelGGL(causal_conv1d_fwd_kernel, dim3((unsigned)rows, (unsigned)((D + 255) / 256)), dim3(256), 0,
-                       (hipStream_t)stream, a);
-  return launch_status();
+  return run_conv_fwd(a, (hipStream_t)stream);
 }
 
 int aussm_causal_conv1d_bwd(const float* dy, const float* x, const float* w, float* dx, float* dw, float* dbias,
@@ -440,17 +380,7 @@ int aussm_causal_conv1d_bwd(const float* dy, const float* x, const float* w, flo
   a.xs_b = xs_b; a.xs_l = xs_l; a.B = B; a.L = L; a.D = D; a.K = K;
   const size_t rows = (size_t)B * L;
   if (rows > 0x7fffffffULL || (D + 255) / 256 > 65535 || (rows + CONV_ROWS - 1) / CONV_ROWS > 65535) return AUSSM_E_SHAPE;
-  hipStream_t s = (hipStream_t)stream;
-  const dim3 wgrid((unsigned)((D + 63) / 64), (unsigned)((rows + CONV_ROWS - 1) / CONV_ROWS));
-  if (K == 4) {
-    const size_t runs = (size_t)B * ((L + CONV_RUN - 1) / CONV_RUN);
-    hipLaunchKernelGGL(causal_conv1d_k4_bwd_data_kernel, dim3((unsigned)runs, (unsigned)((D + 255) / 256)), dim3(256), 0, s, a);
-    hipLaunchKernelGGL(causal_conv1d_k4_bwd_weight_kernel, wgrid, dim3(256), 0, s, a);
-  } else {
-    hipLaunchKernelGGL(causal_conv1d_bwd_data_kernel, dim3((unsigned)rows, (unsigned)((D + 255) / 256)), dim3(256), 0, s, a);
-    hipLaunchKernelGGL(causal_conv1d_bwd_weight_kernel, wgrid, dim3(256), 0, s, a);
-  }
-  return launch_status();
+  return run_conv_bwd(a, (hipStream_t)stream);
 }
 
 int aussm_swap_last2(const float* x, float* y, int B, int R, int C, long long xs_b, long long xs_r, void* stream) {
@@ -458,9 +388,7 @@ int aussm_swap_last2(const float* x, float* y, int B, int R, int C, long long xs
   if ((R + 31) / 32 > 65535) return AUSSM_E_SHAPE;
   if (!x || !y) return AUSSM_E_NULL;
   SwapArgs a{x, y, xs_b, xs_r, R, C};
-  hipLaunchKernelGGL(swap_last2_kernel, dim3((unsigned)((C + 31) / 32), (unsigned)((R + 31) / 32), (unsigned)B), dim3(256), 0,
-                     (hipStream_t)stream, a);
-  return launch_status();
+  return run_swap_last2(a, B, (hipStream_t)stream);
 }
 
 }  // extern "C"

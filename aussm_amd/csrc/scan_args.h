@@ -1,0 +1,141 @@
+// Argument blocks of the kernels and the constants the host side shares with them.  Plain data
+// only: every translation unit of the library includes this header, the kernel headers are
+// included by the one unit that instantiates their kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace aussm {
+
+constexpr int CH = 64;        // channels per workgroup == lanes per wavefront
+constexpr int XT = 32;        // timesteps per chunk of the matrix-core kernels
+constexpr int XN = 16;        // state rows of the matrix tiles (N is zero-padded up to it)
+
+enum { VAR_UNITARY = 0, VAR_COMPLEX = 1, VAR_REAL = 2 };
+
+// The optional auxiliary buffer of the unitary scan holds B*D*L floats followed by AUX_PAD floats;
+// the first of those is AUX_TAG when a forward kernel has filled the buffer, anything else if not.
+constexpr uint32_t AUX_TAG = 0x4f484950u;
+constexpr int AUX_PAD = 64;
+
+typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+
+struct FwdArgs {
+  const void* u;            // [B,D,L]  Tin
+  const void* delta;        // [B,D,L]  Tin
+  const float* theta;       // [B,D,L]  (unitary, complex)
+  const float* rho;         // [B,D,L]  (complex)
+  const float* A;           // [D,N]    (real)
+  const void* Bm;           // [B,N,L(,2)] Tin
+  const void* Cm;           // [B,N,L(,2)] Tin
+  const float* Dskip;       // [D] or null
+  const float* z;           // [B,D,L] or null
+  const float* delta_bias;  // [D] or null (real)
+  const float* h0;          // [B,D,N,C] or null
+  float* y;                 // [B,D,L] or null
+  float* hL;                // [B,D,N,C] or null
+  float* hck;               // [B,nck,N,C,D] or null
+  float* aux;               // unitary, optional: Im(P_t S_t) [B,D,L] followed by a validity tag
+  int B, D, N, L, ck, nck, ncg, delta_softplus;
+  int ld, ns;                // matrix-core unitary kernels: row stride of the [.., L] tensors and segments per
+                             // sequence (B then counts batch x segment pairs and L is the segment length)
+  int hs, ho;                // ... and h0 of pair b is entry b * hs + ho of the state array
+  int urep;                  // generic kernels: u and delta are [B / urep, D, L], shared by urep consecutive batch elements
+};
+
+struct UniBwdArgs {
+  const float* dy;      // [B,D,L]
+  const float* dhL;     // [B,D,N,2] or null
+  const void* u;        // [B,D,L] Tin
+  const void* delta;    // [B,D,L] Tin
+  const float* theta;   // [B,D,L]
+  const void* Bm;       // [B,N,L,2] Tin
+  const void* Cm;       // [B,N,L,2] Tin
+  const float* Dskip;   // [D] or null
+  const float* hck;     // [B,nck,N,2,D]
+  const float* aux;     // optional: what the forward call left in its aux buffer
+  float *du, *ddelta, *dtheta;   // [B,D,L]
+  float *dB, *dC;       // [B,N,L,2]  accumulated into with atomics (caller zero-fills)
+  float* dD;            // [D] or null, accumulated into
+  float* dh0;           // [B,D,N,2] or null
+  int B, D, N, L, ck, nck, ncg;
+  int ld, ns;           // matrix-core kernel: row stride of the [.., L] tensors, segments per sequence
+  int hs, ho;           // ... and dhL of (batch, segment) pair b is entry b * hs + ho of the adjoint array
+  int urep;             // generic kernel: u and delta are [B / urep, D, L], shared by urep consecutive batch elements
+};
+
+struct RecBwdArgs {
+  const float* dy;          // [B,D,L]
+  const float* dhL;         // [B,D,N,C] or null
+  const void* u;            // [B,D,L] Tin
+  const void* delta;        // [B,D,L] Tin
+  const float* theta;       // [B,D,L] (complex)
+  const float* rho;         // [B,D,L] (complex)
+  const float* A;           // [D,N]   (real)
+  const void* Bm;           // [B,N,L(,2)] Tin
+  const void* Cm;           // [B,N,L(,2)] Tin
+  const float* Dskip;       // [D] or null
+  const float* delta_bias;  // [D] or null (real)
+  const float* h0;          // [B,D,N,C] or null
+  const float* hck;         // [B,nck,N,C,D], ck == 16
+  float *du, *ddelta;       // [B,D,L]
+  float *dtheta, *drho;     // [B,D,L] (complex)
+  float* dA;                // [D,N] (real), accumulated into
+  float *dB, *dC;           // [B,N,L(,2)], accumulated into
+  float* dD;                // [D] or null, accumulated into
+  float* dh0;               // [B,D,N,C] or null
+  int B, D, N, L, nck, ncg, delta_softplus;
+};
+
+struct SegArgs {
+  const void* x1;       // forward: delta (Tin), adjoint: dy (float)   [B, D, ld]
+  const void* x2;       // forward: u (Tin), adjoint: unused           [B, D, ld]
+  const float* theta;   //                                    [B, D, ld]
+  const void* M;        // forward: B_t, adjoint: C_t (Tin)            [B, N, ld, 2]
+  float* out;           // Z or Y                             [B * ns, D, N, 2]
+  float* ptot;          // rotation of the segment            [B * ns, D, 2]
+  int D, N, L, ld, ns, ncg;   // L: segment length
+};
+
+// Prepared operands ("images") of the matrix-core kernels, in 16-byte records per (batch, chunk)
+constexpr int PX_NP = 3;                                    // bf16 pieces held by the images
+constexpr int PXF_A = 2 * PX_NP * XN * 4;                   // forward: bt_r, bt_i          (phase A)
+constexpr int PXF_B = 3 * PX_NP * XT * 4;                   //          cs_r, g_re, g_im    (phase B)
+constexpr int PXF_REC = PXF_A + PXF_B;                      // 1536 records = 24 KiB
+constexpr int PXB_A = 4 * PX_NP * XN * 4;                   // backward: bt_r, bt_i, ct_r, ct_i
+constexpr int PXB_B = 3 * PX_NP * XT * 4;                   //           bs, g_r, g_i
+constexpr int PXB_REC = PXB_A + PXB_B;                      // 1920 records = 30 KiB
+
+struct PrepArgs {
+  const void* Bm;       // [B, N, ld, 2] Tin
+  const void* Cm;
+  u4* fimg;             // [B, nch, PXF_REC] or null
+  u4* bimg;             // [B, nch, PXB_REC] or null
+  int N, ld, nch;       // nch = ceil(ld / 32) chunks per batch element
+};
+
+constexpr int CONV_MAX_K = 8;
+constexpr int CONV_ROWS = 128;   // (b, l) rows per workgroup of the weight-gradient kernel
+constexpr int CONV_RUN = 8;      // steps per thread of the kernels for filter length 4
+
+struct ConvArgs {
+  const float* x;      // element (b, l, d) at x[b * xs_b + l * xs_l + d]
+  const float* w;      // [D, K]
+  const float* bias;   // [D] or null
+  const float* dy;     // [B, L, D] contiguous (backward)
+  float* y;            // [B, L, D] contiguous (forward)
+  float* dx;           // [B, L, D] contiguous (backward)
+  float* dw;           // [D, K], accumulated into
+  float* dbias;        // [D] or null, accumulated into
+  long long xs_b, xs_l;
+  int B, L, D, K;
+};
+
+struct SwapArgs {
+  const float* x;      // element (b, r, c) at x[b * xs_b + r * xs_r + c]
+  float* y;            // [B, C, R] contiguous
+  long long xs_b, xs_r;
+  int R, C;
+};
+
+}  // namespace aussm

@@ -24,28 +24,6 @@
 
 namespace aussm {
 
-struct RecBwdArgs {
-  const float* dy;          // [B,D,L]
-  const float* dhL;         // [B,D,N,C] or null
-  const void* u;            // [B,D,L] Tin
-  const void* delta;        // [B,D,L] Tin
-  const float* theta;       // [B,D,L] (complex)
-  const float* rho;         // [B,D,L] (complex)
-  const float* A;           // [D,N]   (real)
-  const void* Bm;           // [B,N,L(,2)] Tin
-  const void* Cm;           // [B,N,L(,2)] Tin
-  const float* Dskip;       // [D] or null
-  const float* delta_bias;  // [D] or null (real)
-  const float* h0;          // [B,D,N,C] or null
-  const float* hck;         // [B,nck,N,C,D], ck == 16
-  float *du, *ddelta;       // [B,D,L]
-  float *dtheta, *drho;     // [B,D,L] (complex)
-  float* dA;                // [D,N] (real), accumulated into
-  float *dB, *dC;           // [B,N,L(,2)], accumulated into
-  float* dD;                // [D] or null, accumulated into
-  float* dh0;               // [B,D,N,C] or null
-  int B, D, N, L, nck, ncg, delta_softplus;
-};
 
 constexpr int RT = 16;       // timesteps per tile == checkpoint interval of these kernels
 

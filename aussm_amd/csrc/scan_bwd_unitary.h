@@ -22,26 +22,6 @@
 
 namespace aussm {
 
-struct UniBwdArgs {
-  const float* dy;      // [B,D,L]
-  const float* dhL;     // [B,D,N,2] or null
-  const void* u;        // [B,D,L] Tin
-  const void* delta;    // [B,D,L] Tin
-  const float* theta;   // [B,D,L]
-  const void* Bm;       // [B,N,L,2] Tin
-  const void* Cm;       // [B,N,L,2] Tin
-  const float* Dskip;   // [D] or null
-  const float* hck;     // [B,nck,N,2,D]
-  const float* aux;     // optional: what the forward call left in its aux buffer
-  float *du, *ddelta, *dtheta;   // [B,D,L]
-  float *dB, *dC;       // [B,N,L,2]  accumulated into with atomics (caller zero-fills)
-  float* dD;            // [D] or null, accumulated into
-  float* dh0;           // [B,D,N,2] or null
-  int B, D, N, L, ck, nck, ncg;
-  int ld, ns;           // matrix-core kernel: row stride of the [.., L] tensors, segments per sequence
-  int hs, ho;           // ... and dhL of (batch, segment) pair b is entry b * hs + ho of the adjoint array
-  int urep;             // generic kernel: u and delta are [B / urep, D, L], shared by urep consecutive batch elements
-};
 
 constexpr int RED_COLS = 4 * TG;        // products per lane per turn: TG x (dB re, dB im) then TG x (dC re, dC im)
 constexpr int RED_RS = RED_COLS + 4;    // padded row stride (floats), keeps rows 16-byte aligned

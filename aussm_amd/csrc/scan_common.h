@@ -14,19 +14,13 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "scan_args.h"
+
 namespace aussm {
 
-constexpr int CH = 64;        // channels per workgroup == lanes per wavefront
 constexpr int T = 32;         // timesteps per staged tile (AUSSM_TILE)
 constexpr int TS = CH + 1;    // padded row stride of [t][channel] LDS tiles (bank-conflict free)
 constexpr int NXCD = 8;       // accelerator complex dies, each with a private L2
-
-enum { VAR_UNITARY = 0, VAR_COMPLEX = 1, VAR_REAL = 2 };
-
-// The optional auxiliary buffer of the unitary scan holds B*D*L floats followed by AUX_PAD floats;
-// the first of those is AUX_TAG when a forward kernel has filled the buffer, anything else if not.
-constexpr uint32_t AUX_TAG = 0x4f484950u;
-constexpr int AUX_PAD = 64;
 
 constexpr float LOG2E = 1.4426950408889634f;
 
@@ -234,6 +228,29 @@ __device__ __forceinline__ void store4(float* __restrict__ p, size_t o, const fl
       if (i < nvalid) p[o + i] = x[i];
   }
 }
+
+typedef float f4 __attribute__((ext_vector_type(4)));
+
+// sin and cos without the large-argument branch: the caller keeps |x| below ~150.
+__device__ __forceinline__ void sincos_small(float x, float* sn, float* cs) {
+  const float kf = rintf(x * 0.636619772367581343f);
+  float r = fmaf(-kf, 1.57079637050628662109375f, x);
+  r = fmaf(-kf, -4.37113900018624283e-8f, r);
+  const float r2 = r * r;
+  float ps = fmaf(-1.9515295891e-4f, r2, 8.3321608736e-3f);
+  ps = fmaf(ps, r2, -1.6666654611e-1f);
+  const float s = fmaf(r * r2, ps, r);
+  float pc = fmaf(2.443315711809948e-5f, r2, -1.388731625493765e-3f);
+  pc = fmaf(pc, r2, 4.166664568298827e-2f);
+  const float c = fmaf(r2 * r2, pc, fmaf(-0.5f, r2, 1.0f));
+  const int q = (int)kf;
+  const float s1 = (q & 1) ? c : s;
+  const float c1 = (q & 1) ? s : c;
+  *sn = (q & 2) ? -s1 : s1;
+  *cs = ((q + 1) & 2) ? -c1 : c1;
+}
+
+__device__ __forceinline__ void touch4(const f4& v) { touch_vgpr(v[0]); touch_vgpr(v[1]); touch_vgpr(v[2]); touch_vgpr(v[3]); }
 
 // Sum `v` over the lanes of each aligned group of 32 lanes; result valid in every lane.
 __device__ __forceinline__ float half_wave_sum(float v) {

@@ -8,28 +8,6 @@
 
 namespace aussm {
 
-struct FwdArgs {
-  const void* u;            // [B,D,L]  Tin
-  const void* delta;        // [B,D,L]  Tin
-  const float* theta;       // [B,D,L]  (unitary, complex)
-  const float* rho;         // [B,D,L]  (complex)
-  const float* A;           // [D,N]    (real)
-  const void* Bm;           // [B,N,L(,2)] Tin
-  const void* Cm;           // [B,N,L(,2)] Tin
-  const float* Dskip;       // [D] or null
-  const float* z;           // [B,D,L] or null
-  const float* delta_bias;  // [D] or null (real)
-  const float* h0;          // [B,D,N,C] or null
-  float* y;                 // [B,D,L] or null
-  float* hL;                // [B,D,N,C] or null
-  float* hck;               // [B,nck,N,C,D] or null
-  float* aux;               // unitary, optional: Im(P_t S_t) [B,D,L] followed by a validity tag
-  int B, D, N, L, ck, nck, ncg, delta_softplus;
-  int ld, ns;                // matrix-core unitary kernels: row stride of the [.., L] tensors and segments per
-                             // sequence (B then counts batch x segment pairs and L is the segment length)
-  int hs, ho;                // ... and h0 of pair b is entry b * hs + ho of the state array
-  int urep;                  // generic kernels: u and delta are [B / urep, D, L], shared by urep consecutive batch elements
-};
 
 // VAR: variant.  NW: states per wavefront.  NT: threads per workgroup.  Tin: float or bf16_t.
 template <int VAR, int NW, int NT, typename Tin>

@@ -26,8 +26,6 @@
 
 namespace aussm {
 
-typedef float f4 __attribute__((ext_vector_type(4)));
-
 __device__ __forceinline__ f4 mfma4(float a, float b, f4 c) {
   return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
 }
@@ -50,27 +48,6 @@ struct MfmaG { float re[MT * M_RT], im[MT * M_RT]; };
 
 __device__ __forceinline__ f4 lds4(const float* p) { return *reinterpret_cast<const f4*>(p); }
 __device__ __forceinline__ f4 ldg4(const float* p) { return *reinterpret_cast<const f4*>(p); }
-
-// sin and cos without the large-argument branch: the caller keeps |x| below ~150.
-__device__ __forceinline__ void sincos_small(float x, float* sn, float* cs) {
-  const float kf = rintf(x * 0.636619772367581343f);
-  float r = fmaf(-kf, 1.57079637050628662109375f, x);
-  r = fmaf(-kf, -4.37113900018624283e-8f, r);
-  const float r2 = r * r;
-  float ps = fmaf(-1.9515295891e-4f, r2, 8.3321608736e-3f);
-  ps = fmaf(ps, r2, -1.6666654611e-1f);
-  const float s = fmaf(r * r2, ps, r);
-  float pc = fmaf(2.443315711809948e-5f, r2, -1.388731625493765e-3f);
-  pc = fmaf(pc, r2, 4.166664568298827e-2f);
-  const float c = fmaf(r2 * r2, pc, fmaf(-0.5f, r2, 1.0f));
-  const int q = (int)kf;
-  const float s1 = (q & 1) ? c : s;
-  const float c1 = (q & 1) ? s : c;
-  *sn = (q & 2) ? -s1 : s1;
-  *cs = ((q + 1) & 2) ? -c1 : c1;
-}
-
-__device__ __forceinline__ void touch4(const f4& v) { touch_vgpr(v[0]); touch_vgpr(v[1]); touch_vgpr(v[2]); touch_vgpr(v[3]); }
 
 // Requires: N <= 16, L % 4 == 0, u/delta/theta/z/y 16-byte aligned, B/C 16-byte aligned,
 // ck % 32 == 0, float inputs.  The launcher checks these and otherwise takes the generic kernel.

@@ -29,19 +29,15 @@
 #pragma once
 #include "scan_common.h"
 #include "scan_fwd.h"
-#include "scan_fwd_mfma.h"
 #include <type_traits>
 
 namespace aussm {
 
 typedef float f2v __attribute__((ext_vector_type(2)));
-typedef uint32_t u4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf2v __attribute__((ext_vector_type(2)));
 typedef __bf16 bf8v __attribute__((ext_vector_type(8)));
 
-constexpr int XT = 32;       // timesteps per chunk
-constexpr int XN = 16;       // state rows of the matrix tiles (N is zero-padded up to it)
 
 __device__ __forceinline__ f4 xdl(const u4& a, const u4& b, f4 c) {
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf8v, a), __builtin_bit_cast(bf8v, b), c, 0, 0, 0);

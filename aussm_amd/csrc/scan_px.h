@@ -1,0 +1,609 @@
+// Unitary scan on the matrix cores with operands prepared once per batch element.
+//
+// Mathematics, operand splitting and lane layout are those of scan_fwd_xdl.h / scan_bwd_xdl.h.
+// Two things differ.
+//
+// 1. The channel-independent operands of a 32-step chunk -- B_t and C_t in the record orders the
+//    products need, G[t,s] = sum_n C_t[n] B_s[n] in both orientations, all split into bf16
+//    pieces -- do not depend on the channel group, yet every workgroup of a batch element used to
+//    rebuild them (staging, two products, a dozen splits per chunk).  A light pre-pass
+//    (unitary_px_prep_kernel, one workgroup per (batch, chunk)) now writes them once, as "images"
+//    that have exactly the layout the scan kernels keep in LDS; a scan workgroup fetches an image
+//    with loads that go from global memory straight into LDS.
+//
+// 2. Two wavefronts per SIMD.  A workgroup still owns (batch b, 64 channels) but has eight
+//    wavefronts: w and w + 4 share the 16 channels of group w and take the chunks in turn.  The
+//    work of a chunk c is cut into a part that does not need the carried state,
+//        phase A:  phases, rotations, V = conj(P) delta u (split), Z = B^T V, then the carry
+//                  H_{c+1} = P_T (H_c + Z)  (a handful of vector instructions),
+//    and the rest,
+//        phase B:  S = C.H_c + G.V, y = Re(P S) + D u.
+//    Time is cut into intervals separated by workgroup barriers; in interval i the wavefront with
+//    i % 2 == its half runs phase A of chunk i while its partner runs phase B of chunk i - 1.
+//    One of the two is busy on the vector ALU while the other feeds the matrix pipe, the carry
+//    passes through LDS once per chunk, and the same barrier publishes the next images.
+#pragma once
+#include "scan_bwd_xdl.h"
+#include "scan_fwd_xdl.h"
+
+namespace aussm {
+
+// One workgroup (256 threads) per (batch element, chunk).
+template <typename Tin>
+__global__ __launch_bounds__(256) void unitary_px_prep_kernel(const PrepArgs p) {
+  constexpr int NP = PX_NP;
+  __shared__ XbBC<NP> s_bc;
+  __shared__ XbG<NP> s_g;
+
+  const int bb = blockIdx.x / p.nch, c = blockIdx.x % p.nch;
+  const int tid = threadIdx.x, lane = tid & 63, wave = wave_index();
+  const int dl = lane & 15, g = lane >> 4;
+  const int N = p.N, L = p.ld;
+  const Tin* __restrict__ gB = static_cast<const Tin*>(p.Bm);
+  const Tin* __restrict__ gC = static_cast<const Tin*>(p.Cm);
+  const SplitK sk = make_splitk();
+
+  for (int i = tid; i < (int)(sizeof(s_g) / 16); i += 256) reinterpret_cast<u4*>(&s_g)[i] = u4{0, 0, 0, 0};
+
+  // ---- records of B_t and C_t (the two thread mappings of scan_bwd_xdl.h)
+  {
+    const int m1_t = tid & 31, m1_g = (tid >> 5) & 3;
+    const bool m1_isB = tid >= 128;
+    const Tin* __restrict__ src = m1_isB ? gB : gC;
+    const int l = c * XT + m1_t;
+    const bool tok = l < L;
+    float x[8];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int n = 4 * m1_g + k;
+      const bool ok = tok && n < N;
+      RawC<Tin> r;
+      r.load(src + (((size_t)bb * N + (ok ? n : 0)) * L + (ok ? l : 0)) * 2);
+      x[k] = ok ? r.re() : 0.0f;
+      x[4 + k] = ok ? r.im() : 0.0f;
+    }
+    u4 pc[NP], pi[NP];
+    split8<NP>(sk, x, pc);                  // [re, im]
+    rot_i<NP>(pc, pi);                      // [-im, re]
+    const int o = xrec(m1_t, m1_g, XT);
+#pragma unroll
+    for (int q = 0; q < NP; ++q) {
+      if (m1_isB) {
+        s_bc.bs[q][o] = pc[q];
+        s_bc.bs_c[q][o] = pi[q];
+      } else {
+        s_bc.cs_r[q][o] = u4{pc[q][0], pc[q][1], pc[q][2] ^ 0x80008000u, pc[q][3] ^ 0x80008000u};   // [re, -im]
+        s_bc.cs_i[q][o] = u4{pc[q][2], pc[q][3], pc[q][0], pc[q][1]};                                // [im, re]
+      }
+    }
+  }
+  {
+    const int m2_n = tid & 15, m2_g = (tid >> 4) & 3, m2_half = (tid >> 6) & 1;
+    const bool m2_isC = tid >= 128;
+    const Tin* __restrict__ src = m2_isC ? gC : gB;
+    const int l2 = c * XT + 16 * m2_half + 4 * m2_g;
+    const bool ok = m2_n < N && l2 < L;               // L is a multiple of 4: a run is in range as a whole
+    RawC4<Tin> r;
+    r.load(src + (((size_t)bb * N + (ok ? m2_n : 0)) * L + (ok ? l2 : 0)) * 2);
+    float re[4], im[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) { re[j] = ok ? r.re(j) : 0.0f; im[j] = ok ? r.im(j) : 0.0f; }
+    uint32_t a0[NP], a1[NP], b0[NP], b1[NP];
+    split2<NP>(sk, re[0], re[1], a0);
+    split2<NP>(sk, re[2], re[3], a1);
+    split2<NP>(sk, im[0], im[1], b0);
+    split2<NP>(sk, im[2], im[3], b1);
+    const int o = xrec(m2_n, m2_g, XN) * 2 + m2_half;   // 8-byte half-record index
+#pragma unroll
+    for (int q = 0; q < NP; ++q) {
+      if (m2_isC) {
+        reinterpret_cast<u2*>(s_bc.ct_r[q])[o] = u2{a0[q], a1[q]};
+        reinterpret_cast<u2*>(s_bc.ct_i[q])[o] = u2{b0[q], b1[q]};
+      } else {
+        reinterpret_cast<u2*>(s_bc.bt_r[q])[o] = u2{a0[q], a1[q]};
+        reinterpret_cast<u2*>(s_bc.bt_i[q])[o] = u2{b0[q], b1[q]};
+      }
+    }
+  }
+  __syncthreads();
+
+  // ---- G in both orientations: wave 0 -> tile (tt 0, st 0), 1 -> (1, 0), 2 -> (1, 1)
+  if (wave < 3) {
+    const int gtt = wave >= 1 ? 1 : 0, gst = wave >= 2 ? 1 : 0;
+    const int g_lim = (gtt == gst) ? dl : 64;          // keep rows s = 4 g + i <= column t = dl
+    const int g_low = (gtt == gst) ? dl : -1;          // keep rows t = 4 g + i >= column s = dl
+    u4 a[NP], cr[NP], ci[NP];
+    ldrec<NP>(s_bc.bs, xrec(16 * gst + dl, g, XT), a);
+    ldrec<NP>(s_bc.cs_r, xrec(16 * gtt + dl, g, XT), cr);
+    ldrec<NP>(s_bc.cs_i, xrec(16 * gtt + dl, g, XT), ci);
+    auto put_half = [&](u4 (*pr)[XT * 4], u4 (*pi)[XT * 4], int h, const f4& vr, const f4& vi) {
+      uint32_t r0[NP], r1[NP], i0[NP], i1[NP];
+      split2<NP>(sk, vr[0], vr[1], r0);
+      split2<NP>(sk, vr[2], vr[3], r1);
+      split2<NP>(sk, vi[0], vi[1], i0);
+      split2<NP>(sk, vi[2], vi[3], i1);
+#pragma unroll
+      for (int q = 0; q < NP; ++q) {
+        reinterpret_cast<u2*>(pr[q])[h] = u2{r0[q], r1[q]};
+        reinterpret_cast<u2*>(pi[q])[h] = u2{i0[q], i1[q]};
+      }
+    };
+    // rows t, columns s  ->  lane: G[t = 4 g + i][s = dl]: half a record of row s (slots t)
+    f4 yr = xmm<NP>(cr, a, f4{0, 0, 0, 0}), yi = xmm<NP>(ci, a, f4{0, 0, 0, 0});
+    // rows s, columns t  ->  lane: G[t = dl][s = 4 g + i]: half a record of row t (slots s)
+    f4 xr = xmm<NP>(a, cr, f4{0, 0, 0, 0}), xi = xmm<NP>(a, ci, f4{0, 0, 0, 0});
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const bool k2 = 4 * g + i >= g_low, k1 = 4 * g + i <= g_lim;
+      yr[i] = k2 ? yr[i] : 0.0f; yi[i] = k2 ? yi[i] : 0.0f;
+      xr[i] = k1 ? xr[i] : 0.0f; xi[i] = k1 ? xi[i] : 0.0f;
+    }
+    put_half(s_g.g_r, s_g.g_i, xrec(16 * gst + dl, g, XT) * 2 + gtt, yr, yi);
+    put_half(s_g.gt_r, s_g.gt_i, xrec(16 * gtt + dl, g, XT) * 2 + gst, xr, xi);
+  }
+  __syncthreads();
+
+  // ---- images
+  const size_t ic = (size_t)bb * p.nch + c;
+  if (p.fimg) {
+    u4* __restrict__ o = p.fimg + ic * PXF_REC;
+    constexpr int S16 = NP * XN * 4, S32 = NP * XT * 4;
+    for (int i = tid; i < S16; i += 256) { o[i] = (&s_bc.bt_r[0][0])[i]; o[S16 + i] = (&s_bc.bt_i[0][0])[i]; }
+    o += PXF_A;
+    for (int i = tid; i < S32; i += 256) {
+      o[i] = (&s_bc.cs_r[0][0])[i];
+      o[S32 + i] = (&s_g.gt_r[0][0])[i];
+      o[2 * S32 + i] = (&s_g.gt_i[0][0])[i];
+    }
+  }
+  if (p.bimg) {
+    u4* __restrict__ o = p.bimg + ic * PXB_REC;
+    constexpr int S16 = NP * XN * 4, S32 = NP * XT * 4;
+    for (int i = tid; i < S16; i += 256) {
+      o[i] = (&s_bc.bt_r[0][0])[i];
+      o[S16 + i] = (&s_bc.bt_i[0][0])[i];
+      o[2 * S16 + i] = (&s_bc.ct_r[0][0])[i];
+      o[3 * S16 + i] = (&s_bc.ct_i[0][0])[i];
+    }
+    o += PXB_A;
+    for (int i = tid; i < S32; i += 256) {
+      o[i] = (&s_bc.bs[0][0])[i];
+      o[S32 + i] = (&s_g.g_r[0][0])[i];
+      o[2 * S32 + i] = (&s_g.g_i[0][0])[i];
+    }
+  }
+}
+
+// ---- global memory -> LDS without passing through registers: a wavefront moves 64 records (1 KiB)
+// per instruction, lane i's record to lds + i.  The data is in LDS once the wavefront's vector-memory
+// counter says so (px_loads_done / px_wait) and a barrier has published it.  The instruction is
+// written out: left to the compiler, every later LDS read of the wavefront waits for ALL of its
+// outstanding loads of this kind, which would serialise the prefetch.
+__device__ __forceinline__ void px_load_block(const u4* __restrict__ src, u4* lds, int lane) {
+  const uint32_t dst = __builtin_amdgcn_readfirstlane(
+      (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)lds);
+  asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src + lane), "s"(dst) : "memory");
+}
+__device__ __forceinline__ void px_loads_done() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+// ... or all but the K youngest vector-memory operations of the wavefront have completed
+template <int K>
+__device__ __forceinline__ void px_wait() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(K) : "memory"); }
+// Workgroup barrier that publishes LDS contents only.  __syncthreads() also drains the
+// vector-memory counter, i.e. waits for every prefetch and store in flight.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+// Input loads whose completion is tracked by hand: the compiler is not told that they are loads, so
+// it places no wait of its own (it cannot count the image loads above and would wait for all of
+// them); every value loaded this way passes through px_landed() before its first use.
+__device__ __forceinline__ void px_ldg(f4& dst, const void* p) {
+  asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(dst) : "v"(p) : "memory");
+}
+__device__ __forceinline__ void px_ldg(float2& dst, const void* p) {
+  asm volatile("global_load_dwordx2 %0, %1, off" : "=v"(dst) : "v"(p) : "memory");
+}
+template <typename Tin> struct PxRaw4;
+template <> struct PxRaw4<float> {
+  f4 v;
+  __device__ __forceinline__ void load(const float* p) { px_ldg(v, p); }
+  __device__ __forceinline__ float get(int i) const { return v[i]; }
+};
+template <> struct PxRaw4<bf16_t> {
+  float2 v;
+  __device__ __forceinline__ void load(const bf16_t* p) { px_ldg(v, p); }
+  __device__ __forceinline__ float get(int i) const {
+    const uint32_t w = __float_as_uint(i < 2 ? v.x : v.y);
+    return (i & 1) ? bf16_hi(w) : bf16_lo(w);
+  }
+};
+
+// [x0..x3, y0..y3] with (x, y) = (Cr, -Ci)  ->  (Ci, Cr): the imaginary-part record of C from the real-part one
+template <int NP>
+__device__ __forceinline__ void cs_i_from_r(const u4 (&a)[NP], u4 (&o)[NP]) {
+#pragma unroll
+  for (int q = 0; q < NP; ++q) o[q] = u4{a[q][2] ^ 0x80008000u, a[q][3] ^ 0x80008000u, a[q][0], a[q][1]};
+}
+
+// Development aid (-DAUSSM_PX_TIMING): lane 0 of wavefronts 0 and 4 of workgroup 0 records the
+// shader clock at marked points of every interval into the hL buffer (which is then not an output).
+#ifdef AUSSM_PX_TIMING
+#define PX_MARK(k) do { if (blockIdx.x == 0 && cg == 0 && lane == 0 && i < 70 && i >= 0) \
+    reinterpret_cast<long long*>(p.hL)[(hf * 70 + i) * 8 + (k)] = clock64(); } while (0)
+#else
+#define PX_MARK(k) do { } while (0)
+#endif
+
+// Requires what unitary_fwd_xdl_kernel requires, and the forward images of the call's B_t / C_t.
+// img: [B / ns batch elements][ceil(ld / 32)] images.
+template <bool GATED, typename Tin = float>
+__global__ __launch_bounds__(512) void unitary_fwd_px_kernel(const FwdArgs p, const u4* __restrict__ img) {
+  constexpr int NP = PX_NP;
+  constexpr int NPA = sizeof(Tin) == 2 ? 1 : NP;   // non-zero pieces of the B / C records
+  __shared__ u4 s_a[3][PXF_A];                     // phase-A part of chunk i in slot i % 3
+  __shared__ u4 s_b[3][PXF_B];                     // phase-B part of chunk i in slot i % 3
+  __shared__ f4 s_h[2][4][2][64];                  // carried state H_c in [c % 2][channel group][re, im][lane]
+
+  const int wg = xcd_remap(blockIdx.x, gridDim.x);
+  const int b = wg / p.ncg, d0 = (wg % p.ncg) * CH;
+  const int tid = threadIdx.x, lane = tid & 63, wave = wave_index();
+  const int cg = wave & 3, hf = wave >> 2;
+  const int dl = lane & 15, g = lane >> 4;
+  const int D = p.D, N = p.N, L = p.L;
+  const int d = d0 + cg * 16 + dl;
+  const bool dok = d < D;
+  const int dc = dok ? d : D - 1;
+  const int bb = b / p.ns;
+  const size_t so = (size_t)(b - bb * p.ns) * L;
+  const size_t row = ((size_t)bb * D + dc) * p.ld + so;
+  const Tin* __restrict__ gu = static_cast<const Tin*>(p.u) + row;
+  const Tin* __restrict__ gdl = static_cast<const Tin*>(p.delta) + row;
+  const float* __restrict__ gth = p.theta + row;
+  const float* __restrict__ gz = GATED ? p.z + row : nullptr;
+  const float dsk = (p.Dskip && dok) ? p.Dskip[dc] : 0.0f;
+  const int nchunks = (L + XT - 1) / XT;
+  const SplitK sk = make_splitk();
+  // images of this (batch element, segment): chunk c of the segment is chunk so / 32 + c of the batch element
+  const u4* __restrict__ gimg = img + ((size_t)bb * ((p.ld + XT - 1) / XT) + so / XT) * PXF_REC;
+
+  // Image traffic of one interval: the phase-A part of chunk ca and the phase-B part of chunk cb,
+  // 24 blocks of 64 records over the eight wavefronts, three per wavefront.  A block is loaded
+  // into registers in one interval (img_load), written to its LDS slot at the start of the next
+  // (img_store, once the load has landed) and published by the barrier that ends that interval.
+  // Chunks past the end are clamped: their slots are free and the data is never used.  (Loads
+  // that write LDS directly would spare the registers, but they are executed one at a time by
+  // the memory pipeline and held up every other load and store of the compute unit.)
+  u4 ireg[3];
+  auto img_load = [&](int ca, int cb) {
+    const int cac = ca < nchunks ? ca : nchunks - 1, cbc = cb < nchunks ? cb : nchunks - 1;
+#pragma unroll
+    for (int k = 0; k < 3; ++k) {
+      const int j = wave + 8 * k;                                     // wave-uniform block index
+      const u4* src = j < PXF_A / 64 ? gimg + (size_t)cac * PXF_REC + j * 64
+                                     : gimg + (size_t)cbc * PXF_REC + PXF_A + (j - PXF_A / 64) * 64;
+      asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(ireg[k]) : "v"(src + lane) : "memory");
+    }
+  };
+  // K: vector-memory operations of the wavefront younger than the image loads being collected
+  auto img_store = [&](int ca, int cb, auto kc) {
+    constexpr int K = decltype(kc)::value;
+    asm volatile("s_waitcnt vmcnt(%3)" : "+v"(ireg[0]), "+v"(ireg[1]), "+v"(ireg[2]) : "n"(K) : "memory");
+#pragma unroll
+    for (int k = 0; k < 3; ++k) {
+      const int j = wave + 8 * k;
+      if (j < PXF_A / 64) s_a[ca % 3][j * 64 + lane] = ireg[k];
+      else s_b[cb % 3][(j - PXF_A / 64) * 64 + lane] = ireg[k];
+    }
+  };
+  constexpr int N_IMG = 3;                          // image loads per wavefront and interval
+  constexpr int N_IN = GATED ? 8 : 6;               // input loads per chunk
+
+  // ---- channel data of one chunk: two runs of four timesteps per lane (clamped, zeroed on use)
+  struct In { PxRaw4<Tin> u[2], de[2]; f4 th[2], z[2]; };
+  auto in_load = [&](In& r, int c) {
+#pragma unroll
+    for (int st = 0; st < 2; ++st) {
+      const int l = c * XT + 16 * st + 4 * g;
+      const int lc = l < L ? l : 0;
+      r.u[st].load(gu + lc);
+      r.de[st].load(gdl + lc);
+      px_ldg(r.th[st], gth + lc);
+      if (GATED) px_ldg(r.z[st], gz + lc);
+    }
+  };
+  // the input loads have landed when at most K younger vector-memory operations are outstanding
+  auto in_landed = [&](In& r, auto kc) {
+    constexpr int K = decltype(kc)::value;
+    if constexpr (GATED)
+      asm volatile("s_waitcnt vmcnt(%8)"
+                   : "+v"(r.u[0].v), "+v"(r.u[1].v), "+v"(r.de[0].v), "+v"(r.de[1].v), "+v"(r.th[0]), "+v"(r.th[1]),
+                     "+v"(r.z[0]), "+v"(r.z[1])
+                   : "n"(K)
+                   : "memory");
+    else
+      asm volatile("s_waitcnt vmcnt(%6)"
+                   : "+v"(r.u[0].v), "+v"(r.u[1].v), "+v"(r.de[0].v), "+v"(r.de[1].v), "+v"(r.th[0]), "+v"(r.th[1])
+                   : "n"(K)
+                   : "memory");
+  };
+
+  // ---- registers that pass from one phase of a wavefront to its next:
+  //   gather (end of phase B, prologue) -> phase A of the next chunk: ph (running phases), w = delta u, un, zn
+  //   phase A -> phase B of the same chunk: cs, sn, Vr, Vi, H (state at the chunk start), uu, zz
+  float ph[8], w[8], un[8], zn[8];
+  float cs[8], sn[8], uu[8], zz[8];
+  u4 Vr[NP], Vi[NP];
+  f4 Hr = {0, 0, 0, 0}, Hi = {0, 0, 0, 0};           // H_c: lane (dl, g) holds n = 4 g + i of channel dl
+  In in;
+
+  // Gather: the loaded inputs of chunk c become masked values and running phases; the same
+  // registers are then refilled with the inputs of chunk cn (clamped).
+  auto gather = [&](int c, int cn, auto kc) {
+    in_landed(in, kc);
+    float th[2][4];
+    bool big = false;
+#pragma unroll
+    for (int st = 0; st < 2; ++st) {
+      const bool ok = c * XT + 16 * st + 4 * g < L;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        th[st][k] = ok ? in.th[st][k] : 0.0f;
+        big |= fabsf(th[st][k]) > 4.0f;
+        un[4 * st + k] = in.u[st].get(k);
+        w[4 * st + k] = ok ? in.de[st].get(k) * un[4 * st + k] : 0.0f;
+        if (GATED) zn[4 * st + k] = in.z[st][k];
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      asm volatile("" : "+v"(un[e]), "+v"(w[e]), "+v"(th[e >> 2][e & 3]));
+      if (GATED) asm volatile("" : "+v"(zn[e]));
+    }
+    in_load(in, cn);
+    // large phases are first reduced to (-pi, pi] so that the running sums stay small enough for
+    // sincos_small and for fp32 sums of 32 terms (rare, uniform branch)
+    if (__builtin_expect(__any(big), 0)) {
+#pragma unroll
+      for (int st = 0; st < 2; ++st)
+#pragma unroll
+        for (int k = 0; k < 4; ++k) th[st][k] = (float)remainder((double)th[st][k], 6.283185307179586476925);
+    }
+#pragma unroll
+    for (int st = 0; st < 2; ++st) { th[st][1] += th[st][0]; th[st][2] += th[st][1]; th[st][3] += th[st][2]; }
+    // exclusive offsets over the order (st 0: g 0..3), (st 1: g 0..3)
+    float sa = th[0][3], sb = th[1][3];
+    {
+      float ta = __shfl_up(sa, 16), tb = __shfl_up(sb, 16);
+      if (g >= 1) { sa += ta; sb += tb; }
+      ta = __shfl_up(sa, 32); tb = __shfl_up(sb, 32);
+      if (g >= 2) { sa += ta; sb += tb; }
+    }
+    const float tot_a = __shfl(sa, 48 + dl);
+    const float off_a = sa - th[0][3];
+    const float off_b = tot_a + sb - th[1][3];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ph[e] = th[e >> 2][e & 3] + ((e >> 2) ? off_b : off_a);
+  };
+
+  // ---- prologue: start state, first images, inputs of this wavefront's first chunk
+  if (hf == 0) {
+    f4 hr = {0, 0, 0, 0}, hi = {0, 0, 0, 0};
+    if (p.h0 && dok) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int n = 4 * g + i;
+        if (n < N) {
+          const size_t o = ((((size_t)b * p.hs + p.ho) * D + d) * N + n) * 2;
+          hr[i] = p.h0[o];
+          hi[i] = p.h0[o + 1];
+        }
+      }
+    }
+    s_h[0][cg][0][lane] = hr;
+    s_h[0][cg][1][lane] = hi;
+  }
+  img_load(0, 0);
+  img_store(0, 0, std::integral_constant<int, 0>{});
+  img_load(1, 0);
+  img_store(1, 0, std::integral_constant<int, 0>{});
+  img_load(2, 1);                                   // collected in interval 0
+  in_load(in, hf);
+  gather(hf, hf + 2, std::integral_constant<int, 0>{});
+  __syncthreads();
+
+  const int ck_chunks = p.ck / XT;
+  f4 yo[2], po[2];                                    // outputs of the last phase B, not yet stored
+  int out_l0 = -1;
+  auto flush_out = [&]() {
+    if (out_l0 >= 0 && dok) {
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt) {
+        const int l = out_l0 + 16 * tt + 4 * g;
+        if (l < L) {
+          if (p.y) *reinterpret_cast<f4*>(p.y + row + l) = yo[tt];
+          if (p.aux) *reinterpret_cast<f4*>(p.aux + row + l) = po[tt];     // Im(P_t S_t) for the backward pass
+        }
+      }
+    }
+    out_l0 = -1;
+  };
+  // ---- phase A of chunk c (interval i = c): rotations, V, Z = B^T V, carry.  Chunks past the end
+  // run on zero input and zero phase: the state passes through unchanged, nothing is stored.
+  auto phase_a = [&](int c) {
+    const int i = c;
+    PX_MARK(0);
+    // (the phase B before it issued the input loads of its gather after the image loads)
+    img_store(i + 2, i + 1, std::integral_constant<int, N_IN>{});
+    flush_out();
+    img_load(i + 3, i + 2);
+    PX_MARK(1);
+    float vr[8], vi[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      sincos_small(ph[e], &sn[e], &cs[e]);
+      vr[e] = cs[e] * w[e];
+      vi[e] = -sn[e] * w[e];
+      uu[e] = un[e];
+      if (GATED) zz[e] = zn[e];
+    }
+    split8<NP>(sk, vr, Vr);
+    split8<NP>(sk, vi, Vi);
+    // rotation over the whole chunk: the element (st 1, g 3, i 3) is timestep 31
+    const float cT = __shfl(cs[7], 48 + dl), sT = __shfl(sn[7], 48 + dl);
+    PX_MARK(2);
+    // ---- Z = B^T V  (four independent accumulation chains)
+    f4 z0 = {0, 0, 0, 0}, z1 = {0, 0, 0, 0}, z2 = {0, 0, 0, 0}, z3 = {0, 0, 0, 0};
+    {
+      const u4* sa_ = s_a[c % 3];
+      u4 b_r[NP], b_i[NP], nVi[NP];
+#pragma unroll
+      for (int q = 0; q < NP; ++q) {
+        b_r[q] = sa_[q * (XN * 4) + xrec(dl, g, XN)];
+        b_i[q] = sa_[(NP + q) * (XN * 4) + xrec(dl, g, XN)];
+        nVi[q] = neg_bf16x8(Vi[q]);
+      }
+#pragma unroll
+      for (int s = NP - 1; s >= 0; --s)
+#pragma unroll
+        for (int k = 0; k <= s; ++k)
+          if (k < NPA) {
+            z0 = xdl(b_r[k], Vr[s - k], z0);
+            z1 = xdl(b_r[k], Vi[s - k], z1);
+            z2 = xdl(b_i[k], nVi[s - k], z2);
+            z3 = xdl(b_i[k], Vr[s - k], z3);
+          }
+    }
+    PX_MARK(3);
+    // ---- carry: H_{c+1} = P_T (H_c + Z)
+    Hr = s_h[c & 1][cg][0][lane];
+    Hi = s_h[c & 1][cg][1][lane];
+    f4 nr, ni;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const float xr = Hr[k] + (z0[k] + z2[k]), xi = Hi[k] + (z1[k] + z3[k]);
+      nr[k] = cT * xr - sT * xi;
+      ni[k] = fmaf(cT, xi, sT * xr);
+    }
+    s_h[(c + 1) & 1][cg][0][lane] = nr;
+    s_h[(c + 1) & 1][cg][1][lane] = ni;
+    // ---- checkpoint: state at the end of every ck-step block and at the end of the sequence
+    if (p.hck && dok && c < nchunks && ((c + 1) % ck_chunks == 0 || c == nchunks - 1)) {
+      float* __restrict__ hp = p.hck + ((((size_t)b * p.nck + c / ck_chunks) * N + 4 * g) * 2) * D + dc;
+#pragma unroll
+      for (int k = 0; k < 4; ++k)
+        if (4 * g + k < N) { hp[(size_t)k * 2 * D] = nr[k]; hp[(size_t)k * 2 * D + D] = ni[k]; }
+    }
+    PX_MARK(4);
+    lds_barrier();
+    PX_MARK(6);
+  };
+
+  // ---- phase B of chunk c (interval i = c + 1): S = C.H + G.V, outputs; then the gather of chunk c + 2
+  auto phase_b = [&](int c) {
+    const int i = c + 1;
+    PX_MARK(0);
+    // (the phase A before it issued nothing after the image loads but, now and then, checkpoint stores)
+    img_store(i + 2, i + 1, std::integral_constant<int, 0>{});
+    img_load(i + 3, i + 2);
+    PX_MARK(1);
+    const u4* sb_ = s_b[c % 3];
+    u4 hk[NP];
+    {
+      const float x[8] = {Hr[0], Hr[1], Hr[2], Hr[3], Hi[0], Hi[1], Hi[2], Hi[3]};
+      split8<NP>(sk, x, hk);
+    }
+    u4 nVi[NP];
+#pragma unroll
+    for (int q = 0; q < NP; ++q) nVi[q] = neg_bf16x8(Vi[q]);
+    f4 Sr[2], Si[2];
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt) {
+      u4 c_r[NP], c_i[NP], g_r[NP], g_i[NP];
+#pragma unroll
+      for (int q = 0; q < NP; ++q) {
+        c_r[q] = sb_[q * (XT * 4) + xrec(16 * tt + dl, g, XT)];
+        g_r[q] = sb_[(NP + q) * (XT * 4) + xrec(16 * tt + dl, g, XT)];
+        g_i[q] = sb_[(2 * NP + q) * (XT * 4) + xrec(16 * tt + dl, g, XT)];
+      }
+      cs_i_from_r<NP>(c_r, c_i);
+      f4 a0 = {0, 0, 0, 0}, a1 = {0, 0, 0, 0}, a2 = {0, 0, 0, 0}, a3 = {0, 0, 0, 0};
+#pragma unroll
+      for (int s = NP - 1; s >= 0; --s)
+#pragma unroll
+        for (int k = 0; k <= s; ++k) {
+          if (k < NPA) {
+            a0 = xdl(c_r[k], hk[s - k], a0);
+            a1 = xdl(c_i[k], hk[s - k], a1);
+          }
+          a2 = xdl(g_r[k], Vr[s - k], a2);
+          a3 = xdl(g_r[k], Vi[s - k], a3);
+          a0 = xdl(g_i[k], nVi[s - k], a0);
+          a1 = xdl(g_i[k], Vr[s - k], a1);
+        }
+      Sr[tt] = a0 + a2;
+      Si[tt] = a1 + a3;
+    }
+    PX_MARK(3);
+    // ---- outputs: rows 16 tt + 4 g + k of channel dl are this lane's own timesteps.  They are
+    // stored at the start of this wavefront's next interval: a store issued here would still be
+    // in flight at the wait that ends the interval (loads and stores share one counter).
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt) {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const int e = 4 * tt + k;
+        float v = cs[e] * Sr[tt][k] - sn[e] * Si[tt][k];
+        v = fmaf(dsk, uu[e], v);
+        if (GATED) v *= siluf_(zz[e]);
+        yo[tt][k] = v;
+        po[tt][k] = cs[e] * Si[tt][k] + sn[e] * Sr[tt][k];
+      }
+    }
+    out_l0 = c * XT;
+    PX_MARK(4);
+    // (younger than the inputs it collects: the image loads of this interval)
+    gather(c + 2, c + 4, std::integral_constant<int, N_IMG>{});
+    PX_MARK(5);
+    lds_barrier();
+    PX_MARK(6);
+  };
+  // an interval in which this wavefront has no chunk: it still takes part in the image loads
+  auto idle = [&](int i) {
+    img_store(i + 2, i + 1, std::integral_constant<int, 0>{});
+    flush_out();
+    img_load(i + 3, i + 2);
+    lds_barrier();
+  };
+
+  // Vector-memory operations of a wavefront are issued in this order.  Phase A: the stores of the
+  // previous phase B, then the image loads.  Phase B: the image loads, then (at its end) the input
+  // loads of the gather.  Every load is collected one interval (images) or two (inputs) after it
+  // was issued, by a wait that leaves the known number of younger operations in flight.  The
+  // loop body is straight-line code on purpose: a join of two paths would make the compiler move
+  // live registers, loads in flight included.
+  const int npairs = (nchunks + 1) / 2;               // chunks per wavefront (the last may be past the end)
+  if (hf == 1) idle(0);
+  for (int k = 0; k < npairs; ++k) {
+    const int c = 2 * k + hf;
+    phase_a(c);
+    phase_b(c);
+  }
+  if (hf == 0) idle(2 * npairs);
+
+  flush_out();
+  if (p.aux && blockIdx.x == 0 && tid == 0) p.aux[(size_t)(p.B / p.ns) * D * p.ld] = __uint_as_float(AUX_TAG);
+#ifndef AUSSM_PX_TIMING
+  if (p.hL && dok && hf == 0) {
+    const f4 hr = s_h[0][cg][0][lane], hi = s_h[0][cg][1][lane];    // state after the last (possibly padding) chunk
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int n = 4 * g + i;
+      if (n < N) {
+        const size_t o = (((size_t)b * D + d) * N + n) * 2;
+        p.hL[o] = hr[i];
+        p.hL[o + 1] = hi[i];
+      }
+    }
+  }
+#endif
+}
+
+}  // namespace aussm

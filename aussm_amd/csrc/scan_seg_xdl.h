@@ -18,15 +18,6 @@
 
 namespace aussm {
 
-struct SegArgs {
-  const void* x1;       // forward: delta (Tin), adjoint: dy (float)   [B, D, ld]
-  const void* x2;       // forward: u (Tin), adjoint: unused           [B, D, ld]
-  const float* theta;   //                                    [B, D, ld]
-  const void* M;        // forward: B_t, adjoint: C_t (Tin)            [B, N, ld, 2]
-  float* out;           // Z or Y                             [B * ns, D, N, 2]
-  float* ptot;          // rotation of the segment            [B * ns, D, 2]
-  int D, N, L, ld, ns, ncg;   // L: segment length
-};
 
 // ADJ = false: Z of each segment, chunks in forward order,  H <- P_T (H + B^T V).
 // ADJ = true:  Y of each segment, chunks in reverse order,  A <- conj(P_T) A + conj(C)^T Q.

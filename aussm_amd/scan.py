@@ -114,7 +114,7 @@ def unitary_aux(u, n: int, ck: int) -> Tensor:
                        dtype=torch.float32)
 
 
-def unitary_fwd_raw(u, delta, theta, Bri, Cri, D=None, z=None, h0=None, want_state=False, ck=0, aux=None):
+def unitary_fwd_raw(u, delta, theta, Bri, Cri, D=None, z=None, h0=None, want_state=False, ck=0, aux=None, ck_arg=0):
     """Launch aussm_unitary_fwd(_aux).  Bri/Cri are real views (b, n, l, 2).  Returns (y, hL, hck);
     hL is (b, d, n, 2) or None, hck is the checkpoint tensor when ck > 0.  u and delta may have a
     batch size that divides theta's: each of their batch elements then serves that many
@@ -129,7 +129,7 @@ def unitary_fwd_raw(u, delta, theta, Bri, Cri, D=None, z=None, h0=None, want_sta
     if ck:
         hck = torch.empty((b, num_checkpoints(l, ck), n, 2, d), device=u.device, dtype=torch.float32)
     check(lib.aussm_unitary_fwd_aux(ptr(u), ptr(delta), ptr(theta), ptr(Bri), ptr(Cri), ptr(D), ptr(z), ptr(h0),
-                                    ptr(y), ptr(hL), ptr(hck), ptr(aux), b, d, n, l, ck or _lib.TILE, _in_dtype(u),
+                                    ptr(y), ptr(hL), ptr(hck), ptr(aux), b, d, n, l, ck or ck_arg or _lib.TILE, _in_dtype(u),
                                     urep, _stream()),
           "aussm_unitary_fwd_aux")
     return y, hL, hck
@@ -221,13 +221,14 @@ def unitary_scan(u: Tensor, delta: Tensor, theta: Tensor, Bc: Tensor, Cc: Tensor
         if z is not None:
             y = y * F.silu(z)
     else:
-        # no backward pass: the auxiliary buffer is only worth allocating when the launch would be split along L
+        # no backward pass: the auxiliary buffer serves as workspace only (prepared operands of the
+        # matrix-core kernels, segment states of a launch that is split along L); no checkpoints are kept
         lib = _lib.load()
         ck = unitary_ck(b, d, n, l)
-        split = lib.aussm_unitary_aux_floats(b, d, n, l, ck) > b * d * l + _lib.AUX_PAD
-        aux = unitary_aux(theta, n, ck) if (split and u.shape[0] == b) else None
+        work = lib.aussm_unitary_aux_floats(b, d, n, l, ck) > b * d * l + _lib.AUX_PAD
+        aux = unitary_aux(theta, n, ck) if (work and u.shape[0] == b) else None
         y, hL, _ = unitary_fwd_raw(u, delta, theta, Bri, Cri, D, z, h0r, want_state=return_last_state,
-                                   ck=ck if aux is not None else 0, aux=aux)
+                                   ck=0, aux=aux, ck_arg=ck if aux is not None else 0)
     if return_last_state:
         return y, torch.view_as_complex(hL)
     return y

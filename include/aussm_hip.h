@@ -56,6 +56,31 @@ int aussm_version(void);
 /* Human-readable text for a return code of this library (host pointer, static storage). */
 const char* aussm_error_string(int code);
 
+/* Process-wide options, for comparisons and tuning; none is needed for normal use.  value < 0
+ * restores "let the library decide".  They are read once per call (atomics), so setting one
+ * while another thread launches is safe; which of two racing values a launch sees is unspecified.
+ * No reference counterpart (the reference fixes its launch table at compile time,
+ * extension-cpp/extension_cpp/csrc/cuda/ssm_adaptive_unitary_forward.cu:215-266).
+ *   AUSSM_OPT_UNITARY_FWD  forward kernel of the unitary scan: 0 vector ALU, 2 / 3 matrix cores on
+ *                          two- / three-piece operands (3 = fp32-accurate, the default choice
+ *                          where the shape allows), 6 matrix cores on operands prepared once per
+ *                          batch element by a pre-pass
+ *   AUSSM_OPT_UNITARY_BWD  backward kernel: 0 vector ALU, 2 two-piece operands, 3 three pieces
+ *                          along the sequence and two in the sums over the channel, 5 three
+ *                          pieces everywhere, 6 prepared operands
+ *   AUSSM_OPT_SPLIT_CAP    largest number of segments a launch may be split into along L
+ *                          (0 or 1: never split)
+ *   AUSSM_OPT_GENERIC_NW / AUSSM_OPT_GENERIC_NT   states per wavefront / threads per workgroup of
+ *                          the vector-ALU kernels (both must be set; one of the built pairs) */
+#define AUSSM_OPT_UNITARY_FWD 0
+#define AUSSM_OPT_UNITARY_BWD 1
+#define AUSSM_OPT_SPLIT_CAP 2
+#define AUSSM_OPT_GENERIC_NW 3
+#define AUSSM_OPT_GENERIC_NT 4
+#define AUSSM_OPT_COUNT 5
+int aussm_set_option(int key, int value);
+int aussm_get_option(int key);   /* -1 = unset */
+
 /* nck = ceil(L / ck): number of checkpoint blocks the hck buffer must hold. */
 int aussm_num_checkpoints(int L, int ck);
 
@@ -74,7 +99,7 @@ int aussm_bwd_checkpoint_interval(int variant);
  * Kernel choice is internal: calls with 6 <= N <= 16, L a multiple of 4, 16-byte aligned
  * tensors and ck a multiple of AUSSM_TILE run on the matrix cores (fp32-accurate, see the
  * kernel headers); every other accepted call runs on the vector ALU.  Results agree to
- * rounding.  The environment variables AUSSM_MFMA / AUSSM_MFMA_BWD force one for comparisons.
+ * rounding.  aussm_set_option(AUSSM_OPT_UNITARY_FWD / _BWD, ...) forces one for comparisons.
  * ------------------------------------------------------------------------------------- */
 int aussm_unitary_fwd(const void* u, const void* delta, const float* theta,
                       const void* Bc, const void* Cc, const float* Dskip, const float* z,
@@ -111,7 +136,7 @@ int aussm_unitary_bwd(const float* dy, const float* dhL,
  *    the scan of every segment from its true incoming state - the two-level scan of
  *    ssm_adaptive_unitary_forward.cu:122-162 one level up); the segment states live behind the
  *    per-(b,d,l) part of the buffer, during the call only.  Each call writes there: two calls
- *    that share one buffer must not overlap.  AUSSM_SPLIT=0 (environment) switches the split off.
+ *    that share one buffer must not overlap.  aussm_set_option(AUSSM_OPT_SPLIT_CAP, 0) switches the split off.
  * urep (>= 1, divides B): u and delta are [B / urep, D, L] and shared by urep consecutive batch
  * elements (theta, z, y, dy and every gradient stay [B, D, L]).  This is how the drop-in operator
  * runs its n states per channel, each with its own phase, as n batch elements of one launch without

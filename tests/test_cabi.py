@@ -21,7 +21,8 @@ def test_header_declares_the_expected_entry_points():
     for must in ("aussm_unitary_fwd", "aussm_unitary_bwd", "aussm_complex_fwd", "aussm_complex_bwd",
                  "aussm_real_fwd", "aussm_real_bwd", "aussm_version", "aussm_error_string",
                  "aussm_unitary_fwd_aux", "aussm_unitary_bwd_aux", "aussm_unitary_aux_floats",
-                 "aussm_causal_conv1d_fwd", "aussm_causal_conv1d_bwd", "aussm_swap_last2", "aussm_unitary_split_segments"):
+                 "aussm_causal_conv1d_fwd", "aussm_causal_conv1d_bwd", "aussm_swap_last2", "aussm_unitary_split_segments",
+                 "aussm_set_option", "aussm_get_option"):
         assert must in names
 
 
@@ -63,13 +64,19 @@ def test_argument_checks_without_a_device():
                                1, 1, 1, 32, 32, 0, null)
     assert rc == -5
     # the auxiliary buffer: size query, alignment check, NULL accepted like the plain entry points
-    assert lib.aussm_unitary_aux_floats(32, 512, 16, 2048, 256) == 32 * 512 * 2048 + 64
+    # per-(b,d,l) part + tag, then one 30 KiB image of prepared operands per (batch element, 32-step chunk)
+    img = lambda b, l: b * ((l + 31) // 32) * 1920 * 4
+    assert lib.aussm_unitary_aux_floats(32, 512, 16, 2048, 256) == 32 * 512 * 2048 + 64 + img(32, 2048)
     assert lib.aussm_unitary_aux_floats(0, 1, 1, 1, 32) == 0
     # few (batch, channel) pairs and a long sequence: room for the states of 64 segments of 256 steps
-    assert lib.aussm_unitary_aux_floats(4, 256, 16, 16384, 256) == 4 * 256 * 16384 + 64 + 4 * 64 * 256 * (2 * 16 + 2)
+    assert lib.aussm_unitary_aux_floats(4, 256, 16, 16384, 256) == (4 * 256 * 16384 + 64 + 4 * 64 * 256 * (2 * 16 + 2)
+                                                                    + img(4, 16384))
     # ... which needs whole checkpoint blocks per segment, and states the matrix-core kernels serve
-    assert lib.aussm_unitary_aux_floats(4, 256, 16, 16384 + 4, 256) == 4 * 256 * (16384 + 4) + 64
+    assert lib.aussm_unitary_aux_floats(4, 256, 16, 16384 + 4, 256) == 4 * 256 * (16384 + 4) + 64 + img(4, 16388)
     assert lib.aussm_unitary_aux_floats(4, 256, 4, 16384, 256) == 4 * 256 * 16384 + 64
+    # options: unset by default, settable, restorable
+    assert lib.aussm_get_option(0) == -1 and lib.aussm_set_option(0, 3) == 0 and lib.aussm_get_option(0) == 3
+    assert lib.aussm_set_option(0, -1) == 0 and lib.aussm_get_option(0) == -1 and lib.aussm_set_option(99, 1) == -2
     assert lib.aussm_unitary_split_segments(4, 256, 16, 16384, 256) == 16
     assert lib.aussm_unitary_split_segments(16, 128, 16, 1024, 256) == 4
     assert lib.aussm_unitary_split_segments(16, 128, 16, 1024, 128) == 8

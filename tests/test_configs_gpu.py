@@ -6,8 +6,6 @@ gradients at L=16384 are compared on a slice of the channels, and the full sizes
 size-independent properties: splitting the sequence with a carried state, linearity in the
 input, independence of batch elements, and the adjoint identity <dy, J v> = <J^T dy, v>.
 float32 tolerance: atol = rtol = 1e-4; bfloat16 inputs: 2e-2."""
-import os
-
 import pytest
 import torch
 
@@ -126,12 +124,10 @@ def test_headline_shape_batch_slice_and_independence():
     y_all, g_all = run(scan.unitary_scan, "cuda", slice(0, B))
     _close(y_all[0:2], y_dev.cpu(), "y full batch vs slice", tol=1e-5)
     # bit for bit when the same kernels run: small batches are otherwise split along the sequence
-    os.environ["AUSSM_SPLIT"] = "0"
-    try:
+    from aussm_amd import _lib
+    with _lib.options(split_cap=0):
         y_head, _ = run(scan.unitary_scan, "cuda", slice(0, 2))
         y_tail, _ = run(scan.unitary_scan, "cuda", slice(B - 3, B))
-    finally:
-        del os.environ["AUSSM_SPLIT"]
     assert torch.equal(y_all[0:2], y_head), "forward output must not depend on the other batch elements"
     assert torch.equal(y_all[B - 3:], y_tail)
     for k, ga, gs in zip(names, g_all, g_dev):
@@ -181,3 +177,78 @@ def test_bf16_inputs(variant):
         if w.is_complex():
             w = torch.view_as_real(w)
         _close(g, w, f"grad of input {i}", tol=2e-2)
+
+
+def _variant_case(variant, bf16):
+    """(names of the differentiable inputs, oracle callable, device callable, input dict) for one
+    variant of configuration 3; bf16 rounds u / delta / B / C once so that oracle and device see
+    the same values."""
+    from aussm_amd import scan
+    B, D, N, L = 32, 512, 16, 2048
+    p = O.make_core_inputs(B, D, N, L, seed=11, variant=variant)
+    bf = lambda t: t.to(torch.bfloat16)
+    if variant == "real":
+        names = ["u", "delta", "A", "Bm", "Cm", "Dskip"]
+        low = ("u", "delta", "Bm", "Cm")
+        ref_fn = lambda *a: O.real_core_loop(*a)[0]
+        dev_fn = scan.selective_scan_fn
+    else:
+        names = ["u", "delta"] + (["theta"] if variant == "unitary" else ["rho", "theta"]) + ["Bc", "Cc", "Dskip"]
+        low = ("u", "delta", "Bc", "Cc")
+        ref_fn = (lambda *a: O.unitary_core_loop(*a)[0]) if variant == "unitary" else (lambda *a: O.complex_core_loop(*a)[0])
+        dev_fn = scan.unitary_scan if variant == "unitary" else scan.complex_scan
+    ref_in, dev_in = {}, {}
+    for k in names:
+        t = p[k]
+        if bf16 and k in low:
+            if t.is_complex():
+                r = bf(torch.view_as_real(t))                       # (b, n, l, 2) bfloat16: the device layout
+                dev_in[k] = r
+                ref_in[k] = torch.view_as_complex(r.float().contiguous())
+            else:
+                dev_in[k] = bf(t)
+                ref_in[k] = dev_in[k].float()
+        else:
+            ref_in[k] = dev_in[k] = t
+    return names, ref_fn, dev_fn, ref_in, dev_in, p["dy"]
+
+
+@pytest.mark.parametrize("variant,bf16", [("unitary", True), ("complex", False), ("complex", True),
+                                          ("real", False), ("real", True)])
+def test_headline_shape_other_variants_and_bf16(variant, bf16):
+    """Configuration 3 (B=32 D=512 N=16 L=2048) for the complex and real scans and for bfloat16
+    u / delta / B / C: two batch elements against the oracle (outputs and every gradient), then the
+    full batch against that slice (batch elements are independent; the gradients of the shared A and
+    D are excluded from the slice comparison since they sum over the batch)."""
+    names, ref_fn, dev_fn, ref_in, dev_in, dy = _variant_case(variant, bf16)
+    tol = 2e-2 if bf16 else 1e-4
+    shared = ("A", "Dskip")
+    print(f"case headline {variant} bf16={bf16} slice", flush=True)
+
+    def run(fn, ins, dev, sl):
+        lv = [(ins[k] if k in shared else ins[k][sl]).clone().to(dev).requires_grad_(True) for k in names]
+        y = fn(*lv)
+        (y.float() * dy[sl].to(dev)).sum().backward()
+        return y.detach(), [t.grad for t in lv]
+
+    y_ref, g_ref = run(ref_fn, ref_in, "cpu", slice(0, 2))
+    y_dev, g_dev = run(dev_fn, dev_in, "cuda", slice(0, 2))
+    _close(y_dev, y_ref, "y[0:2]", tol=tol)
+    for k, w, g in zip(names, g_ref, g_dev):
+        if w.is_complex():
+            w = torch.view_as_real(w)
+        if g.is_complex():
+            g = torch.view_as_real(g)
+        _close(g, w, f"d{k}[0:2]", tol=tol)
+    print(f"case headline {variant} bf16={bf16} full batch", flush=True)
+    y_all, g_all = run(dev_fn, dev_in, "cuda", slice(0, 32))
+    _close(y_all[0:2], y_dev.cpu(), "y full batch vs slice", tol=1e-5)
+    y_tail, _ = run(dev_fn, dev_in, "cuda", slice(29, 32))
+    _close(y_all[29:], y_tail.cpu(), "y full batch vs tail slice", tol=1e-5)
+    for k, ga, gs in zip(names, g_all, g_dev):
+        if k in shared:
+            continue
+        a, s = ga[0:2], gs
+        if a.is_complex():
+            a, s = torch.view_as_real(a), torch.view_as_real(s)
+        _close(a, s.cpu(), f"d{k} full batch vs slice", tol=2e-2 if bf16 else 1e-5)

