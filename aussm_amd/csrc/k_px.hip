@@ -23,8 +23,10 @@ int run_px_fwd(const FwdArgs& a, const u4* img, int in_dtype, hipStream_t s) {
 }
 
 int run_px_bwd(const UniBwdArgs& a, const u4* img, int in_dtype, hipStream_t s) {
-  (void)a; (void)img; (void)in_dtype; (void)s;
-  return -2;
+  const dim3 grid((unsigned)(a.B * a.ncg));
+  if (in_dtype == 1) hipLaunchKernelGGL((unitary_bwd_px_kernel<2, bf16_t>), grid, dim3(512), 0, s, a, img);
+  else hipLaunchKernelGGL((unitary_bwd_px_kernel<2, float>), grid, dim3(512), 0, s, a, img);
+  return launch_status();
 }
 
 }  // namespace aussm

@@ -63,6 +63,7 @@ inline bool misaligned(const void* p, size_t a) { return p && (reinterpret_cast<
 // The matrix-core kernels cost the same for every N <= 16 while the vector-ALU ones scale with N:
 // measured, the crossover is between N = 4 (vector ALU 15 % faster) and N = 8 (matrix 30 % faster).
 constexpr int MATRIX_MIN_STATE = 6;
+constexpr int DEFAULT_FWD_MODE = 3, DEFAULT_BWD_MODE = 6;   // (6 falls back to 3 where the call brings no workspace)
 inline int kernel_mode(int key, int dflt, int N) {
   const int e = opt(key);
   if (e >= 0) return e;                        // an explicit choice is honoured for every N <= 16
@@ -125,7 +126,7 @@ inline AuxLayout aux_layout(float* aux, int B, int D, int N, int L, int ck) {
 }
 
 inline int mfma_fwd_mode(const FwdArgs& a, int in_dtype, bool have_img) {
-  int mode = kernel_mode(AUSSM_OPT_UNITARY_FWD, have_img ? 6 : 3, a.N);
+  int mode = kernel_mode(AUSSM_OPT_UNITARY_FWD, DEFAULT_FWD_MODE, a.N);
   if (mode <= 0 || a.urep != 1 || !matrix_shape(a.N, a.L, a.ck)) return 0;
   if (mode == 6 && !have_img) mode = 3;
   if (in_dtype != AUSSM_F32 && mode != 6) mode = 3;       // bf16 inputs: three-piece kernels only
@@ -291,8 +292,11 @@ int aussm_unitary_bwd_aux(const float* dy, const float* dhL, const void* u, cons
   a.ld = L; a.ns = 1; a.hs = 1; a.ho = 0; a.urep = 1;
   a.urep = urep;
   const AuxLayout ws = aux_layout(aux, B, D, N, L, ck);
-  int mode = kernel_mode(AUSSM_OPT_UNITARY_BWD, ws.img ? 6 : 3, N);   // matrix-core kernels for the common case
-  if (mode == 6 && !ws.img) mode = 3;
+  int mode = kernel_mode(AUSSM_OPT_UNITARY_BWD, DEFAULT_BWD_MODE, N);   // matrix-core kernels for the common case
+  // (the prepared-operand kernel addresses its tensors with 32-bit byte offsets)
+  if (mode == 6 && (!ws.img || (unsigned long long)B * D * L * 4 >= (1ull << 32) ||
+                    (unsigned long long)B * N * L * 8 >= (1ull << 32)))
+    mode = 3;
   if (mode > 0 && urep == 1 && matrix_shape(N, L, ck) &&
       !(misaligned(dy, 16) || misaligned(u, 16) || misaligned(delta, 16) || misaligned(theta, 16) ||
         misaligned(du, 16) || misaligned(ddelta, 16) || misaligned(dtheta, 16) || misaligned(Bc, 16) ||
@@ -310,9 +314,15 @@ int aussm_unitary_bwd_aux(const float* dy, const float* dhL, const void* u, cons
       a.B = B * ns; a.L = Ls; a.ns = ns; a.nck = Ls / ck; a.dhL = seg; a.dh0 = nullptr; a.hs = r; a.ho = r - 1;
     }
     if (mode == 6) {
+      // The prepared-operand kernel needs Im(P S) from the forward call in the auxiliary buffer; its
+      // workgroups leave at once if the buffer's tag says it is not there, and the kernel that
+      // recomputes it (launched behind, leaving at once in the opposite case) does the work.
       PrepArgs pa{Bc, Cc, nullptr, ws.img, N, L, (L + XT - 1) / XT};
       run_px_prep(pa, B, in_dtype, s);
-      return run_px_bwd(a, ws.img, in_dtype, s);
+      a.tag_mode = 1;
+      if (int e = run_px_bwd(a, ws.img, in_dtype, s)) return e;
+      a.tag_mode = 2;
+      return run_xdl_bwd(3, a, in_dtype, s);
     }
     return run_xdl_bwd(mode, a, in_dtype, s);
   }

@@ -62,6 +62,8 @@ struct UniBwdArgs {
   int ld, ns;           // matrix-core kernel: row stride of the [.., L] tensors, segments per sequence
   int hs, ho;           // ... and dhL of (batch, segment) pair b is entry b * hs + ho of the adjoint array
   int urep;             // generic kernel: u and delta are [B / urep, D, L], shared by urep consecutive batch elements
+  int tag_mode;         // matrix-core kernels: 0 use the auxiliary buffer if its tag is valid; 1 leave at once
+                        // unless it is; 2 leave at once if it is
 };
 
 struct RecBwdArgs {

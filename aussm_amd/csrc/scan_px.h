@@ -201,15 +201,25 @@ __device__ __forceinline__ void px_ldg(f4& dst, const void* p) {
 __device__ __forceinline__ void px_ldg(float2& dst, const void* p) {
   asm volatile("global_load_dwordx2 %0, %1, off" : "=v"(dst) : "v"(p) : "memory");
 }
+// ... with a wave-uniform base pointer and a 32-bit byte offset per lane (one address register
+// instead of two, and no 64-bit pointer kept per tensor)
+__device__ __forceinline__ void px_ldg(f4& dst, const void* base, uint32_t off) {
+  asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(dst) : "v"(off), "s"(base) : "memory");
+}
+__device__ __forceinline__ void px_ldg(float2& dst, const void* base, uint32_t off) {
+  asm volatile("global_load_dwordx2 %0, %1, %2" : "=v"(dst) : "v"(off), "s"(base) : "memory");
+}
 template <typename Tin> struct PxRaw4;
 template <> struct PxRaw4<float> {
   f4 v;
   __device__ __forceinline__ void load(const float* p) { px_ldg(v, p); }
+  __device__ __forceinline__ void load(const void* base, uint32_t off) { px_ldg(v, base, off); }
   __device__ __forceinline__ float get(int i) const { return v[i]; }
 };
 template <> struct PxRaw4<bf16_t> {
   float2 v;
   __device__ __forceinline__ void load(const bf16_t* p) { px_ldg(v, p); }
+  __device__ __forceinline__ void load(const void* base, uint32_t off) { px_ldg(v, base, off); }
   __device__ __forceinline__ float get(int i) const {
     const uint32_t w = __float_as_uint(i < 2 ? v.x : v.y);
     return (i & 1) ? bf16_hi(w) : bf16_lo(w);
@@ -604,6 +614,643 @@ __global__ __launch_bounds__(512) void unitary_fwd_px_kernel(const FwdArgs p, co
     }
   }
 #endif
+}
+
+
+// ---------------------------------------------------------------------------------------------
+// Backward scan on prepared operands, same organisation: eight wavefronts, partners w / w + 4 take
+// the chunks in turn (in reverse order), intervals separated by one workgroup barrier.  With the
+// notation of scan_bwd_xdl.h,
+//   phase A of chunk c:  V, Q (split), Z = B^T V, W = conj(C)^T Q, then the carry
+//                        J = conj(P_T) A',  H = conj(P_T) H_end - Z,  A = J + W   (H: state at the
+//                        chunk start, recomputed backwards; A: its adjoint), then
+//                        gV = conj(B) J + conj(G)^T Q and du / ddelta / dtheta
+//   phase B of chunk c:  the sums over the channel behind dB, dC; then the rotations of the
+//                        wavefront's next chunk.
+// Every wavefront closes its own 16 channels' share of dB / dC (M conj(B), M^T conj(C)) and adds
+// hands it over through LDS at the end of the interval.
+// Im(P_t S_t) must have been left in p.aux by the forward call: a workgroup leaves at once when
+// the buffer's tag says otherwise (p.tag_mode == 1; the launcher then lets the kernel of
+// scan_bwd_xdl.h do the work, with tag_mode == 2).
+//
+// Memory operations.  All loads of a wavefront are issued at the start of its phase A: the images
+// for two intervals ahead (straight into LDS), the inputs of its next chunk, the checkpoint that
+// chunk may need, and Im(P S) for the phase B that follows.  They are collected by ONE wait in the
+// middle of the next phase B, before that phase issues its first store or atomic: everything
+// outstanding at that point is at least an interval old.  (A wait by count would have to know how
+// many stores and atomics, which depend on masks, were issued after the loads.)
+constexpr int PXB_TS = 33;                 // rows per channel group of the [t][d] scratch (32 + pad)
+constexpr int PXB_TD = 4 * PXB_TS * 4;     // floats of one [t][d] array
+constexpr int PXB_WS = 4 * PXB_TD;         // floats of a channel group's scratch: Q re, Q im, V re, V im
+constexpr int PXB_NS = 17;                 // rows per channel group of the [n][d] arrays that later reuse it
+constexpr int PXB_ND = 4 * PXB_NS * 4;
+constexpr int PXB_RS = 68;                 // row stride of the dB / dC shares (64 floats + pad)
+static_assert(4 * PXB_ND <= PXB_WS, "the scratch is reused");
+
+#ifdef AUSSM_PX_TIMING
+#define PXB_MARK(k) do { if (blockIdx.x == 0 && cg == 0 && lane == 0 && i_ < 40) \
+    reinterpret_cast<long long*>(p.dh0)[(hf * 40 + i_) * 12 + (k)] = clock64(); } while (0)
+#else
+#define PXB_MARK(k) do { } while (0)
+#endif
+
+template <int NPC, typename Tin = float>
+__global__ __launch_bounds__(512) void unitary_bwd_px_kernel(const UniBwdArgs p, const u4* __restrict__ img) {
+  constexpr int NP = PX_NP;
+  constexpr int NPA = sizeof(Tin) == 2 ? 1 : NP, NPAC = sizeof(Tin) == 2 ? 1 : NPC;
+  __shared__ u4 s_a[3][PXB_A];                     // bt, ct of chunk index r in slot r % 3 (phase A and the closing of phase B)
+  __shared__ u4 s_b[2][PXB_B];                     // bs, g of chunk index r in slot r % 2 (phase A)
+  __shared__ f4 s_x[4][4][64];                     // carry per channel group: H re, H im, A re, A im
+  __shared__ __attribute__((aligned(16))) float s_ws[4][PXB_WS];   // per channel group: transposes
+  // dC (rows 0..15) and dB (rows 16..31) of the chunk of one interval, one copy per channel group:
+  // the wavefronts in phase B leave their shares here at the end of the interval, the wavefronts
+  // that start the next interval add the four up and send the sums to global memory
+  __shared__ __attribute__((aligned(16))) float s_tile[4][2 * XN * PXB_RS];
+
+  const int wg = xcd_remap(blockIdx.x, gridDim.x);
+  const int b = wg / p.ncg, d0 = (wg % p.ncg) * CH;
+  const int tid = threadIdx.x, lane = tid & 63, wave = wave_index();
+  const int cg = wave & 3, hf = wave >> 2;
+  const int dl = lane & 15, g = lane >> 4;
+  const int D = p.D, N = p.N, L = p.L;
+  const int d = d0 + cg * 16 + dl;
+  const bool dok = d < D;
+  const int dc = dok ? d : D - 1;
+  const int bb = b / p.ns;
+  const size_t so = (size_t)(b - bb * p.ns) * L;
+  const size_t row = ((size_t)bb * D + dc) * p.ld + so;
+  const size_t tagpos = (size_t)(p.B / p.ns) * D * p.ld;
+  if (p.tag_mode == 1 &&
+      __builtin_amdgcn_readfirstlane(__float_as_uint(p.aux[tagpos])) != AUX_TAG)
+    return;
+  // (the launcher only takes this kernel for tensors below 4 GiB: 32-bit byte offsets per lane)
+  const uint32_t rowf = (uint32_t)(row * 4), rowt = (uint32_t)(row * sizeof(Tin));
+  const float dsk = (p.Dskip && dok) ? p.Dskip[dc] : 0.0f;
+  const int nchunks = (L + XT - 1) / XT;
+  const int ck_chunks = p.ck / XT;
+  const SplitK sk = make_splitk();
+  float* __restrict__ ws = s_ws[cg];
+  // images of this (batch element, segment); chunk index r counts from the END of the segment
+  const u4* __restrict__ gimg = img + ((size_t)bb * ((p.ld + XT - 1) / XT) + so / XT) * PXB_REC;
+  auto chunk_of = [&](int r) { const int c = nchunks - 1 - r; return c < 0 ? 0 : c; };   // clamped for the loads
+
+  // Image loads, issued by the four wavefronts that start a phase B: parts of chunk indices ra (A
+  // part) and rb (B part), 30 blocks of 64 records, up to eight per wavefront.
+  auto img_load = [&](int ra, int rb) {
+    const u4* __restrict__ ia = gimg + (size_t)chunk_of(ra) * PXB_REC;
+    const u4* __restrict__ ib = gimg + (size_t)chunk_of(rb) * PXB_REC + PXB_A;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const int j = cg + 4 * k;                                       // wave-uniform block index
+      if (j < PXB_A / 64) px_load_block(ia + j * 64, &s_a[ra % 3][j * 64], lane);
+      else if (j < PXB_REC / 64) px_load_block(ib + (j - PXB_A / 64) * 64, &s_b[rb & 1][(j - PXB_A / 64) * 64], lane);
+    }
+  };
+
+  // ---- channel data of one chunk; issued at the start of a phase B, collected by the wait that ends it
+  struct In { PxRaw4<Tin> u[2], de[2]; f4 th[2], dy[2]; };
+  In in;
+  f4 phi[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};
+  const size_t ck_stride = (size_t)N * 2 * D;
+  auto in_load = [&](int r) {
+    const int c = chunk_of(r);
+#pragma unroll
+    for (int st = 0; st < 2; ++st) {
+      const int l = c * XT + 16 * st + 4 * g;
+      const uint32_t lc = l < L ? l : 0;
+      in.u[st].load(p.u, rowt + lc * (uint32_t)sizeof(Tin));
+      in.de[st].load(p.delta, rowt + lc * (uint32_t)sizeof(Tin));
+      px_ldg(in.th[st], p.theta, rowf + lc * 4);
+      px_ldg(in.dy[st], p.dy, rowf + lc * 4);
+      px_ldg(phi[st], p.aux, rowf + lc * 4);            // Im(P S) left by the forward call
+    }
+  };
+  // everything the wavefront has loaded so far has landed
+  auto all_landed = [&]() {
+    asm volatile("s_waitcnt vmcnt(0)"
+                 : "+v"(in.u[0].v), "+v"(in.u[1].v), "+v"(in.de[0].v), "+v"(in.de[1].v), "+v"(in.th[0]), "+v"(in.th[1]),
+                   "+v"(in.dy[0]), "+v"(in.dy[1]), "+v"(phi[0]), "+v"(phi[1])
+                 :
+                 : "memory");
+  };
+
+  // ---- registers that pass between the phases of a wavefront
+  float cs[8], sn[8], dy[8], uu[8], de[8];           // phase A -> phase B
+  f4 Hr, Hi, Jr, Ji;                                 // state at the chunk start and J, lane (dl, g): n = 4 g + i
+  float tq = 0.0f, accD = 0.0f;
+
+  // What the phase-B wavefronts of interval i - 1 accumulated (the chunk of index i - 2) goes to
+  // global memory: one wavefront per channel group takes eight of the 32 rows, one atomic
+  // instruction per row (64 floats = the row's 32 timesteps x (re, im), two whole 128-byte lines).
+  auto flush_acc = [&](int i) {
+    const int rr = i - 2;
+    if (rr < 0) return;
+    const int c = nchunks - 1 - rr;
+    float v[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const int o = (8 * cg + k) * PXB_RS + lane;
+      v[k] = (s_tile[0][o] + s_tile[1][o]) + (s_tile[2][o] + s_tile[3][o]);
+    }
+    if (c >= 0 && c * XT + (lane >> 1) < L) {
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        const int rowi = 8 * cg + k, n = rowi & 15;
+        if (n < N) {
+          float* __restrict__ dst = (rowi < XN ? p.dC : p.dB) +
+              (size_t)((uint32_t)((((size_t)bb * N + n) * p.ld + so) * 2) + (uint32_t)(c * XT) * 2 + lane);
+          atomicAdd(dst, v[k]);
+        }
+      }
+    }
+  };
+
+  // ---- gather of chunk index r (end of a phase B, prologue): the loaded inputs become masked
+  // values, rotations and Im(P S) in the registers that phase A of the chunk starts from
+  float ph_s[8];
+  auto gather = [&](int r) {
+    const int c = nchunks - 1 - r;                   // may be negative: a padding chunk (zero input, no stores)
+    float th[2][4];
+    bool big = false;
+#pragma unroll
+    for (int st = 0; st < 2; ++st) {
+      const bool ok = dok && c >= 0 && (c * XT + 16 * st + 4 * g < L);   // idle lanes must not feed the channel sums
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const int e = 4 * st + k;
+        th[st][k] = ok ? in.th[st][k] : 0.0f;
+        big |= fabsf(th[st][k]) > 4.0f;
+        uu[e] = ok ? in.u[st].get(k) : 0.0f;
+        de[e] = ok ? in.de[st].get(k) : 0.0f;
+        dy[e] = ok ? in.dy[st][k] : 0.0f;
+        ph_s[e] = phi[st][k];
+      }
+    }
+    if (__builtin_expect(__any(big), 0)) {
+#pragma unroll
+      for (int st = 0; st < 2; ++st)
+#pragma unroll
+        for (int k = 0; k < 4; ++k) th[st][k] = (float)remainder((double)th[st][k], 6.283185307179586476925);
+    }
+#pragma unroll
+    for (int st = 0; st < 2; ++st) { th[st][1] += th[st][0]; th[st][2] += th[st][1]; th[st][3] += th[st][2]; }
+    float sa = th[0][3], sb = th[1][3];
+    {
+      float ta = __shfl_up(sa, 16), tb = __shfl_up(sb, 16);
+      if (g >= 1) { sa += ta; sb += tb; }
+      ta = __shfl_up(sa, 32); tb = __shfl_up(sb, 32);
+      if (g >= 2) { sa += ta; sb += tb; }
+    }
+    const float tot_a = __shfl(sa, 48 + dl);
+    const float off_a = sa - th[0][3];
+    const float off_b = tot_a + sb - th[1][3];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float ph = th[e >> 2][e & 3] + ((e >> 2) ? off_b : off_a);
+      sincos_small(ph, &sn[e], &cs[e]);
+      accD = fmaf(dy[e], uu[e], accD);
+    }
+  };
+
+  // ---- phase A of chunk index r
+  auto phase_a = [&](int r) {
+    const int c = nchunks - 1 - r;
+    const int i_ = r;
+    PXB_MARK(0);
+    // A chunk that starts a checkpoint block hands the stored state on instead of the recomputed
+    // one (this stops the drift of the backward recomputation).  Plain loads, once per block.
+    const bool ck_here = c > 0 && c % ck_chunks == 0;     // (uniform)
+    float ckv[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (ck_here) {
+      const float* __restrict__ cp = p.hck + ((size_t)b * p.nck + (c / ck_chunks - 1)) * ck_stride + dc;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int n = 4 * g + i;
+        if (n < N) { ckv[i] = cp[(size_t)n * 2 * D]; ckv[4 + i] = cp[(size_t)n * 2 * D + D]; }
+      }
+    }
+    PXB_MARK(1);
+    u4 Vr[NP], Vi[NP], Qr[NP], Qi[NP];
+    float vr[8], vi[8];
+    {
+      float qr[8], qi[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float w = de[e] * uu[e];
+        vr[e] = cs[e] * w;
+        vi[e] = -sn[e] * w;
+        qr[e] = cs[e] * dy[e];
+        qi[e] = -sn[e] * dy[e];
+      }
+      split8<NP>(sk, vr, Vr); split8<NP>(sk, vi, Vi); split8<NP>(sk, qr, Qr); split8<NP>(sk, qi, Qi);
+    }
+    const float cT = __shfl(cs[7], 48 + dl), sT = __shfl(sn[7], 48 + dl);
+    PXB_MARK(2);
+    // ---- Z = B^T V, then W = conj(C)^T Q  (four independent accumulation chains each; one after
+    // the other so that only one set of operand records is live at a time)
+    f4 z0 = {0, 0, 0, 0}, z1 = z0, z2 = z0, z3 = z0, w0 = z0, w1 = z0, w2 = z0, w3 = z0;
+    const u4* sa_ = s_a[r % 3];
+    {
+      u4 b_r[NP], b_i[NP], nVi[NP];
+#pragma unroll
+      for (int q = 0; q < NP; ++q) {
+        b_r[q] = sa_[q * (XN * 4) + xrec(dl, g, XN)];
+        b_i[q] = sa_[(NP + q) * (XN * 4) + xrec(dl, g, XN)];
+        nVi[q] = neg_bf16x8(Vi[q]);
+      }
+#pragma unroll
+      for (int s = NP - 1; s >= 0; --s)
+#pragma unroll
+        for (int k = 0; k <= s; ++k)
+          if (k < NPA) {
+            z0 = xdl(b_r[k], Vr[s - k], z0);
+            z1 = xdl(b_r[k], Vi[s - k], z1);
+            z2 = xdl(b_i[k], nVi[s - k], z2);
+            z3 = xdl(b_i[k], Vr[s - k], z3);
+          }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    {
+      u4 c_r[NP], c_i[NP], nQr[NP];
+#pragma unroll
+      for (int q = 0; q < NP; ++q) {
+        c_r[q] = sa_[(2 * NP + q) * (XN * 4) + xrec(dl, g, XN)];
+        c_i[q] = sa_[(3 * NP + q) * (XN * 4) + xrec(dl, g, XN)];
+        nQr[q] = neg_bf16x8(Qr[q]);
+      }
+#pragma unroll
+      for (int s = NP - 1; s >= 0; --s)
+#pragma unroll
+        for (int k = 0; k <= s; ++k)
+          if (k < NPA) {
+            w0 = xdl(c_r[k], Qr[s - k], w0);
+            w1 = xdl(c_r[k], Qi[s - k], w1);
+            w2 = xdl(c_i[k], Qi[s - k], w2);
+            w3 = xdl(c_i[k], nQr[s - k], w3);
+          }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    PXB_MARK(3);
+    // (here rather than at the start of the interval, where every wavefront of the workgroup has
+    // memory operations to issue)
+    flush_acc(r);
+    // ---- carry
+    const f4 er = s_x[cg][0][lane], ei = s_x[cg][1][lane], ar = s_x[cg][2][lane], ai = s_x[cg][3][lane];
+    float t = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) t -= ar[i] * ei[i] - ai[i] * er[i];   // - sum_n Im(conj(A') H_end): phase gradient at the last step
+    t += __shfl_xor(t, 16);
+    t += __shfl_xor(t, 32);
+    tq = t;
+    f4 nAr, nAi;
+    f4 pr, pi;                                            // what the next chunk takes as its end state
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      Hr[i] = cT * er[i] + sT * ei[i] - (z0[i] + z2[i]);
+      Hi[i] = cT * ei[i] - sT * er[i] - (z1[i] + z3[i]);
+      Jr[i] = cT * ar[i] + sT * ai[i];
+      Ji[i] = cT * ai[i] - sT * ar[i];
+      nAr[i] = Jr[i] + (w0[i] + w2[i]);
+      nAi[i] = Ji[i] + (w1[i] + w3[i]);
+      pr[i] = ck_here ? ckv[i] : Hr[i];
+      pi[i] = ck_here ? ckv[4 + i] : Hi[i];
+    }
+    s_x[cg][0][lane] = pr;
+    s_x[cg][1][lane] = pi;
+    s_x[cg][2][lane] = nAr;
+    s_x[cg][3][lane] = nAi;
+    __builtin_amdgcn_sched_barrier(0);
+    PXB_MARK(4);
+    const u4* sb_ = s_b[r & 1];
+    // ---- gV = sum_n conj(B_s[n]) J[n] + sum_{t>=s} conj(G[t,s]) Q_t   (one set of operand records live at a time)
+    f4 gVr[2], gVi[2];
+    {
+      u4 jk[NP];
+      const float x[8] = {Jr[0], Jr[1], Jr[2], Jr[3], Ji[0], Ji[1], Ji[2], Ji[3]};
+      split8<NP>(sk, x, jk);
+#pragma unroll
+      for (int st = 0; st < 2; ++st) {
+        u4 a[NP], ac[NP];
+#pragma unroll
+        for (int q = 0; q < NP; ++q) a[q] = sb_[q * (XT * 4) + xrec(16 * st + dl, g, XT)];
+        rot_i<NP>(a, ac);                                  // [-Bi, Br]
+        gVr[st] = xmm_p<NP, NPA>(a, jk, f4{0, 0, 0, 0});
+        gVi[st] = xmm_p<NP, NPA>(ac, jk, f4{0, 0, 0, 0});
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    {
+      u4 nQr[NP];
+#pragma unroll
+      for (int q = 0; q < NP; ++q) nQr[q] = neg_bf16x8(Qr[q]);
+#pragma unroll
+      for (int st = 0; st < 2; ++st) {
+        u4 gr[NP], gi[NP];
+#pragma unroll
+        for (int q = 0; q < NP; ++q) {
+          gr[q] = sb_[(NP + q) * (XT * 4) + xrec(16 * st + dl, g, XT)];
+          gi[q] = sb_[(2 * NP + q) * (XT * 4) + xrec(16 * st + dl, g, XT)];
+        }
+        f4 a2 = {0, 0, 0, 0}, a3 = a2;
+#pragma unroll
+        for (int s = NP - 1; s >= 0; --s)
+#pragma unroll
+          for (int k = 0; k <= s; ++k) {
+            a2 = xdl(gr[k], Qr[s - k], a2);
+            a3 = xdl(gr[k], Qi[s - k], a3);
+            gVr[st] = xdl(gi[k], Qi[s - k], gVr[st]);
+            gVi[st] = xdl(gi[k], nQr[s - k], gVi[st]);
+          }
+        gVr[st] += a2;
+        gVi[st] += a3;
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    PXB_MARK(5);
+    // ---- per-element results
+    {
+      float dw[8], gth[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float gr = gVr[e >> 2][e & 3], gi = gVi[e >> 2][e & 3];
+        dw[e] = gr * cs[e] - gi * sn[e];
+        gth[e] = gr * vi[e] - gi * vr[e] - dy[e] * ph_s[e];
+      }
+      gth[7] += (g == 3) ? tq : 0.0f;
+      // suffix sums over the chunk: runs (st 1: g 3..0) then (st 0: g 3..0) in reverse time
+      gth[2] += gth[3]; gth[1] += gth[2]; gth[0] += gth[1];
+      gth[6] += gth[7]; gth[5] += gth[6]; gth[4] += gth[5];
+      float ra = gth[0], rb = gth[4];
+      {
+        float ta = __shfl_down(ra, 16), tb = __shfl_down(rb, 16);
+        if (g <= 2) { ra += ta; rb += tb; }
+        ta = __shfl_down(ra, 32); tb = __shfl_down(rb, 32);
+        if (g <= 1) { ra += ta; rb += tb; }
+      }
+      const float tot_b = __shfl(rb, dl);
+      const float offb = rb - gth[4];
+      const float offa = tot_b + ra - gth[0];
+      if (dok && c >= 0) {
+#pragma unroll
+        for (int st = 0; st < 2; ++st) {
+          const int l = c * XT + 16 * st + 4 * g;
+          if (l < L) {
+            f4 o_du, o_dd, o_dt;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+              const int e = 4 * st + k;
+              o_du[k] = fmaf(de[e], dw[e], dsk * dy[e]);
+              o_dd[k] = uu[e] * dw[e];
+              o_dt[k] = gth[e] + (st ? offb : offa);
+            }
+            const size_t ob = (size_t)(rowf + (uint32_t)l * 4);
+            *reinterpret_cast<f4*>(reinterpret_cast<char*>(p.du) + ob) = o_du;
+            *reinterpret_cast<f4*>(reinterpret_cast<char*>(p.ddelta) + ob) = o_dd;
+            *reinterpret_cast<f4*>(reinterpret_cast<char*>(p.dtheta) + ob) = o_dt;
+          }
+        }
+      }
+    }
+    PXB_MARK(6);
+    lds_barrier();                 // (the shares of dB / dC of the interval before have been read)
+    lds_barrier();
+    PXB_MARK(7);
+  };
+
+  // ---- phase B of chunk index r
+  auto phase_b = [&](int r) {
+    const int c = nchunks - 1 - r;
+    const int i_ = r + 1;
+    PXB_MARK(0);
+    // ---- this wavefront's loads: the images of the next interval, the inputs of its next chunk
+    img_load(r + 2, r + 2);
+    const u4* sa_ = s_a[r % 3];
+    f4 tr[4], ti[4];                                  // the four result tiles: dC 0, dC 1, dB 0, dB 1
+    float vr[8], vi[8], qr[8], qi[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float w = de[e] * uu[e];
+      vr[e] = cs[e] * w;
+      vi[e] = -sn[e] * w;
+      qr[e] = cs[e] * dy[e];
+      qi[e] = -sn[e] * dy[e];
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    // ---- sums over the channel: Q, V through the group's scratch with the channel in the K slots
+    u4 Q0[NPC], Q1[NPC], V0[NPC], V1[NPC];
+    {
+      float* tqr = ws;
+      float* tqi = ws + PXB_TD;
+      float* tvr = ws + 2 * PXB_TD;
+      float* tvi = ws + 3 * PXB_TD;
+      const int dg = dl >> 2, dm = dl & 3;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int t = 16 * (e >> 2) + 4 * g + (e & 3);
+        const int o = (dg * PXB_TS + t) * 4 + dm;
+        tqr[o] = qr[e]; tqi[o] = qi[e]; tvr[o] = vr[e]; tvi[o] = vi[e];
+      }
+      __builtin_amdgcn_wave_barrier();
+      auto rec_t = [&](const float* re, const float* im, int tile, u4 (&o)[NPC]) {
+        const f4 a = *reinterpret_cast<const f4*>(re + (g * PXB_TS + 16 * tile + dl) * 4);
+        const f4 bq = *reinterpret_cast<const f4*>(im + (g * PXB_TS + 16 * tile + dl) * 4);
+        const float x[8] = {a[0], a[1], a[2], a[3], bq[0], bq[1], bq[2], bq[3]};
+        split8<NPC>(sk, x, o);
+      };
+      rec_t(tqr, tqi, 0, Q0); rec_t(tqr, tqi, 1, Q1); rec_t(tvr, tvi, 0, V0); rec_t(tvr, tvi, 1, V1);
+      __builtin_amdgcn_wave_barrier();
+    }
+    // M[t,s] = sum_d Q_t conj(V_s) in both orientations, as operands of the closing products:
+    //   rows t, slots s (for dC): products with V as the row operand -> lane (col t = dl, rows s = 4 g + i)
+    //   rows s, slots t (for dB): products with Q as the row operand -> lane (col s = dl, rows t = 4 g + i)
+    const f4 z4 = {0, 0, 0, 0};
+    // ---- X1[t,n] = sum_d Q_t conj(H[n]),  X2[s,n] = sum_d conj(V_s) J[n]: H, J through the scratch
+    u4 Hc[NPC], Jc[NPC];
+    {
+      float* thr = ws;
+      float* thi = ws + PXB_ND;
+      float* tjr = ws + 2 * PXB_ND;
+      float* tji = ws + 3 * PXB_ND;
+      const int dg = dl >> 2, dm = dl & 3;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int o = (dg * PXB_NS + 4 * g + i) * 4 + dm;
+        thr[o] = Hr[i]; thi[o] = Hi[i]; tjr[o] = Jr[i]; tji[o] = Ji[i];
+      }
+      __builtin_amdgcn_wave_barrier();
+      auto rec_n = [&](const float* re, const float* im, u4 (&o)[NPC]) {
+        const f4 a = *reinterpret_cast<const f4*>(re + (g * PXB_NS + dl) * 4);
+        const f4 bq = *reinterpret_cast<const f4*>(im + (g * PXB_NS + dl) * 4);
+        const float x[8] = {a[0], a[1], a[2], a[3], bq[0], bq[1], bq[2], bq[3]};
+        split8<NPC>(sk, x, o);
+      };
+      rec_n(thr, thi, Hc); rec_n(tjr, tji, Jc);
+      __builtin_amdgcn_wave_barrier();
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    in_load(r + 2);                // (not at the start of the interval, where every wavefront has loads to issue)
+    PXB_MARK(1);
+    // One output tile at a time: (dC, timesteps 16 tile ..), then (dB, ...).  The closing product
+    // takes M with rows = the tile's timesteps and the other time index in the K slots: two 16 x 16
+    // blocks of M side by side (the second one is zero above the block diagonal).
+    auto close_tile = [&](bool isC, int tile) {
+      // X term: lane (col n = dl, rows 4 g + i of the tile)
+      const u4 (&R)[NPC] = tile ? (isC ? Q1 : V1) : (isC ? Q0 : V0);
+      u4 Xi[NPC];                                           // [-Hi, Hr] or [Ji, -Jr]
+      if (isC) rot_i<NPC>(Hc, Xi); else rot_mi<NPC>(Jc, Xi);
+      f4 xr = isC ? xmm<NPC>(R, Hc, z4) : xmm<NPC>(R, Jc, z4);
+      f4 xi = xmm<NPC>(R, Xi, z4);
+      // M blocks with this tile's index in the rows (lane column = row index of the closing operand)
+      f4 m0r, m0i, m1r, m1i;       // K-slot halves: other index 0..15, 16..31
+      if (isC) {
+        // rows t (tile), slots s: M[t][s] = sum_d Q_t conj(V_s), lane (col t = dl, rows s = 4 g + i)
+        u4 Vx[NPC];                                         // [-Vi, Vr]
+        rot_i<NPC>(V0, Vx);
+        m0r = xmm<NPC>(V0, R, z4);  m0i = xmm<NPC>(Vx, R, z4);
+        if (tile) { rot_i<NPC>(V1, Vx); m1r = xmm<NPC>(V1, R, z4); m1i = xmm<NPC>(Vx, R, z4); } else { m1r = z4; m1i = z4; }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          // causal mask of the diagonal block: keep s = 4 g + i <= t = dl
+          const bool keep = 4 * g + i <= dl;
+          if (tile) { m1r[i] = keep ? m1r[i] : 0.0f; m1i[i] = keep ? m1i[i] : 0.0f; }
+          else { m0r[i] = keep ? m0r[i] : 0.0f; m0i[i] = keep ? m0i[i] : 0.0f; }
+        }
+      } else {
+        // rows s (tile), slots t: M[t][s], lane (col s = dl, rows t = 4 g + i)
+        u4 Ri[NPC];                                         // [-Vi, Vr] of the tile
+        rot_i<NPC>(R, Ri);
+        if (tile) { m0r = z4; m0i = z4; } else { m0r = xmm<NPC>(Q0, R, z4); m0i = xmm<NPC>(Q0, Ri, z4); }
+        m1r = xmm<NPC>(Q1, R, z4);  m1i = xmm<NPC>(Q1, Ri, z4);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          // keep t = 4 g + i >= s = dl in the diagonal block
+          const bool keep = 4 * g + i >= dl;
+          if (tile) { m1r[i] = keep ? m1r[i] : 0.0f; m1i[i] = keep ? m1i[i] : 0.0f; }
+          else { m0r[i] = keep ? m0r[i] : 0.0f; m0i[i] = keep ? m0i[i] : 0.0f; }
+        }
+      }
+      u4 mr[NPC], mi[NPC], nmr[NPC];
+      {
+        const float x[8] = {m0r[0], m0r[1], m0r[2], m0r[3], m1r[0], m1r[1], m1r[2], m1r[3]};
+        const float y[8] = {m0i[0], m0i[1], m0i[2], m0i[3], m1i[0], m1i[1], m1i[2], m1i[3]};
+        split8<NPC>(sk, x, mr);
+        split8<NPC>(sk, y, mi);
+        nega<NPC>(mr, nmr);
+      }
+      // dC = X1 + M conj(B);  dB = X2 + M^T conj(C): B or C of the chunk with the timestep in the K slots
+      u4 er_[NPC], ei_[NPC];
+#pragma unroll
+      for (int q = 0; q < NPC; ++q) {
+        er_[q] = sa_[((isC ? 0 : 2 * NP) + q) * (XN * 4) + xrec(dl, g, XN)];
+        ei_[q] = sa_[((isC ? NP : 3 * NP) + q) * (XN * 4) + xrec(dl, g, XN)];
+      }
+      xr = xmm_q<NPC, NPAC>(mr, er_, xr);  xr = xmm_q<NPC, NPAC>(mi, ei_, xr);
+      xi = xmm_q<NPC, NPAC>(mi, er_, xi);  xi = xmm_q<NPC, NPAC>(nmr, ei_, xi);
+      tr[(isC ? 0 : 2) + tile] = xr;
+      ti[(isC ? 0 : 2) + tile] = xi;
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    close_tile(true, 0);
+    PXB_MARK(3);
+    close_tile(true, 1);
+    PXB_MARK(4);
+    close_tile(false, 0);
+    PXB_MARK(5);
+    close_tile(false, 1);
+    PXB_MARK(6);
+    // ---- the one wait for this wavefront's loads: they were issued at the start of the phase, and
+    // nothing else of it is in flight (the stores of the phase A before are an interval old)
+    all_landed();
+    gather(r + 2);
+    lds_barrier();                 // the wavefronts in phase A have read the shares of the interval before
+    // lane (row n = dl, timesteps 16 tile + 4 g + i) of each tile
+    {
+      float* __restrict__ tl = s_tile[cg];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        float* __restrict__ at = tl + ((q >> 1) * XN + dl) * PXB_RS + (16 * (q & 1) + 4 * g) * 2;
+        *reinterpret_cast<f4*>(at) = f4{tr[q][0], ti[q][0], tr[q][1], ti[q][1]};
+        *reinterpret_cast<f4*>(at + 4) = f4{tr[q][2], ti[q][2], tr[q][3], ti[q][3]};
+      }
+    }
+    lds_barrier();
+    PXB_MARK(7);
+  };
+  // an interval in which this wavefront has no chunk
+  auto idle = [&](int i) { flush_acc(i); lds_barrier(); lds_barrier(); };
+
+  // ---- prologue: end state and its adjoint into the carry, first images, first inputs
+  if (hf == 0) {
+    f4 hr = {0, 0, 0, 0}, hi = hr, ar = hr, ai = hr;
+    const float* __restrict__ cp = p.hck + ((size_t)b * p.nck + (p.nck - 1)) * ck_stride + dc;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int n = 4 * g + i;
+      if (n < N) {
+        hr[i] = cp[(size_t)n * 2 * D];
+        hi[i] = cp[(size_t)n * 2 * D + D];
+        if (p.dhL && dok) {
+          const size_t o = ((((size_t)b * p.hs + p.ho) * D + d) * N + n) * 2;
+          ar[i] = p.dhL[o];
+          ai[i] = p.dhL[o + 1];
+        }
+      }
+    }
+    s_x[cg][0][lane] = hr; s_x[cg][1][lane] = hi; s_x[cg][2][lane] = ar; s_x[cg][3][lane] = ai;
+  }
+  // images of chunk indices 0 and 1 (all eight wavefronts take part, here only)
+  {
+    const u4* __restrict__ i0 = gimg + (size_t)chunk_of(0) * PXB_REC;
+    const u4* __restrict__ i1 = gimg + (size_t)chunk_of(1) * PXB_REC;
+    for (int j = wave; j < PXB_REC / 64; j += 8) {
+      if (j < PXB_A / 64) {
+        px_load_block(i0 + j * 64, &s_a[0][j * 64], lane);
+        px_load_block(i1 + j * 64, &s_a[1][j * 64], lane);
+      } else {
+        px_load_block(i0 + j * 64, &s_b[0][(j - PXB_A / 64) * 64], lane);
+        px_load_block(i1 + j * 64, &s_b[1][(j - PXB_A / 64) * 64], lane);
+      }
+    }
+  }
+  in_load(hf);
+  all_landed();
+  gather(hf);
+  __syncthreads();
+
+  // Straight-line loop body (phase A, then phase B of the same chunk); the second half starts one
+  // interval late and the first half idles through the last one.
+  const int npairs = (nchunks + 1) / 2;
+  if (hf == 1) idle(0);
+  for (int k = 0; k < npairs; ++k) {
+    const int r = 2 * k + hf;
+    phase_a(r);
+    phase_b(r);
+  }
+  if (hf == 0) {
+    idle(2 * npairs);
+    flush_acc(2 * npairs + 1);          // (what the second half accumulated in the last interval)
+  }
+
+#ifndef AUSSM_PX_TIMING
+  if (p.dh0 && dok && hf == 0) {
+    const f4 ar = s_x[cg][2][lane], ai = s_x[cg][3][lane];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int n = 4 * g + i;
+      if (n < N) {
+        const size_t o = (((size_t)b * D + d) * N + n) * 2;
+        p.dh0[o] = ar[i];
+        p.dh0[o + 1] = ai[i];
+      }
+    }
+  }
+#endif
+  if (p.dD && dok) {
+    accD += __shfl_xor(accD, 16);
+    accD += __shfl_xor(accD, 32);
+    if (g == 0) atomicAdd(p.dD + d, accD);
+  }
 }
 
 }  // namespace aussm
