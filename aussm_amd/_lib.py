@@ -35,6 +35,8 @@ _SIGNATURES = {
     "aussm_unitary_bwd": [_P] * 16 + [_I] * 6 + [_P],
     "aussm_unitary_fwd_aux": [_P] * 12 + [_I] * 7 + [_P],
     "aussm_unitary_bwd_aux": [_P] * 17 + [_I] * 7 + [_P],
+    "aussm_static_init": [],
+    "aussm_unitary_fwd_static": [_P] * 10 + [_I] * 6 + [_P],
     "aussm_complex_fwd": [_P] * 12 + [_I] * 6 + [_P],
     "aussm_complex_bwd": [_P] * 19 + [_I] * 6 + [_P],
     "aussm_real_fwd": [_P] * 8 + [_I] + [_P] * 4 + [_I] * 6 + [_P],

@@ -169,6 +169,32 @@ int launch_unitary_fwd(FwdArgs a, int in_dtype, hipStream_t s, AuxLayout ws) {
   return run_xdl_fwd(mode, a, in_dtype, s);
 }
 
+// ---- static workspace of aussm_unitary_fwd_static ---------------------------------------------
+// A file-scope device array: every GPU the library runs on holds its own copy at its own address
+// until the process ends.  In host code the array's NAME is only a handle for the runtime, not a
+// device address: the address is looked up once per device (hipGetSymbolAddress) and that pointer
+// is what the launches are given.
+constexpr size_t STATIC_SCRATCH_FLOATS = AUSSM_STATIC_SCRATCH_BYTES / sizeof(float);
+static __device__ __align__(256) float g_static_scratch[STATIC_SCRATCH_FLOATS];
+constexpr int MAX_DEVICES = 64;
+std::atomic<float*> g_static_scratch_ptr[MAX_DEVICES];
+
+int static_scratch(float** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= MAX_DEVICES) return AUSSM_E_SHAPE;
+  float* ptr = g_static_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!ptr) {
+    e = hipGetSymbolAddress(reinterpret_cast<void**>(&ptr), HIP_SYMBOL(g_static_scratch));
+    if (e != hipSuccess) return (int)e;
+    if (!ptr) return AUSSM_E_NULL;
+    g_static_scratch_ptr[dev].store(ptr, std::memory_order_release);
+  }
+  *out = ptr;
+  return AUSSM_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -183,6 +209,7 @@ const char* aussm_error_string(int code) {
     case AUSSM_E_CK: return "checkpoint interval must be a multiple of 32 accepted by this function";
     case AUSSM_E_DTYPE: return "in_dtype must be AUSSM_F32 or AUSSM_BF16";
     case AUSSM_E_ALIGN: return "pointer not aligned to its element size";
+    case AUSSM_E_SCRATCH: return "the call needs more workspace than the static scratch holds (use the _aux entry point)";
     default: return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown aussm error";
   }
 }
@@ -233,6 +260,35 @@ int aussm_unitary_fwd_aux(const void* u, const void* delta, const float* theta, 
   a.B = B; a.D = D; a.N = N; a.L = L; a.ck = ck; a.nck = (L + ck - 1) / ck; a.ncg = (D + CH - 1) / CH;
   a.ld = L; a.ns = 1; a.hs = 1; a.ho = 0; a.urep = urep;
   return launch_unitary_fwd(a, in_dtype, (hipStream_t)stream, aux_layout(aux, B, D, N, L, ck));
+}
+
+int aussm_static_init(void) {
+  float* ptr = nullptr;
+  return static_scratch(&ptr);
+}
+
+int aussm_unitary_fwd_static(const void* u, const void* delta, const float* theta, const void* Bc, const void* Cc,
+                             const float* Dskip, const float* z, const float* h0, float* y, float* hL,
+                             int B, int D, int N, int L, int ck, int in_dtype, void* stream) {
+  if (int e = check_common(B, D, N, L, ck, in_dtype)) return e;
+  if (!u || !delta || !theta || !Bc || !Cc) return AUSSM_E_NULL;
+  const size_t ca = in_dtype == AUSSM_BF16 ? 4 : 8;
+  if (misaligned(Bc, ca) || misaligned(Cc, ca)) return AUSSM_E_ALIGN;
+  // the only workspace a forward call without checkpoints uses: the segment states of a launch
+  // that is split along L
+  const size_t need = seg_floats(B, D, N, L, seg_capacity(B, D, N, L, ck));
+  if (need > STATIC_SCRATCH_FLOATS) return AUSSM_E_SCRATCH;
+  float* scratch = nullptr;
+  if (need > 0)
+    if (int e = static_scratch(&scratch)) return e;
+  FwdArgs a{};
+  a.u = u; a.delta = delta; a.theta = theta; a.Bm = Bc; a.Cm = Cc; a.Dskip = Dskip; a.z = z;
+  a.h0 = h0; a.y = y; a.hL = hL; a.hck = nullptr; a.aux = nullptr;
+  a.B = B; a.D = D; a.N = N; a.L = L; a.ck = ck; a.nck = (L + ck - 1) / ck; a.ncg = (D + CH - 1) / CH;
+  a.ld = L; a.ns = 1; a.hs = 1; a.ho = 0; a.urep = 1;
+  // (every segment state the scan reads is written earlier in the same call: nothing in the
+  // scratch has to start at zero)
+  return launch_unitary_fwd(a, in_dtype, (hipStream_t)stream, AuxLayout{scratch, nullptr});
 }
 
 int aussm_complex_fwd(const void* u, const void* delta, const float* rho, const float* theta, const void* Bc,

@@ -45,6 +45,7 @@ extern "C" {
 #define AUSSM_E_CK (-3)        /* checkpoint interval not accepted by this function  */
 #define AUSSM_E_DTYPE (-4)     /* unknown in_dtype                                   */
 #define AUSSM_E_ALIGN (-5)     /* a pointer is not aligned to its element size       */
+#define AUSSM_E_SCRATCH (-6)   /* the call needs more workspace than the static scratch holds */
 
 #define AUSSM_TILE 32          /* timesteps per staged tile; ck is a multiple of it, */
                                /* or exactly AUSSM_TILE / 2                          */
@@ -162,6 +163,28 @@ int aussm_unitary_bwd_aux(const float* dy, const float* dhL,
                           float* du, float* ddelta, float* dtheta, float* dB, float* dC,
                           float* dD, float* dh0,
                           int B, int D, int N, int L, int ck, int in_dtype, int urep, void* stream);
+
+/* Forward unitary scan that ALLOCATES NOTHING and takes no workspace argument: the variant of
+ * aussm_unitary_fwd_aux (called with hck == NULL, i.e. outputs and final state only) for callers
+ * that cannot allocate device memory - code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc.  It has no counterpart in the reference (whose launcher
+ * allocates its outputs per call, ssm_adaptive_unitary_forward.cu:215-222).
+ * The one workspace such a call uses - the segment states of a launch with few (batch, channel)
+ * pairs that is split along L, see above - lives in a device array of AUSSM_STATIC_SCRATCH_BYTES
+ * inside the library, which every GPU the library runs on holds from the first use to the end of
+ * the process.  Same arguments, results and kernel choice as aussm_unitary_fwd_aux with a buffer
+ * sized for (B, D, N, L, ck); a call whose segment states do not fit returns AUSSM_E_SCRATCH.
+ * All calls on one GPU share that GPU's array: calls that overlap there (different streams,
+ * different threads) race; calls in one stream are ordered and safe.  Nothing in the array has
+ * to start at zero (every state read is written earlier in the same call).
+ * aussm_static_init() looks the array up for the CURRENT device (once per device; the entry point
+ * does the same on its first use there): call it before a graph capture starts. */
+#define AUSSM_STATIC_SCRATCH_BYTES (4u << 20)
+int aussm_static_init(void);
+int aussm_unitary_fwd_static(const void* u, const void* delta, const float* theta,
+                             const void* Bc, const void* Cc, const float* Dskip, const float* z,
+                             const float* h0, float* y, float* hL,
+                             int B, int D, int N, int L, int ck, int in_dtype, void* stream);
 
 /* ---------------------------------------------------------------------------------------
  * Complex scan:  a_l = exp(rho_l[b,d] + i*theta_l[b,d]), otherwise as the unitary scan.
