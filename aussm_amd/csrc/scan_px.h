@@ -597,6 +597,11 @@ __global__ __launch_bounds__(512) void unitary_fwd_px_kernel(const FwdArgs p, co
     phase_b(c);
   }
   if (hf == 0) idle(2 * npairs);
+  // The loads issued last (images and inputs of chunks past the end) are never used, but they are
+  // still in flight: their destination registers must stay reserved until they have landed, or
+  // whatever the code below keeps there - the addresses of the final stores - is overwritten.
+  asm volatile("s_waitcnt vmcnt(0)" : "+v"(ireg[0]), "+v"(ireg[1]), "+v"(ireg[2])::"memory");
+  in_landed(in, std::integral_constant<int, 0>{});
 
   flush_out();
   if (p.aux && blockIdx.x == 0 && tid == 0) p.aux[(size_t)(p.B / p.ns) * D * p.ld] = __uint_as_float(AUX_TAG);
