@@ -44,9 +44,12 @@ _SIGNATURES = {
     "aussm_causal_conv1d_fwd": [_P] * 4 + [_I] * 4 + [_LL] * 2 + [_P],
     "aussm_causal_conv1d_bwd": [_P] * 6 + [_I] * 4 + [_LL] * 2 + [_P],
     "aussm_swap_last2": [_P] * 2 + [_I] * 3 + [_LL] * 2 + [_P],
+    "aussm_ssm_adaptive_unitary_fwd": [_P] * 16 + [_I] * 4 + [_P],
+    "aussm_ssm_adaptive_unitary_bwd": [_P] * 30 + [_I] * 4 + [_P],
 }
 
-EXPORTED = tuple(_SIGNATURES) + ("aussm_error_string", "aussm_unitary_aux_floats")
+EXPORTED = tuple(_SIGNATURES) + ("aussm_error_string", "aussm_unitary_aux_floats",
+                                 "aussm_ssm_adaptive_unitary_workspace_floats")
 
 
 OPT_UNITARY_FWD, OPT_UNITARY_BWD, OPT_SPLIT_CAP, OPT_GENERIC_NW, OPT_GENERIC_NT = range(5)
@@ -76,6 +79,8 @@ def load() -> ctypes.CDLL:
         fn.restype = c_int
     lib.aussm_unitary_aux_floats.argtypes = [_I, _I, _I, _I, _I]
     lib.aussm_unitary_aux_floats.restype = ctypes.c_size_t
+    lib.aussm_ssm_adaptive_unitary_workspace_floats.argtypes = [_I, _I, _I, _I, _I]
+    lib.aussm_ssm_adaptive_unitary_workspace_floats.restype = ctypes.c_size_t
     lib.aussm_error_string.argtypes = [c_int]
     lib.aussm_error_string.restype = c_char_p
     _lib = lib

@@ -4,6 +4,7 @@
     python -m aussm_amd.build --only k_px     # recompile one unit (the others' objects must exist) and relink
     python -m aussm_amd.build --asm DIR       # also keep the compiler's gfx950 assembly in DIR
     python -m aussm_amd.build --experimental  # also build the measured-and-dropped alternative kernels
+    python -m aussm_amd.build --check         # compile k_px.hip to assembly and check its listings (below)
 
 hipcc cross-compiles without a GPU, so this runs on a CPU-only machine.
 """
@@ -21,7 +22,7 @@ LIBNAME = "libaussm_hip.so"
 
 # One translation unit per kernel family: they compile side by side, and a change in one family
 # does not recompile the others' objects by hand (`--only k_px` rebuilds one unit and relinks).
-SOURCES = ["scan_api.hip", "k_generic.hip", "k_xdl.hip", "k_px.hip"]
+SOURCES = ["scan_api.hip", "k_generic.hip", "k_xdl.hip", "k_px.hip", "k_dropin.hip"]
 
 # Packed-FP32 instructions are switched off on purpose (see the flag): the kernels are written
 # with scalar float arithmetic only.
@@ -77,8 +78,97 @@ def build(verbose: bool = True, asm_dir: str | None = None, only=None, extra=())
     return out
 
 
+# ---- listing check of the kernels that track their own loads ------------------------------------
+#
+# The kernels of scan_px.h issue some global loads as hand-written instructions and wait for them
+# by count, so that the compiler neither sees a load nor places a wait.  Two things the compiler is
+# then free to do would silently break them, and both are visible in the assembly it emits:
+#   * spilling vector registers (a register that is the destination of a load in flight would be
+#     saved before the data has arrived);
+#   * touching a load's destination registers between the load and the wait that retires it
+#     (copying them, or - when it considers the value dead - reusing them for something else,
+#     which the landing data then overwrites).
+# check_px_listing() compiles k_px.hip to assembly and looks for both in every kernel of the unit.
+
+def scan_listing(text: str):
+    """Findings [(line number, instruction)] of one kernel listing: vector registers touched while
+    they are the destination of a hand-written (ASMSTART ... ASMEND) global load that no
+    s_waitcnt vmcnt has retired yet.  The scan follows the file order, not the control flow."""
+    import re
+
+    def regs(tok):
+        out = set()
+        for m in re.finditer(r"\bv\[(\d+):(\d+)\]|\bv(\d+)\b", tok):
+            if m.group(1):
+                out.update(range(int(m.group(1)), int(m.group(2)) + 1))
+            else:
+                out.add(int(m.group(3)))
+        return out
+
+    inflight, in_asm, found = {}, False, []
+    for i, line in enumerate(text.split("\n")):
+        s = line.strip()
+        if "ASMSTART" in s:
+            in_asm = True
+            continue
+        if "ASMEND" in s:
+            in_asm = False
+            continue
+        if not s or s[0] in ";.":
+            continue
+        ins = s.split(";")[0]
+        if ins.startswith("s_waitcnt") and "vmcnt" in ins:
+            k = int(re.search(r"vmcnt\((\d+)\)", ins).group(1))
+            issued = sorted(set(inflight.values()))
+            keep = set(issued[len(issued) - k:]) if k > 0 else set()
+            inflight = {r: ln for r, ln in inflight.items() if ln in keep}
+            continue
+        if in_asm and re.match(r"global_load_dwordx[24] ", ins):
+            ops = ins.split(None, 1)[1].split(",")
+            if any(r in inflight for r in regs(ops[1])):
+                found.append((i + 1, ins))
+            for r in regs(ops[0]):
+                inflight[r] = i + 1
+            continue
+        if any(r in inflight for r in regs(ins)):
+            found.append((i + 1, ins))
+    return found
+
+
+def check_px_listing(verbose: bool = True) -> None:
+    """Raises RuntimeError if a kernel of k_px.hip spills vector registers or touches registers
+    with a load in flight."""
+    import re
+    import tempfile
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    with tempfile.TemporaryDirectory() as tmp:
+        out = os.path.join(tmp, "k_px.s")
+        cmd = [hipcc] + HIPCC_FLAGS + ["-S", "--cuda-device-only", os.path.join(CSRC, "k_px.hip"), "-o", out]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        subprocess.run(cmd, check=True, cwd=tmp)
+        text = open(out).read()
+    problems = []
+    kernels = re.findall(r"^(_ZN5aussm\w+):[^\n]*\n(.*?)s_endpgm", text, flags=re.S | re.M)
+    if not kernels:
+        raise RuntimeError("no kernels found in the listing of k_px.hip")
+    for name, body in kernels:
+        for ln, ins in scan_listing(body):
+            problems.append(f"{name}: line {ln}: `{ins.strip()}` touches registers with a load in flight")
+    for name, count in re.findall(r"^\s*\.name:\s+(_ZN5aussm\w+)\n(?:.*\n)*?\s*\.vgpr_spill_count:\s+(\d+)", text, flags=re.M):
+        if "_px_" in name and int(count):
+            problems.append(f"{name}: {count} vector registers spilled")
+    if problems:
+        raise RuntimeError("k_px.hip: " + "; ".join(problems))
+    if verbose:
+        print(f"k_px.hip: {len(kernels)} kernel listings checked", flush=True)
+
+
 if __name__ == "__main__":
     argv = sys.argv[1:]
+    if "--check" in argv:
+        check_px_listing()
+        sys.exit(0)
     only = [argv[i + 1] for i, a in enumerate(argv) if a == "--only"]
     extra = ["-DAUSSM_EXPERIMENTAL_KERNELS"] if "--experimental" in argv else []
     build(asm_dir=os.path.abspath(argv[argv.index("--asm") + 1]) if "--asm" in argv else None, only=only or None,

@@ -1,0 +1,553 @@
+// The reference's operator, extension_cpp::ssm_adaptive_unitary, as fused kernels.
+//
+// Semantics (extension-cpp/extension_cpp/csrc/cuda/ssm_adaptive_unitary_forward.cu:83-181), per batch
+// b, channel i, state j, with ut = silu(u), Bt_j = B_r[j] e^{i B_theta[j]}, Ct_j likewise:
+//     theta_l[b,i,j] = sum_r x[i,j,r] u_l[b,r] + x_bias[i,j]
+//     h_l[b,i,j]     = exp(i theta_l) h_{l-1}[b,i,j] + Bt_j dt_l[b,i] ut_l[b,i]
+//     y_l[b,i]       = silu(z_l[b,i]) ( sum_j Re(Ct_j h_l[b,i,j]) + D_i ut_l[b,i] )
+//
+// The phase tensor theta[b,i,j,l] (n times the size of every other tensor) never exists in memory.
+// A wavefront owns one (batch, channel) pair and walks the sequence in tiles of 16 timesteps:
+//   * the tile's phases, a (16 states) x (16 timesteps) block, are one small matrix product
+//     x[i] (16 x d) . u[b][:, tile] (d x 16) on the bf16 matrix cores with both operands split exactly
+//     into three bf16 pieces (scan_fwd_xdl.h), i.e. fp32-accurate.  The wavefront keeps its rows of x
+//     in registers for the whole sequence; the tile of u, which all wavefronts of the workgroup
+//     share, is split and staged in LDS once per workgroup;
+//   * the result lands with the timestep along the lanes of a 16-lane row (lane = (timestep l,
+//     state group g), states 4 g .. 4 g + 3 in registers), so the recurrence becomes two prefix sums
+//     along the row (DPP row shifts, no LDS): G = prefix(theta), E = e^{iG}, p = conj(E) Bt w,
+//     R = h_in + prefix(p), h = E R.  This is the cumulative-sum form the reference itself uses
+//     (:122-162), tile by tile, with the state h handed from tile to tile - so G restarts at every
+//     tile and stays small;
+//   * one sincos per (state, timestep), the sum over the states inside the wavefront, the gates
+//     and the skip fused into the store.
+#pragma once
+#include "dropin_args.h"
+#include "scan_fwd_xdl.h"
+
+namespace aussm {
+
+
+// ---- prefix / suffix sums along a row of 16 lanes
+template <int CTRL>
+__device__ __forceinline__ float dpp_mov0(float v) {   // lanes that have no source read 0
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float row_prefix(float v) {   // inclusive, towards higher lanes
+  v += dpp_mov0<0x111>(v);    // row_shr:1
+  v += dpp_mov0<0x112>(v);
+  v += dpp_mov0<0x114>(v);
+  v += dpp_mov0<0x118>(v);
+  return v;
+}
+__device__ __forceinline__ float row_suffix(float v) {   // inclusive, towards lower lanes
+  v += dpp_mov0<0x101>(v);    // row_shl:1
+  v += dpp_mov0<0x102>(v);
+  v += dpp_mov0<0x104>(v);
+  v += dpp_mov0<0x108>(v);
+  return v;
+}
+// value of the row's last / first lane in every lane of the row
+__device__ __forceinline__ float row_last(float v, int lane) { return __shfl(v, (lane & 48) | 15); }
+__device__ __forceinline__ float row_first(float v, int lane) { return __shfl(v, lane & 48); }
+
+
+// x (d, n, d) -> operand records.  Record (i, ks, piece, lane = (row j = lane % 16, g = lane / 16))
+// holds x[i, j, 32 ks + 8 g .. + 7] (zero past the ends).  One thread per (i, ks, lane).
+__global__ __launch_bounds__(256) void dropin_xprep_kernel(const float* __restrict__ x, u4* __restrict__ xp, int d, int n, int ks) {
+  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (size_t)d * ks * 64) return;
+  const int lane = (int)(idx & 63);
+  const int k = (int)((idx >> 6) % ks), i = (int)((idx >> 6) / ks);
+  const int j = lane & 15, g = lane >> 4;
+  const SplitK sk = make_splitk();
+  float v[8];
+#pragma unroll
+  for (int q = 0; q < 8; ++q) {
+    const int r = 32 * k + 8 * g + q;
+    v[q] = (j < n && r < d) ? x[((size_t)i * n + j) * d + r] : 0.0f;
+  }
+  u4 pc[3];
+  split8<3>(sk, v, pc);
+#pragma unroll
+  for (int q = 0; q < 3; ++q) xp[(((size_t)i * ks + k) * 3 + q) * 64 + lane] = pc[q];
+}
+
+// Stage the tile u[b][:, l0 .. l0 + 15] as the second operand of the phase product: record
+// (ks, piece, lane = (column l = lane % 16, g)) holds u[b, 32 ks + 8 g .. + 7, l0 + l].  In two steps so
+// that the loads of the next tile fly while the current one is computed: stage_load requests the
+// values (NREC records of eight per thread), stage_store splits them and writes the records.
+template <int NT, int NREC>
+__device__ __forceinline__ void stage_load(const float* __restrict__ ub, float (&v)[NREC][8], int d, int L, int ks, int l0, int tid) {
+#pragma unroll
+  for (int e = 0; e < NREC; ++e) {
+    const int rec = tid + e * NT;
+    const int lane = rec & 63, k = rec >> 6;
+    const int l = l0 + (lane & 15), g = lane >> 4;
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      const int r = 32 * k + 8 * g + q;
+      v[e][q] = (k < ks && r < d && l < L) ? ub[(size_t)r * L + l] : 0.0f;
+    }
+  }
+}
+template <int NT, int NREC>
+__device__ __forceinline__ void stage_store(const float (&v)[NREC][8], u4* __restrict__ dst, int ks, int tid, const SplitK& sk) {
+#pragma unroll
+  for (int e = 0; e < NREC; ++e) {
+    const int rec = tid + e * NT;
+    const int lane = rec & 63, k = rec >> 6;
+    if (k < ks) {
+      u4 pc[3];
+      split8<3>(sk, v[e], pc);
+#pragma unroll
+      for (int q = 0; q < 3; ++q) dst[(k * 3 + q) * 64 + lane] = pc[q];
+    }
+  }
+}
+
+// Workgroup = (batch b, NW consecutive channels), one channel per wavefront.  KS: 32-wide steps of
+// the contraction over r (d <= 32 KS).  n <= 16.
+template <int KS, int NW>
+__global__ __launch_bounds__(NW * 64) void dropin_fwd_kernel(const DropinArgs p) {
+  __shared__ u4 s_u[2][KS * 3 * 64];
+  const int tid = threadIdx.x, lane = tid & 63, wave = wave_index();
+  const int ncg = (p.d + NW - 1) / NW;
+  const int b = blockIdx.x / ncg, i = (blockIdx.x % ncg) * NW + wave;
+  const bool iok = i < p.d;
+  const int ic = iok ? i : p.d - 1;
+  const int l_ = lane & 15, g = lane >> 4;
+  const int d = p.d, n = p.n, L = p.L;
+  const SplitK sk = make_splitk();
+  const float* __restrict__ ub = p.u + (size_t)b * d * L;
+  const size_t row = ((size_t)b * d + ic) * L;
+
+  // this wavefront's rows of x, split, for the whole sequence
+  u4 xa[KS][3];
+#pragma unroll
+  for (int k = 0; k < KS; ++k)
+#pragma unroll
+    for (int q = 0; q < 3; ++q)
+      xa[k][q] = (k < p.ks) ? p.xp[(((size_t)ic * p.ks + k) * 3 + q) * 64 + lane] : u4{0, 0, 0, 0};
+  // per state j = 4 g + a: bias, Bt, Ct, carried state
+  float xb[4], btr[4], bti[4], ctr[4], cti[4], hr[4], hi[4];
+#pragma unroll
+  for (int a = 0; a < 4; ++a) {
+    const int j = 4 * g + a;
+    const bool ok = j < n;
+    const int jc = ok ? j : 0;
+    xb[a] = ok ? p.x_bias[(size_t)ic * n + jc] : 0.0f;
+    float s, c;
+    fast_sincosf(p.B_th[jc], &s, &c);
+    btr[a] = ok ? p.B_r[jc] * c : 0.0f;
+    bti[a] = ok ? p.B_r[jc] * s : 0.0f;
+    fast_sincosf(p.C_th[jc], &s, &c);
+    ctr[a] = ok ? p.C_r[jc] * c : 0.0f;
+    cti[a] = ok ? p.C_r[jc] * s : 0.0f;
+    hr[a] = ok ? p.h_re[((size_t)b * d + ic) * n + jc] : 0.0f;
+    hi[a] = ok ? p.h_im[((size_t)b * d + ic) * n + jc] : 0.0f;
+  }
+  const float Di = p.Dp[ic];
+  const int ntiles = (L + DT - 1) / DT;
+
+  constexpr int NT = NW * 64, NREC = (KS * 64 + NT - 1) / NT;
+  float sv[NREC][8];
+  stage_load<NT, NREC>(ub, sv, d, L, p.ks, 0, tid);
+  stage_store<NT, NREC>(sv, s_u[0], p.ks, tid, sk);
+  __syncthreads();
+  // the wavefront's own inputs, requested one tile ahead
+  float un = l_ < L ? p.u[row + l_] : 0.0f, dtn = l_ < L ? p.dt[row + l_] : 0.0f, zn = l_ < L ? p.z[row + l_] : 0.0f;
+  for (int t = 0; t < ntiles; ++t) {
+    const int l0 = t * DT, l = l0 + l_;
+    const bool lok = l < L;
+    const float uv = un, dtv = dtn, zv = zn;
+    {
+      const bool nok = l + DT < L;
+      un = nok ? p.u[row + l + DT] : 0.0f;
+      dtn = nok ? p.dt[row + l + DT] : 0.0f;
+      zn = nok ? p.z[row + l + DT] : 0.0f;
+    }
+    if (t + 1 < ntiles) stage_load<NT, NREC>(ub, sv, d, L, p.ks, l0 + DT, tid);
+    // ---- phases of the tile: lane (column l, rows j = 4 g + a)
+    f4 th = {0, 0, 0, 0};
+    const u4* su = s_u[t & 1];
+#pragma unroll
+    for (int k = 0; k < KS; ++k) {
+      if (k < p.ks) {
+        u4 ubk[3];
+#pragma unroll
+        for (int q = 0; q < 3; ++q) ubk[q] = su[(k * 3 + q) * 64 + lane];
+        th = xmm<3>(xa[k], ubk, th);
+      }
+    }
+    const float ut = siluf_(uv), w = dtv * ut;
+    float ysum = 0.0f;
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+      const float thv = lok ? th[a] + xb[a] : 0.0f;
+      const float G = row_prefix(thv);
+      float sn, cs;
+      fast_sincosf(G, &sn, &cs);
+      // p = conj(E) Bt w
+      const float pr = (cs * btr[a] + sn * bti[a]) * w, pi = (cs * bti[a] - sn * btr[a]) * w;
+      const float Rr = hr[a] + row_prefix(pr), Ri = hi[a] + row_prefix(pi);
+      // h = E R
+      const float her = cs * Rr - sn * Ri, hei = cs * Ri + sn * Rr;
+      ysum += ctr[a] * her - cti[a] * hei;
+      hr[a] = row_last(her, lane);
+      hi[a] = row_last(hei, lane);
+    }
+    ysum += __shfl_xor(ysum, 16);
+    ysum += __shfl_xor(ysum, 32);
+    if (p.y && iok && lok && g == 0) p.y[row + l] = siluf_(zv) * (ysum + Di * ut);
+    if (t + 1 < ntiles) stage_store<NT, NREC>(sv, s_u[(t + 1) & 1], p.ks, tid, sk);
+    __syncthreads();
+  }
+  if (p.nh_re && iok && l_ == 0) {
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+      const int j = 4 * g + a;
+      if (j < n) {
+        p.nh_re[((size_t)b * d + i) * n + j] = hr[a];
+        p.nh_im[((size_t)b * d + i) * n + j] = hi[a];
+      }
+    }
+  }
+}
+
+// ---- backward ---------------------------------------------------------------------------------
+//
+// Reverse sweep of the same tiles (the reference's ssm_adaptive_unitary_backward.cu:90-330 computes the
+// same gradients from the same twelve inputs).  With hats for adjoints (hat h = dL/dRe h + i dL/dIm h),
+// a_l = grad_y_l silu(z_l), and inside a tile G, E, p, R, h as in the forward kernel:
+//     hat R_l = conj(E_l) a_l conj(Ct)                      (+ conj(E_last) hat h_out at the tile's last step)
+//     hat p_s = sum_{l >= s} hat R_l,      hat h_in = hat p_first
+//     hat w_s = Re(E_s conj(Bt) hat p_s)   summed over the states
+//     hat G_l = -Im(conj(a_l conj(Ct)) h_l) + Im(conj(hat p_l) p_l)   (- Im(conj(hat h_out) h_last) at the last step)
+//     hat theta_s = sum_{l >= s} hat G_l                    (suffix sum inside the tile only: the state handed
+//                                                            to the next tile carries the rotation)
+//     hat Bt += E_s w_s hat p_s,   hat Ct += a_l conj(h_l),   hat D += a_l ut_l
+// The state at the end of each tile is recovered backwards (the recurrence is unitary, so this is
+// stable): R_last = conj(E_last) h_out, h_in = R_last - sum p.  h at the end of the sequence comes from
+// one forward sweep without outputs.
+//
+// hat theta is what the two products with x and u need:
+//     grad_x[i,j,r] = sum_{b,l} hat theta[b,i,j,l] u[b,r,l],   grad_u[b,r,l] += sum_{i,j} x[i,j,r] hat theta[b,i,j,l].
+// The second one sums over every channel of a batch element, so hat theta has to leave the wavefront
+// that made it: it goes to a workspace that holds it for a GROUP of batch elements only (tens of MB,
+// cache resident), and a matrix-core GEMM kernel consumes it before the next group overwrites it.
+
+__device__ __forceinline__ float row_sum(float v) {     // total of the row in its first lane (others: partial)
+  return row_suffix(v);
+}
+
+#ifndef DROPIN_BWD_WAVES
+#define DROPIN_BWD_WAVES 1
+#endif
+template <int KS, int NW>
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DROPIN_BWD_WAVES, DROPIN_BWD_WAVES))) void dropin_bwd_kernel(const DropinBwdArgs q) {
+  __shared__ u4 s_u[2][KS * 3 * 64];
+  const DropinArgs& p = q.f;
+  const int tid = threadIdx.x, lane = tid & 63, wave = wave_index();
+  const int ncg = (p.d + NW - 1) / NW;
+  const int zb = blockIdx.x / ncg, b = q.b0 + zb, i = (blockIdx.x % ncg) * NW + wave;
+  const bool iok = i < p.d;
+  const int ic = iok ? i : p.d - 1;
+  const int l_ = lane & 15, g = lane >> 4;
+  const int d = p.d, n = p.n, L = p.L;
+  const SplitK sk = make_splitk();
+  const float* __restrict__ ub = p.u + (size_t)b * d * L;
+  const size_t row = ((size_t)b * d + ic) * L;
+
+  u4 xa[KS][3];
+#pragma unroll
+  for (int k = 0; k < KS; ++k)
+#pragma unroll
+    for (int c = 0; c < 3; ++c)
+      xa[k][c] = (k < p.ks) ? p.xp[(((size_t)ic * p.ks + k) * 3 + c) * 64 + lane] : u4{0, 0, 0, 0};
+  float xb[4], btr[4], bti[4], ctr[4], cti[4], hr[4], hi[4], ar[4], ai[4];
+  float gBr[4], gBi[4], gCr[4], gCi[4], gxb[4];
+  bool jok[4];
+#pragma unroll
+  for (int a = 0; a < 4; ++a) {
+    const int j = 4 * g + a;
+    const bool ok = j < n;
+    jok[a] = ok;
+    const int jc = ok ? j : 0;
+    const size_t sidx = ((size_t)b * d + ic) * n + jc;
+    xb[a] = ok ? p.x_bias[(size_t)ic * n + jc] : 0.0f;
+    float s, c;
+    fast_sincosf(p.B_th[jc], &s, &c);
+    btr[a] = ok ? p.B_r[jc] * c : 0.0f;
+    bti[a] = ok ? p.B_r[jc] * s : 0.0f;
+    fast_sincosf(p.C_th[jc], &s, &c);
+    ctr[a] = ok ? p.C_r[jc] * c : 0.0f;
+    cti[a] = ok ? p.C_r[jc] * s : 0.0f;
+    hr[a] = ok ? q.hfin_re[sidx] : 0.0f;           // state at the end of the tile being processed
+    hi[a] = ok ? q.hfin_im[sidx] : 0.0f;
+    ar[a] = (ok && q.gnh_re) ? q.gnh_re[sidx] : 0.0f;   // its adjoint
+    ai[a] = (ok && q.gnh_im) ? q.gnh_im[sidx] : 0.0f;
+    gBr[a] = gBi[a] = gCr[a] = gCi[a] = gxb[a] = 0.0f;
+  }
+  const float Di = p.Dp[ic];
+  float gD = 0.0f;
+  const int ntiles = (L + DT - 1) / DT;
+  float* __restrict__ dth = q.dth + ((size_t)zb * d + ic) * n * L;
+
+  constexpr int NT = NW * 64, NREC = (KS * 64 + NT - 1) / NT;
+  float sv[NREC][8];
+  stage_load<NT, NREC>(ub, sv, d, L, p.ks, (ntiles - 1) * DT, tid);
+  stage_store<NT, NREC>(sv, s_u[(ntiles - 1) & 1], p.ks, tid, sk);
+  __syncthreads();
+  // the wavefront's own inputs, requested one tile ahead
+  float un, dtn, zn, gyn;
+  {
+    const int l = (ntiles - 1) * DT + l_;
+    const bool ok = l < L;
+    un = ok ? p.u[row + l] : 0.0f;
+    dtn = ok ? p.dt[row + l] : 0.0f;
+    zn = ok ? p.z[row + l] : 0.0f;
+    gyn = ok ? q.gy[row + l] : 0.0f;
+  }
+  for (int t = ntiles - 1; t >= 0; --t) {
+    const int l0 = t * DT, l = l0 + l_;
+    const bool lok = l < L;
+    const float uv = un, dtv = dtn, zv = zn, gyv = gyn;
+    if (t > 0) {                       // l - DT < L holds
+      un = p.u[row + l - DT];
+      dtn = p.dt[row + l - DT];
+      zn = p.z[row + l - DT];
+      gyn = q.gy[row + l - DT];
+    }
+    if (t > 0) stage_load<NT, NREC>(ub, sv, d, L, p.ks, l0 - DT, tid);
+    f4 th = {0, 0, 0, 0};
+    const u4* su = s_u[t & 1];
+#pragma unroll
+    for (int k = 0; k < KS; ++k) {
+      if (k < p.ks) {
+        u4 ubk[3];
+#pragma unroll
+        for (int c = 0; c < 3; ++c) ubk[c] = su[(k * 3 + c) * 64 + lane];
+        th = xmm<3>(xa[k], ubk, th);
+      }
+    }
+    const float ut = siluf_(uv), w = dtv * ut, sz = siluf_(zv), av = gyv * sz;
+    float ysum = 0.0f, wsum = 0.0f;
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+      const float thv = lok ? th[a] + xb[a] : 0.0f;
+      const float G = row_prefix(thv);
+      float sn, cs;
+      fast_sincosf(G, &sn, &cs);
+      const float csl = row_last(cs, lane), snl = row_last(sn, lane);
+      // forward quantities of the tile from the state at its end
+      const float pr = (cs * btr[a] + sn * bti[a]) * w, pi = (cs * bti[a] - sn * btr[a]) * w;
+      const float Ppr = row_prefix(pr), Ppi = row_prefix(pi);
+      const float Ptr = row_last(Ppr, lane), Pti = row_last(Ppi, lane);
+      const float Rer = csl * hr[a] + snl * hi[a], Rei = csl * hi[a] - snl * hr[a];   // conj(E_last) h_out
+      const float hinr = Rer - Ptr, hini = Rei - Pti;
+      const float Rr = hinr + Ppr, Ri = hini + Ppi;
+      const float her = cs * Rr - sn * Ri, hei = cs * Ri + sn * Rr;                  // h_l
+      ysum += ctr[a] * her - cti[a] * hei;
+      // adjoints
+      const float hdr = av * ctr[a], hdi = -av * cti[a];                              // a conj(Ct)
+      const float Rhr = cs * hdr + sn * hdi, Rhi = cs * hdi - sn * hdr;               // conj(E_l) (a conj(Ct))
+      const float Kr = csl * ar[a] + snl * ai[a], Ki = csl * ai[a] - snl * ar[a];     // conj(E_last) hat h_out
+      const float phr = row_suffix(Rhr) + Kr, phi = row_suffix(Rhi) + Ki;             // hat p_s
+      // hat w: Re(E conj(Bt) hat p)
+      const float ebr = cs * btr[a] + sn * bti[a], ebi = sn * btr[a] - cs * bti[a];   // E conj(Bt)
+      wsum += ebr * phr - ebi * phi;
+      // hat G
+      float Gh = -(hdr * hei - hdi * her) + (phr * pi - phi * pr);
+      if (l_ == 15) Gh -= ar[a] * hi[a] - ai[a] * hr[a];                              // h at the last step is h_out
+      const float thh = row_suffix(Gh);
+      if (lok && iok && jok[a]) dth[(size_t)(4 * g + a) * L + l] = thh;
+      gxb[a] += lok ? thh : 0.0f;
+      // hat Bt += E w hat p ; hat Ct += a conj(h)
+      const float ewr = cs * w, ewi = sn * w;
+      gBr[a] += ewr * phr - ewi * phi;
+      gBi[a] += ewr * phi + ewi * phr;
+      gCr[a] += av * her;
+      gCi[a] -= av * hei;
+      // hand over to the previous tile
+      hr[a] = hinr;
+      hi[a] = hini;
+      ar[a] = row_first(phr, lane);
+      ai[a] = row_first(phi, lane);
+    }
+    ysum += __shfl_xor(ysum, 16);
+    ysum += __shfl_xor(ysum, 32);
+    wsum += __shfl_xor(wsum, 16);
+    wsum += __shfl_xor(wsum, 32);
+    if (iok && lok && g == 0) {
+      const float pre = ysum + Di * ut;
+      q.dz[row + l] = gyv * pre * dsiluf_(zv);
+      q.ddt[row + l] = wsum * ut;
+      q.du[row + l] = (wsum * dtv + av * Di) * dsiluf_(uv);
+      gD += av * ut;
+    }
+    if (t > 0) stage_store<NT, NREC>(sv, s_u[(t - 1) & 1], p.ks, tid, sk);
+    __syncthreads();
+  }
+  // ---- reductions over the timesteps (lanes of a row) and hand-off
+#pragma unroll
+  for (int a = 0; a < 4; ++a) {
+    gxb[a] = row_sum(gxb[a]);
+    gBr[a] = row_sum(gBr[a]);
+    gBi[a] = row_sum(gBi[a]);
+    gCr[a] = row_sum(gCr[a]);
+    gCi[a] = row_sum(gCi[a]);
+  }
+  gD = row_sum(gD);
+  if (iok && l_ == 0) {
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+      const int j = 4 * g + a;
+      if (j < n) {
+        const size_t sidx = ((size_t)b * d + i) * n + j;
+        q.dh_re[sidx] = ar[a];
+        q.dh_im[sidx] = ai[a];
+        atomicAdd(q.dxb + (size_t)i * n + j, gxb[a]);
+        // polar parameters: Bt = B_r e^{i B_theta}
+        float ebr, ebi, ecr, eci;
+        fast_sincosf(p.B_th[j], &ebi, &ebr);
+        fast_sincosf(p.C_th[j], &eci, &ecr);
+        atomicAdd(q.dB_r + j, gBr[a] * ebr + gBi[a] * ebi);
+        atomicAdd(q.dB_th + j, gBi[a] * btr[a] - gBr[a] * bti[a]);
+        atomicAdd(q.dC_r + j, gCr[a] * ecr + gCi[a] * eci);
+        atomicAdd(q.dC_th + j, gCi[a] * ctr[a] - gCr[a] * cti[a]);
+      }
+    }
+    if (g == 0) atomicAdd(q.dD + i, gD);
+  }
+}
+
+__global__ __launch_bounds__(256) void fill_zero_kernel(float* __restrict__ p, size_t n) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) p[i] = 0.0f;
+}
+
+// ---- fp32-accurate GEMM on the bf16 matrix cores, operands in fp32 with arbitrary strides -------
+//     C_z[m][n] (+)= sum_k A_z(m, k) B_z(k, n)           z = 0 .. Z-1
+//     C[m][n]    += sum_z sum_k A_z(m, k) B_z(k, n)      (reduce_z)
+// Workgroup tile 128 x 64, four wavefronts of 64 x 32 each, 32 of k per step, one workgroup per
+// (tile, z, k slice); with more than one k slice, or with reduce_z, the results are summed into C with
+// atomics (C holds the addend beforehand).  Both operands are split into three bf16 pieces while
+// they are staged in LDS; the values of the next step are requested before the products of the
+// current one.
+// K1: both operands are contiguous along k.  Then four neighbouring lanes fetch the 32 values of
+// one row as 16-byte vectors (VEC: every row start is 16-byte aligned) - a wavefront request covers 16
+// cache lines.  Otherwise both are contiguous along m / n and a 16-lane row of the wavefront
+// fetches 16 neighbouring rows' values of one k.
+template <bool K1, bool VEC>
+__global__ __launch_bounds__(256) void split_gemm_kernel(const GemmArgs p) {
+  __shared__ u4 s_a[8 * 3 * 64], s_b[4 * 3 * 64];
+  const int tid = threadIdx.x, lane = tid & 63, wave = wave_index();
+  const int m0 = blockIdx.x * 128, n0 = blockIdx.y * 64;
+  const int z = blockIdx.z / p.ksplit, ksl = blockIdx.z % p.ksplit;
+  const int wm = (wave >> 1) * 4, wn = (wave & 1) * 2;       // this wavefront's first 16-wide tiles
+  const SplitK sk = make_splitk();
+  f4 acc[4][2];
+#pragma unroll
+  for (int e = 0; e < 4; ++e)
+#pragma unroll
+    for (int f = 0; f < 2; ++f) acc[e][f] = f4{0, 0, 0, 0};
+  // the three records this thread stages: rows ra, ra + 64 of the A tile and row rb of the B tile, k slots kq ..
+  const int ra = K1 ? tid >> 2 : wave * 16 + (lane & 15);
+  const int kq = 8 * (K1 ? tid & 3 : lane >> 4);
+  const int ma = m0 + ra, mb = ma + 64, nb = n0 + ra;
+  // ... and where they go in LDS: [16-row tile][piece][lane = 16 (kq / 8) + row % 16]
+  const int slot = (ra >> 4) * 192 + (kq >> 3) * 16 + (ra & 15);
+  // uniform bases, 32-bit per-thread offsets (a z-slice of either operand is below 2^31 elements)
+  const float* __restrict__ Az = p.A + z * p.saz;
+  const float* __restrict__ Bz = p.Bm + z * p.sbz;
+  const unsigned sak = (unsigned)p.sak, sbk = (unsigned)p.sbk;
+  const unsigned oa0 = (unsigned)ma * (unsigned)p.sam + (unsigned)kq * sak;
+  const unsigned oa1 = (unsigned)mb * (unsigned)p.sam + (unsigned)kq * sak;
+  const unsigned ob0 = (unsigned)nb * (unsigned)p.sbn + (unsigned)kq * sbk;
+  const int nk = (p.K + 31) / 32, per = (nk + p.ksplit - 1) / p.ksplit;
+  const int it0 = ksl * per, it1 = it0 + per < nk ? it0 + per : nk;
+  const bool inside = m0 + 128 <= p.M && n0 + 64 <= p.N;      // uniform over the workgroup
+  float va[2][8], vb[8];
+  auto fetch = [&](int it) {
+    const unsigned ka = (unsigned)(it * 32) * sak, kb = (unsigned)(it * 32) * sbk;
+    if (inside && it * 32 + 32 <= p.K) {
+      if constexpr (K1 && VEC) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const f4 x0 = *reinterpret_cast<const f4*>(Az + (oa0 + ka + 4 * h));
+          const f4 x1 = *reinterpret_cast<const f4*>(Az + (oa1 + ka + 4 * h));
+          const f4 x2 = *reinterpret_cast<const f4*>(Bz + (ob0 + kb + 4 * h));
+#pragma unroll
+          for (int c = 0; c < 4; ++c) {
+            va[0][4 * h + c] = x0[c];
+            va[1][4 * h + c] = x1[c];
+            vb[4 * h + c] = x2[c];
+          }
+        }
+      } else {
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+          va[0][c] = Az[oa0 + ka + (unsigned)c * sak];
+          va[1][c] = Az[oa1 + ka + (unsigned)c * sak];
+          vb[c] = Bz[ob0 + kb + (unsigned)c * sbk];
+        }
+      }
+    } else {
+#pragma unroll
+      for (int c = 0; c < 8; ++c) {
+        const bool kok = it * 32 + kq + c < p.K;
+        va[0][c] = (ma < p.M && kok) ? Az[oa0 + ka + (unsigned)c * sak] : 0.0f;
+        va[1][c] = (mb < p.M && kok) ? Az[oa1 + ka + (unsigned)c * sak] : 0.0f;
+        vb[c] = (nb < p.N && kok) ? Bz[ob0 + kb + (unsigned)c * sbk] : 0.0f;
+      }
+    }
+  };
+  if (it0 < it1) fetch(it0);
+  for (int it = it0; it < it1; ++it) {
+    u4 pa[2][3], pb[3];
+    split8<3>(sk, va[0], pa[0]);
+    split8<3>(sk, va[1], pa[1]);
+    split8<3>(sk, vb, pb);
+    __syncthreads();
+#pragma unroll
+    for (int c = 0; c < 3; ++c) {
+      s_a[slot + c * 64] = pa[0][c];
+      s_a[slot + 4 * 192 + c * 64] = pa[1][c];
+      s_b[slot + c * 64] = pb[c];
+    }
+    __syncthreads();
+    if (it + 1 < it1) fetch(it + 1);      // in flight during the products
+    u4 rb[2][3];
+#pragma unroll
+    for (int f = 0; f < 2; ++f)
+#pragma unroll
+      for (int c = 0; c < 3; ++c) rb[f][c] = s_b[((wn + f) * 3 + c) * 64 + lane];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      u4 rA[3];
+#pragma unroll
+      for (int c = 0; c < 3; ++c) rA[c] = s_a[((wm + e) * 3 + c) * 64 + lane];
+#pragma unroll
+      for (int f = 0; f < 2; ++f) acc[e][f] = xmm<3>(rA, rb[f], acc[e][f]);
+    }
+  }
+  // result tile (e, f): lane (column = lane % 16, rows 4 (lane / 16) + a)
+  float* __restrict__ C = p.C + (p.reduce_z ? 0 : z * p.scz);
+  const bool atomic = p.reduce_z || p.ksplit > 1;
+#pragma unroll
+  for (int e = 0; e < 4; ++e)
+#pragma unroll
+    for (int f = 0; f < 2; ++f)
+#pragma unroll
+      for (int a = 0; a < 4; ++a) {
+        const int m = m0 + (wm + e) * 16 + 4 * (lane >> 4) + a, nn = n0 + (wn + f) * 16 + (lane & 15);
+        if (m < p.M && nn < p.N) {
+          float* c = C + m * p.scm + nn * p.scn;
+          if (atomic) atomicAdd(c, acc[e][f][a]);
+          else *c = p.accumulate ? *c + acc[e][f][a] : acc[e][f][a];
+        }
+      }
+}
+
+}  // namespace aussm

@@ -1,0 +1,62 @@
+// Argument blocks of the fused operator kernels (dropin.h), shared with the host side.
+#pragma once
+#include "scan_args.h"
+
+namespace aussm {
+
+constexpr int DT = 16;            // timesteps per tile
+constexpr int D_MAXKS = 16;       // 32-wide steps of the contraction over r held in registers: d <= 512
+constexpr int D_MAXN = 16;        // states per channel
+
+struct DropinArgs {
+  const float* u;        // [b, d, L]
+  const float* dt;       // [b, d, L]
+  const float* z;        // [b, d, L]
+  const float* x_bias;   // [d, n]
+  const float* B_r;      // [n]
+  const float* B_th;
+  const float* C_r;
+  const float* C_th;
+  const float* Dp;       // [d]
+  const float* h_re;     // [b, d, n]
+  const float* h_im;
+  float* y;              // [b, d, L] or null (states only)
+  float* nh_re;          // [b, d, n] or null
+  float* nh_im;
+  const u4* xp;          // rows of x as matrix operands: [d][ks][piece][64 lanes]
+  int b, d, n, L, ks;    // ks = ceil(d / 32)
+};
+
+struct DropinBwdArgs {
+  DropinArgs f;            // inputs (y, nh_* unused)
+  const float* gy;         // [b, d, L]
+  const float* gnh_re;     // [b, d, n] or null
+  const float* gnh_im;
+  const float* hfin_re;    // [b, d, n] state at the end of the sequence
+  const float* hfin_im;
+  float* dth;              // workspace [bg][d n][L]
+  float* du;               // [b, d, L] direct part (the product with x is added afterwards)
+  float* ddt;
+  float* dz;
+  float* dxb;              // [d, n]   accumulated with atomics (zeroed by the host)
+  float* dB_r;             // [n] each, accumulated with atomics
+  float* dB_th;
+  float* dC_r;
+  float* dC_th;
+  float* dD;               // [d]      (atomics)
+  float* dh_re;            // [b, d, n]
+  float* dh_im;
+  int b0, bg;              // batch elements b0 .. b0 + bg - 1
+};
+
+struct GemmArgs {
+  const float* A; const float* Bm; float* C;
+  long sam, sak, saz;     // element strides of A over m, k, z
+  long sbk, sbn, sbz;
+  long scm, scn, scz;
+  int M, N, K, Z;
+  int reduce_z, accumulate;
+  int ksplit;             // workgroups along k per (tile, z); > 1 sums into C with atomics
+};
+
+}  // namespace aussm

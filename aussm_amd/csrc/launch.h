@@ -5,6 +5,7 @@
 #include <hip/hip_runtime.h>
 
 #include "scan_args.h"
+#include "dropin_args.h"
 
 namespace aussm {
 
@@ -38,5 +39,12 @@ void run_seg_carry_bwd(float* seg, const float* ptot, const float* dhL, float* d
 void run_px_prep(const PrepArgs& a, int B, int in_dtype, hipStream_t s);
 int run_px_fwd(const FwdArgs& a, const u4* img, int in_dtype, hipStream_t s);
 int run_px_bwd(const UniBwdArgs& a, const u4* img, int in_dtype, hipStream_t s);
+
+// ---- k_dropin.hip: the reference's 12-input operator as fused kernels
+void run_dropin_xprep(const float* x, u4* xp, int d, int n, int ks, hipStream_t s);
+int run_dropin_fwd(const DropinArgs& a, hipStream_t s);
+int run_dropin_bwd(const DropinBwdArgs& a, hipStream_t s);
+void run_fill_zero(float* p, size_t n, hipStream_t s);
+int run_split_gemm(const GemmArgs& a, hipStream_t s);
 
 }  // namespace aussm

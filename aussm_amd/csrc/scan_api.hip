@@ -457,4 +457,129 @@ int aussm_swap_last2(const float* x, float* y, int B, int R, int C, long long xs
   return run_swap_last2(a, B, (hipStream_t)stream);
 }
 
+// ---- the reference's operator extension_cpp::ssm_adaptive_unitary as fused kernels (dropin.h)
+
+static size_t dropin_xp_floats(int d) { return (size_t)d * ((d + 31) / 32) * 3 * 64 * 4; }
+// batch elements whose phase adjoints the workspace holds at a time: at most about 96 MiB of them, in
+// groups of equal size
+static int dropin_group(int b, int d, int n, int L) {
+  const size_t per = (size_t)d * n * L, cap = (size_t)24 << 20;
+  size_t gmax = cap / per;
+  if (gmax < 1) gmax = 1;
+  const size_t ng = ((size_t)b + gmax - 1) / gmax;
+  return (int)(((size_t)b + ng - 1) / ng);
+}
+// k slices of a GEMM launch: enough workgroups for about three per compute unit, at least four steps each
+static int gemm_ksplit(int M, int N, int K, int Z) {
+  const long tiles = (long)((M + 127) / 128) * ((N + 63) / 64) * Z;
+  const int nk = (K + 31) / 32;
+  long s = (768 + tiles - 1) / tiles;
+  if (s > nk / 4) s = nk / 4;
+  if (s < 1) s = 1;
+  while (s > 1 && (long)Z * s > 65535) --s;
+  return (int)s;
+}
+static size_t round4(size_t v) { return (v + 3) & ~(size_t)3; }
+static int dropin_check(int b, int d, int n, int L) {
+  if (b < 1 || d < 1 || n < 1 || L < 1) return AUSSM_E_SHAPE;
+  if (n > D_MAXN || d > 32 * D_MAXKS) return AUSSM_E_SHAPE;
+  if ((long long)b * ((d + 3) / 4) > 0x7fffffffLL || (long long)d * n * L > 0x7fffffffLL) return AUSSM_E_SHAPE;
+  return AUSSM_OK;
+}
+
+size_t aussm_ssm_adaptive_unitary_workspace_floats(int b, int d, int n, int L, int backward) {
+  if (dropin_check(b, d, n, L) != AUSSM_OK) return 0;
+  size_t f = dropin_xp_floats(d);
+  if (backward) f += 2 * round4((size_t)b * d * n) + (size_t)dropin_group(b, d, n, L) * d * n * L;
+  return f;
+}
+
+int aussm_ssm_adaptive_unitary_fwd(const float* u, const float* dt, const float* x, const float* x_bias,
+                                   const float* B_r, const float* B_theta, const float* C_r, const float* C_theta,
+                                   const float* D, const float* z, const float* h_re, const float* h_im,
+                                   float* y, float* nh_re, float* nh_im, float* workspace,
+                                   int b, int d, int n, int L, void* stream) {
+  if (int e = dropin_check(b, d, n, L)) return e;
+  if (!u || !dt || !x || !x_bias || !B_r || !B_theta || !C_r || !C_theta || !D || !z || !h_re || !h_im || !y ||
+      !nh_re || !nh_im || !workspace)
+    return AUSSM_E_NULL;
+  if (misaligned(workspace, 16)) return AUSSM_E_ALIGN;
+  hipStream_t s = (hipStream_t)stream;
+  const int ks = (d + 31) / 32;
+  run_dropin_xprep(x, (u4*)workspace, d, n, ks, s);
+  DropinArgs a{u, dt, z, x_bias, B_r, B_theta, C_r, C_theta, D, h_re, h_im, y, nh_re, nh_im, (const u4*)workspace,
+               b, d, n, L, ks};
+  return run_dropin_fwd(a, s);
+}
+
+int aussm_ssm_adaptive_unitary_bwd(const float* grad_y, const float* grad_nh_re, const float* grad_nh_im,
+                                   const float* u, const float* dt, const float* x, const float* x_bias,
+                                   const float* B_r, const float* B_theta, const float* C_r, const float* C_theta,
+                                   const float* D, const float* z, const float* h_re, const float* h_im,
+                                   const float* nh_re, const float* nh_im,
+                                   float* du, float* ddt, float* dx, float* dx_bias, float* dB_r, float* dB_theta,
+                                   float* dC_r, float* dC_theta, float* dD, float* dz, float* dh_re, float* dh_im,
+                                   float* workspace, int b, int d, int n, int L, void* stream) {
+  if (int e = dropin_check(b, d, n, L)) return e;
+  if (!grad_y || !u || !dt || !x || !x_bias || !B_r || !B_theta || !C_r || !C_theta || !D || !z || !h_re || !h_im ||
+      !du || !ddt || !dx || !dx_bias || !dB_r || !dB_theta || !dC_r || !dC_theta || !dD || !dz || !dh_re || !dh_im ||
+      !workspace)
+    return AUSSM_E_NULL;
+  if (misaligned(workspace, 16)) return AUSSM_E_ALIGN;
+  hipStream_t s = (hipStream_t)stream;
+  const int ks = (d + 31) / 32, bg = dropin_group(b, d, n, L);
+  const size_t nstate = (size_t)b * d * n;
+  u4* xp = (u4*)workspace;
+  float* ws_re = workspace + dropin_xp_floats(d);
+  float* ws_im = ws_re + round4(nstate);
+  float* dth = ws_im + round4(nstate);
+  run_dropin_xprep(x, xp, d, n, ks, s);
+  DropinArgs f{u, dt, z, x_bias, B_r, B_theta, C_r, C_theta, D, h_re, h_im, nullptr, ws_re, ws_im, xp, b, d, n, L, ks};
+  const float* hfin_re = nh_re;
+  const float* hfin_im = nh_im;
+  if (!nh_re || !nh_im) {
+    // the state at the end of the sequence: one forward sweep without outputs
+    if (int e = run_dropin_fwd(f, s)) return e;
+    hfin_re = ws_re;
+    hfin_im = ws_im;
+  }
+  run_fill_zero(dx, (size_t)d * n * d, s);
+  run_fill_zero(dx_bias, (size_t)d * n, s);
+  run_fill_zero(dB_r, n, s);
+  run_fill_zero(dB_theta, n, s);
+  run_fill_zero(dC_r, n, s);
+  run_fill_zero(dC_theta, n, s);
+  run_fill_zero(dD, d, s);
+  const long dn = (long)d * n;
+  for (int b0 = 0; b0 < b; b0 += bg) {
+    const int g = b - b0 < bg ? b - b0 : bg;
+    DropinBwdArgs q{};
+    q.f = f;
+    q.f.nh_re = q.f.nh_im = nullptr;
+    q.gy = grad_y; q.gnh_re = grad_nh_re; q.gnh_im = grad_nh_im;
+    q.hfin_re = hfin_re; q.hfin_im = hfin_im; q.dth = dth;
+    q.du = du; q.ddt = ddt; q.dz = dz; q.dxb = dx_bias;
+    q.dB_r = dB_r; q.dB_th = dB_theta; q.dC_r = dC_r; q.dC_th = dC_theta; q.dD = dD;
+    q.dh_re = dh_re; q.dh_im = dh_im; q.b0 = b0; q.bg = g;
+    if (int e = run_dropin_bwd(q, s)) return e;
+    // grad_u[b, r, l] += sum_(i j) x[(i j), r] hat theta[b, (i j), l]
+    GemmArgs gu{};
+    gu.A = x; gu.sam = 1; gu.sak = d; gu.saz = 0;
+    gu.Bm = dth; gu.sbk = L; gu.sbn = 1; gu.sbz = dn * L;
+    gu.C = du + (size_t)b0 * d * L; gu.scm = L; gu.scn = 1; gu.scz = (long)d * L;
+    gu.M = d; gu.N = L; gu.K = (int)dn; gu.Z = g; gu.reduce_z = 0; gu.accumulate = 1;
+    gu.ksplit = gemm_ksplit(gu.M, gu.N, gu.K, g);
+    if (int e = run_split_gemm(gu, s)) return e;
+    // grad_x[(i j), r] += sum_b sum_l hat theta[b, (i j), l] u[b, r, l]
+    GemmArgs gx{};
+    gx.A = dth; gx.sam = L; gx.sak = 1; gx.saz = dn * L;
+    gx.Bm = u + (size_t)b0 * d * L; gx.sbk = 1; gx.sbn = L; gx.sbz = (long)d * L;
+    gx.C = dx; gx.scm = d; gx.scn = 1; gx.scz = 0;
+    gx.M = (int)dn; gx.N = d; gx.K = L; gx.Z = g; gx.reduce_z = 1; gx.accumulate = 1;
+    gx.ksplit = gemm_ksplit(gx.M, gx.N, gx.K, g);
+    if (int e = run_split_gemm(gx, s)) return e;
+  }
+  return AUSSM_OK;
+}
+
 }  // extern "C"

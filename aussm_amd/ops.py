@@ -13,12 +13,16 @@ Operator semantics (ssm_adaptive_unitary_forward.cu:83-181), per batch b, channe
     h_l[b,i,j]     = exp(i theta_l) h_{l-1}[b,i,j] + Bt_j dt_l[b,i] silu(u_l[b,i]),   Bt_j = B_r[j] e^{i B_theta[j]}
     y_l[b,i]       = silu(z_l[b,i]) * ( sum_j Re(Ct_j h_l[b,i,j]) + D_i silu(u_l[b,i]) )
 
-How it maps onto the core scan kernel: dividing the state by the constant Bt_j is not needed --
-instead every (batch, state) pair becomes one batch element of a core scan with ONE state per
-channel: its phase is theta[b, j] (channels x time), its B_t and C_t are the constants Bt_j and
-Ct_j, and the sum over j is taken afterwards.  The phase projection is a plain GEMM
-(x as a (d n) x d matrix times u), done by the BLAS behind torch.matmul.  The backward operator
-re-runs this composition under autograd, so its scan gradients come from the HIP reverse scan.
+The two dispatcher ops run the library's fused kernels (aussm_ssm_adaptive_unitary_fwd / _bwd,
+include/aussm_hip.h): the phase tensor theta (b, d, n, l) is formed tile by tile inside the scan
+kernel and never stored, and the backward op recomputes from the twelve inputs as the reference's
+does.  Shapes beyond the fused kernels' limits (n > 16 or d > 512) raise.
+
+`_composite` is a second, independent route to the same numbers, kept for the interface's
+save_intermediates=True mode and as a cross-check in the tests: every (batch, state) pair becomes
+one batch element of a core scan with ONE state per channel - its phase is theta[b, j]
+(channels x time), its B_t and C_t are the constants Bt_j and Ct_j - the phase projection is a
+BLAS GEMM, and the sum over j is taken afterwards.
 """
 from __future__ import annotations
 
@@ -28,6 +32,7 @@ import torch
 import torch.nn.functional as F
 from torch import Tensor
 
+from . import _lib as L
 from . import scan
 
 __all__ = ["ssm_adaptive_unitary", "ssm_adaptive_interface", "pad_to_multiple_of"]
@@ -96,23 +101,58 @@ _lib.define(_FWD_SCHEMA)
 _lib.define(_BWD_SCHEMA)
 
 
+def _workspace(b, d, n, l, backward, device):
+    floats = L.load().aussm_ssm_adaptive_unitary_workspace_floats(b, d, n, l, int(backward))
+    if floats == 0:
+        raise RuntimeError(f"ssm_adaptive_unitary: shape (b={b}, d={d}, n={n}, l={l}) is outside the fused kernels' "
+                           "range (n <= 16, d <= 512)")
+    return torch.empty(floats, device=device, dtype=torch.float32)
+
+
 def _fwd_impl(u, dt, x, x_bias, B_r, B_theta, C_r, C_theta, D, z, h_r, h_i):
-    with torch.no_grad():
-        return _composite(u, dt, x, x_bias, B_r, B_theta, C_r, C_theta, D, z, h_r, h_i)
+    args = [t.contiguous() for t in (u, dt, x, x_bias, B_r, B_theta, C_r, C_theta, D, z, h_r, h_i)]
+    b, d, n, l = _check_op_inputs(args)
+    with torch.cuda.device(u.device):
+        y, nh_r, nh_i = torch.empty_like(args[0]), torch.empty_like(args[10]), torch.empty_like(args[11])
+        ws = _workspace(b, d, n, l, False, u.device)
+        L.check(L.load().aussm_ssm_adaptive_unitary_fwd(
+            *[L.ptr(t) for t in args], L.ptr(y), L.ptr(nh_r), L.ptr(nh_i), L.ptr(ws), b, d, n, l,
+            scan._stream()), "aussm_ssm_adaptive_unitary_fwd")
+    return y, nh_r, nh_i
 
 
-def _bwd_impl(grad_y, grad_hr, grad_hi, u, dt, x, x_bias, B_r, B_theta, C_r, C_theta, D, z, h_r, h_i):
-    with torch.enable_grad():
-        leaves = [t.detach().requires_grad_(True) for t in (u, dt, x, x_bias, B_r, B_theta, C_r, C_theta, D, z,
-                                                              h_r, h_i)]
-        outs = _composite(*leaves)
-        grads = torch.autograd.grad(outs, leaves, [grad_y.contiguous(), grad_hr.contiguous(), grad_hi.contiguous()],
-                                    allow_unused=True)
-    return tuple(torch.zeros_like(t) if g is None else g.contiguous() for g, t in zip(grads, leaves))
+def _bwd_impl(grad_y, grad_hr, grad_hi, u, dt, x, x_bias, B_r, B_theta, C_r, C_theta, D, z, h_r, h_i,
+              nh_r=None, nh_i=None):
+    args = [t.contiguous() for t in (u, dt, x, x_bias, B_r, B_theta, C_r, C_theta, D, z, h_r, h_i)]
+    b, d, n, l = _check_op_inputs(args)
+    grads_in = [grad_y.contiguous(), grad_hr.contiguous(), grad_hi.contiguous()]
+    for name, t, like in zip(("grad_y", "grad_next_hid_real", "grad_next_hid_imag"), grads_in,
+                             (args[0], args[10], args[11])):
+        if t.dtype != torch.float32 or tuple(t.shape) != tuple(like.shape):
+            raise RuntimeError(f"expected {name} float32 of shape {tuple(like.shape)}, got {t.dtype} {tuple(t.shape)}")
+    with torch.cuda.device(u.device):
+        outs = [torch.empty_like(t) for t in args]
+        ws = _workspace(b, d, n, l, True, u.device)
+        L.check(L.load().aussm_ssm_adaptive_unitary_bwd(
+            *[L.ptr(t) for t in grads_in], *[L.ptr(t) for t in args],
+            L.ptr(None if nh_r is None else nh_r.contiguous()), L.ptr(None if nh_i is None else nh_i.contiguous()),
+            *[L.ptr(t) for t in outs], L.ptr(ws),
+            b, d, n, l, scan._stream()), "aussm_ssm_adaptive_unitary_bwd")
+    return tuple(outs)
 
 
 _lib.impl("ssm_adaptive_unitary", _fwd_impl, "CUDA")
 _lib.impl("ssm_adaptive_backward_unitary", _bwd_impl, "CUDA")
+
+# The backward operator above gets what the reference's gets: gradients and the twelve inputs, so it
+# first re-runs the forward recurrence to find the state at the end of the sequence, where the
+# reverse sweep starts.  The autograd formula has that state already (it is an output of the forward
+# operator), so it calls this variant, which takes it as two more inputs and skips the re-run.
+_own = torch.library.Library("aussm_amd", "FRAGMENT")
+_own.define(_BWD_SCHEMA.replace("ssm_adaptive_backward_unitary(", "ssm_adaptive_backward_unitary_from_state(")
+            .replace("Tensor prev_hidden_state_imag) ->", "Tensor prev_hidden_state_imag, Tensor next_hid_real, "
+                     "Tensor next_hid_imag) ->"))
+_own.impl("ssm_adaptive_backward_unitary_from_state", _bwd_impl, "CUDA")
 
 
 @torch.library.register_fake(f"{_NS}::ssm_adaptive_unitary")
@@ -122,6 +162,11 @@ def _fwd_fake(u, dt, x, x_bias, B_r, B_theta, C_r, C_theta, D, z, h_r, h_i):
 
 @torch.library.register_fake(f"{_NS}::ssm_adaptive_backward_unitary")
 def _bwd_fake(grad_y, grad_hr, grad_hi, u, dt, x, x_bias, B_r, B_theta, C_r, C_theta, D, z, h_r, h_i):
+    return tuple(torch.empty_like(t) for t in (u, dt, x, x_bias, B_r, B_theta, C_r, C_theta, D, z, h_r, h_i))
+
+
+@torch.library.register_fake("aussm_amd::ssm_adaptive_backward_unitary_from_state")
+def _bwd_state_fake(grad_y, grad_hr, grad_hi, u, dt, x, x_bias, B_r, B_theta, C_r, C_theta, D, z, h_r, h_i, nh_r, nh_i):
     return tuple(torch.empty_like(t) for t in (u, dt, x, x_bias, B_r, B_theta, C_r, C_theta, D, z, h_r, h_i))
 
 
@@ -137,18 +182,19 @@ def backward_unitary(ctx, grad_y, grad_next_hidden_state_real, grad_next_hidden_
     """Autograd formula (ops.py:109-146): gradients for the 12 inputs, in input order."""
     saved = ctx.saved_tensors
     try:
-        return torch.ops.extension_cpp.ssm_adaptive_backward_unitary.default(
+        return torch.ops.aussm_amd.ssm_adaptive_backward_unitary_from_state.default(
             grad_y, grad_next_hidden_state_real, grad_next_hidden_state_imag, *saved)
     except RuntimeError:
-        shapes = {k: tuple(t.shape) for k, t in zip(_INPUT_NAMES, saved)}
+        shapes = {k: tuple(t.shape) for k, t in zip(_INPUT_NAMES, saved[:12])}
         shapes["grad_y"] = tuple(grad_y.shape)
         print(f"Runtime Error for {shapes}")
         raise
 
 
 def setup_context_unitary(ctx, inputs, output):
-    # like the reference (ops.py:148-151): only the 12 inputs are kept for the backward pass
-    ctx.save_for_backward(*inputs)
+    # like the reference (ops.py:148-151) the 12 inputs are kept for the backward pass - no intermediate of
+    # the size of the sequence - plus the two (b, d, n) end states, where the reverse sweep starts
+    ctx.save_for_backward(*inputs, output[1], output[2])
 
 
 torch.library.register_autograd(f"{_NS}::ssm_adaptive_unitary", backward_unitary,
@@ -166,7 +212,7 @@ def pad_to_multiple_of(tensor: Tensor, multiple_of: int) -> Tensor:
 
 def ssm_adaptive_interface(u: Tensor, dt: Tensor, x: Tensor, x_bias: Tensor, B: Tensor, C: Tensor, D: Tensor,
                            z: Tensor, unitary: bool = True, preal: bool = False,
-                           max_parallel_length: int = 2048, save_intermediates: bool = True, **kwargs) -> Tensor:
+                           max_parallel_length: int = 2048, save_intermediates: bool = False, **kwargs) -> Tensor:
     """Front-end of the adaptive-unitary operator (ops.py:28-93).
 
     u, dt, z: (b, d, l) float32; x: (d, n, d); x_bias: (d, n); B, C: (n,) complex64; D: (d,).
@@ -177,10 +223,12 @@ def ssm_adaptive_interface(u: Tensor, dt: Tensor, x: Tensor, x_bias: Tensor, B: 
     (The reference zero-pads the sequence to a multiple of 16 for its kernel; this kernel takes
     any length, and the padded steps never influence the returned y.)
 
-    save_intermediates (not in the reference): True keeps the phase tensor (b, n, d, l) and the
-    scan's checkpoints for the backward pass; False goes through the dispatcher operator, whose
-    backward pass keeps only the twelve inputs and recomputes, as the reference's does
-    (ops.py:148-151) - less memory, one more phase projection and forward scan per step.
+    save_intermediates (not in the reference): False, the default, goes through the dispatcher
+    operator, i.e. the fused kernels: the phase tensor (b, d, n, l) is never stored and the backward
+    pass keeps only the twelve inputs and the end state and recomputes, as the reference's does
+    (ops.py:148-151).  True takes the composite route instead (BLAS phase projection + core scan),
+    which holds the phase tensor and the scan's checkpoints for the backward pass - n times the
+    memory, and slower at the benchmark's training shape; it is kept as an independent cross-check.
     """
     assert not (unitary and preal), "Both unitary and preal cannot be used at the same time"
     if not unitary:

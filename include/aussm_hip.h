@@ -255,6 +255,47 @@ int aussm_causal_conv1d_bwd(const float* dy, const float* x, const float* w,
 int aussm_swap_last2(const float* x, float* y, int B, int R, int C,
                      long long xs_b, long long xs_r, void* stream);
 
+/* ---------------------------------------------------------------------------------------
+ * The reference's custom operator itself, as two calls: what
+ *   torch.ops.extension_cpp.ssm_adaptive_unitary           (12 tensors -> y, next_hid_real, next_hid_imag)
+ *   torch.ops.extension_cpp.ssm_adaptive_backward_unitary  (3 + 12 tensors -> 12 gradients)
+ * bind to - extension-cpp/extension_cpp/csrc/cuda/ssm_adaptive_unitary_forward.cu:184-286 and
+ * ssm_adaptive_unitary_backward.cu:333-497, Python side extension-cpp/extension_cpp/ops.py:97-154.
+ * Arguments in the operator's order; all tensors fp32 and contiguous:
+ *   u, dt, z (b, d, L);  x (d, n, d);  x_bias (d, n);  B_r, B_theta, C_r, C_theta (n);  D (d);
+ *   h_re, h_im (b, d, n) the state before the first step;  y (b, d, L);  nh_* (b, d, n).
+ *     theta_l[b,i,j] = sum_r x[i,j,r] u_l[b,r] + x_bias[i,j]
+ *     h_l[b,i,j]     = exp(i theta_l) h_{l-1}[b,i,j] + B_r[j] e^{i B_theta[j]} dt_l[b,i] silu(u_l[b,i])
+ *     y_l[b,i]       = silu(z_l[b,i]) ( sum_j Re(C_r[j] e^{i C_theta[j]} h_l[b,i,j]) + D[i] silu(u_l[b,i]) )
+ * The phase tensor theta (b, d, n, L) is never stored: the forward call forms it tile by tile on
+ * the matrix cores inside the scan kernel.  The backward call recomputes from the twelve inputs,
+ * as the reference does, and needs the phase adjoints of a few batch elements at a time (for the
+ * product that sums over all channels); they live in the workspace, at most about 96 MiB.
+ * Limits: n <= 16, d <= 512 (AUSSM_E_SHAPE beyond).  L is arbitrary (the reference needs a
+ * multiple of 16 and pads).  `workspace` holds aussm_ssm_adaptive_unitary_workspace_floats(...)
+ * floats, 16-byte aligned; nothing in it has to be initialised, nothing in it is kept between calls.
+ * grad_nh_re / grad_nh_im may be NULL (zero).  Every gradient buffer is fully written.
+ * nh_re / nh_im of the backward call: the state after the last step as the forward call returned it,
+ * or NULL - then the backward call recomputes it with one forward sweep (the reference's backward
+ * operator gets the twelve inputs only), which costs about one forward call more.
+ * ------------------------------------------------------------------------------------- */
+size_t aussm_ssm_adaptive_unitary_workspace_floats(int b, int d, int n, int L, int backward);
+
+int aussm_ssm_adaptive_unitary_fwd(const float* u, const float* dt, const float* x, const float* x_bias,
+                                   const float* B_r, const float* B_theta, const float* C_r, const float* C_theta,
+                                   const float* D, const float* z, const float* h_re, const float* h_im,
+                                   float* y, float* nh_re, float* nh_im, float* workspace,
+                                   int b, int d, int n, int L, void* stream);
+
+int aussm_ssm_adaptive_unitary_bwd(const float* grad_y, const float* grad_nh_re, const float* grad_nh_im,
+                                   const float* u, const float* dt, const float* x, const float* x_bias,
+                                   const float* B_r, const float* B_theta, const float* C_r, const float* C_theta,
+                                   const float* D, const float* z, const float* h_re, const float* h_im,
+                                   const float* nh_re, const float* nh_im,
+                                   float* du, float* ddt, float* dx, float* dx_bias, float* dB_r, float* dB_theta,
+                                   float* dC_r, float* dC_theta, float* dD, float* dz, float* dh_re, float* dh_im,
+                                   float* workspace, int b, int d, int n, int L, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -93,9 +93,9 @@ def test_error_behaviour():
 
 
 def test_dispatcher_operators_pass_opcheck():
-    """torch.library.opcheck on the forward dispatcher operator: schema (no input is mutated),
-    autograd registration, the shape-only implementation against the real one, and tracing.  (The
-    backward operator's shape-only implementation is covered by tests/test_ops_fake.py.)"""
+    """torch.library.opcheck on the dispatcher operators: schema (no input is mutated), autograd
+    registration of the forward one, the shape-only implementations against the real ones, and
+    tracing."""
     from aussm_amd import ops  # noqa: F401
     u, dt, x, xb, Bp, Cp, D, z = O.make_adaptive_inputs(b=2, d=8, n=4, l=32, binary_u=False, seed=7)
     Br, Bt, Cr, Ct = O.polar_params(Bp, Cp)
@@ -104,3 +104,11 @@ def test_dispatcher_operators_pass_opcheck():
     print("case opcheck forward", flush=True)
     torch.library.opcheck(torch.ops.extension_cpp.ssm_adaptive_unitary.default,
                           tuple(a.clone().requires_grad_(True) for a in args), atol=1e-4, rtol=1e-4)
+    g = torch.Generator().manual_seed(3)
+    grads = _cuda([torch.randn(2, 8, 32, generator=g), torch.randn(2, 8, 4, generator=g), torch.randn(2, 8, 4, generator=g)])
+    print("case opcheck backward", flush=True)
+    torch.library.opcheck(torch.ops.extension_cpp.ssm_adaptive_backward_unitary.default, tuple(grads + args),
+                          atol=1e-4, rtol=1e-4)
+    nh = list(torch.ops.extension_cpp.ssm_adaptive_unitary(*args)[1:])
+    torch.library.opcheck(torch.ops.aussm_amd.ssm_adaptive_backward_unitary_from_state.default,
+                          tuple(grads + args + nh), atol=1e-4, rtol=1e-4)

@@ -1,0 +1,136 @@
+"""The fused operator kernels (aussm_ssm_adaptive_unitary_fwd / _bwd behind
+torch.ops.extension_cpp.ssm_adaptive_unitary and ssm_adaptive_backward_unitary) against the CPU oracle's
+sequential-loop restatement of the operator in float64 (oracle.scan_oracle.adaptive_unitary_op_loop) and
+its autograd gradients: all three outputs, all twelve gradients, explicit start state and state
+gradients, ragged shapes (l not a multiple of the 16-step tile, d not a multiple of 32 or of the
+channels per workgroup, n < 16).  Tolerance: the benchmark contract's 1e-4 after normalising each
+tensor by its largest oracle entry (the reference's own forward tolerance is atol 7e-5, rtol 5e-5,
+extension-cpp/test/test_extension.py:95).  A last case at the benchmark's training shape checks the
+fused kernels against the package's composite route (BLAS phase projection + core scan)."""
+import pytest
+import torch
+
+from oracle import scan_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+IN_NAMES = ["u", "dt", "x", "x_bias", "B_r", "B_theta", "C_r", "C_theta", "D", "z", "h_re", "h_im"]
+
+
+def _inputs(b, d, n, l, seed, dtype=torch.float64, xscale=None):
+    u, dt, x, xb, Bp, Cp, D, z = O.make_adaptive_inputs(b=b, d=d, n=n, l=l, binary_u=False, seed=seed, dtype=dtype)
+    if xscale is not None:
+        x = x * xscale
+    Br, Bt, Cr, Ct = O.polar_params(Bp, Cp)
+    g = torch.Generator().manual_seed(seed + 100)
+    hr = torch.randn(b, d, n, generator=g, dtype=torch.float64).to(dtype)
+    hi = torch.randn(b, d, n, generator=g, dtype=torch.float64).to(dtype)
+    return [u, dt, x, xb, Br, Bt, Cr, Ct, D, z, hr, hi]
+
+
+def _close(got, want, name, tol=1e-4):
+    scale = max(1e-3, float(want.abs().max()))
+    torch.testing.assert_close(got.double().cpu() / scale, want.double() / scale, atol=tol, rtol=tol,
+                               msg=lambda m: f"{name}: {m}")
+
+
+SHAPES = [(2, 8, 4, 256), (3, 20, 5, 48), (2, 37, 16, 45), (1, 70, 11, 130), (2, 16, 16, 14)]
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+def test_fused_forward_matches_oracle(shape):
+    from aussm_amd import ops  # noqa: F401
+    b, d, n, l = shape
+    print(f"case fused fwd b={b} d={d} n={n} l={l}", flush=True)
+    args = _inputs(b, d, n, l, seed=3, xscale=d ** -0.5)
+    want = O.adaptive_unitary_op_loop(*args)
+    got = torch.ops.extension_cpp.ssm_adaptive_unitary(*[a.float().cuda() for a in args])
+    for w, g_, name in zip(want, got, ("y", "next_hid_real", "next_hid_imag")):
+        _close(g_, w, name)
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+def test_fused_backward_matches_oracle_autograd(shape):
+    from aussm_amd import ops  # noqa: F401
+    b, d, n, l = shape
+    print(f"case fused bwd b={b} d={d} n={n} l={l}", flush=True)
+    args = _inputs(b, d, n, l, seed=5, xscale=d ** -0.5)
+    g = torch.Generator().manual_seed(9)
+    gy = torch.randn(b, d, l, generator=g, dtype=torch.float64)
+    ghr = torch.randn(b, d, n, generator=g, dtype=torch.float64)
+    ghi = torch.randn(b, d, n, generator=g, dtype=torch.float64)
+    leaves = [a.clone().requires_grad_(True) for a in args]
+    outs = O.adaptive_unitary_op_loop(*leaves)
+    want = torch.autograd.grad(outs, leaves, [gy, ghr, ghi])
+    got = torch.ops.extension_cpp.ssm_adaptive_backward_unitary(
+        *[t.float().cuda() for t in (gy, ghr, ghi)], *[a.float().cuda() for a in args])
+    assert len(got) == 12
+    for w, g_, name in zip(want, got, IN_NAMES):
+        assert g_.shape == w.shape, name
+        _close(g_, w, "gradient wrt " + name)
+
+
+def test_backward_from_saved_state_equals_backward_from_inputs():
+    """The autograd formula hands the forward call's end state to the backward kernels; the reference-shaped
+    backward operator recomputes it.  Same gradients either way."""
+    from aussm_amd import ops  # noqa: F401
+    args = [a.float().cuda() for a in _inputs(3, 24, 16, 100, seed=8, xscale=24 ** -0.5)]
+    g = torch.Generator().manual_seed(4)
+    grads = [torch.randn(3, 24, 100, generator=g).cuda(), torch.randn(3, 24, 16, generator=g).cuda(),
+             torch.randn(3, 24, 16, generator=g).cuda()]
+    _, nh_r, nh_i = torch.ops.extension_cpp.ssm_adaptive_unitary(*args)
+    a = torch.ops.extension_cpp.ssm_adaptive_backward_unitary(*grads, *args)
+    b = torch.ops.aussm_amd.ssm_adaptive_backward_unitary_from_state(*grads, *args, nh_r, nh_i)
+    for x, y, name in zip(a, b, IN_NAMES):
+        _close(y, x.cpu(), "gradient wrt " + name, tol=1e-5)
+
+
+def test_fused_autograd_through_the_operator():
+    """loss.backward() through torch.ops.extension_cpp.ssm_adaptive_unitary reaches the fused backward."""
+    from aussm_amd import ops
+    args = _inputs(2, 12, 6, 40, seed=7, xscale=12 ** -0.5)
+    leaves = [a.clone().requires_grad_(True) for a in args]
+    y, hr, hi = O.adaptive_unitary_op_loop(*leaves)
+    (y.square().mean() + (hr * hi).mean()).backward()
+    dev = [a.float().cuda().requires_grad_(True) for a in args]
+    y2, hr2, hi2 = ops.ssm_adaptive_unitary(*dev)
+    (y2.square().mean() + (hr2 * hi2).mean()).backward()
+    for w, g_, name in zip(leaves, dev, IN_NAMES):
+        _close(g_.grad, w.grad, "gradient wrt " + name)
+
+
+def test_fused_matches_composite_at_training_shape():
+    """b=32, d=256, n=16, l=720 (the benchmark's training configuration of one block): the fused kernels
+    against the composite route, forward and the gradients of the large tensors."""
+    from aussm_amd import ops
+    b, d, n, l = 32, 256, 16, 720
+    print("case fused vs composite b=32 d=256 n=16 l=720", flush=True)
+    args = [a.float().cuda() for a in _inputs(b, d, n, l, seed=1, dtype=torch.float32, xscale=d ** -0.5)]
+    g = torch.Generator().manual_seed(2)
+    gy = torch.randn(b, d, l, generator=g).cuda()
+    zeros = torch.zeros(b, d, n, device="cuda")
+    torch.cuda.reset_peak_memory_stats()
+    base = torch.cuda.memory_allocated()
+    y, hr, hi = torch.ops.extension_cpp.ssm_adaptive_unitary(*args)
+    grads = torch.ops.extension_cpp.ssm_adaptive_backward_unitary(gy, zeros, zeros, *args)
+    torch.cuda.synchronize()
+    peak = torch.cuda.max_memory_allocated() - base
+    inputs_bytes = sum(a.numel() * 4 for a in args)
+    # the fused route never holds the phase tensor (b d n l floats = 377 MB here): everything it allocates
+    # (outputs, twelve gradients, workspace) stays within three times the operator's input footprint
+    assert peak < 3 * inputs_bytes, (peak, inputs_bytes)
+    leaves = [a.clone().requires_grad_(True) for a in args]
+    yc, hrc, hic = ops._composite(*leaves)
+    want = torch.autograd.grad([yc], leaves, [gy], allow_unused=True)
+    _close(y, yc.detach().cpu(), "y")
+    _close(hr, hrc.detach().cpu(), "next_hid_real")
+    _close(hi, hic.detach().cpu(), "next_hid_imag")
+    for w, g_, name in zip(want, grads, IN_NAMES):
+        _close(g_, w.cpu(), "gradient wrt " + name, tol=2e-4)
+
+
+def test_fused_rejects_shapes_beyond_the_kernels():
+    from aussm_amd import ops  # noqa: F401
+    args = [a.float().cuda() for a in _inputs(1, 4, 17, 8, seed=1)]
+    with pytest.raises(RuntimeError, match="outside the fused kernels' range"):
+        torch.ops.extension_cpp.ssm_adaptive_unitary(*args)
