@@ -31,6 +31,7 @@ _SIGNATURES = {
     "aussm_num_checkpoints": [_I, _I],
     "aussm_bwd_checkpoint_interval": [_I],
     "aussm_unitary_split_segments": [_I] * 5,
+    "aussm_unitary_kernel_mode": [_I] * 9,
     "aussm_unitary_fwd": [_P] * 11 + [_I] * 6 + [_P],
     "aussm_unitary_bwd": [_P] * 16 + [_I] * 6 + [_P],
     "aussm_unitary_fwd_aux": [_P] * 12 + [_I] * 7 + [_P],

@@ -234,8 +234,10 @@ __global__ __launch_bounds__(NW * 64) void dropin_fwd_kernel(const DropinArgs p)
 // hat theta is what the two products with x and u need:
 //     grad_x[i,j,r] = sum_{b,l} hat theta[b,i,j,l] u[b,r,l],   grad_u[b,r,l] += sum_{i,j} x[i,j,r] hat theta[b,i,j,l].
 // The second one sums over every channel of a batch element, so hat theta has to leave the wavefront
-// that made it: it goes to a workspace that holds it for a GROUP of batch elements only (tens of MB,
-// cache resident), and a matrix-core GEMM kernel consumes it before the next group overwrites it.
+// that made it: it goes to a workspace that holds it for a CHUNK of the sequence only (tens of MB,
+// cache resident), and a matrix-core GEMM kernel consumes it before the next chunk overwrites it.
+// A launch therefore covers the tiles t0 .. t1 - 1 of every (batch, channel) pair; the state and its
+// adjoint pass from launch to launch through two small buffers.
 
 __device__ __forceinline__ float row_sum(float v) {     // total of the row in its first lane (others: partial)
   return row_suffix(v);
@@ -265,61 +267,64 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DROPIN_
 #pragma unroll
     for (int c = 0; c < 3; ++c)
       xa[k][c] = (k < p.ks) ? p.xp[(((size_t)ic * p.ks + k) * 3 + c) * 64 + lane] : u4{0, 0, 0, 0};
-  float xb[4], btr[4], bti[4], ctr[4], cti[4], hr[4], hi[4], ar[4], ai[4];
+  // per state: (Re Bt, Im Bt, Re Ct, Im Ct), shared by the workgroup, and the bias of this wavefront's channel.
+  // They are read from LDS where they are used: in registers they would push the kernel over 256.
+  __shared__ f4 s_par[D_MAXN];
+  __shared__ float s_xb[NW][D_MAXN];
+  if (tid < D_MAXN) {
+    const bool ok = tid < n;
+    const int jc = ok ? tid : 0;
+    float sb, cb, sc, cc;
+    fast_sincosf(p.B_th[jc], &sb, &cb);
+    fast_sincosf(p.C_th[jc], &sc, &cc);
+    s_par[tid] = ok ? f4{p.B_r[jc] * cb, p.B_r[jc] * sb, p.C_r[jc] * cc, p.C_r[jc] * sc} : f4{0, 0, 0, 0};
+  }
+  if (lane < D_MAXN) s_xb[wave][lane] = lane < n ? p.x_bias[(size_t)ic * n + lane] : 0.0f;
+  float hr[4], hi[4], ar[4], ai[4];
   float gBr[4], gBi[4], gCr[4], gCi[4], gxb[4];
-  bool jok[4];
 #pragma unroll
   for (int a = 0; a < 4; ++a) {
     const int j = 4 * g + a;
     const bool ok = j < n;
-    jok[a] = ok;
     const int jc = ok ? j : 0;
     const size_t sidx = ((size_t)b * d + ic) * n + jc;
-    xb[a] = ok ? p.x_bias[(size_t)ic * n + jc] : 0.0f;
-    float s, c;
-    fast_sincosf(p.B_th[jc], &s, &c);
-    btr[a] = ok ? p.B_r[jc] * c : 0.0f;
-    bti[a] = ok ? p.B_r[jc] * s : 0.0f;
-    fast_sincosf(p.C_th[jc], &s, &c);
-    ctr[a] = ok ? p.C_r[jc] * c : 0.0f;
-    cti[a] = ok ? p.C_r[jc] * s : 0.0f;
-    hr[a] = ok ? q.hfin_re[sidx] : 0.0f;           // state at the end of the tile being processed
-    hi[a] = ok ? q.hfin_im[sidx] : 0.0f;
-    ar[a] = (ok && q.gnh_re) ? q.gnh_re[sidx] : 0.0f;   // its adjoint
-    ai[a] = (ok && q.gnh_im) ? q.gnh_im[sidx] : 0.0f;
+    hr[a] = ok ? q.hc_re[sidx] : 0.0f;             // state at the end of the tile being processed
+    hi[a] = ok ? q.hc_im[sidx] : 0.0f;
+    ar[a] = ok ? q.dh_re[sidx] : 0.0f;             // its adjoint
+    ai[a] = ok ? q.dh_im[sidx] : 0.0f;
     gBr[a] = gBi[a] = gCr[a] = gCi[a] = gxb[a] = 0.0f;
   }
   const float Di = p.Dp[ic];
   float gD = 0.0f;
-  const int ntiles = (L + DT - 1) / DT;
-  float* __restrict__ dth = q.dth + ((size_t)zb * d + ic) * n * L;
+  const int t_first = q.t0, t_last = q.t1 - 1;
+  float* __restrict__ dth = q.dth + ((size_t)zb * d + ic) * n * q.lc - (size_t)t_first * DT;
 
   constexpr int NT = NW * 64, NREC = (KS * 64 + NT - 1) / NT;
   float sv[NREC][8];
-  stage_load<NT, NREC>(ub, sv, d, L, p.ks, (ntiles - 1) * DT, tid);
-  stage_store<NT, NREC>(sv, s_u[(ntiles - 1) & 1], p.ks, tid, sk);
+  stage_load<NT, NREC>(ub, sv, d, L, p.ks, t_last * DT, tid);
+  stage_store<NT, NREC>(sv, s_u[t_last & 1], p.ks, tid, sk);
   __syncthreads();
   // the wavefront's own inputs, requested one tile ahead
   float un, dtn, zn, gyn;
   {
-    const int l = (ntiles - 1) * DT + l_;
+    const int l = t_last * DT + l_;
     const bool ok = l < L;
     un = ok ? p.u[row + l] : 0.0f;
     dtn = ok ? p.dt[row + l] : 0.0f;
     zn = ok ? p.z[row + l] : 0.0f;
     gyn = ok ? q.gy[row + l] : 0.0f;
   }
-  for (int t = ntiles - 1; t >= 0; --t) {
+  for (int t = t_last; t >= t_first; --t) {
     const int l0 = t * DT, l = l0 + l_;
     const bool lok = l < L;
     const float uv = un, dtv = dtn, zv = zn, gyv = gyn;
-    if (t > 0) {                       // l - DT < L holds
+    if (t > t_first) {                 // l - DT < L holds
       un = p.u[row + l - DT];
       dtn = p.dt[row + l - DT];
       zn = p.z[row + l - DT];
       gyn = q.gy[row + l - DT];
     }
-    if (t > 0) stage_load<NT, NREC>(ub, sv, d, L, p.ks, l0 - DT, tid);
+    if (t > t_first) stage_load<NT, NREC>(ub, sv, d, L, p.ks, l0 - DT, tid);
     f4 th = {0, 0, 0, 0};
     const u4* su = s_u[t & 1];
 #pragma unroll
@@ -335,33 +340,35 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DROPIN_
     float ysum = 0.0f, wsum = 0.0f;
 #pragma unroll
     for (int a = 0; a < 4; ++a) {
-      const float thv = lok ? th[a] + xb[a] : 0.0f;
+      const f4 par = s_par[4 * g + a];
+      const float btr_ = par[0], bti_ = par[1], ctr_ = par[2], cti_ = par[3];
+      const float thv = lok ? th[a] + s_xb[wave][4 * g + a] : 0.0f;
       const float G = row_prefix(thv);
       float sn, cs;
       fast_sincosf(G, &sn, &cs);
       const float csl = row_last(cs, lane), snl = row_last(sn, lane);
       // forward quantities of the tile from the state at its end
-      const float pr = (cs * btr[a] + sn * bti[a]) * w, pi = (cs * bti[a] - sn * btr[a]) * w;
+      const float pr = (cs * btr_ + sn * bti_) * w, pi = (cs * bti_ - sn * btr_) * w;
       const float Ppr = row_prefix(pr), Ppi = row_prefix(pi);
       const float Ptr = row_last(Ppr, lane), Pti = row_last(Ppi, lane);
       const float Rer = csl * hr[a] + snl * hi[a], Rei = csl * hi[a] - snl * hr[a];   // conj(E_last) h_out
       const float hinr = Rer - Ptr, hini = Rei - Pti;
       const float Rr = hinr + Ppr, Ri = hini + Ppi;
       const float her = cs * Rr - sn * Ri, hei = cs * Ri + sn * Rr;                  // h_l
-      ysum += ctr[a] * her - cti[a] * hei;
+      ysum += ctr_ * her - cti_ * hei;
       // adjoints
-      const float hdr = av * ctr[a], hdi = -av * cti[a];                              // a conj(Ct)
+      const float hdr = av * ctr_, hdi = -av * cti_;                              // a conj(Ct)
       const float Rhr = cs * hdr + sn * hdi, Rhi = cs * hdi - sn * hdr;               // conj(E_l) (a conj(Ct))
       const float Kr = csl * ar[a] + snl * ai[a], Ki = csl * ai[a] - snl * ar[a];     // conj(E_last) hat h_out
       const float phr = row_suffix(Rhr) + Kr, phi = row_suffix(Rhi) + Ki;             // hat p_s
       // hat w: Re(E conj(Bt) hat p)
-      const float ebr = cs * btr[a] + sn * bti[a], ebi = sn * btr[a] - cs * bti[a];   // E conj(Bt)
+      const float ebr = cs * btr_ + sn * bti_, ebi = sn * btr_ - cs * bti_;   // E conj(Bt)
       wsum += ebr * phr - ebi * phi;
       // hat G
       float Gh = -(hdr * hei - hdi * her) + (phr * pi - phi * pr);
       if (l_ == 15) Gh -= ar[a] * hi[a] - ai[a] * hr[a];                              // h at the last step is h_out
       const float thh = row_suffix(Gh);
-      if (lok && iok && jok[a]) dth[(size_t)(4 * g + a) * L + l] = thh;
+      if (lok && iok && 4 * g + a < n) dth[(size_t)(4 * g + a) * q.lc + l] = thh;
       gxb[a] += lok ? thh : 0.0f;
       // hat Bt += E w hat p ; hat Ct += a conj(h)
       const float ewr = cs * w, ewi = sn * w;
@@ -386,10 +393,15 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DROPIN_
       q.du[row + l] = (wsum * dtv + av * Di) * dsiluf_(uv);
       gD += av * ut;
     }
-    if (t > 0) stage_store<NT, NREC>(sv, s_u[(t - 1) & 1], p.ks, tid, sk);
+    if (t > t_first) stage_store<NT, NREC>(sv, s_u[(t - 1) & 1], p.ks, tid, sk);
     __syncthreads();
   }
-  // ---- reductions over the timesteps (lanes of a row) and hand-off
+  // ---- reductions over the timesteps (lanes of a row) and hand-off.  The gradients of the 4 n shared
+  // parameters are first summed over the workgroup's channels in LDS: every workgroup of the launch adds
+  // to the same few addresses.
+  __shared__ float s_red[4][D_MAXN];
+  if (tid < 4 * D_MAXN) (&s_red[0][0])[tid] = 0.0f;
+  __syncthreads();
 #pragma unroll
   for (int a = 0; a < 4; ++a) {
     gxb[a] = row_sum(gxb[a]);
@@ -407,32 +419,42 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DROPIN_
         const size_t sidx = ((size_t)b * d + i) * n + j;
         q.dh_re[sidx] = ar[a];
         q.dh_im[sidx] = ai[a];
+        q.hc_re[sidx] = hr[a];
+        q.hc_im[sidx] = hi[a];
         atomicAdd(q.dxb + (size_t)i * n + j, gxb[a]);
         // polar parameters: Bt = B_r e^{i B_theta}
         float ebr, ebi, ecr, eci;
         fast_sincosf(p.B_th[j], &ebi, &ebr);
         fast_sincosf(p.C_th[j], &eci, &ecr);
-        atomicAdd(q.dB_r + j, gBr[a] * ebr + gBi[a] * ebi);
-        atomicAdd(q.dB_th + j, gBi[a] * btr[a] - gBr[a] * bti[a]);
-        atomicAdd(q.dC_r + j, gCr[a] * ecr + gCi[a] * eci);
-        atomicAdd(q.dC_th + j, gCi[a] * ctr[a] - gCr[a] * cti[a]);
+        const f4 par = s_par[j];
+        atomicAdd(&s_red[0][j], gBr[a] * ebr + gBi[a] * ebi);
+        atomicAdd(&s_red[1][j], gBi[a] * par[0] - gBr[a] * par[1]);
+        atomicAdd(&s_red[2][j], gCr[a] * ecr + gCi[a] * eci);
+        atomicAdd(&s_red[3][j], gCi[a] * par[2] - gCr[a] * par[3]);
       }
     }
     if (g == 0) atomicAdd(q.dD + i, gD);
   }
+  __syncthreads();
+  if (tid < 4 * D_MAXN && (tid & (D_MAXN - 1)) < n) {
+    float* dst = (tid >> 4) == 0 ? q.dB_r : (tid >> 4) == 1 ? q.dB_th : (tid >> 4) == 2 ? q.dC_r : q.dC_th;
+    atomicAdd(dst + (tid & (D_MAXN - 1)), (&s_red[0][0])[tid]);
+  }
 }
 
-__global__ __launch_bounds__(256) void fill_zero_kernel(float* __restrict__ p, size_t n) {
+// p[i] = src ? src[i] : 0
+__global__ __launch_bounds__(256) void fill_kernel(float* __restrict__ p, const float* __restrict__ src, size_t n) {
   const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-  if (i < n) p[i] = 0.0f;
+  if (i < n) p[i] = src ? src[i] : 0.0f;
 }
 
 // ---- fp32-accurate GEMM on the bf16 matrix cores, operands in fp32 with arbitrary strides -------
 //     C_z[m][n] (+)= sum_k A_z(m, k) B_z(k, n)           z = 0 .. Z-1
 //     C[m][n]    += sum_z sum_k A_z(m, k) B_z(k, n)      (reduce_z)
 // Workgroup tile 128 x 64, four wavefronts of 64 x 32 each, 32 of k per step, one workgroup per
-// (tile, z, k slice); with more than one k slice, or with reduce_z, the results are summed into C with
-// atomics (C holds the addend beforehand).  Both operands are split into three bf16 pieces while
+// (tile, slice of z, slice of k): zper consecutive z per workgroup (1 unless reduce_z) and ksplit slices
+// of k.  With more than one slice per element of C the results are summed into C with atomics (C holds
+// the addend beforehand).  Both operands are split into three bf16 pieces while
 // they are staged in LDS; the values of the next step are requested before the products of the
 // current one.
 // K1: both operands are contiguous along k.  Then four neighbouring lanes fetch the 32 values of
@@ -444,7 +466,8 @@ __global__ __launch_bounds__(256) void split_gemm_kernel(const GemmArgs p) {
   __shared__ u4 s_a[8 * 3 * 64], s_b[4 * 3 * 64];
   const int tid = threadIdx.x, lane = tid & 63, wave = wave_index();
   const int m0 = blockIdx.x * 128, n0 = blockIdx.y * 64;
-  const int z = blockIdx.z / p.ksplit, ksl = blockIdx.z % p.ksplit;
+  const int zs = blockIdx.z / p.ksplit, ksl = blockIdx.z % p.ksplit;
+  const int z_lo = zs * p.zper, z_hi = z_lo + p.zper < p.Z ? z_lo + p.zper : p.Z;
   const int wm = (wave >> 1) * 4, wn = (wave & 1) * 2;       // this wavefront's first 16-wide tiles
   const SplitK sk = make_splitk();
   f4 acc[4][2];
@@ -459,17 +482,19 @@ __global__ __launch_bounds__(256) void split_gemm_kernel(const GemmArgs p) {
   // ... and where they go in LDS: [16-row tile][piece][lane = 16 (kq / 8) + row % 16]
   const int slot = (ra >> 4) * 192 + (kq >> 3) * 16 + (ra & 15);
   // uniform bases, 32-bit per-thread offsets (a z-slice of either operand is below 2^31 elements)
-  const float* __restrict__ Az = p.A + z * p.saz;
-  const float* __restrict__ Bz = p.Bm + z * p.sbz;
   const unsigned sak = (unsigned)p.sak, sbk = (unsigned)p.sbk;
   const unsigned oa0 = (unsigned)ma * (unsigned)p.sam + (unsigned)kq * sak;
   const unsigned oa1 = (unsigned)mb * (unsigned)p.sam + (unsigned)kq * sak;
   const unsigned ob0 = (unsigned)nb * (unsigned)p.sbn + (unsigned)kq * sbk;
   const int nk = (p.K + 31) / 32, per = (nk + p.ksplit - 1) / p.ksplit;
   const int it0 = ksl * per, it1 = it0 + per < nk ? it0 + per : nk;
+  const int nit = it1 > it0 ? (it1 - it0) * (z_hi - z_lo) : 0;      // steps of this workgroup: (z, k step) pairs
   const bool inside = m0 + 128 <= p.M && n0 + 64 <= p.N;      // uniform over the workgroup
   float va[2][8], vb[8];
-  auto fetch = [&](int it) {
+  auto fetch = [&](int step) {
+    const int z = z_lo + step / (it1 - it0), it = it0 + step % (it1 - it0);
+    const float* __restrict__ Az = p.A + z * p.saz;
+    const float* __restrict__ Bz = p.Bm + z * p.sbz;
     const unsigned ka = (unsigned)(it * 32) * sak, kb = (unsigned)(it * 32) * sbk;
     if (inside && it * 32 + 32 <= p.K) {
       if constexpr (K1 && VEC) {
@@ -503,8 +528,8 @@ __global__ __launch_bounds__(256) void split_gemm_kernel(const GemmArgs p) {
       }
     }
   };
-  if (it0 < it1) fetch(it0);
-  for (int it = it0; it < it1; ++it) {
+  if (nit > 0) fetch(0);
+  for (int step = 0; step < nit; ++step) {
     u4 pa[2][3], pb[3];
     split8<3>(sk, va[0], pa[0]);
     split8<3>(sk, va[1], pa[1]);
@@ -517,7 +542,7 @@ __global__ __launch_bounds__(256) void split_gemm_kernel(const GemmArgs p) {
       s_b[slot + c * 64] = pb[c];
     }
     __syncthreads();
-    if (it + 1 < it1) fetch(it + 1);      // in flight during the products
+    if (step + 1 < nit) fetch(step + 1);      // in flight during the products
     u4 rb[2][3];
 #pragma unroll
     for (int f = 0; f < 2; ++f)
@@ -533,8 +558,8 @@ __global__ __launch_bounds__(256) void split_gemm_kernel(const GemmArgs p) {
     }
   }
   // result tile (e, f): lane (column = lane % 16, rows 4 (lane / 16) + a)
-  float* __restrict__ C = p.C + (p.reduce_z ? 0 : z * p.scz);
-  const bool atomic = p.reduce_z || p.ksplit > 1;
+  float* __restrict__ C = p.C + (p.reduce_z ? 0 : z_lo * p.scz);
+  const bool atomic = p.ksplit > 1 || (p.reduce_z && p.zper < p.Z);
 #pragma unroll
   for (int e = 0; e < 4; ++e)
 #pragma unroll

@@ -30,11 +30,9 @@ struct DropinArgs {
 struct DropinBwdArgs {
   DropinArgs f;            // inputs (y, nh_* unused)
   const float* gy;         // [b, d, L]
-  const float* gnh_re;     // [b, d, n] or null
-  const float* gnh_im;
-  const float* hfin_re;    // [b, d, n] state at the end of the sequence
-  const float* hfin_im;
-  float* dth;              // workspace [bg][d n][L]
+  float* hc_re;            // [b, d, n] in: state after tile t1 - 1; out: state before tile t0
+  float* hc_im;
+  float* dth;              // workspace [bg][d n][lc]: phase adjoints of the launch
   float* du;               // [b, d, L] direct part (the product with x is added afterwards)
   float* ddt;
   float* dz;
@@ -44,9 +42,11 @@ struct DropinBwdArgs {
   float* dC_r;
   float* dC_th;
   float* dD;               // [d]      (atomics)
-  float* dh_re;            // [b, d, n]
+  float* dh_re;            // [b, d, n] in: adjoint of the state after tile t1 - 1; out: of the state before tile t0
   float* dh_im;
-  int b0, bg;              // batch elements b0 .. b0 + bg - 1
+  int b0, bg;              // batch elements b0 .. b0 + bg - 1 ...
+  int t0, t1;              // ... and tiles of 16 timesteps t0 .. t1 - 1 (in reverse) are this launch's
+  int lc;                  // row length of dth (>= 16 (t1 - t0))
 };
 
 struct GemmArgs {
@@ -56,7 +56,8 @@ struct GemmArgs {
   long scm, scn, scz;
   int M, N, K, Z;
   int reduce_z, accumulate;
-  int ksplit;             // workgroups along k per (tile, z); > 1 sums into C with atomics
+  int ksplit;             // slices of k per (tile, slice of z)
+  int zper;               // z per workgroup (summed inside it; 1 unless reduce_z)
 };
 
 }  // namespace aussm

@@ -9,8 +9,8 @@ void run_dropin_xprep(const float* x, u4* xp, int d, int n, int ks, hipStream_t 
   hipLaunchKernelGGL(dropin_xprep_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, x, xp, d, n, ks);
 }
 
-void run_fill_zero(float* p, size_t n, hipStream_t s) {
-  if (n) hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, p, n);
+void run_fill(float* p, const float* src, size_t n, hipStream_t s) {
+  if (n) hipLaunchKernelGGL(fill_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, p, src, n);
 }
 
 #ifndef DROPIN_NW_
@@ -18,16 +18,21 @@ void run_fill_zero(float* p, size_t n, hipStream_t s) {
 #endif
 constexpr int DROPIN_NW = DROPIN_NW_;     // channels (wavefronts) per workgroup
 
+// (d > 256: the rows of x take 192 registers, which leaves room for one wavefront per SIMD only)
 template <int KS>
 static void launch_fwd(const DropinArgs& a, hipStream_t s) {
-  const unsigned grid = (unsigned)(a.b * ((a.d + DROPIN_NW - 1) / DROPIN_NW));
-  hipLaunchKernelGGL((dropin_fwd_kernel<KS, DROPIN_NW>), dim3(grid), dim3(DROPIN_NW * 64), 0, s, a);
+  constexpr int NW = KS > 8 ? 4 : DROPIN_NW;
+  const unsigned grid = (unsigned)(a.b * ((a.d + NW - 1) / NW));
+  hipLaunchKernelGGL((dropin_fwd_kernel<KS, NW>), dim3(grid), dim3(NW * 64), 0, s, a);
 }
 template <int KS>
 static void launch_bwd(const DropinBwdArgs& a, hipStream_t s) {
-  const unsigned grid = (unsigned)(a.bg * ((a.f.d + DROPIN_NW - 1) / DROPIN_NW));
-  hipLaunchKernelGGL((dropin_bwd_kernel<KS, DROPIN_NW>), dim3(grid), dim3(DROPIN_NW * 64), 0, s, a);
+  constexpr int NW = KS > 8 ? 4 : DROPIN_NW;
+  const unsigned grid = (unsigned)(a.bg * ((a.f.d + NW - 1) / NW));
+  hipLaunchKernelGGL((dropin_bwd_kernel<KS, NW>), dim3(grid), dim3(NW * 64), 0, s, a);
 }
+
+int dropin_channels_per_workgroup(int ks) { return ks > 8 ? 4 : DROPIN_NW; }
 
 int run_dropin_fwd(const DropinArgs& a, hipStream_t s) {
   if (a.ks <= 1) launch_fwd<1>(a, s);
@@ -48,8 +53,10 @@ int run_dropin_bwd(const DropinBwdArgs& a, hipStream_t s) {
 }
 
 int run_split_gemm(const GemmArgs& a, hipStream_t s) {
-  if (a.ksplit < 1 || (long)a.Z * a.ksplit > 65535) return -2;
-  const dim3 grid((unsigned)((a.M + 127) / 128), (unsigned)((a.N + 63) / 64), (unsigned)(a.Z * a.ksplit));
+  if (a.ksplit < 1 || a.zper < 1 || (!a.reduce_z && a.zper != 1)) return -2;
+  const long gz = (long)((a.Z + a.zper - 1) / a.zper) * a.ksplit;
+  if (gz > 65535) return -2;
+  const dim3 grid((unsigned)((a.M + 127) / 128), (unsigned)((a.N + 63) / 64), (unsigned)gz);
   const bool k1 = a.sak == 1 && a.sbk == 1;
   const bool vec = k1 && a.sam % 4 == 0 && a.sbn % 4 == 0 && a.saz % 4 == 0 && a.sbz % 4 == 0 &&
                    (reinterpret_cast<uintptr_t>(a.A) | reinterpret_cast<uintptr_t>(a.Bm)) % 16 == 0;

@@ -125,11 +125,26 @@ inline AuxLayout aux_layout(float* aux, int B, int D, int N, int L, int ck) {
   return AuxLayout{seg, img_floats(B, N, L, ck) ? reinterpret_cast<u4*>(img) : nullptr};
 }
 
-inline int mfma_fwd_mode(const FwdArgs& a, int in_dtype, bool have_img) {
-  int mode = kernel_mode(AUSSM_OPT_UNITARY_FWD, DEFAULT_FWD_MODE, a.N);
-  if (mode <= 0 || a.urep != 1 || !matrix_shape(a.N, a.L, a.ck)) return 0;
+// Kernel family of a call whose tensors are 16-byte aligned: 0 vector ALU, 2 / 3 / 5 matrix-core kernels
+// that prepare their operands themselves, 6 prepared-operand kernels.
+inline int fwd_mode_for(int N, int L, int ck, int in_dtype, int urep, bool have_img) {
+  int mode = kernel_mode(AUSSM_OPT_UNITARY_FWD, DEFAULT_FWD_MODE, N);
+  if (mode <= 0 || urep != 1 || !matrix_shape(N, L, ck)) return 0;
   if (mode == 6 && !have_img) mode = 3;
   if (in_dtype != AUSSM_F32 && mode != 6) mode = 3;       // bf16 inputs: three-piece kernels only
+  return mode;
+}
+inline int bwd_mode_for(int B, int D, int N, int L, int ck, int urep, bool have_img) {
+  int mode = kernel_mode(AUSSM_OPT_UNITARY_BWD, DEFAULT_BWD_MODE, N);   // matrix-core kernels for the common case
+  if (mode <= 0 || urep != 1 || !matrix_shape(N, L, ck)) return 0;
+  // (the prepared-operand kernel addresses its tensors with 32-bit byte offsets)
+  if (mode == 6 && (!have_img || (unsigned long long)B * D * L * 4 >= (1ull << 32) ||
+                    (unsigned long long)B * N * L * 8 >= (1ull << 32)))
+    mode = 3;
+  return mode;
+}
+inline int mfma_fwd_mode(const FwdArgs& a, int in_dtype, bool have_img) {
+  const int mode = fwd_mode_for(a.N, a.L, a.ck, in_dtype, a.urep, have_img);
   if (misaligned(a.u, 16) || misaligned(a.delta, 16) || misaligned(a.theta, 16) || misaligned(a.z, 16) ||
       misaligned(a.y, 16) || misaligned(a.Bm, 16) || misaligned(a.Cm, 16))
     return 0;
@@ -236,6 +251,12 @@ int aussm_unitary_split_segments(int B, int D, int N, int L, int ck) {
 size_t aussm_unitary_aux_floats(int B, int D, int N, int L, int ck) {
   if (B < 1 || D < 1 || N < 1 || L < 1) return 0;
   return (size_t)B * D * L + AUX_PAD + seg_floats(B, D, N, L, seg_capacity(B, D, N, L, ck)) + img_floats(B, N, L, ck);
+}
+
+int aussm_unitary_kernel_mode(int backward, int B, int D, int N, int L, int ck, int in_dtype, int urep, int have_aux) {
+  if (check_common(B, D, N, L, ck, in_dtype) != AUSSM_OK || urep < 1) return 0;
+  const bool have_img = have_aux && img_floats(B, N, L, ck) > 0;
+  return backward ? bwd_mode_for(B, D, N, L, ck, urep, have_img) : fwd_mode_for(N, L, ck, in_dtype, urep, have_img);
 }
 
 int aussm_unitary_fwd(const void* u, const void* delta, const float* theta, const void* Bc, const void* Cc,
@@ -348,12 +369,8 @@ int aussm_unitary_bwd_aux(const float* dy, const float* dhL, const void* u, cons
   a.ld = L; a.ns = 1; a.hs = 1; a.ho = 0; a.urep = 1;
   a.urep = urep;
   const AuxLayout ws = aux_layout(aux, B, D, N, L, ck);
-  int mode = kernel_mode(AUSSM_OPT_UNITARY_BWD, DEFAULT_BWD_MODE, N);   // matrix-core kernels for the common case
-  // (the prepared-operand kernel addresses its tensors with 32-bit byte offsets)
-  if (mode == 6 && (!ws.img || (unsigned long long)B * D * L * 4 >= (1ull << 32) ||
-                    (unsigned long long)B * N * L * 8 >= (1ull << 32)))
-    mode = 3;
-  if (mode > 0 && urep == 1 && matrix_shape(N, L, ck) &&
+  const int mode = bwd_mode_for(B, D, N, L, ck, urep, ws.img != nullptr);
+  if (mode > 0 &&
       !(misaligned(dy, 16) || misaligned(u, 16) || misaligned(delta, 16) || misaligned(theta, 16) ||
         misaligned(du, 16) || misaligned(ddelta, 16) || misaligned(dtheta, 16) || misaligned(Bc, 16) ||
         misaligned(Cc, 16))) {
@@ -460,24 +477,47 @@ int aussm_swap_last2(const float* x, float* y, int B, int R, int C, long long xs
 // ---- the reference's operator extension_cpp::ssm_adaptive_unitary as fused kernels (dropin.h)
 
 static size_t dropin_xp_floats(int d) { return (size_t)d * ((d + 31) / 32) * 3 * 64 * 4; }
-// batch elements whose phase adjoints the workspace holds at a time: at most about 96 MiB of them, in
-// groups of equal size
-static int dropin_group(int b, int d, int n, int L) {
-  const size_t per = (size_t)d * n * L, cap = (size_t)24 << 20;
-  size_t gmax = cap / per;
-  if (gmax < 1) gmax = 1;
-  const size_t ng = ((size_t)b + gmax - 1) / gmax;
-  return (int)(((size_t)b + ng - 1) / ng);
+// The backward call works through the (batch, sequence) plane in blocks of bg batch elements x ct tiles
+// of 16 timesteps: the workspace holds the phase adjoints of one block (about 96 MiB at most).  bg is
+// what fills the chip with one workgroup per compute unit (fewer would idle units, more would only
+// shorten the blocks and repeat the per-launch set-up, the rows of x among it, more often).
+struct DropinBlocks { int bg, ct; };
+static DropinBlocks dropin_blocks(int b, int d, int n, int L) {
+  const int nw = dropin_channels_per_workgroup((d + 31) / 32);
+  const int wgs_per_b = (d + nw - 1) / nw;
+  int bg = (256 + wgs_per_b - 1) / wgs_per_b;
+  if (bg > b) bg = b;
+  const int ng = (b + bg - 1) / bg;
+  bg = (b + ng - 1) / ng;
+  const size_t per_tile = (size_t)bg * d * n * DT, cap = (size_t)24 << 20;
+  const int ntiles = (L + DT - 1) / DT;
+  size_t tmax = cap / per_tile;
+  if (tmax < 1) tmax = 1;
+  const size_t nc = ((size_t)ntiles + tmax - 1) / tmax;
+  return DropinBlocks{bg, (int)(((size_t)ntiles + nc - 1) / nc)};
 }
-// k slices of a GEMM launch: enough workgroups for about three per compute unit, at least four steps each
-static int gemm_ksplit(int M, int N, int K, int Z) {
-  const long tiles = (long)((M + 127) / 128) * ((N + 63) / 64) * Z;
-  const int nk = (K + 31) / 32;
-  long s = (768 + tiles - 1) / tiles;
+// How a GEMM launch is cut: about three workgroups per compute unit.  Without reduce_z every z is a
+// slice of its own and k is cut (at least four steps per slice); with reduce_z the z are dealt to the
+// slices first and k is cut only when there are too few z.
+static void gemm_slices(GemmArgs& g) {
+  const long tiles = (long)((g.M + 127) / 128) * ((g.N + 63) / 64);
+  const int nk = (g.K + 31) / 32;
+  long zs = 1;                                   // slices of z
+  g.zper = 1;
+  if (g.reduce_z) {
+    zs = (768 + tiles - 1) / tiles;
+    if (zs > g.Z) zs = g.Z;
+    if (zs < 1) zs = 1;
+    g.zper = (int)((g.Z + zs - 1) / zs);
+    zs = (g.Z + g.zper - 1) / g.zper;
+  } else {
+    zs = g.Z;
+  }
+  long s = (768 + tiles * zs - 1) / (tiles * zs);
   if (s > nk / 4) s = nk / 4;
   if (s < 1) s = 1;
-  while (s > 1 && (long)Z * s > 65535) --s;
-  return (int)s;
+  while (s > 1 && zs * s > 65535) --s;
+  g.ksplit = (int)s;
 }
 static size_t round4(size_t v) { return (v + 3) & ~(size_t)3; }
 static int dropin_check(int b, int d, int n, int L) {
@@ -490,7 +530,10 @@ static int dropin_check(int b, int d, int n, int L) {
 size_t aussm_ssm_adaptive_unitary_workspace_floats(int b, int d, int n, int L, int backward) {
   if (dropin_check(b, d, n, L) != AUSSM_OK) return 0;
   size_t f = dropin_xp_floats(d);
-  if (backward) f += 2 * round4((size_t)b * d * n) + (size_t)dropin_group(b, d, n, L) * d * n * L;
+  if (backward) {
+    const DropinBlocks k = dropin_blocks(b, d, n, L);
+    f += 2 * round4((size_t)b * d * n) + (size_t)k.bg * k.ct * DT * d * n;
+  }
   return f;
 }
 
@@ -527,56 +570,61 @@ int aussm_ssm_adaptive_unitary_bwd(const float* grad_y, const float* grad_nh_re,
     return AUSSM_E_NULL;
   if (misaligned(workspace, 16)) return AUSSM_E_ALIGN;
   hipStream_t s = (hipStream_t)stream;
-  const int ks = (d + 31) / 32, bg = dropin_group(b, d, n, L);
+  const DropinBlocks blk = dropin_blocks(b, d, n, L);
+  const int ks = (d + 31) / 32, ct = blk.ct, lc = ct * DT;
+  const int ntiles = (L + DT - 1) / DT;
   const size_t nstate = (size_t)b * d * n;
   u4* xp = (u4*)workspace;
-  float* ws_re = workspace + dropin_xp_floats(d);
-  float* ws_im = ws_re + round4(nstate);
-  float* dth = ws_im + round4(nstate);
+  float* hc_re = workspace + dropin_xp_floats(d);
+  float* hc_im = hc_re + round4(nstate);
+  float* dth = hc_im + round4(nstate);
   run_dropin_xprep(x, xp, d, n, ks, s);
-  DropinArgs f{u, dt, z, x_bias, B_r, B_theta, C_r, C_theta, D, h_re, h_im, nullptr, ws_re, ws_im, xp, b, d, n, L, ks};
-  const float* hfin_re = nh_re;
-  const float* hfin_im = nh_im;
-  if (!nh_re || !nh_im) {
+  DropinArgs f{u, dt, z, x_bias, B_r, B_theta, C_r, C_theta, D, h_re, h_im, nullptr, hc_re, hc_im, xp, b, d, n, L, ks};
+  if (nh_re && nh_im) {
+    run_fill(hc_re, nh_re, nstate, s);
+    run_fill(hc_im, nh_im, nstate, s);
+  } else {
     // the state at the end of the sequence: one forward sweep without outputs
     if (int e = run_dropin_fwd(f, s)) return e;
-    hfin_re = ws_re;
-    hfin_im = ws_im;
   }
-  run_fill_zero(dx, (size_t)d * n * d, s);
-  run_fill_zero(dx_bias, (size_t)d * n, s);
-  run_fill_zero(dB_r, n, s);
-  run_fill_zero(dB_theta, n, s);
-  run_fill_zero(dC_r, n, s);
-  run_fill_zero(dC_theta, n, s);
-  run_fill_zero(dD, d, s);
+  run_fill(dh_re, grad_nh_re, nstate, s);           // the adjoint of the state travels in the output buffers
+  run_fill(dh_im, grad_nh_im, nstate, s);
+  run_fill(dx, nullptr, (size_t)d * n * d, s);
+  run_fill(dx_bias, nullptr, (size_t)d * n, s);
+  run_fill(dB_r, nullptr, n, s);
+  run_fill(dB_theta, nullptr, n, s);
+  run_fill(dC_r, nullptr, n, s);
+  run_fill(dC_theta, nullptr, n, s);
+  run_fill(dD, nullptr, d, s);
   const long dn = (long)d * n;
-  for (int b0 = 0; b0 < b; b0 += bg) {
-    const int g = b - b0 < bg ? b - b0 : bg;
+  for (int b0 = 0; b0 < b; b0 += blk.bg)
+  for (int t1 = ntiles; t1 > 0; t1 -= ct) {
+    const int bg = b - b0 < blk.bg ? b - b0 : blk.bg;
+    const int t0 = t1 - ct > 0 ? t1 - ct : 0;
+    const int l0 = t0 * DT, len = (t1 * DT < L ? t1 * DT : L) - l0;
     DropinBwdArgs q{};
     q.f = f;
     q.f.nh_re = q.f.nh_im = nullptr;
-    q.gy = grad_y; q.gnh_re = grad_nh_re; q.gnh_im = grad_nh_im;
-    q.hfin_re = hfin_re; q.hfin_im = hfin_im; q.dth = dth;
+    q.gy = grad_y; q.hc_re = hc_re; q.hc_im = hc_im; q.dth = dth;
     q.du = du; q.ddt = ddt; q.dz = dz; q.dxb = dx_bias;
     q.dB_r = dB_r; q.dB_th = dB_theta; q.dC_r = dC_r; q.dC_th = dC_theta; q.dD = dD;
-    q.dh_re = dh_re; q.dh_im = dh_im; q.b0 = b0; q.bg = g;
+    q.dh_re = dh_re; q.dh_im = dh_im; q.b0 = b0; q.bg = bg; q.t0 = t0; q.t1 = t1; q.lc = lc;
     if (int e = run_dropin_bwd(q, s)) return e;
-    // grad_u[b, r, l] += sum_(i j) x[(i j), r] hat theta[b, (i j), l]
+    // grad_u[b, r, l0 + l] += sum_(i j) x[(i j), r] hat theta[b, (i j), l]
     GemmArgs gu{};
     gu.A = x; gu.sam = 1; gu.sak = d; gu.saz = 0;
-    gu.Bm = dth; gu.sbk = L; gu.sbn = 1; gu.sbz = dn * L;
-    gu.C = du + (size_t)b0 * d * L; gu.scm = L; gu.scn = 1; gu.scz = (long)d * L;
-    gu.M = d; gu.N = L; gu.K = (int)dn; gu.Z = g; gu.reduce_z = 0; gu.accumulate = 1;
-    gu.ksplit = gemm_ksplit(gu.M, gu.N, gu.K, g);
+    gu.Bm = dth; gu.sbk = lc; gu.sbn = 1; gu.sbz = dn * lc;
+    gu.C = du + (size_t)b0 * d * L + l0; gu.scm = L; gu.scn = 1; gu.scz = (long)d * L;
+    gu.M = d; gu.N = len; gu.K = (int)dn; gu.Z = bg; gu.reduce_z = 0; gu.accumulate = 1;
+    gemm_slices(gu);
     if (int e = run_split_gemm(gu, s)) return e;
-    // grad_x[(i j), r] += sum_b sum_l hat theta[b, (i j), l] u[b, r, l]
+    // grad_x[(i j), r] += sum_b sum_l hat theta[b, (i j), l] u[b, r, l0 + l]
     GemmArgs gx{};
-    gx.A = dth; gx.sam = L; gx.sak = 1; gx.saz = dn * L;
-    gx.Bm = u + (size_t)b0 * d * L; gx.sbk = 1; gx.sbn = L; gx.sbz = (long)d * L;
+    gx.A = dth; gx.sam = lc; gx.sak = 1; gx.saz = dn * lc;
+    gx.Bm = u + (size_t)b0 * d * L + l0; gx.sbk = 1; gx.sbn = L; gx.sbz = (long)d * L;
     gx.C = dx; gx.scm = d; gx.scn = 1; gx.scz = 0;
-    gx.M = (int)dn; gx.N = d; gx.K = L; gx.Z = g; gx.reduce_z = 1; gx.accumulate = 1;
-    gx.ksplit = gemm_ksplit(gx.M, gx.N, gx.K, g);
+    gx.M = (int)dn; gx.N = d; gx.K = len; gx.Z = bg; gx.reduce_z = 1; gx.accumulate = 1;
+    gemm_slices(gx);
     if (int e = run_split_gemm(gx, s)) return e;
   }
   return AUSSM_OK;

@@ -16,7 +16,7 @@ Operator semantics (ssm_adaptive_unitary_forward.cu:83-181), per batch b, channe
 The two dispatcher ops run the library's fused kernels (aussm_ssm_adaptive_unitary_fwd / _bwd,
 include/aussm_hip.h): the phase tensor theta (b, d, n, l) is formed tile by tile inside the scan
 kernel and never stored, and the backward op recomputes from the twelve inputs as the reference's
-does.  Shapes beyond the fused kernels' limits (n > 16 or d > 512) raise.
+does.  Shapes beyond the fused kernels' limits (n > 16 or d > 512) take the composite route below.
 
 `_composite` is a second, independent route to the same numbers, kept for the interface's
 save_intermediates=True mode and as a cross-check in the tests: every (batch, state) pair becomes
@@ -101,17 +101,23 @@ _lib.define(_FWD_SCHEMA)
 _lib.define(_BWD_SCHEMA)
 
 
+def fused_supported(b: int, d: int, n: int, l: int) -> bool:
+    """Whether the fused kernels take this shape (n <= 16, d <= 512); beyond it the dispatcher ops run
+    the composite route (same HIP core scan, phase tensor materialised)."""
+    return L.load().aussm_ssm_adaptive_unitary_workspace_floats(b, d, n, l, 0) > 0
+
+
 def _workspace(b, d, n, l, backward, device):
     floats = L.load().aussm_ssm_adaptive_unitary_workspace_floats(b, d, n, l, int(backward))
-    if floats == 0:
-        raise RuntimeError(f"ssm_adaptive_unitary: shape (b={b}, d={d}, n={n}, l={l}) is outside the fused kernels' "
-                           "range (n <= 16, d <= 512)")
     return torch.empty(floats, device=device, dtype=torch.float32)
 
 
 def _fwd_impl(u, dt, x, x_bias, B_r, B_theta, C_r, C_theta, D, z, h_r, h_i):
     args = [t.contiguous() for t in (u, dt, x, x_bias, B_r, B_theta, C_r, C_theta, D, z, h_r, h_i)]
     b, d, n, l = _check_op_inputs(args)
+    if not fused_supported(b, d, n, l):
+        with torch.no_grad():
+            return _composite(*args)
     with torch.cuda.device(u.device):
         y, nh_r, nh_i = torch.empty_like(args[0]), torch.empty_like(args[10]), torch.empty_like(args[11])
         ws = _workspace(b, d, n, l, False, u.device)
@@ -126,6 +132,11 @@ def _bwd_impl(grad_y, grad_hr, grad_hi, u, dt, x, x_bias, B_r, B_theta, C_r, C_t
     args = [t.contiguous() for t in (u, dt, x, x_bias, B_r, B_theta, C_r, C_theta, D, z, h_r, h_i)]
     b, d, n, l = _check_op_inputs(args)
     grads_in = [grad_y.contiguous(), grad_hr.contiguous(), grad_hi.contiguous()]
+    if not fused_supported(b, d, n, l):
+        with torch.enable_grad():
+            leaves = [t.detach().requires_grad_(True) for t in args]
+            grads = torch.autograd.grad(_composite(*leaves), leaves, grads_in, allow_unused=True)
+        return tuple(torch.zeros_like(t) if g is None else g.contiguous() for g, t in zip(grads, leaves))
     for name, t, like in zip(("grad_y", "grad_next_hid_real", "grad_next_hid_imag"), grads_in,
                              (args[0], args[10], args[11])):
         if t.dtype != torch.float32 or tuple(t.shape) != tuple(like.shape):

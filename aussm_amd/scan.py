@@ -114,6 +114,15 @@ def unitary_aux(u, n: int, ck: int) -> Tensor:
                        dtype=torch.float32)
 
 
+def unitary_aux_useful(b: int, d: int, n: int, l: int, ck: int, in_dtype: int, urep: int = 1) -> bool:
+    """False when neither direction of the scan would touch an auxiliary buffer for this shape (the
+    vector-ALU kernels do not use it, e.g. n > 16 or inputs shared between batch elements), so that
+    the autograd wrapper does not allocate and keep b d l floats for nothing."""
+    lib = _lib.load()
+    return bool(lib.aussm_unitary_kernel_mode(0, b, d, n, l, ck, in_dtype, urep, 1)
+                or lib.aussm_unitary_kernel_mode(1, b, d, n, l, ck, in_dtype, urep, 1))
+
+
 def unitary_fwd_raw(u, delta, theta, Bri, Cri, D=None, z=None, h0=None, want_state=False, ck=0, aux=None, ck_arg=0):
     """Launch aussm_unitary_fwd(_aux).  Bri/Cri are real views (b, n, l, 2).  Returns (y, hL, hck);
     hL is (b, d, n, 2) or None, hck is the checkpoint tensor when ck > 0.  u and delta may have a
@@ -166,7 +175,9 @@ class _UnitaryScanFn(torch.autograd.Function):
     @staticmethod
     def forward(ctx, u, delta, theta, Bri, Cri, D, h0):
         ck = unitary_ck(theta.shape[0], theta.shape[1], Bri.shape[1], theta.shape[2])
-        aux = unitary_aux(theta, Bri.shape[1], ck)
+        b, d, l = theta.shape
+        n = Bri.shape[1]
+        aux = unitary_aux(theta, n, ck) if unitary_aux_useful(b, d, n, l, ck, _in_dtype(u), b // u.shape[0]) else None
         y, hL, hck = unitary_fwd_raw(u, delta, theta, Bri, Cri, D, None, h0, want_state=True, ck=ck, aux=aux)
         ctx.save_for_backward(u, delta, theta, Bri, Cri, D, hck, aux)
         ctx.ck = ck

@@ -13,17 +13,26 @@ resident in HBM.  Prints ONE JSON line.
 
   value          (b,d,l) samples per second over forward+backward (B*D*L / step time)
   roofline       dominant kernel (the backward scan): algorithmic bytes (28E + 32S + 4D,
-                 E = B*D*L, S = B*N*L) / its average launch duration, measured here with HIP
-                 events on the launch stream, against the 8 TB/s HBM peak.  "traffic" is the HBM
-                 bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE passes over this same
-                 script (profiles/), scaled by what the counters read for the 256 MiB device copy
-                 that --copy-probe adds to the run; it is a recorded figure, not measured live.
+                 E = B*D*L, S = B*N*L) / the average duration of one backward call (the scan kernel
+                 and, for the prepared-operand kernel, its light operand pre-pass), measured here
+                 with HIP events on the launch stream, against the 8 TB/s HBM peak.  "traffic" is
+                 the HBM bytes per call from rocprofv3 FETCH_SIZE / WRITE_SIZE passes over this same
+                 script, scaled by what the counters read for the 256 MiB device copy that
+                 --copy-probe adds to the run.  It is read from profiles/traffic.json, which
+                 `bench.py --summarize-traffic FETCH_DIR WRITE_DIR` writes from the two passes'
+                 output; the file records the kernels it saw and a digest of the kernel sources,
+                 and the figure is reported as null when either no longer matches this build.
   cpu_baseline   the CPU oracle (sequential-loop PyTorch scan + autograd) timed on this host's
-                 cores on a bounded slice of the batch
+                 cores on a bounded slice of the batch: one warm-up run, then the median of three
+
+Before the W warm-up steps the step is repeated for --prewarm-ms (default 200 ms, reported as
+prewarm_ms) so that clocks and caches are where a long run has them.
 """
 from __future__ import annotations
 
 import argparse
+import glob
+import hashlib
 import json
 import os
 import sys
@@ -34,12 +43,76 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 SHAPE = dict(B=32, D=512, N=16, L=2048)
-# HBM bytes per launch at SHAPE from the counter passes summarised in
-# profiles/unitary_fwd_bwd_B32_D512_N16_L2048_hbm_traffic.md (FETCH_SIZE x 2.00, WRITE_SIZE x 1.00 after
-# calibration on a 256 MiB copy): forward 427 MB read + 286 MB written, backward 818 MB read +
-# 547 MB written.  Both include the auxiliary buffer (134 MB written forward, read backward) and the
-# checkpoints; the dB/dC atomics of the eight workgroups of a batch element count as writes.
-TRAFFIC_BYTES = {"unitary_fwd": 713e6, "unitary_bwd": 1366e6}
+TRAFFIC_JSON = os.path.join(ROOT, "profiles", "traffic.json")
+# kernels of one call, by the kernel family the library reports (aussm_unitary_kernel_mode)
+FWD_KERNELS = {0: ["core_fwd_kernel<0"], 2: ["unitary_fwd_xdl_kernel<2"], 3: ["unitary_fwd_xdl_kernel<3"],
+               6: ["unitary_px_prep_kernel", "unitary_fwd_px_kernel"]}
+BWD_KERNELS = {0: ["unitary_bwd_kernel"], 2: ["unitary_bwd_xdl_kernel<2"], 3: ["unitary_bwd_xdl_kernel<3, 2"],
+               5: ["unitary_bwd_xdl_kernel<3, 3"],
+               6: ["unitary_px_prep_kernel", "unitary_bwd_px_kernel", "unitary_bwd_xdl_kernel<3, 2"]}
+
+
+def source_digest() -> str:
+    """Digest of the kernel sources: a traffic record is only valid for the sources it was taken with."""
+    h = hashlib.sha256()
+    for f in sorted(glob.glob(os.path.join(ROOT, "aussm_amd", "csrc", "*"))):
+        h.update(os.path.basename(f).encode())
+        h.update(open(f, "rb").read())
+    return h.hexdigest()[:16]
+
+
+def summarize_traffic(fetch_dir: str, write_dir: str) -> None:
+    """profiles/traffic.json from the counter_collection.csv files of two rocprofv3 --pmc passes
+    (FETCH_SIZE, WRITE_SIZE) over `bench.py --copy-probe`."""
+    import csv
+
+    def per_kernel(d, counter):
+        files = glob.glob(os.path.join(d, "**", "*counter_collection.csv"), recursive=True)
+        if not files:
+            sys.exit(f"no counter_collection.csv under {d}")
+        acc = {}
+        for row in csv.DictReader(open(max(files, key=os.path.getmtime))):
+            if row["Counter_Name"] == counter:
+                acc.setdefault(row["Kernel_Name"], []).append(float(row["Counter_Value"]))
+        return {k: (sum(v) / len(v), len(v)) for k, v in acc.items()}
+
+    fetch, write = per_kernel(fetch_dir, "FETCH_SIZE"), per_kernel(write_dir, "WRITE_SIZE")
+    copy = [k for k in fetch if "copyBuffer" in k]
+    if not copy or copy[0] not in write:
+        sys.exit("the passes do not contain the 256 MiB copy (run bench.py with --copy-probe)")
+    copy_kib = 256.0 * 1024
+    scale = {"FETCH_SIZE": copy_kib / fetch[copy[0]][0], "WRITE_SIZE": copy_kib / write[copy[0]][0]}
+    kernels = {}
+    for k in fetch:
+        if "aussm::" in k and k in write:
+            kernels[k] = {"fetch_KiB": fetch[k][0], "write_KiB": write[k][0], "dispatches": fetch[k][1],
+                          "read_bytes": fetch[k][0] * scale["FETCH_SIZE"] * 1024,
+                          "written_bytes": write[k][0] * scale["WRITE_SIZE"] * 1024}
+    rec = {"shape": SHAPE, "sources": source_digest(), "scale": scale, "copy_kernel": copy[0],
+           "copy_KiB": {"FETCH_SIZE": fetch[copy[0]][0], "WRITE_SIZE": write[copy[0]][0]}, "kernels": kernels,
+           "command": "rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE --kernel-trace --output-format csv -d <out> -- "
+                      "python3 bench.py --steps 3 --warmup 1 --prewarm-ms 0 --no-cpu --copy-probe"}
+    json.dump(rec, open(TRAFFIC_JSON, "w"), indent=1)
+    print(f"wrote {TRAFFIC_JSON}: {len(kernels)} kernels")
+
+
+def recorded_traffic(kernel_substrings):
+    """(bytes per call, note): sum over the named kernels of read + written bytes in profiles/traffic.json, or
+    (None, why) when the record does not cover this build or these kernels."""
+    if not os.path.exists(TRAFFIC_JSON):
+        return None, "profiles/traffic.json missing"
+    rec = json.load(open(TRAFFIC_JSON))
+    if rec.get("sources") != source_digest():
+        return None, "profiles/traffic.json was taken with other kernel sources"
+    if rec.get("shape") != SHAPE:
+        return None, "profiles/traffic.json was taken at another shape"
+    total = 0.0
+    for sub in kernel_substrings:
+        hit = [v for k, v in rec["kernels"].items() if sub in k and "float" in k]
+        if len(hit) != 1:
+            return None, f"profiles/traffic.json has {len(hit)} kernels matching {sub!r}"
+        total += hit[0]["read_bytes"] + hit[0]["written_bytes"]
+    return total, "profiles/traffic.json"
 
 
 def cpu_baseline(B_sample: int):
@@ -51,18 +124,23 @@ def cpu_baseline(B_sample: int):
     threads = min(cores, 16)
     torch.set_num_threads(threads)
     p = O.make_core_inputs(B_sample, D, N, L, seed=0)
-    leaves = [p[k].clone().requires_grad_(True) for k in ("u", "delta", "theta", "Bc", "Cc", "Dskip")]
-    t0 = time.perf_counter()
-    y, _ = O.unitary_core_loop(*leaves)
-    (y * p["dy"]).sum().backward()
-    dt = time.perf_counter() - t0
+    times = []
+    for run in range(4):                      # one warm-up run, three timed
+        leaves = [p[k].clone().requires_grad_(True) for k in ("u", "delta", "theta", "Bc", "Cc", "Dskip")]
+        t0 = time.perf_counter()
+        y, _ = O.unitary_core_loop(*leaves)
+        (y * p["dy"]).sum().backward()
+        if run:
+            times.append(time.perf_counter() - t0)
+    dt = sorted(times)[1]
     return {
         "value": B_sample * D * L / dt,
         "unit": "(b,d,l) samples/s, forward+backward",
         "cores": threads,
         "kind": "port",
-        "sample": f"B={B_sample} of {SHAPE['B']} batch elements at D={D} N={N} L={L}, one run, {dt:.1f} s wall, "
-                  f"torch {threads} threads on a host with {cores} cores",
+        "sample": f"B={B_sample} of {SHAPE['B']} batch elements at D={D} N={N} L={L}, one warm-up run then the median of "
+                  f"three ({', '.join(f'{t:.1f}' for t in times)} s wall), torch {threads} threads on a host with "
+                  f"{cores} cores",
     }
 
 
@@ -73,6 +151,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-batch", type=int, default=8)
+    ap.add_argument("--prewarm-ms", type=float, default=200.0, help="repeat the step for this long before the warm-up steps")
+    ap.add_argument("--summarize-traffic", nargs=2, metavar=("FETCH_DIR", "WRITE_DIR"),
+                    help="write profiles/traffic.json from the output of the two counter passes and exit")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one 256 MiB device-to-device copy (calibrates FETCH_SIZE / WRITE_SIZE under rocprofv3)")
     ap.add_argument("--shape", default=None, help="B,D,N,L instead of the headline shape (no recorded traffic figure then)")
@@ -80,6 +161,9 @@ def main():
     headline = args.shape is None
     if not headline:
         SHAPE.update(zip("BDNL", (int(v) for v in args.shape.split(","))))
+    if args.summarize_traffic:
+        summarize_traffic(*args.summarize_traffic)
+        return
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus must be 1 (no multi-GPU path exists)", file=sys.stderr)
         sys.exit(2)
@@ -113,6 +197,11 @@ def main():
         return scan.unitary_bwd_raw(p["dy"], None, p["u"], p["delta"], p["theta"], Bri, Cri, p["Dskip"], hck, ck,
                                     aux=aux)
 
+    t_pre = time.perf_counter()
+    while (time.perf_counter() - t_pre) * 1e3 < args.prewarm_ms:
+        step()
+        torch.cuda.synchronize()
+    prewarm_ms = (time.perf_counter() - t_pre) * 1e3
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -165,6 +254,11 @@ def main():
     bytes_fwd = 16 * E + 16 * S + 4 * D
     bytes_bwd = 28 * E + 32 * S + 4 * D
     ach = bytes_bwd / (t_bwd * 1e-6) / 1e9
+    # which kernels these calls ran, and what the counter passes recorded for them
+    fmode = lib.aussm_unitary_kernel_mode(0, B, D, N, L, ck, 0, 1, 1)
+    bmode = lib.aussm_unitary_kernel_mode(1, B, D, N, L, ck, 0, 1, 1)
+    traffic_fwd, note_fwd = recorded_traffic(FWD_KERNELS[fmode])
+    traffic_bwd, note_bwd = recorded_traffic(BWD_KERNELS[bmode])
 
     out = {
         "metric": f"unitary scan fwd+bwd elements/s + achieved HBM GB/s (% peak), B{B} D{D} N{N} L{L}",
@@ -173,6 +267,7 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "prewarm_ms": prewarm_ms,
         "ms_per_step": dt * 1e3,
         "higher_is_better": True,
         "scaling": "weak",
@@ -186,13 +281,14 @@ def main():
         "fwd_bwd_algorithmic_GBps": (bytes_fwd + bytes_bwd) / ((t_fwd + t_bwd) * 1e-6) / 1e9,
         "fwd_bwd_frac_of_hbm_peak": (bytes_fwd + bytes_bwd) / ((t_fwd + t_bwd) * 1e-6) / 1e9 / HBM_PEAK_GBS,
         "kernels_us": {"unitary_fwd": t_fwd, "unitary_bwd": t_bwd},
-        "roofline": {"bound": "hbm", "kernel": "unitary_bwd_xdl_kernel<3, 2, float>", "achieved": ach, "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": ach / HBM_PEAK_GBS, "traffic": TRAFFIC_BYTES["unitary_bwd"] if headline else None,
+        "roofline": {"bound": "hbm", "kernel": " + ".join(BWD_KERNELS[bmode][:2 if bmode == 6 else 1]) + " (one backward call)",
+                     "achieved": ach, "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": ach / HBM_PEAK_GBS, "traffic": traffic_bwd, "traffic_source": note_bwd,
                      "algorithmic_bytes": bytes_bwd,
-                     "fwd_kernel": {"kernel": "unitary_fwd_xdl_kernel<3, false, float>",
+                     "fwd_kernel": {"kernel": " + ".join(FWD_KERNELS[fmode]) + " (one forward call)",
                                     "achieved": bytes_fwd / (t_fwd * 1e-6) / 1e9,
                                     "frac": bytes_fwd / (t_fwd * 1e-6) / 1e9 / HBM_PEAK_GBS,
-                                    "traffic": TRAFFIC_BYTES["unitary_fwd"] if headline else None,
+                                    "traffic": traffic_fwd, "traffic_source": note_fwd,
                                     "algorithmic_bytes": bytes_fwd}},
     }
     if not args.no_cpu:

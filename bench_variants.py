@@ -4,10 +4,22 @@ once with float32 inputs and once with bfloat16 u / delta / B / C (float32 phase
 states, outputs and gradients): configuration 3 of the benchmark contract.
 
     python bench_variants.py [--reps R] [--shape B,D,N,L] [--variants real,...] [--model | --only-model]
+    python bench_variants.py --scaling [--runs 50] [--bdn 16,32,64 --bdn 32,256,16] [--lengths 10,...]
 
 With --model it also times configuration 4 of the contract: one training step (forward, MSE loss,
 backward) of SSMTS(d_model=256, input_dim=21, output_dim=21, layers="a|m|a|m") on x ~ N(0,1) of
 shape (32, 720, 21), random-init weights, wall clock around synchronised steps.
+
+With --scaling it runs the protocol of the reference's sweep, extension-cpp/test/scaling_benchmark.py:99-189,
+instead: for each system and each sequence length (20 log-spaced points in [10, 2048] as there, plus
+4096 and 16384), 5 warm-up and --runs timed repetitions of the operator's forward pass and of
+`y.sum().backward()`, device time of each (HIP events on the launch stream) and peak device memory after
+each (torch.cuda.max_memory_allocated, reset before every repetition).  Systems (the reference's are
+"mamba", "SSMau-cuda", "SSMau-pytorch", :193-216): "SSMau-hip" = ssm_adaptive_interface on the fused
+kernels, "SSMau-hip-composite" = the same interface on the composite route (phase tensor materialised),
+"mamba-hip" = selective_scan_fn.  Shapes: the reference's default b=16, d=32, n=64 (:259-262; n > 16 runs on
+the composite route for both SSMau systems) and the training configuration's b=32, d=256, n=16.  One JSON
+line per (system, shape, length).
 
 Prints one JSON line per (variant, input dtype): the duration of the forward and of the backward
 call (HIP events on the launch stream, mean of R launches after a warm-up long enough for the
@@ -42,6 +54,71 @@ def algorithmic_bytes(variant: str, w: int, E: int, S: int):
     return 2 * w * E + 4 * E + 2 * w * S, 2 * w * E + 12 * E + 2 * w * S + 8 * S
 
 
+def scaling(args):
+    """The sweep of extension-cpp/test/scaling_benchmark.py:99-189 on this package's operators."""
+    import numpy as np
+    import torch
+    from aussm_amd import ops, scan
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    lengths = ([int(v) for v in args.lengths.split(",")] if args.lengths else
+               [int(v) for v in np.logspace(np.log10(10), np.log10(2048), 20)] + [4096, 16384])
+    shapes = [tuple(int(v) for v in s.split(",")) for s in (args.bdn or ["16,32,64", "32,256,16"])]
+    systems = args.systems.split(",")
+    for b, d, n in shapes:
+        for system in systems:
+            for l in lengths:
+                g = torch.Generator(device=dev).manual_seed(0)
+                rn = lambda *s: torch.randn(*s, generator=g, device=dev)
+                leaf = lambda t: t.requires_grad_(True)
+                u, dt, z, D = leaf(rn(b, d, l)), leaf(rn(b, d, l)), leaf(rn(b, d, l)), leaf(rn(d))
+                if system == "mamba-hip":
+                    A, Bm, Cm = leaf(-torch.exp(rn(d, n))), leaf(rn(b, n, l)), leaf(rn(b, n, l))
+                    params = [u, dt, A, Bm, Cm, D, z]
+                    fn = lambda: scan.selective_scan_fn(u, dt, A, Bm, Cm, D, z=z, delta_softplus=True)
+                else:
+                    x, xb = leaf(rn(d, n, d) * d ** -0.5), leaf(rn(d, n))
+                    Bp, Cp = leaf(torch.complex(rn(n), rn(n))), leaf(torch.complex(rn(n), rn(n)))
+                    params = [u, dt, x, xb, Bp, Cp, D, z]
+                    save = system == "SSMau-hip-composite"
+                    fn = lambda: ops.ssm_adaptive_interface(u, dt, x, xb, Bp, Cp, D, z, unitary=True,
+                                                            save_intermediates=save)
+                tf = tb = mf = mb = 0.0
+                ev = lambda: torch.cuda.Event(enable_timing=True)
+                try:
+                    for run in range(args.runs + 5):
+                        for t in params:
+                            t.grad = None
+                        torch.cuda.synchronize()
+                        torch.cuda.reset_peak_memory_stats()
+                        e0, e1, e2 = ev(), ev(), ev()
+                        e0.record()
+                        y = fn()
+                        e1.record()
+                        mem_f = torch.cuda.max_memory_allocated()
+                        y.sum().backward()
+                        e2.record()
+                        torch.cuda.synchronize()
+                        if run >= 5:
+                            tf += e0.elapsed_time(e1)
+                            tb += e1.elapsed_time(e2)
+                            mf += mem_f
+                            mb += torch.cuda.max_memory_allocated()
+                        del y
+                except RuntimeError as e:           # out of memory, or a shape an operator does not take
+                    print(json.dumps({"system": system, "b": b, "d": d, "n": n, "L": l,
+                                      "error": str(e).split("\n")[0][:160]}), flush=True)
+                    torch.cuda.empty_cache()
+                    continue
+                r = args.runs
+                print(json.dumps({"system": system, "b": b, "d": d, "n": n, "L": l, "runs": r,
+                                  "fwd_us": round(tf / r * 1e3, 1), "bwd_us": round(tb / r * 1e3, 1),
+                                  "fwd_peak_MB": round(mf / r * 1e-6, 2), "bwd_peak_MB": round(mb / r * 1e-6, 2)}),
+                      flush=True)
+                del params, u, dt, z, D
+                torch.cuda.empty_cache()
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--reps", type=int, default=30)
@@ -49,6 +126,11 @@ def main():
     ap.add_argument("--model", action="store_true", help="also time the hybrid SSMTS training step (configuration 4)")
     ap.add_argument("--only-model", action="store_true", help="time only the SSMTS training step")
     ap.add_argument("--variants", default="unitary,complex,real", help="comma-separated subset of the variants")
+    ap.add_argument("--scaling", action="store_true", help="the sequence-length sweep of the reference's scaling benchmark")
+    ap.add_argument("--runs", type=int, default=50, help="timed repetitions per point of the sweep (after 5 warm-ups)")
+    ap.add_argument("--bdn", action="append", help="b,d,n of the sweep (repeatable)")
+    ap.add_argument("--lengths", default=None, help="comma-separated sequence lengths of the sweep")
+    ap.add_argument("--systems", default="SSMau-hip,SSMau-hip-composite,mamba-hip")
     args = ap.parse_args()
     B, D, N, L = (int(v) for v in args.shape.split(","))
 
@@ -60,6 +142,9 @@ def main():
         sys.exit(1)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.scaling:
+        scaling(args)
+        return
 
     def timed(fn):
         for _ in range(40):

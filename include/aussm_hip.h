@@ -146,6 +146,12 @@ int aussm_unitary_bwd(const float* dy, const float* dhL,
  * No counterpart in the reference (its backward kernel recomputes,
  * ssm_adaptive_unitary_backward.cu:113-181, and its launches cover at most 2048 steps). */
 size_t aussm_unitary_aux_floats(int B, int D, int N, int L, int ck);
+/* Which kernel family a unitary call of this shape runs (tensors 16-byte aligned, current options):
+ * 0 vector-ALU kernels, 2 / 3 / 5 matrix-core kernels that build their operands themselves,
+ * 6 matrix-core kernels on operands prepared by a pre-pass.  have_aux: the call gets an auxiliary
+ * buffer.  A caller can skip allocating that buffer when both directions answer 0 (the vector-ALU
+ * kernels neither fill nor read it) and aussm_unitary_split_segments() answers 1. */
+int aussm_unitary_kernel_mode(int backward, int B, int D, int N, int L, int ck, int in_dtype, int urep, int have_aux);
 
 /* Number of segments a call of this shape is split into along L when it is given an auxiliary
  * buffer (1 = not split); lets a caller choose ck (a segment is a whole number of checkpoint blocks). */

@@ -129,8 +129,18 @@ def test_fused_matches_composite_at_training_shape():
         _close(g_, w.cpu(), "gradient wrt " + name, tol=2e-4)
 
 
-def test_fused_rejects_shapes_beyond_the_kernels():
-    from aussm_amd import ops  # noqa: F401
-    args = [a.float().cuda() for a in _inputs(1, 4, 17, 8, seed=1)]
-    with pytest.raises(RuntimeError, match="outside the fused kernels' range"):
-        torch.ops.extension_cpp.ssm_adaptive_unitary(*args)
+def test_shapes_beyond_the_fused_kernels_take_the_composite_route():
+    """n > 16: the dispatcher operators still answer (through the core scan), forward and backward."""
+    from aussm_amd import ops
+    b, d, n, l = 2, 8, 24, 40
+    assert not ops.fused_supported(b, d, n, l) and ops.fused_supported(b, d, 16, l)
+    args = _inputs(b, d, n, l, seed=6, xscale=d ** -0.5)
+    leaves = [a.clone().requires_grad_(True) for a in args]
+    y, hr, hi = O.adaptive_unitary_op_loop(*leaves)
+    (y.square().mean() + (hr * hi).mean()).backward()
+    dev = [a.float().cuda().requires_grad_(True) for a in args]
+    y2, hr2, hi2 = ops.ssm_adaptive_unitary(*dev)
+    _close(y2.detach(), y.detach(), "y")
+    (y2.square().mean() + (hr2 * hi2).mean()).backward()
+    for w, g_, name in zip(leaves, dev, IN_NAMES):
+        _close(g_.grad, w.grad, "gradient wrt " + name)
