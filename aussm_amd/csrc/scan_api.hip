@@ -478,9 +478,12 @@ int aussm_swap_last2(const float* x, float* y, int B, int R, int C, long long xs
 
 static size_t dropin_xp_floats(int d) { return (size_t)d * ((d + 31) / 32) * 3 * 64 * 4; }
 // The backward call works through the (batch, sequence) plane in blocks of bg batch elements x ct tiles
-// of 16 timesteps: the workspace holds the phase adjoints of one block (about 96 MiB at most).  bg is
+// of 16 timesteps: the workspace holds the phase adjoints of one block (about 50 MiB at most).  bg is
 // what fills the chip with one workgroup per compute unit (fewer would idle units, more would only
 // shorten the blocks and repeat the per-launch set-up, the rows of x among it, more often).
+#ifndef DROPIN_BLOCK_FLOATS
+#define DROPIN_BLOCK_FLOATS (25u << 19)
+#endif
 struct DropinBlocks { int bg, ct; };
 static DropinBlocks dropin_blocks(int b, int d, int n, int L) {
   const int nw = dropin_channels_per_workgroup((d + 31) / 32);
@@ -489,7 +492,7 @@ static DropinBlocks dropin_blocks(int b, int d, int n, int L) {
   if (bg > b) bg = b;
   const int ng = (b + bg - 1) / bg;
   bg = (b + ng - 1) / ng;
-  const size_t per_tile = (size_t)bg * d * n * DT, cap = (size_t)24 << 20;
+  const size_t per_tile = (size_t)bg * d * n * DT, cap = (size_t)DROPIN_BLOCK_FLOATS;
   const int ntiles = (L + DT - 1) / DT;
   size_t tmax = cap / per_tile;
   if (tmax < 1) tmax = 1;

@@ -109,16 +109,24 @@ def test_fused_matches_composite_at_training_shape():
     g = torch.Generator().manual_seed(2)
     gy = torch.randn(b, d, l, generator=g).cuda()
     zeros = torch.zeros(b, d, n, device="cuda")
+    inputs_bytes = sum(a.numel() * 4 for a in args)
+    # The fused route never holds the phase tensor (b d n l floats = 377 MB here).  What a call allocates on top of
+    # its inputs - outputs and workspace - stays within the operator's input footprint for the forward call and
+    # within twice that for the backward call (twelve gradients the size of the inputs, plus the workspace).
+    torch.cuda.synchronize()
     torch.cuda.reset_peak_memory_stats()
     base = torch.cuda.memory_allocated()
     y, hr, hi = torch.ops.extension_cpp.ssm_adaptive_unitary(*args)
+    torch.cuda.synchronize()
+    peak_fwd = torch.cuda.max_memory_allocated() - base
+    torch.cuda.reset_peak_memory_stats()
+    base = torch.cuda.memory_allocated()
     grads = torch.ops.extension_cpp.ssm_adaptive_backward_unitary(gy, zeros, zeros, *args)
     torch.cuda.synchronize()
-    peak = torch.cuda.max_memory_allocated() - base
-    inputs_bytes = sum(a.numel() * 4 for a in args)
-    # the fused route never holds the phase tensor (b d n l floats = 377 MB here): everything it allocates
-    # (outputs, twelve gradients, workspace) stays within three times the operator's input footprint
-    assert peak < 3 * inputs_bytes, (peak, inputs_bytes)
+    peak_bwd = torch.cuda.max_memory_allocated() - base
+    print(f"inputs {inputs_bytes / 1e6:.0f} MB, forward call +{peak_fwd / 1e6:.0f} MB, backward call +{peak_bwd / 1e6:.0f} MB", flush=True)
+    assert peak_fwd <= inputs_bytes, (peak_fwd, inputs_bytes)
+    assert peak_bwd <= 2 * inputs_bytes, (peak_bwd, inputs_bytes)
     leaves = [a.clone().requires_grad_(True) for a in args]
     yc, hrc, hic = ops._composite(*leaves)
     want = torch.autograd.grad([yc], leaves, [gy], allow_unused=True)
