@@ -7,7 +7,8 @@
 //     y_l[b,i]       = silu(z_l[b,i]) ( sum_j Re(Ct_j h_l[b,i,j]) + D_i ut_l[b,i] )
 //
 // The phase tensor theta[b,i,j,l] (n times the size of every other tensor) never exists in memory.
-// A wavefront owns one (batch, channel) pair and walks the sequence in tiles of 16 timesteps:
+// A wavefront owns one (batch, channel) pair - with more than 16 states per channel, one block of 16
+// states of it - and walks the sequence in tiles of 16 timesteps:
 //   * the tile's phases, a (16 states) x (16 timesteps) block, are one small matrix product
 //     x[i] (16 x d) . u[b][:, tile] (d x 16) on the bf16 matrix cores with both operands split exactly
 //     into three bf16 pieces (scan_fwd_xdl.h), i.e. fp32-accurate.  The wavefront keeps its rows of x
@@ -52,14 +53,14 @@ __device__ __forceinline__ float row_last(float v, int lane) { return __shfl(v, 
 __device__ __forceinline__ float row_first(float v, int lane) { return __shfl(v, lane & 48); }
 
 
-// x (d, n, d) -> operand records.  Record (i, ks, piece, lane = (row j = lane % 16, g = lane / 16))
-// holds x[i, j, 32 ks + 8 g .. + 7] (zero past the ends).  One thread per (i, ks, lane).
-__global__ __launch_bounds__(256) void dropin_xprep_kernel(const float* __restrict__ x, u4* __restrict__ xp, int d, int n, int ks) {
+// x (d, n, d) -> operand records.  Record (v = i nb + sb, ks, piece, lane = (row = lane % 16, g = lane / 16))
+// holds x[i, 16 sb + row, 32 ks + 8 g .. + 7] (zero past the ends).  One thread per (v, ks, lane).
+__global__ __launch_bounds__(256) void dropin_xprep_kernel(const float* __restrict__ x, u4* __restrict__ xp, int d, int n, int ks, int nb) {
   const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
-  if (idx >= (size_t)d * ks * 64) return;
+  if (idx >= (size_t)d * nb * ks * 64) return;
   const int lane = (int)(idx & 63);
-  const int k = (int)((idx >> 6) % ks), i = (int)((idx >> 6) / ks);
-  const int j = lane & 15, g = lane >> 4;
+  const int k = (int)((idx >> 6) % ks), vc = (int)((idx >> 6) / ks);
+  const int i = vc / nb, j = 16 * (vc % nb) + (lane & 15), g = lane >> 4;
   const SplitK sk = make_splitk();
   float v[8];
 #pragma unroll
@@ -70,7 +71,7 @@ __global__ __launch_bounds__(256) void dropin_xprep_kernel(const float* __restri
   u4 pc[3];
   split8<3>(sk, v, pc);
 #pragma unroll
-  for (int q = 0; q < 3; ++q) xp[(((size_t)i * ks + k) * 3 + q) * 64 + lane] = pc[q];
+  for (int q = 0; q < 3; ++q) xp[(((size_t)vc * ks + k) * 3 + q) * 64 + lane] = pc[q];
 }
 
 // Stage the tile u[b][:, l0 .. l0 + 15] as the second operand of the phase product: record
@@ -106,16 +107,19 @@ __device__ __forceinline__ void stage_store(const float (&v)[NREC][8], u4* __res
   }
 }
 
-// Workgroup = (batch b, NW consecutive channels), one channel per wavefront.  KS: 32-wide steps of
-// the contraction over r (d <= 32 KS).  n <= 16.
+// Workgroup = (batch b, NW consecutive (channel, state block) pairs), one pair per wavefront; the nb
+// wavefronts of a channel are neighbours (nb divides NW) and add their shares of y through LDS.
+// KS: 32-wide steps of the contraction over r (d <= 32 KS).
 template <int KS, int NW>
 __global__ __launch_bounds__(NW * 64) void dropin_fwd_kernel(const DropinArgs p) {
   __shared__ u4 s_u[2][KS * 3 * 64];
+  __shared__ float s_y[2][NW][DT];                     // shares of y of the tile, by tile parity (nb > 1)
   const int tid = threadIdx.x, lane = tid & 63, wave = wave_index();
-  const int ncg = (p.d + NW - 1) / NW;
-  const int b = blockIdx.x / ncg, i = (blockIdx.x % ncg) * NW + wave;
+  const int nb = p.nb, ncg = (p.d * nb + NW - 1) / NW;
+  const int b = blockIdx.x / ncg, v = (blockIdx.x % ncg) * NW + wave;
+  const int i = v / nb, sb = v % nb, j0 = 16 * sb;
   const bool iok = i < p.d;
-  const int ic = iok ? i : p.d - 1;
+  const int ic = iok ? i : p.d - 1, vc = ic * nb + sb;
   const int l_ = lane & 15, g = lane >> 4;
   const int d = p.d, n = p.n, L = p.L;
   const SplitK sk = make_splitk();
@@ -128,12 +132,12 @@ __global__ __launch_bounds__(NW * 64) void dropin_fwd_kernel(const DropinArgs p)
   for (int k = 0; k < KS; ++k)
 #pragma unroll
     for (int q = 0; q < 3; ++q)
-      xa[k][q] = (k < p.ks) ? p.xp[(((size_t)ic * p.ks + k) * 3 + q) * 64 + lane] : u4{0, 0, 0, 0};
-  // per state j = 4 g + a: bias, Bt, Ct, carried state
+      xa[k][q] = (k < p.ks) ? p.xp[(((size_t)vc * p.ks + k) * 3 + q) * 64 + lane] : u4{0, 0, 0, 0};
+  // per state j = j0 + 4 g + a: bias, Bt, Ct, carried state
   float xb[4], btr[4], bti[4], ctr[4], cti[4], hr[4], hi[4];
 #pragma unroll
   for (int a = 0; a < 4; ++a) {
-    const int j = 4 * g + a;
+    const int j = j0 + 4 * g + a;
     const bool ok = j < n;
     const int jc = ok ? j : 0;
     xb[a] = ok ? p.x_bias[(size_t)ic * n + jc] : 0.0f;
@@ -199,14 +203,23 @@ __global__ __launch_bounds__(NW * 64) void dropin_fwd_kernel(const DropinArgs p)
     }
     ysum += __shfl_xor(ysum, 16);
     ysum += __shfl_xor(ysum, 32);
-    if (p.y && iok && lok && g == 0) p.y[row + l] = siluf_(zv) * (ysum + Di * ut);
+    if (nb == 1) {
+      if (p.y && iok && lok && g == 0) p.y[row + l] = siluf_(zv) * (ysum + Di * ut);
+    } else if (g == 0) {
+      s_y[t & 1][wave][l_] = ysum;
+    }
     if (t + 1 < ntiles) stage_store<NT, NREC>(sv, s_u[(t + 1) & 1], p.ks, tid, sk);
     __syncthreads();
+    if (nb > 1 && sb == 0 && g == 0 && p.y && iok && lok) {      // the channel's first wavefront adds the shares up
+      float tot = ysum;
+      for (int k = 1; k < nb; ++k) tot += s_y[t & 1][wave + k][l_];
+      p.y[row + l] = siluf_(zv) * (tot + Di * ut);
+    }
   }
   if (p.nh_re && iok && l_ == 0) {
 #pragma unroll
     for (int a = 0; a < 4; ++a) {
-      const int j = 4 * g + a;
+      const int j = j0 + 4 * g + a;
       if (j < n) {
         p.nh_re[((size_t)b * d + i) * n + j] = hr[a];
         p.nh_im[((size_t)b * d + i) * n + j] = hi[a];
@@ -249,12 +262,14 @@ __device__ __forceinline__ float row_sum(float v) {     // total of the row in i
 template <int KS, int NW>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DROPIN_BWD_WAVES, DROPIN_BWD_WAVES))) void dropin_bwd_kernel(const DropinBwdArgs q) {
   __shared__ u4 s_u[2][KS * 3 * 64];
+  __shared__ float2 s_yw[2][NW][DT];                   // shares of (sum_j Re(Ct h), sum_j hat w) of the tile (nb > 1)
   const DropinArgs& p = q.f;
   const int tid = threadIdx.x, lane = tid & 63, wave = wave_index();
-  const int ncg = (p.d + NW - 1) / NW;
-  const int zb = blockIdx.x / ncg, b = q.b0 + zb, i = (blockIdx.x % ncg) * NW + wave;
+  const int nb = p.nb, ncg = (p.d * nb + NW - 1) / NW;
+  const int zb = blockIdx.x / ncg, b = q.b0 + zb, v = (blockIdx.x % ncg) * NW + wave;
+  const int i = v / nb, sb = v % nb, j0 = 16 * sb;
   const bool iok = i < p.d;
-  const int ic = iok ? i : p.d - 1;
+  const int ic = iok ? i : p.d - 1, vc = ic * nb + sb;
   const int l_ = lane & 15, g = lane >> 4;
   const int d = p.d, n = p.n, L = p.L;
   const SplitK sk = make_splitk();
@@ -266,11 +281,11 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DROPIN_
   for (int k = 0; k < KS; ++k)
 #pragma unroll
     for (int c = 0; c < 3; ++c)
-      xa[k][c] = (k < p.ks) ? p.xp[(((size_t)ic * p.ks + k) * 3 + c) * 64 + lane] : u4{0, 0, 0, 0};
+      xa[k][c] = (k < p.ks) ? p.xp[(((size_t)vc * p.ks + k) * 3 + c) * 64 + lane] : u4{0, 0, 0, 0};
   // per state: (Re Bt, Im Bt, Re Ct, Im Ct), shared by the workgroup, and the bias of this wavefront's channel.
   // They are read from LDS where they are used: in registers they would push the kernel over 256.
   __shared__ f4 s_par[D_MAXN];
-  __shared__ float s_xb[NW][D_MAXN];
+  __shared__ float s_xb[NW][16];
   if (tid < D_MAXN) {
     const bool ok = tid < n;
     const int jc = ok ? tid : 0;
@@ -279,12 +294,12 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DROPIN_
     fast_sincosf(p.C_th[jc], &sc, &cc);
     s_par[tid] = ok ? f4{p.B_r[jc] * cb, p.B_r[jc] * sb, p.C_r[jc] * cc, p.C_r[jc] * sc} : f4{0, 0, 0, 0};
   }
-  if (lane < D_MAXN) s_xb[wave][lane] = lane < n ? p.x_bias[(size_t)ic * n + lane] : 0.0f;
+  if (lane < 16) s_xb[wave][lane] = j0 + lane < n ? p.x_bias[(size_t)ic * n + j0 + lane] : 0.0f;
   float hr[4], hi[4], ar[4], ai[4];
   float gBr[4], gBi[4], gCr[4], gCi[4], gxb[4];
 #pragma unroll
   for (int a = 0; a < 4; ++a) {
-    const int j = 4 * g + a;
+    const int j = j0 + 4 * g + a;
     const bool ok = j < n;
     const int jc = ok ? j : 0;
     const size_t sidx = ((size_t)b * d + ic) * n + jc;
@@ -340,7 +355,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DROPIN_
     float ysum = 0.0f, wsum = 0.0f;
 #pragma unroll
     for (int a = 0; a < 4; ++a) {
-      const f4 par = s_par[4 * g + a];
+      const f4 par = s_par[j0 + 4 * g + a];
       const float btr_ = par[0], bti_ = par[1], ctr_ = par[2], cti_ = par[3];
       const float thv = lok ? th[a] + s_xb[wave][4 * g + a] : 0.0f;
       const float G = row_prefix(thv);
@@ -368,7 +383,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DROPIN_
       float Gh = -(hdr * hei - hdi * her) + (phr * pi - phi * pr);
       if (l_ == 15) Gh -= ar[a] * hi[a] - ai[a] * hr[a];                              // h at the last step is h_out
       const float thh = row_suffix(Gh);
-      if (lok && iok && 4 * g + a < n) dth[(size_t)(4 * g + a) * q.lc + l] = thh;
+      if (lok && iok && j0 + 4 * g + a < n) dth[(size_t)(j0 + 4 * g + a) * q.lc + l] = thh;
       gxb[a] += lok ? thh : 0.0f;
       // hat Bt += E w hat p ; hat Ct += a conj(h)
       const float ewr = cs * w, ewi = sn * w;
@@ -386,15 +401,24 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DROPIN_
     ysum += __shfl_xor(ysum, 32);
     wsum += __shfl_xor(wsum, 16);
     wsum += __shfl_xor(wsum, 32);
-    if (iok && lok && g == 0) {
+    if (nb > 1 && g == 0) s_yw[t & 1][wave][l_] = make_float2(ysum, wsum);
+    if (t > t_first) stage_store<NT, NREC>(sv, s_u[(t - 1) & 1], p.ks, tid, sk);
+    if (nb > 1) {                                      // the channel's first wavefront adds the shares up
+      __syncthreads();
+      for (int k = 1; k < nb; ++k) {
+        const float2 o = s_yw[t & 1][(wave + k) & (NW - 1)][l_];
+        ysum += o.x;
+        wsum += o.y;
+      }
+    }
+    if (iok && lok && g == 0 && sb == 0) {
       const float pre = ysum + Di * ut;
       q.dz[row + l] = gyv * pre * dsiluf_(zv);
       q.ddt[row + l] = wsum * ut;
       q.du[row + l] = (wsum * dtv + av * Di) * dsiluf_(uv);
       gD += av * ut;
     }
-    if (t > t_first) stage_store<NT, NREC>(sv, s_u[(t - 1) & 1], p.ks, tid, sk);
-    __syncthreads();
+    if (nb == 1) __syncthreads();
   }
   // ---- reductions over the timesteps (lanes of a row) and hand-off.  The gradients of the 4 n shared
   // parameters are first summed over the workgroup's channels in LDS: every workgroup of the launch adds
@@ -414,7 +438,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DROPIN_
   if (iok && l_ == 0) {
 #pragma unroll
     for (int a = 0; a < 4; ++a) {
-      const int j = 4 * g + a;
+      const int j = j0 + 4 * g + a;
       if (j < n) {
         const size_t sidx = ((size_t)b * d + i) * n + j;
         q.dh_re[sidx] = ar[a];
@@ -433,11 +457,12 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DROPIN_
         atomicAdd(&s_red[3][j], gCi[a] * par[2] - gCr[a] * par[3]);
       }
     }
-    if (g == 0) atomicAdd(q.dD + i, gD);
+    if (g == 0 && sb == 0) atomicAdd(q.dD + i, gD);
   }
   __syncthreads();
   if (tid < 4 * D_MAXN && (tid & (D_MAXN - 1)) < n) {
-    float* dst = (tid >> 4) == 0 ? q.dB_r : (tid >> 4) == 1 ? q.dB_th : (tid >> 4) == 2 ? q.dC_r : q.dC_th;
+    constexpr int SH = 6;                              // log2(D_MAXN)
+    float* dst = (tid >> SH) == 0 ? q.dB_r : (tid >> SH) == 1 ? q.dB_th : (tid >> SH) == 2 ? q.dC_r : q.dC_th;
     atomicAdd(dst + (tid & (D_MAXN - 1)), (&s_red[0][0])[tid]);
   }
 }

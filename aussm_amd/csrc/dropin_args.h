@@ -6,7 +6,7 @@ namespace aussm {
 
 constexpr int DT = 16;            // timesteps per tile
 constexpr int D_MAXKS = 16;       // 32-wide steps of the contraction over r held in registers: d <= 512
-constexpr int D_MAXN = 16;        // states per channel
+constexpr int D_MAXN = 64;        // states per channel: up to four blocks of 16, one block per wavefront
 
 struct DropinArgs {
   const float* u;        // [b, d, L]
@@ -23,8 +23,9 @@ struct DropinArgs {
   float* y;              // [b, d, L] or null (states only)
   float* nh_re;          // [b, d, n] or null
   float* nh_im;
-  const u4* xp;          // rows of x as matrix operands: [d][ks][piece][64 lanes]
+  const u4* xp;          // rows of x as matrix operands: [d nb][ks][piece][64 lanes]
   int b, d, n, L, ks;    // ks = ceil(d / 32)
+  int nb;                // blocks of 16 states per channel: 1, 2 or 4 (>= ceil(n / 16))
 };
 
 struct DropinBwdArgs {

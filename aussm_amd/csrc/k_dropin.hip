@@ -4,9 +4,9 @@
 
 namespace aussm {
 
-void run_dropin_xprep(const float* x, u4* xp, int d, int n, int ks, hipStream_t s) {
-  const size_t total = (size_t)d * ks * 64;
-  hipLaunchKernelGGL(dropin_xprep_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, x, xp, d, n, ks);
+void run_dropin_xprep(const float* x, u4* xp, int d, int n, int ks, int nb, hipStream_t s) {
+  const size_t total = (size_t)d * nb * ks * 64;
+  hipLaunchKernelGGL(dropin_xprep_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, x, xp, d, n, ks, nb);
 }
 
 void run_fill(float* p, const float* src, size_t n, hipStream_t s) {
@@ -22,13 +22,13 @@ constexpr int DROPIN_NW = DROPIN_NW_;     // channels (wavefronts) per workgroup
 template <int KS>
 static void launch_fwd(const DropinArgs& a, hipStream_t s) {
   constexpr int NW = KS > 8 ? 4 : DROPIN_NW;
-  const unsigned grid = (unsigned)(a.b * ((a.d + NW - 1) / NW));
+  const unsigned grid = (unsigned)(a.b * ((a.d * a.nb + NW - 1) / NW));
   hipLaunchKernelGGL((dropin_fwd_kernel<KS, NW>), dim3(grid), dim3(NW * 64), 0, s, a);
 }
 template <int KS>
 static void launch_bwd(const DropinBwdArgs& a, hipStream_t s) {
   constexpr int NW = KS > 8 ? 4 : DROPIN_NW;
-  const unsigned grid = (unsigned)(a.bg * ((a.f.d + NW - 1) / NW));
+  const unsigned grid = (unsigned)(a.bg * ((a.f.d * a.f.nb + NW - 1) / NW));
   hipLaunchKernelGGL((dropin_bwd_kernel<KS, NW>), dim3(grid), dim3(NW * 64), 0, s, a);
 }
 

@@ -41,7 +41,7 @@ int run_px_fwd(const FwdArgs& a, const u4* img, int in_dtype, hipStream_t s);
 int run_px_bwd(const UniBwdArgs& a, const u4* img, int in_dtype, hipStream_t s);
 
 // ---- k_dropin.hip: the reference's 12-input operator as fused kernels
-void run_dropin_xprep(const float* x, u4* xp, int d, int n, int ks, hipStream_t s);
+void run_dropin_xprep(const float* x, u4* xp, int d, int n, int ks, int nb, hipStream_t s);
 int dropin_channels_per_workgroup(int ks);
 int run_dropin_fwd(const DropinArgs& a, hipStream_t s);
 int run_dropin_bwd(const DropinBwdArgs& a, hipStream_t s);

@@ -476,7 +476,9 @@ int aussm_swap_last2(const float* x, float* y, int B, int R, int C, long long xs
 
 // ---- the reference's operator extension_cpp::ssm_adaptive_unitary as fused kernels (dropin.h)
 
-static size_t dropin_xp_floats(int d) { return (size_t)d * ((d + 31) / 32) * 3 * 64 * 4; }
+// blocks of 16 states per channel, one per wavefront: 1, 2 or 4 (they have to divide the wavefronts of a workgroup)
+static int dropin_state_blocks(int n) { const int k = (n + 15) / 16; return k == 3 ? 4 : k; }
+static size_t dropin_xp_floats(int d, int n) { return (size_t)d * dropin_state_blocks(n) * ((d + 31) / 32) * 3 * 64 * 4; }
 // The backward call works through the (batch, sequence) plane in blocks of bg batch elements x ct tiles
 // of 16 timesteps: the workspace holds the phase adjoints of one block (about 50 MiB at most).  bg is
 // what fills the chip with one workgroup per compute unit (fewer would idle units, more would only
@@ -487,7 +489,7 @@ static size_t dropin_xp_floats(int d) { return (size_t)d * ((d + 31) / 32) * 3 *
 struct DropinBlocks { int bg, ct; };
 static DropinBlocks dropin_blocks(int b, int d, int n, int L) {
   const int nw = dropin_channels_per_workgroup((d + 31) / 32);
-  const int wgs_per_b = (d + nw - 1) / nw;
+  const int wgs_per_b = (d * dropin_state_blocks(n) + nw - 1) / nw;
   int bg = (256 + wgs_per_b - 1) / wgs_per_b;
   if (bg > b) bg = b;
   const int ng = (b + bg - 1) / bg;
@@ -526,13 +528,13 @@ static size_t round4(size_t v) { return (v + 3) & ~(size_t)3; }
 static int dropin_check(int b, int d, int n, int L) {
   if (b < 1 || d < 1 || n < 1 || L < 1) return AUSSM_E_SHAPE;
   if (n > D_MAXN || d > 32 * D_MAXKS) return AUSSM_E_SHAPE;
-  if ((long long)b * ((d + 3) / 4) > 0x7fffffffLL || (long long)d * n * L > 0x7fffffffLL) return AUSSM_E_SHAPE;
+  if ((long long)b * d > 0x7fffffffLL || (long long)d * n * L > 0x7fffffffLL) return AUSSM_E_SHAPE;
   return AUSSM_OK;
 }
 
 size_t aussm_ssm_adaptive_unitary_workspace_floats(int b, int d, int n, int L, int backward) {
   if (dropin_check(b, d, n, L) != AUSSM_OK) return 0;
-  size_t f = dropin_xp_floats(d);
+  size_t f = dropin_xp_floats(d, n);
   if (backward) {
     const DropinBlocks k = dropin_blocks(b, d, n, L);
     f += 2 * round4((size_t)b * d * n) + (size_t)k.bg * k.ct * DT * d * n;
@@ -551,10 +553,10 @@ int aussm_ssm_adaptive_unitary_fwd(const float* u, const float* dt, const float*
     return AUSSM_E_NULL;
   if (misaligned(workspace, 16)) return AUSSM_E_ALIGN;
   hipStream_t s = (hipStream_t)stream;
-  const int ks = (d + 31) / 32;
-  run_dropin_xprep(x, (u4*)workspace, d, n, ks, s);
+  const int ks = (d + 31) / 32, nb = dropin_state_blocks(n);
+  run_dropin_xprep(x, (u4*)workspace, d, n, ks, nb, s);
   DropinArgs a{u, dt, z, x_bias, B_r, B_theta, C_r, C_theta, D, h_re, h_im, y, nh_re, nh_im, (const u4*)workspace,
-               b, d, n, L, ks};
+               b, d, n, L, ks, nb};
   return run_dropin_fwd(a, s);
 }
 
@@ -574,15 +576,15 @@ int aussm_ssm_adaptive_unitary_bwd(const float* grad_y, const float* grad_nh_re,
   if (misaligned(workspace, 16)) return AUSSM_E_ALIGN;
   hipStream_t s = (hipStream_t)stream;
   const DropinBlocks blk = dropin_blocks(b, d, n, L);
-  const int ks = (d + 31) / 32, ct = blk.ct, lc = ct * DT;
+  const int ks = (d + 31) / 32, nb = dropin_state_blocks(n), ct = blk.ct, lc = ct * DT;
   const int ntiles = (L + DT - 1) / DT;
   const size_t nstate = (size_t)b * d * n;
   u4* xp = (u4*)workspace;
-  float* hc_re = workspace + dropin_xp_floats(d);
+  float* hc_re = workspace + dropin_xp_floats(d, n);
   float* hc_im = hc_re + round4(nstate);
   float* dth = hc_im + round4(nstate);
-  run_dropin_xprep(x, xp, d, n, ks, s);
-  DropinArgs f{u, dt, z, x_bias, B_r, B_theta, C_r, C_theta, D, h_re, h_im, nullptr, hc_re, hc_im, xp, b, d, n, L, ks};
+  run_dropin_xprep(x, xp, d, n, ks, nb, s);
+  DropinArgs f{u, dt, z, x_bias, B_r, B_theta, C_r, C_theta, D, h_re, h_im, nullptr, hc_re, hc_im, xp, b, d, n, L, ks, nb};
   if (nh_re && nh_im) {
     run_fill(hc_re, nh_re, nstate, s);
     run_fill(hc_im, nh_im, nstate, s);

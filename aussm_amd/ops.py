@@ -16,7 +16,7 @@ Operator semantics (ssm_adaptive_unitary_forward.cu:83-181), per batch b, channe
 The two dispatcher ops run the library's fused kernels (aussm_ssm_adaptive_unitary_fwd / _bwd,
 include/aussm_hip.h): the phase tensor theta (b, d, n, l) is formed tile by tile inside the scan
 kernel and never stored, and the backward op recomputes from the twelve inputs as the reference's
-does.  Shapes beyond the fused kernels' limits (n > 16 or d > 512) take the composite route below.
+does.  Shapes beyond the fused kernels' limits (n > 64 or d > 512) take the composite route below.
 
 `_composite` is a second, independent route to the same numbers, kept for the interface's
 save_intermediates=True mode and as a cross-check in the tests: every (batch, state) pair becomes
@@ -102,7 +102,7 @@ _lib.define(_BWD_SCHEMA)
 
 
 def fused_supported(b: int, d: int, n: int, l: int) -> bool:
-    """Whether the fused kernels take this shape (n <= 16, d <= 512); beyond it the dispatcher ops run
+    """Whether the fused kernels take this shape (n <= 64, d <= 512); beyond it the dispatcher ops run
     the composite route (same HIP core scan, phase tensor materialised)."""
     return L.load().aussm_ssm_adaptive_unitary_workspace_floats(b, d, n, l, 0) > 0
 

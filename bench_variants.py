@@ -17,9 +17,8 @@ instead: for each system and each sequence length (20 log-spaced points in [10, 
 each (torch.cuda.max_memory_allocated, reset before every repetition).  Systems (the reference's are
 "mamba", "SSMau-cuda", "SSMau-pytorch", :193-216): "SSMau-hip" = ssm_adaptive_interface on the fused
 kernels, "SSMau-hip-composite" = the same interface on the composite route (phase tensor materialised),
-"mamba-hip" = selective_scan_fn.  Shapes: the reference's default b=16, d=32, n=64 (:259-262; n > 16 runs on
-the composite route for both SSMau systems) and the training configuration's b=32, d=256, n=16.  One JSON
-line per (system, shape, length).
+"mamba-hip" = selective_scan_fn.  Shapes: the reference's default b=16, d=32, n=64 (:259-262) and the training
+configuration's b=32, d=256, n=16.  One JSON line per (system, shape, length).
 
 Prints one JSON line per (variant, input dtype): the duration of the forward and of the backward
 call (HIP events on the launch stream, mean of R launches after a warm-up long enough for the

@@ -277,7 +277,7 @@ int aussm_swap_last2(const float* x, float* y, int B, int R, int C,
  * the matrix cores inside the scan kernel.  The backward call recomputes from the twelve inputs,
  * as the reference does, and needs the phase adjoints of a few batch elements at a time (for the
  * product that sums over all channels); they live in the workspace, at most about 50 MiB.
- * Limits: n <= 16, d <= 512 (AUSSM_E_SHAPE beyond).  L is arbitrary (the reference needs a
+ * Limits: n <= 64, d <= 512 (AUSSM_E_SHAPE beyond).  L is arbitrary (the reference needs a
  * multiple of 16 and pads).  `workspace` holds aussm_ssm_adaptive_unitary_workspace_floats(...)
  * floats, 16-byte aligned; nothing in it has to be initialised, nothing in it is kept between calls.
  * grad_nh_re / grad_nh_im may be NULL (zero).  Every gradient buffer is fully written.

@@ -34,7 +34,8 @@ def _close(got, want, name, tol=1e-4):
                                msg=lambda m: f"{name}: {m}")
 
 
-SHAPES = [(2, 8, 4, 256), (3, 20, 5, 48), (2, 37, 16, 45), (1, 70, 11, 130), (2, 16, 16, 14)]
+SHAPES = [(2, 8, 4, 256), (3, 20, 5, 48), (2, 37, 16, 45), (1, 70, 11, 130), (2, 16, 16, 14),
+          (2, 12, 64, 70), (2, 9, 24, 33), (1, 21, 40, 50)]          # more than 16 states: 4, 2 and 4 (3 padded) blocks per channel
 
 
 @pytest.mark.parametrize("shape", SHAPES)
@@ -138,10 +139,10 @@ def test_fused_matches_composite_at_training_shape():
 
 
 def test_shapes_beyond_the_fused_kernels_take_the_composite_route():
-    """n > 16: the dispatcher operators still answer (through the core scan), forward and backward."""
+    """n > 64: the dispatcher operators still answer (through the core scan), forward and backward."""
     from aussm_amd import ops
-    b, d, n, l = 2, 8, 24, 40
-    assert not ops.fused_supported(b, d, n, l) and ops.fused_supported(b, d, 16, l)
+    b, d, n, l = 2, 8, 72, 40
+    assert not ops.fused_supported(b, d, n, l) and ops.fused_supported(b, d, 64, l)
     args = _inputs(b, d, n, l, seed=6, xscale=d ** -0.5)
     leaves = [a.clone().requires_grad_(True) for a in args]
     y, hr, hi = O.adaptive_unitary_op_loop(*leaves)
