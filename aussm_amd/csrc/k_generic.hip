@@ -60,15 +60,25 @@ int run_unitary_bwd_generic(const UniBwdArgs& a, int in_dtype, Cfg c, hipStream_
 #define AUSSM_RBWD_CASE(NW_)                                                                         \
   if (nw == NW_) {                                                                                   \
     hipLaunchKernelGGL((recompute_bwd_kernel<VAR, NW_, 256, Tin>), grid, dim3(256), 0, s, a);        \
-    return launch_status();                                                                          \
+    done = true;                                                                                     \
   }
 
 template <int VAR, typename Tin>
-static int rec_bwd_t(const RecBwdArgs& a, hipStream_t s) {
-  const dim3 grid((unsigned)(a.B * a.ncg));
-  const int nw = a.N <= 4 ? 1 : (a.N <= 8 ? 2 : 4);
-  AUSSM_RBWD_CASE(1) AUSSM_RBWD_CASE(2) AUSSM_RBWD_CASE(4)
-  return -2;
+static int rec_bwd_t(const RecBwdArgs& args, hipStream_t s) {
+  const dim3 grid((unsigned)(args.B * args.ncg));
+  // one launch per block of 16 states (stream order makes the later blocks' additions safe)
+  for (int nbase = 0; nbase < args.N; nbase += 16) {
+    RecBwdArgs a = args;
+    a.nbase = nbase;
+    a.accum = nbase > 0;
+    const int left = args.N - nbase;
+    const int nw = left <= 4 ? 1 : (left <= 8 ? 2 : 4);
+    bool done = false;
+    AUSSM_RBWD_CASE(1) AUSSM_RBWD_CASE(2) AUSSM_RBWD_CASE(4)
+    if (!done) return -2;
+    if (int e = launch_status()) return e;
+  }
+  return 0;
 }
 
 int run_rec_bwd(int variant, const RecBwdArgs& a, int in_dtype, hipStream_t s) {

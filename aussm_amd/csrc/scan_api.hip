@@ -45,7 +45,6 @@ inline int check_common(int B, int D, int N, int L, int ck, int in_dtype) {
 
 // The recomputing backward kernels (complex, real) keep a tile of states in registers: four
 // wavefronts of at most four states each.
-constexpr int REC_MAX_STATE = 16;
 constexpr int REC_CK = AUSSM_TILE / 2;
 
 inline bool misaligned(const void* p, size_t a) { return p && (reinterpret_cast<uintptr_t>(p) % a) != 0; }
@@ -410,7 +409,6 @@ int aussm_complex_bwd(const float* dy, const float* dhL, const void* u, const vo
                       int B, int D, int N, int L, int ck, int in_dtype, void* stream) {
   if (int e = check_common(B, D, N, L, ck, in_dtype)) return e;
   if (ck != REC_CK) return AUSSM_E_CK;
-  if (N > REC_MAX_STATE) return AUSSM_E_SHAPE;
   if (!dy || !u || !delta || !rho || !theta || !Bc || !Cc || !hck || !du || !ddelta || !drho || !dtheta ||
       !dB || !dC)
     return AUSSM_E_NULL;
@@ -431,7 +429,6 @@ int aussm_real_bwd(const float* dy, const float* dhL, const void* u, const void*
                    int B, int D, int N, int L, int ck, int in_dtype, void* stream) {
   if (int e = check_common(B, D, N, L, ck, in_dtype)) return e;
   if (ck != REC_CK) return AUSSM_E_CK;
-  if (N > REC_MAX_STATE) return AUSSM_E_SHAPE;
   if (!dy || !u || !delta || !A || !Bm || !Cm || !hck || !du || !ddelta || !dB || !dC) return AUSSM_E_NULL;
   RecBwdArgs a{};
   a.dy = dy; a.dhL = dhL; a.u = u; a.delta = delta; a.A = A; a.Bm = Bm; a.Cm = Cm; a.Dskip = Dskip;

@@ -87,6 +87,11 @@ struct RecBwdArgs {
   float* dD;                // [D] or null, accumulated into
   float* dh0;               // [B,D,N,C] or null
   int B, D, N, L, nck, ncg, delta_softplus;
+  // A launch handles the states nbase .. nbase + 15 (a workgroup's four wavefronts of up to four states);
+  // larger N takes one launch per block of 16 states.  accum: a later block - the sums over the states
+  // (du, ddelta, dtheta, drho) are added to what the earlier blocks wrote, and the terms that do not
+  // depend on the state (the D skip, dD) are left out.
+  int nbase, accum;
 };
 
 struct SegArgs {

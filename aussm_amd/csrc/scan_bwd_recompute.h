@@ -85,9 +85,9 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
   const int wg = xcd_remap(blockIdx.x, gridDim.x);
   const int b = wg / p.ncg, d0 = (wg % p.ncg) * CH;
   const int N = p.N, L = p.L, D = p.D;
-  const int n0 = wave * NW;
+  const int n0 = p.nbase + wave * NW;
   const bool active = n0 < N;
-  const int nwa = (N + NW - 1) / NW;
+  const int nwa = (N - p.nbase + NW - 1) / NW;         // wavefronts of this launch that own existing states
   const int d = d0 + lane;
   const bool dok = d < D;
 
@@ -400,15 +400,16 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
       for (int w = 0; w < NWV; ++w) { kk += pv[k][w].x; xx += pv[k][w].y; zz += pv[k][w].z; }
       if (rowok[k] && ll < L) {
         const size_t o = goff[k] + ll;
-        p.du[o] = fmaf(kk, edl[k], dsk[k] * egy[k]);
+        const bool acc = p.accum != 0;                   // uniform
+        p.du[o] = acc ? fmaf(kk, edl[k], p.du[o]) : fmaf(kk, edl[k], dsk[k] * egy[k]);
         if (VAR == VAR_REAL) {
           float dd = fmaf(kk, eu[k], xx);
           if (p.delta_softplus) dd *= (eraw[k] > 20.0f) ? 1.0f : sigmoidf_(eraw[k]);
-          p.ddelta[o] = dd;
+          p.ddelta[o] = acc ? p.ddelta[o] + dd : dd;
         } else {
-          p.ddelta[o] = kk * eu[k];
-          p.dtheta[o] = xx;
-          p.drho[o] = zz;
+          p.ddelta[o] = acc ? fmaf(kk, eu[k], p.ddelta[o]) : kk * eu[k];
+          p.dtheta[o] = acc ? p.dtheta[o] + xx : xx;
+          p.drho[o] = acc ? p.drho[o] + zz : zz;
         }
         accD[k] = fmaf(egy[k], eu[k], accD[k]);
       }
@@ -430,7 +431,7 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
       }
     }
   }
-  if (p.dD) {
+  if (p.dD && !p.accum) {
 #pragma unroll
     for (int k = 0; k < E; ++k) {
       float s = accD[k];

@@ -250,7 +250,7 @@ def unitary_scan(u: Tensor, delta: Tensor, theta: Tensor, Bc: Tensor, Cc: Tensor
 # --------------------------------------------------------------------------------------------
 
 REC_CK = 16          # checkpoint interval the recomputing backward kernels (complex, real) need
-REC_MAX_STATE = 16   # largest state size those kernels take
+REC_MAX_STATE = _lib.MAX_STATE   # largest state size those kernels take (16 states per launch, one launch per block)
 
 
 def complex_fwd_raw(u, delta, rho, theta, Bri, Cri, D=None, z=None, h0=None, want_state=False, ck=0):

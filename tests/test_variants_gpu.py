@@ -28,6 +28,9 @@ SHAPES = [
     (2, 128, 1, 33),
     (1, 40, 16, 16),
     (1, 33, 2, 17),
+    (2, 40, 64, 50),          # more than 16 states: the backward pass takes one launch per block of 16
+    (1, 70, 24, 33),
+    (2, 20, 37, 40),
 ]
 
 
@@ -135,13 +138,12 @@ def test_real_gradients(B, D, N, L, softplus, gate):
         _close(got[k], want[k], f"d{k}")
 
 
-def test_backward_state_limit():
+def test_state_limit():
+    """64 states per channel is the limit of both directions (AUSSM_MAX_STATE)."""
     from aussm_amd import scan
-    p = {k: v.cuda() for k, v in O.make_core_inputs(1, 8, 32, 16, variant="real").items()}
-    y = scan.selective_scan_fn(p["u"], p["delta"], p["A"], p["Bm"], p["Cm"])          # forward is fine
-    assert y.shape == (1, 8, 16)
+    p = {k: v.cuda() for k, v in O.make_core_inputs(1, 8, 65, 16, variant="real").items()}
     with pytest.raises(RuntimeError):
-        scan.selective_scan_fn(p["u"].requires_grad_(True), p["delta"], p["A"], p["Bm"], p["Cm"])
+        scan.selective_scan_fn(p["u"], p["delta"], p["A"], p["Bm"], p["Cm"])
 
 
 @pytest.mark.parametrize("seed", range(20))
