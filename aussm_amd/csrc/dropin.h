@@ -467,10 +467,12 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DROPIN_
   }
 }
 
-// p[i] = src ? src[i] : 0
-__global__ __launch_bounds__(256) void fill_kernel(float* __restrict__ p, const float* __restrict__ src, size_t n) {
-  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-  if (i < n) p[i] = src ? src[i] : 0.0f;
+// Several small buffers set in one launch (blockIdx.y picks the buffer): dst[i] = src ? src[i] : 0.
+__global__ __launch_bounds__(256) void fill_kernel(const FillArgs a) {
+  float* __restrict__ dst = a.dst[blockIdx.y];
+  const float* __restrict__ src = a.src[blockIdx.y];
+  const size_t n = a.n[blockIdx.y];
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) dst[i] = src ? src[i] : 0.0f;
 }
 
 // ---- fp32-accurate GEMM on the bf16 matrix cores, operands in fp32 with arbitrary strides -------
@@ -504,8 +506,11 @@ __global__ __launch_bounds__(256) void split_gemm_kernel(const GemmArgs p) {
   const int ra = K1 ? tid >> 2 : wave * 16 + (lane & 15);
   const int kq = 8 * (K1 ? tid & 3 : lane >> 4);
   const int ma = m0 + ra, mb = ma + 64, nb = n0 + ra;
-  // ... and where they go in LDS: [16-row tile][piece][lane = 16 (kq / 8) + row % 16]
-  const int slot = (ra >> 4) * 192 + (kq >> 3) * 16 + (ra & 15);
+  // ... and where they go in LDS: [16-row tile][piece][16 g + (row + 4 g) % 16], g = kq / 8.  The rotation by
+  // 4 g keeps the 16-byte writes of the K1 mapping (four neighbouring lanes = the four g of one row) and the
+  // reads (16 neighbouring lanes = 16 rows of one g) both free of bank conflicts.
+  const int slot = (ra >> 4) * 192 + (kq >> 3) * 16 + ((ra + (kq >> 1)) & 15);
+  const int rslot = (lane & 48) + ((lane + (lane >> 4) * 4) & 15);       // the record of (row lane % 16, g lane / 16)
   // uniform bases, 32-bit per-thread offsets (a z-slice of either operand is below 2^31 elements)
   const unsigned sak = (unsigned)p.sak, sbk = (unsigned)p.sbk;
   const unsigned oa0 = (unsigned)ma * (unsigned)p.sam + (unsigned)kq * sak;
@@ -572,12 +577,12 @@ __global__ __launch_bounds__(256) void split_gemm_kernel(const GemmArgs p) {
 #pragma unroll
     for (int f = 0; f < 2; ++f)
 #pragma unroll
-      for (int c = 0; c < 3; ++c) rb[f][c] = s_b[((wn + f) * 3 + c) * 64 + lane];
+      for (int c = 0; c < 3; ++c) rb[f][c] = s_b[((wn + f) * 3 + c) * 64 + rslot];
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       u4 rA[3];
 #pragma unroll
-      for (int c = 0; c < 3; ++c) rA[c] = s_a[((wm + e) * 3 + c) * 64 + lane];
+      for (int c = 0; c < 3; ++c) rA[c] = s_a[((wm + e) * 3 + c) * 64 + rslot];
 #pragma unroll
       for (int f = 0; f < 2; ++f) acc[e][f] = xmm<3>(rA, rb[f], acc[e][f]);
     }

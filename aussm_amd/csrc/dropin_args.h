@@ -50,6 +50,14 @@ struct DropinBwdArgs {
   int lc;                  // row length of dth (>= 16 (t1 - t0))
 };
 
+// Up to 12 buffers set in one launch: dst[i] = src ? src[i] : 0 for i < n.
+struct FillArgs {
+  float* dst[12];
+  const float* src[12];
+  unsigned long long n[12];
+  int count;
+};
+
 struct GemmArgs {
   const float* A; const float* Bm; float* C;
   long sam, sak, saz;     // element strides of A over m, k, z

@@ -9,8 +9,13 @@ void run_dropin_xprep(const float* x, u4* xp, int d, int n, int ks, int nb, hipS
   hipLaunchKernelGGL(dropin_xprep_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, x, xp, d, n, ks, nb);
 }
 
-void run_fill(float* p, const float* src, size_t n, hipStream_t s) {
-  if (n) hipLaunchKernelGGL(fill_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, p, src, n);
+void run_fill(const FillArgs& a, hipStream_t s) {
+  size_t most = 0;
+  for (int i = 0; i < a.count; ++i) most = a.n[i] > most ? a.n[i] : most;
+  if (!a.count || !most) return;
+  size_t blocks = (most + 255) / 256;
+  if (blocks > 4096) blocks = 4096;
+  hipLaunchKernelGGL(fill_kernel, dim3((unsigned)blocks, (unsigned)a.count), dim3(256), 0, s, a);
 }
 
 #ifndef DROPIN_NW_

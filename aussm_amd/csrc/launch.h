@@ -45,7 +45,7 @@ void run_dropin_xprep(const float* x, u4* xp, int d, int n, int ks, int nb, hipS
 int dropin_channels_per_workgroup(int ks);
 int run_dropin_fwd(const DropinArgs& a, hipStream_t s);
 int run_dropin_bwd(const DropinBwdArgs& a, hipStream_t s);
-void run_fill(float* p, const float* src, size_t n, hipStream_t s);   // p[i] = src ? src[i] : 0
+void run_fill(const FillArgs& a, hipStream_t s);   // several buffers set (zero or a copy) in one launch
 int run_split_gemm(const GemmArgs& a, hipStream_t s);
 
 }  // namespace aussm

@@ -582,22 +582,27 @@ int aussm_ssm_adaptive_unitary_bwd(const float* grad_y, const float* grad_nh_re,
   float* dth = hc_im + round4(nstate);
   run_dropin_xprep(x, xp, d, n, ks, nb, s);
   DropinArgs f{u, dt, z, x_bias, B_r, B_theta, C_r, C_theta, D, h_re, h_im, nullptr, hc_re, hc_im, xp, b, d, n, L, ks, nb};
+  FillArgs fa{};
+  auto fill = [&](float* dst, const float* src, size_t cnt) {
+    fa.dst[fa.count] = dst; fa.src[fa.count] = src; fa.n[fa.count] = cnt; ++fa.count;
+  };
   if (nh_re && nh_im) {
-    run_fill(hc_re, nh_re, nstate, s);
-    run_fill(hc_im, nh_im, nstate, s);
+    fill(hc_re, nh_re, nstate);
+    fill(hc_im, nh_im, nstate);
   } else {
     // the state at the end of the sequence: one forward sweep without outputs
     if (int e = run_dropin_fwd(f, s)) return e;
   }
-  run_fill(dh_re, grad_nh_re, nstate, s);           // the adjoint of the state travels in the output buffers
-  run_fill(dh_im, grad_nh_im, nstate, s);
-  run_fill(dx, nullptr, (size_t)d * n * d, s);
-  run_fill(dx_bias, nullptr, (size_t)d * n, s);
-  run_fill(dB_r, nullptr, n, s);
-  run_fill(dB_theta, nullptr, n, s);
-  run_fill(dC_r, nullptr, n, s);
-  run_fill(dC_theta, nullptr, n, s);
-  run_fill(dD, nullptr, d, s);
+  fill(dh_re, grad_nh_re, nstate);                  // the adjoint of the state travels in the output buffers
+  fill(dh_im, grad_nh_im, nstate);
+  fill(dx, nullptr, (size_t)d * n * d);
+  fill(dx_bias, nullptr, (size_t)d * n);
+  fill(dB_r, nullptr, n);
+  fill(dB_theta, nullptr, n);
+  fill(dC_r, nullptr, n);
+  fill(dC_theta, nullptr, n);
+  fill(dD, nullptr, d);
+  run_fill(fa, s);
   const long dn = (long)d * n;
   for (int b0 = 0; b0 < b; b0 += blk.bg)
   for (int t1 = ntiles; t1 > 0; t1 -= ct) {

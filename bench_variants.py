@@ -14,7 +14,8 @@ With --scaling it runs the protocol of the reference's sweep, extension-cpp/test
 instead: for each system and each sequence length (20 log-spaced points in [10, 2048] as there, plus
 4096 and 16384), 5 warm-up and --runs timed repetitions of the operator's forward pass and of
 `y.sum().backward()`, device time of each (HIP events on the launch stream) and peak device memory after
-each (torch.cuda.max_memory_allocated, reset before every repetition).  Systems (the reference's are
+each (torch.cuda.max_memory_allocated, reset before every repetition; `inputs_MB` is what was allocated at
+that moment, i.e. the point's inputs).  Systems (the reference's are
 "mamba", "SSMau-cuda", "SSMau-pytorch", :193-216): "SSMau-hip" = ssm_adaptive_interface on the fused
 kernels, "SSMau-hip-composite" = the same interface on the composite route (phase tensor materialised),
 "mamba-hip" = selective_scan_fn.  Shapes: the reference's default b=16, d=32, n=64 (:259-262) and the training
@@ -64,57 +65,68 @@ def scaling(args):
                [int(v) for v in np.logspace(np.log10(10), np.log10(2048), 20)] + [4096, 16384])
     shapes = [tuple(int(v) for v in s.split(",")) for s in (args.bdn or ["16,32,64", "32,256,16"])]
     systems = args.systems.split(",")
+    def point(system, b, d, n, l):
+        """One (system, shape, length) point; its tensors die with this frame."""
+        g = torch.Generator(device=dev).manual_seed(0)
+        rn = lambda *s: torch.randn(*s, generator=g, device=dev)
+        leaf = lambda t: t.requires_grad_(True)
+        u, dt, z, D = leaf(rn(b, d, l)), leaf(rn(b, d, l)), leaf(rn(b, d, l)), leaf(rn(d))
+        if system == "mamba-hip":
+            A, Bm, Cm = leaf(-torch.exp(rn(d, n))), leaf(rn(b, n, l)), leaf(rn(b, n, l))
+            params = [u, dt, A, Bm, Cm, D, z]
+            fn = lambda: scan.selective_scan_fn(u, dt, A, Bm, Cm, D, z=z, delta_softplus=True)
+        else:
+            x, xb = leaf(rn(d, n, d) * d ** -0.5), leaf(rn(d, n))
+            Bp, Cp = leaf(torch.complex(rn(n), rn(n))), leaf(torch.complex(rn(n), rn(n)))
+            params = [u, dt, x, xb, Bp, Cp, D, z]
+            save = system == "SSMau-hip-composite"
+            fn = lambda: ops.ssm_adaptive_interface(u, dt, x, xb, Bp, Cp, D, z, unitary=True, save_intermediates=save)
+        tf = tb = mf = mb = 0.0
+        ev = lambda: torch.cuda.Event(enable_timing=True)
+        for run in range(args.runs + 5):
+            for t in params:
+                t.grad = None
+            torch.cuda.synchronize()
+            torch.cuda.reset_peak_memory_stats()
+            base = torch.cuda.memory_allocated()          # the inputs (and nothing else of this point)
+            e0, e1, e2 = ev(), ev(), ev()
+            e0.record()
+            y = fn()
+            e1.record()
+            mem_f = torch.cuda.max_memory_allocated()
+            y.sum().backward()
+            e2.record()
+            torch.cuda.synchronize()
+            if run >= 5:
+                tf += e0.elapsed_time(e1)
+                tb += e1.elapsed_time(e2)
+                mf += mem_f
+                mb += torch.cuda.max_memory_allocated()
+            del y
+        r = args.runs
+        return {"system": system, "b": b, "d": d, "n": n, "L": l, "runs": r,
+                "fwd_us": round(tf / r * 1e3, 1), "bwd_us": round(tb / r * 1e3, 1),
+                "inputs_MB": round(base * 1e-6, 2),
+                "fwd_peak_MB": round(mf / r * 1e-6, 2), "bwd_peak_MB": round(mb / r * 1e-6, 2)}
+
+    import gc
+    import time
+    # the clocks of the part ramp up over tens of milliseconds of load: the first points would read slow
+    warm = torch.randn(4096, 4096, device=dev)
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < 0.3:
+        warm = torch.mm(warm, warm).clamp_(-1, 1)
+        torch.cuda.synchronize()
+    del warm
     for b, d, n in shapes:
         for system in systems:
             for l in lengths:
-                g = torch.Generator(device=dev).manual_seed(0)
-                rn = lambda *s: torch.randn(*s, generator=g, device=dev)
-                leaf = lambda t: t.requires_grad_(True)
-                u, dt, z, D = leaf(rn(b, d, l)), leaf(rn(b, d, l)), leaf(rn(b, d, l)), leaf(rn(d))
-                if system == "mamba-hip":
-                    A, Bm, Cm = leaf(-torch.exp(rn(d, n))), leaf(rn(b, n, l)), leaf(rn(b, n, l))
-                    params = [u, dt, A, Bm, Cm, D, z]
-                    fn = lambda: scan.selective_scan_fn(u, dt, A, Bm, Cm, D, z=z, delta_softplus=True)
-                else:
-                    x, xb = leaf(rn(d, n, d) * d ** -0.5), leaf(rn(d, n))
-                    Bp, Cp = leaf(torch.complex(rn(n), rn(n))), leaf(torch.complex(rn(n), rn(n)))
-                    params = [u, dt, x, xb, Bp, Cp, D, z]
-                    save = system == "SSMau-hip-composite"
-                    fn = lambda: ops.ssm_adaptive_interface(u, dt, x, xb, Bp, Cp, D, z, unitary=True,
-                                                            save_intermediates=save)
-                tf = tb = mf = mb = 0.0
-                ev = lambda: torch.cuda.Event(enable_timing=True)
                 try:
-                    for run in range(args.runs + 5):
-                        for t in params:
-                            t.grad = None
-                        torch.cuda.synchronize()
-                        torch.cuda.reset_peak_memory_stats()
-                        e0, e1, e2 = ev(), ev(), ev()
-                        e0.record()
-                        y = fn()
-                        e1.record()
-                        mem_f = torch.cuda.max_memory_allocated()
-                        y.sum().backward()
-                        e2.record()
-                        torch.cuda.synchronize()
-                        if run >= 5:
-                            tf += e0.elapsed_time(e1)
-                            tb += e1.elapsed_time(e2)
-                            mf += mem_f
-                            mb += torch.cuda.max_memory_allocated()
-                        del y
-                except RuntimeError as e:           # out of memory, or a shape an operator does not take
-                    print(json.dumps({"system": system, "b": b, "d": d, "n": n, "L": l,
-                                      "error": str(e).split("\n")[0][:160]}), flush=True)
-                    torch.cuda.empty_cache()
-                    continue
-                r = args.runs
-                print(json.dumps({"system": system, "b": b, "d": d, "n": n, "L": l, "runs": r,
-                                  "fwd_us": round(tf / r * 1e3, 1), "bwd_us": round(tb / r * 1e3, 1),
-                                  "fwd_peak_MB": round(mf / r * 1e-6, 2), "bwd_peak_MB": round(mb / r * 1e-6, 2)}),
-                      flush=True)
-                del params, u, dt, z, D
+                    rec = point(system, b, d, n, l)
+                except RuntimeError as e:               # out of memory, or a shape an operator does not take
+                    rec = {"system": system, "b": b, "d": d, "n": n, "L": l, "error": str(e).split("\n")[0][:160]}
+                print(json.dumps(rec), flush=True)
+                gc.collect()
                 torch.cuda.empty_cache()
 
 
