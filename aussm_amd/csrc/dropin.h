@@ -485,7 +485,7 @@ __global__ __launch_bounds__(256) void fill_kernel(const FillArgs a) {
 // they are staged in LDS; the values of the next step are requested before the products of the
 // current one.
 // K1: both operands are contiguous along k.  Then four neighbouring lanes fetch the 32 values of
-// one row as 16-byte vectors (VEC: every row start is 16-byte aligned) - a wavefront request covers 16
+// one row as 16-byte vectors (VEC; rows need not be 16-byte aligned) - a wavefront request covers 16
 // cache lines.  Otherwise both are contiguous along m / n and a 16-lane row of the wavefront
 // fetches 16 neighbouring rows' values of one k.
 template <bool K1, bool VEC>
@@ -528,11 +528,14 @@ __global__ __launch_bounds__(256) void split_gemm_kernel(const GemmArgs p) {
     const unsigned ka = (unsigned)(it * 32) * sak, kb = (unsigned)(it * 32) * sbk;
     if (inside && it * 32 + 32 <= p.K) {
       if constexpr (K1 && VEC) {
+        // 16-byte loads that are only known to be 4-byte aligned (rows start anywhere when the row length is
+        // not a multiple of four): the memory pipeline takes them, the type tells the compiler so
+        typedef float f4u __attribute__((ext_vector_type(4), aligned(4)));
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
-          const f4 x0 = *reinterpret_cast<const f4*>(Az + (oa0 + ka + 4 * h));
-          const f4 x1 = *reinterpret_cast<const f4*>(Az + (oa1 + ka + 4 * h));
-          const f4 x2 = *reinterpret_cast<const f4*>(Bz + (ob0 + kb + 4 * h));
+          const f4u x0 = *reinterpret_cast<const f4u*>(Az + (oa0 + ka + 4 * h));
+          const f4u x1 = *reinterpret_cast<const f4u*>(Az + (oa1 + ka + 4 * h));
+          const f4u x2 = *reinterpret_cast<const f4u*>(Bz + (ob0 + kb + 4 * h));
 #pragma unroll
           for (int c = 0; c < 4; ++c) {
             va[0][4 * h + c] = x0[c];

@@ -63,10 +63,7 @@ int run_split_gemm(const GemmArgs& a, hipStream_t s) {
   if (gz > 65535) return -2;
   const dim3 grid((unsigned)((a.M + 127) / 128), (unsigned)((a.N + 63) / 64), (unsigned)gz);
   const bool k1 = a.sak == 1 && a.sbk == 1;
-  const bool vec = k1 && a.sam % 4 == 0 && a.sbn % 4 == 0 && a.saz % 4 == 0 && a.sbz % 4 == 0 &&
-                   (reinterpret_cast<uintptr_t>(a.A) | reinterpret_cast<uintptr_t>(a.Bm)) % 16 == 0;
-  if (k1 && vec) hipLaunchKernelGGL((split_gemm_kernel<true, true>), grid, dim3(256), 0, s, a);
-  else if (k1) hipLaunchKernelGGL((split_gemm_kernel<true, false>), grid, dim3(256), 0, s, a);
+  if (k1) hipLaunchKernelGGL((split_gemm_kernel<true, true>), grid, dim3(256), 0, s, a);
   else hipLaunchKernelGGL((split_gemm_kernel<false, false>), grid, dim3(256), 0, s, a);
   return launch_status();
 }
