@@ -92,13 +92,15 @@ __device__ __forceinline__ void stage_load(const float* __restrict__ ub, float (
     }
   }
 }
-template <int NT, int NREC>
-__device__ __forceinline__ void stage_store(const float (&v)[NREC][8], u4* __restrict__ dst, int ks, int tid, const SplitK& sk) {
+// (all KS steps the kernel was compiled for are written, the ones past ceil(d / 32) as zeros, so that the
+// kernel's product loop needs no run-time bound)
+template <int NT, int NREC, int KS>
+__device__ __forceinline__ void stage_store(const float (&v)[NREC][8], u4* __restrict__ dst, int tid, const SplitK& sk) {
 #pragma unroll
   for (int e = 0; e < NREC; ++e) {
     const int rec = tid + e * NT;
     const int lane = rec & 63, k = rec >> 6;
-    if (k < ks) {
+    if (k < KS) {
       u4 pc[3];
       split8<3>(sk, v[e], pc);
 #pragma unroll
@@ -157,7 +159,7 @@ __global__ __launch_bounds__(NW * 64) void dropin_fwd_kernel(const DropinArgs p)
   constexpr int NT = NW * 64, NREC = (KS * 64 + NT - 1) / NT;
   float sv[NREC][8];
   stage_load<NT, NREC>(ub, sv, d, L, p.ks, 0, tid);
-  stage_store<NT, NREC>(sv, s_u[0], p.ks, tid, sk);
+  stage_store<NT, NREC, KS>(sv, s_u[0], tid, sk);
   __syncthreads();
   // the wavefront's own inputs, requested one tile ahead
   float un = l_ < L ? p.u[row + l_] : 0.0f, dtn = l_ < L ? p.dt[row + l_] : 0.0f, zn = l_ < L ? p.z[row + l_] : 0.0f;
@@ -177,12 +179,10 @@ __global__ __launch_bounds__(NW * 64) void dropin_fwd_kernel(const DropinArgs p)
     const u4* su = s_u[t & 1];
 #pragma unroll
     for (int k = 0; k < KS; ++k) {
-      if (k < p.ks) {
-        u4 ubk[3];
+      u4 ubk[3];
 #pragma unroll
-        for (int q = 0; q < 3; ++q) ubk[q] = su[(k * 3 + q) * 64 + lane];
-        th = xmm<3>(xa[k], ubk, th);
-      }
+      for (int q = 0; q < 3; ++q) ubk[q] = su[(k * 3 + q) * 64 + lane];
+      th = xmm<3>(xa[k], ubk, th);
     }
     const float ut = siluf_(uv), w = dtv * ut;
     float ysum = 0.0f;
@@ -208,7 +208,7 @@ __global__ __launch_bounds__(NW * 64) void dropin_fwd_kernel(const DropinArgs p)
     } else if (g == 0) {
       s_y[t & 1][wave][l_] = ysum;
     }
-    if (t + 1 < ntiles) stage_store<NT, NREC>(sv, s_u[(t + 1) & 1], p.ks, tid, sk);
+    if (t + 1 < ntiles) stage_store<NT, NREC, KS>(sv, s_u[(t + 1) & 1], tid, sk);
     __syncthreads();
     if (nb > 1 && sb == 0 && g == 0 && p.y && iok && lok) {      // the channel's first wavefront adds the shares up
       float tot = ysum;
@@ -317,7 +317,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DROPIN_
   constexpr int NT = NW * 64, NREC = (KS * 64 + NT - 1) / NT;
   float sv[NREC][8];
   stage_load<NT, NREC>(ub, sv, d, L, p.ks, t_last * DT, tid);
-  stage_store<NT, NREC>(sv, s_u[t_last & 1], p.ks, tid, sk);
+  stage_store<NT, NREC, KS>(sv, s_u[t_last & 1], tid, sk);
   __syncthreads();
   // the wavefront's own inputs, requested one tile ahead
   float un, dtn, zn, gyn;
@@ -344,12 +344,10 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DROPIN_
     const u4* su = s_u[t & 1];
 #pragma unroll
     for (int k = 0; k < KS; ++k) {
-      if (k < p.ks) {
-        u4 ubk[3];
+      u4 ubk[3];
 #pragma unroll
-        for (int c = 0; c < 3; ++c) ubk[c] = su[(k * 3 + c) * 64 + lane];
-        th = xmm<3>(xa[k], ubk, th);
-      }
+      for (int c = 0; c < 3; ++c) ubk[c] = su[(k * 3 + c) * 64 + lane];
+      th = xmm<3>(xa[k], ubk, th);
     }
     const float ut = siluf_(uv), w = dtv * ut, sz = siluf_(zv), av = gyv * sz;
     float ysum = 0.0f, wsum = 0.0f;
@@ -402,7 +400,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DROPIN_
     wsum += __shfl_xor(wsum, 16);
     wsum += __shfl_xor(wsum, 32);
     if (nb > 1 && g == 0) s_yw[t & 1][wave][l_] = make_float2(ysum, wsum);
-    if (t > t_first) stage_store<NT, NREC>(sv, s_u[(t - 1) & 1], p.ks, tid, sk);
+    if (t > t_first) stage_store<NT, NREC, KS>(sv, s_u[(t - 1) & 1], tid, sk);
     if (nb > 1) {                                      // the channel's first wavefront adds the shares up
       __syncthreads();
       for (int k = 1; k < nb; ++k) {

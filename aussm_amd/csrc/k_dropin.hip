@@ -39,21 +39,24 @@ static void launch_bwd(const DropinBwdArgs& a, hipStream_t s) {
 
 int dropin_channels_per_workgroup(int ks) { return ks > 8 ? 4 : DROPIN_NW; }
 
+// compiled sizes of the contraction over r, in steps of 32: the smallest one >= ceil(d / 32) runs
+#define DROPIN_KS_DISPATCH(LAUNCH, ks)          \
+  if (ks <= 1) LAUNCH<1>(a, s);                 \
+  else if (ks <= 2) LAUNCH<2>(a, s);            \
+  else if (ks <= 3) LAUNCH<3>(a, s);            \
+  else if (ks <= 4) LAUNCH<4>(a, s);            \
+  else if (ks <= 6) LAUNCH<6>(a, s);            \
+  else if (ks <= 8) LAUNCH<8>(a, s);            \
+  else if (ks <= 12) LAUNCH<12>(a, s);          \
+  else LAUNCH<16>(a, s);
+
 int run_dropin_fwd(const DropinArgs& a, hipStream_t s) {
-  if (a.ks <= 1) launch_fwd<1>(a, s);
-  else if (a.ks <= 2) launch_fwd<2>(a, s);
-  else if (a.ks <= 4) launch_fwd<4>(a, s);
-  else if (a.ks <= 8) launch_fwd<8>(a, s);
-  else launch_fwd<16>(a, s);
+  DROPIN_KS_DISPATCH(launch_fwd, a.ks)
   return launch_status();
 }
 
 int run_dropin_bwd(const DropinBwdArgs& a, hipStream_t s) {
-  if (a.f.ks <= 1) launch_bwd<1>(a, s);
-  else if (a.f.ks <= 2) launch_bwd<2>(a, s);
-  else if (a.f.ks <= 4) launch_bwd<4>(a, s);
-  else if (a.f.ks <= 8) launch_bwd<8>(a, s);
-  else launch_bwd<16>(a, s);
+  DROPIN_KS_DISPATCH(launch_bwd, a.f.ks)
   return launch_status();
 }
 
