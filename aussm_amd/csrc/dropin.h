@@ -29,6 +29,16 @@
 namespace aussm {
 
 
+// sin and cos of any argument without a branch: reduction by 2 pi in two fused steps (the result is as exact
+// as the fp32 argument itself), then the polynomial kernel for small arguments.  A branch here would cut the
+// four state groups of a lane into separate blocks that the scheduler cannot interleave.
+__device__ __forceinline__ void sincos_any(float x, float* sn, float* cs) {
+  const float k = rintf(x * 0.15915494309189535f);
+  float r = fmaf(-k, 6.2831854820251465f, x);
+  r = fmaf(-k, -1.7484555e-07f, r);
+  sincos_small(r, sn, cs);
+}
+
 // ---- prefix / suffix sums along a row of 16 lanes
 template <int CTRL>
 __device__ __forceinline__ float dpp_mov0(float v) {   // lanes that have no source read 0
@@ -191,7 +201,7 @@ __global__ __launch_bounds__(NW * 64) void dropin_fwd_kernel(const DropinArgs p)
       const float thv = lok ? th[a] + xb[a] : 0.0f;
       const float G = row_prefix(thv);
       float sn, cs;
-      fast_sincosf(G, &sn, &cs);
+      sincos_any(G, &sn, &cs);
       // p = conj(E) Bt w
       const float pr = (cs * btr[a] + sn * bti[a]) * w, pi = (cs * bti[a] - sn * btr[a]) * w;
       const float Rr = hr[a] + row_prefix(pr), Ri = hi[a] + row_prefix(pi);
@@ -358,7 +368,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DROPIN_
       const float thv = lok ? th[a] + s_xb[wave][4 * g + a] : 0.0f;
       const float G = row_prefix(thv);
       float sn, cs;
-      fast_sincosf(G, &sn, &cs);
+      sincos_any(G, &sn, &cs);
       const float csl = row_last(cs, lane), snl = row_last(sn, lane);
       // forward quantities of the tile from the state at its end
       const float pr = (cs * btr_ + sn * bti_) * w, pi = (cs * bti_ - sn * btr_) * w;
