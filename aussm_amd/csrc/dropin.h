@@ -9,17 +9,17 @@
 // The phase tensor theta[b,i,j,l] (n times the size of every other tensor) never exists in memory.
 // A wavefront owns one (batch, channel) pair - with more than 16 states per channel, one block of 16
 // states of it - and walks the sequence in tiles of 16 timesteps:
-//   * the tile's phases, a (16 states) x (16 timesteps) block, are one small matrix product
-//     x[i] (16 x d) . u[b][:, tile] (d x 16) on the bf16 matrix cores with both operands split exactly
-//     into three bf16 pieces (scan_fwd_xdl.h), i.e. fp32-accurate.  The wavefront keeps its rows of x
-//     in registers for the whole sequence; the tile of u, which all wavefronts of the workgroup
-//     share, is split and staged in LDS once per workgroup;
-//   * the result lands with the timestep along the lanes of a 16-lane row (lane = (timestep l,
-//     state group g), states 4 g .. 4 g + 3 in registers), so the recurrence becomes two prefix sums
-//     along the row (DPP row shifts, no LDS): G = prefix(theta), E = e^{iG}, p = conj(E) Bt w,
-//     R = h_in + prefix(p), h = E R.  This is the cumulative-sum form the reference itself uses
-//     (:122-162), tile by tile, with the state h handed from tile to tile - so G restarts at every
-//     tile and stays small;
+//   * the tile's RUNNING phases G = prefix(theta), a (16 states) x (16 timesteps) block, are one small matrix
+//     product x[i] (16 x d) . U (d x 16) on the bf16 matrix cores with both operands split exactly into
+//     three bf16 pieces (scan_fwd_xdl.h), i.e. fp32-accurate, where U is the tile of u[b] prefix-summed along
+//     the tile (sum_{l' <= l} x.u_{l'} = x.U_l), plus (l + 1) x_bias.  The wavefront keeps its rows of x in
+//     registers for the whole launch; the tiles of U, which all wavefronts of a batch element share, are
+//     prepared once per call by a pre-pass (dropin_uprep_kernel) and copied into LDS once per workgroup;
+//   * the product lands with the timestep along the lanes of a 16-lane row (lane = (timestep l,
+//     state group g), states 4 g .. 4 g + 3 in registers), so the rest of the recurrence is prefix sums
+//     along the row (DPP row shifts, no LDS): E = e^{iG}, p = conj(E) Bt w, R = h_in + prefix(p), h = E R.
+//     This is the cumulative-sum form the reference itself uses (:122-162), tile by tile, with the state h
+//     handed from tile to tile - so G restarts at every tile and stays small;
 //   * one sincos per (state, timestep), the sum over the states inside the wavefront, the gates
 //     and the skip fused into the store.
 #pragma once
@@ -38,6 +38,11 @@ __device__ __forceinline__ void sincos_any(float x, float* sn, float* cs) {
   r = fmaf(-k, -1.7484555e-07f, r);
   sincos_small(r, sn, cs);
 }
+
+// silu and its derivative with the hardware reciprocal (1 ulp) instead of an IEEE division (ten instructions)
+__device__ __forceinline__ float sigm_fast(float v) { return __builtin_amdgcn_rcpf(1.0f + __expf(-v)); }
+__device__ __forceinline__ float silu_fast(float v) { return v * sigm_fast(v); }
+__device__ __forceinline__ float dsilu_fast(float v) { const float sg = sigm_fast(v); return sg * (1.0f + v * (1.0f - sg)); }
 
 // ---- prefix / suffix sums along a row of 16 lanes
 template <int CTRL>
@@ -84,38 +89,50 @@ __global__ __launch_bounds__(256) void dropin_xprep_kernel(const float* __restri
   for (int q = 0; q < 3; ++q) xp[(((size_t)vc * ks + k) * 3 + q) * 64 + lane] = pc[q];
 }
 
-// Stage the tile u[b][:, l0 .. l0 + 15] as the second operand of the phase product: record
-// (ks, piece, lane = (column l = lane % 16, g)) holds u[b, 32 ks + 8 g .. + 7, l0 + l].  In two steps so
-// that the loads of the next tile fly while the current one is computed: stage_load requests the
-// values (NREC records of eight per thread), stage_store splits them and writes the records.
-template <int NT, int NREC>
-__device__ __forceinline__ void stage_load(const float* __restrict__ ub, float (&v)[NREC][8], int d, int L, int ks, int l0, int tid) {
-#pragma unroll
-  for (int e = 0; e < NREC; ++e) {
-    const int rec = tid + e * NT;
+// Tiles of u as the second operand of the phase product, prepared once per call (one workgroup of 256
+// threads per (batch element, tile)): record (k, piece, lane = (column l = lane % 16, g)) holds
+// U[32 k + 8 g .. + 7][l], U[r][l] = sum_{l' <= l} u[b, r, l0 + l'] - the prefix sum along the tile - so that
+// the matrix product hands the scan kernels the running phase G = prefix(theta) directly
+// (sum_{l' <= l} sum_r x[i,j,r] u[r,l'] = sum_r x[i,j,r] U[r,l]); timesteps past L count as zero.  All KS steps the
+// kernels are compiled for are written, the ones past ceil(d / 32) as zeros.
+__global__ __launch_bounds__(256) void dropin_uprep_kernel(const float* __restrict__ u, u4* __restrict__ up, int d, int L,
+                                                           int KS, int b0, int t0, int nt) {
+  const int zb = blockIdx.x / nt, t = t0 + blockIdx.x % nt;
+  const float* __restrict__ ub = u + (size_t)(b0 + zb) * d * L;
+  u4* __restrict__ dst = up + (size_t)blockIdx.x * KS * 3 * 64;
+  const SplitK sk = make_splitk();
+  for (int rec = threadIdx.x; rec < KS * 64; rec += 256) {        // (whole wavefronts: 64 records per k)
     const int lane = rec & 63, k = rec >> 6;
-    const int l = l0 + (lane & 15), g = lane >> 4;
+    const int l = t * DT + (lane & 15), g = lane >> 4;
+    float v[8];
 #pragma unroll
     for (int q = 0; q < 8; ++q) {
       const int r = 32 * k + 8 * g + q;
-      v[e][q] = (k < ks && r < d && l < L) ? ub[(size_t)r * L + l] : 0.0f;
+      v[q] = row_prefix((r < d && l < L) ? ub[(size_t)r * L + l] : 0.0f);
     }
+    u4 pc[3];
+    split8<3>(sk, v, pc);
+#pragma unroll
+    for (int q = 0; q < 3; ++q) dst[(k * 3 + q) * 64 + lane] = pc[q];
   }
 }
-// (all KS steps the kernel was compiled for are written, the ones past ceil(d / 32) as zeros, so that the
-// kernel's product loop needs no run-time bound)
+
+// A tile's records, global memory -> registers -> LDS, in two steps so that the loads of the next tile fly
+// while the current one is computed.
 template <int NT, int NREC, int KS>
-__device__ __forceinline__ void stage_store(const float (&v)[NREC][8], u4* __restrict__ dst, int tid, const SplitK& sk) {
+__device__ __forceinline__ void tile_load(const u4* __restrict__ src, u4 (&v)[NREC], int tid) {
 #pragma unroll
   for (int e = 0; e < NREC; ++e) {
     const int rec = tid + e * NT;
-    const int lane = rec & 63, k = rec >> 6;
-    if (k < KS) {
-      u4 pc[3];
-      split8<3>(sk, v[e], pc);
+    if (rec < KS * 3 * 64) v[e] = src[rec];
+  }
+}
+template <int NT, int NREC, int KS>
+__device__ __forceinline__ void tile_store(const u4 (&v)[NREC], u4* __restrict__ dst, int tid) {
 #pragma unroll
-      for (int q = 0; q < 3; ++q) dst[(k * 3 + q) * 64 + lane] = pc[q];
-    }
+  for (int e = 0; e < NREC; ++e) {
+    const int rec = tid + e * NT;
+    if (rec < KS * 3 * 64) dst[rec] = v[e];
   }
 }
 
@@ -128,17 +145,16 @@ __global__ __launch_bounds__(NW * 64) void dropin_fwd_kernel(const DropinArgs p)
   __shared__ float s_y[2][NW][DT];                     // shares of y of the tile, by tile parity (nb > 1)
   const int tid = threadIdx.x, lane = tid & 63, wave = wave_index();
   const int nb = p.nb, ncg = (p.d * nb + NW - 1) / NW;
-  const int b = blockIdx.x / ncg, v = (blockIdx.x % ncg) * NW + wave;
+  const int b = p.b0 + blockIdx.x / ncg, v = (blockIdx.x % ncg) * NW + wave;
   const int i = v / nb, sb = v % nb, j0 = 16 * sb;
   const bool iok = i < p.d;
   const int ic = iok ? i : p.d - 1, vc = ic * nb + sb;
   const int l_ = lane & 15, g = lane >> 4;
   const int d = p.d, n = p.n, L = p.L;
-  const SplitK sk = make_splitk();
-  const float* __restrict__ ub = p.u + (size_t)b * d * L;
   const size_t row = ((size_t)b * d + ic) * L;
+  const u4* __restrict__ upb = p.up + ((size_t)(b - p.up_b0) * p.up_nt - p.up_t0) * (KS * 3 * 64);   // + tile * (KS 3 64)
 
-  // this wavefront's rows of x, split, for the whole sequence
+  // this wavefront's rows of x, split, for the whole launch
   u4 xa[KS][3];
 #pragma unroll
   for (int k = 0; k < KS; ++k)
@@ -164,16 +180,17 @@ __global__ __launch_bounds__(NW * 64) void dropin_fwd_kernel(const DropinArgs p)
     hi[a] = ok ? p.h_im[((size_t)b * d + ic) * n + jc] : 0.0f;
   }
   const float Di = p.Dp[ic];
-  const int ntiles = (L + DT - 1) / DT;
+  const int ntiles = p.t1;
 
-  constexpr int NT = NW * 64, NREC = (KS * 64 + NT - 1) / NT;
-  float sv[NREC][8];
-  stage_load<NT, NREC>(ub, sv, d, L, p.ks, 0, tid);
-  stage_store<NT, NREC, KS>(sv, s_u[0], tid, sk);
+  constexpr int NT = NW * 64, NREC = (KS * 3 * 64 + NT - 1) / NT;
+  u4 sv[NREC];
+  tile_load<NT, NREC, KS>(upb + (size_t)p.t0 * (KS * 3 * 64), sv, tid);
+  tile_store<NT, NREC, KS>(sv, s_u[p.t0 & 1], tid);
   __syncthreads();
   // the wavefront's own inputs, requested one tile ahead
-  float un = l_ < L ? p.u[row + l_] : 0.0f, dtn = l_ < L ? p.dt[row + l_] : 0.0f, zn = l_ < L ? p.z[row + l_] : 0.0f;
-  for (int t = 0; t < ntiles; ++t) {
+  const int lf = p.t0 * DT + l_;
+  float un = lf < L ? p.u[row + lf] : 0.0f, dtn = lf < L ? p.dt[row + lf] : 0.0f, zn = lf < L ? p.z[row + lf] : 0.0f;
+  for (int t = p.t0; t < ntiles; ++t) {
     const int l0 = t * DT, l = l0 + l_;
     const bool lok = l < L;
     const float uv = un, dtv = dtn, zv = zn;
@@ -183,8 +200,8 @@ __global__ __launch_bounds__(NW * 64) void dropin_fwd_kernel(const DropinArgs p)
       dtn = nok ? p.dt[row + l + DT] : 0.0f;
       zn = nok ? p.z[row + l + DT] : 0.0f;
     }
-    if (t + 1 < ntiles) stage_load<NT, NREC>(ub, sv, d, L, p.ks, l0 + DT, tid);
-    // ---- phases of the tile: lane (column l, rows j = 4 g + a)
+    if (t + 1 < ntiles) tile_load<NT, NREC, KS>(upb + (size_t)(t + 1) * (KS * 3 * 64), sv, tid);
+    // ---- running phases of the tile, less the bias: lane (column l, rows j = 4 g + a)
     f4 th = {0, 0, 0, 0};
     const u4* su = s_u[t & 1];
 #pragma unroll
@@ -194,12 +211,12 @@ __global__ __launch_bounds__(NW * 64) void dropin_fwd_kernel(const DropinArgs p)
       for (int q = 0; q < 3; ++q) ubk[q] = su[(k * 3 + q) * 64 + lane];
       th = xmm<3>(xa[k], ubk, th);
     }
-    const float ut = siluf_(uv), w = dtv * ut;
+    const float ut = silu_fast(uv), w = dtv * ut;
+    const float cnt = (float)(min(l_ + 1, L - l0));      // timesteps of the tile up to this one that exist
     float ysum = 0.0f;
 #pragma unroll
     for (int a = 0; a < 4; ++a) {
-      const float thv = lok ? th[a] + xb[a] : 0.0f;
-      const float G = row_prefix(thv);
+      const float G = fmaf(xb[a], cnt, th[a]);
       float sn, cs;
       sincos_any(G, &sn, &cs);
       // p = conj(E) Bt w
@@ -214,16 +231,16 @@ __global__ __launch_bounds__(NW * 64) void dropin_fwd_kernel(const DropinArgs p)
     ysum += __shfl_xor(ysum, 16);
     ysum += __shfl_xor(ysum, 32);
     if (nb == 1) {
-      if (p.y && iok && lok && g == 0) p.y[row + l] = siluf_(zv) * (ysum + Di * ut);
+      if (p.y && iok && lok && g == 0) p.y[row + l] = silu_fast(zv) * (ysum + Di * ut);
     } else if (g == 0) {
       s_y[t & 1][wave][l_] = ysum;
     }
-    if (t + 1 < ntiles) stage_store<NT, NREC, KS>(sv, s_u[(t + 1) & 1], tid, sk);
+    if (t + 1 < ntiles) tile_store<NT, NREC, KS>(sv, s_u[(t + 1) & 1], tid);
     __syncthreads();
     if (nb > 1 && sb == 0 && g == 0 && p.y && iok && lok) {      // the channel's first wavefront adds the shares up
       float tot = ysum;
       for (int k = 1; k < nb; ++k) tot += s_y[t & 1][wave + k][l_];
-      p.y[row + l] = siluf_(zv) * (tot + Di * ut);
+      p.y[row + l] = silu_fast(zv) * (tot + Di * ut);
     }
   }
   if (p.nh_re && iok && l_ == 0) {
@@ -282,9 +299,8 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DROPIN_
   const int ic = iok ? i : p.d - 1, vc = ic * nb + sb;
   const int l_ = lane & 15, g = lane >> 4;
   const int d = p.d, n = p.n, L = p.L;
-  const SplitK sk = make_splitk();
-  const float* __restrict__ ub = p.u + (size_t)b * d * L;
   const size_t row = ((size_t)b * d + ic) * L;
+  const u4* __restrict__ upb = p.up + ((size_t)(b - p.up_b0) * p.up_nt - p.up_t0) * (KS * 3 * 64);   // + tile * (KS 3 64)
 
   u4 xa[KS][3];
 #pragma unroll
@@ -324,10 +340,10 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DROPIN_
   const int t_first = q.t0, t_last = q.t1 - 1;
   float* __restrict__ dth = q.dth + ((size_t)zb * d + ic) * n * q.lc - (size_t)t_first * DT;
 
-  constexpr int NT = NW * 64, NREC = (KS * 64 + NT - 1) / NT;
-  float sv[NREC][8];
-  stage_load<NT, NREC>(ub, sv, d, L, p.ks, t_last * DT, tid);
-  stage_store<NT, NREC, KS>(sv, s_u[t_last & 1], tid, sk);
+  constexpr int NT = NW * 64, NREC = (KS * 3 * 64 + NT - 1) / NT;
+  u4 sv[NREC];
+  tile_load<NT, NREC, KS>(upb + (size_t)t_last * (KS * 3 * 64), sv, tid);
+  tile_store<NT, NREC, KS>(sv, s_u[t_last & 1], tid);
   __syncthreads();
   // the wavefront's own inputs, requested one tile ahead
   float un, dtn, zn, gyn;
@@ -349,7 +365,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DROPIN_
       zn = p.z[row + l - DT];
       gyn = q.gy[row + l - DT];
     }
-    if (t > t_first) stage_load<NT, NREC>(ub, sv, d, L, p.ks, l0 - DT, tid);
+    if (t > t_first) tile_load<NT, NREC, KS>(upb + (size_t)(t - 1) * (KS * 3 * 64), sv, tid);
     f4 th = {0, 0, 0, 0};
     const u4* su = s_u[t & 1];
 #pragma unroll
@@ -359,14 +375,14 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DROPIN_
       for (int c = 0; c < 3; ++c) ubk[c] = su[(k * 3 + c) * 64 + lane];
       th = xmm<3>(xa[k], ubk, th);
     }
-    const float ut = siluf_(uv), w = dtv * ut, sz = siluf_(zv), av = gyv * sz;
+    const float ut = silu_fast(uv), w = dtv * ut, sz = silu_fast(zv), av = gyv * sz;
+    const float cnt = (float)(min(l_ + 1, L - l0));      // timesteps of the tile up to this one that exist
     float ysum = 0.0f, wsum = 0.0f;
 #pragma unroll
     for (int a = 0; a < 4; ++a) {
       const f4 par = s_par[j0 + 4 * g + a];
       const float btr_ = par[0], bti_ = par[1], ctr_ = par[2], cti_ = par[3];
-      const float thv = lok ? th[a] + s_xb[wave][4 * g + a] : 0.0f;
-      const float G = row_prefix(thv);
+      const float G = fmaf(s_xb[wave][4 * g + a], cnt, th[a]);
       float sn, cs;
       sincos_any(G, &sn, &cs);
       const float csl = row_last(cs, lane), snl = row_last(sn, lane);
@@ -410,7 +426,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DROPIN_
     wsum += __shfl_xor(wsum, 16);
     wsum += __shfl_xor(wsum, 32);
     if (nb > 1 && g == 0) s_yw[t & 1][wave][l_] = make_float2(ysum, wsum);
-    if (t > t_first) stage_store<NT, NREC, KS>(sv, s_u[(t - 1) & 1], tid, sk);
+    if (t > t_first) tile_store<NT, NREC, KS>(sv, s_u[(t - 1) & 1], tid);
     if (nb > 1) {                                      // the channel's first wavefront adds the shares up
       __syncthreads();
       for (int k = 1; k < nb; ++k) {
@@ -421,9 +437,9 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DROPIN_
     }
     if (iok && lok && g == 0 && sb == 0) {
       const float pre = ysum + Di * ut;
-      q.dz[row + l] = gyv * pre * dsiluf_(zv);
+      q.dz[row + l] = gyv * pre * dsilu_fast(zv);
       q.ddt[row + l] = wsum * ut;
-      q.du[row + l] = (wsum * dtv + av * Di) * dsiluf_(uv);
+      q.du[row + l] = (wsum * dtv + av * Di) * dsilu_fast(uv);
       gD += av * ut;
     }
     if (nb == 1) __syncthreads();

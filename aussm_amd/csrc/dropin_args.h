@@ -18,14 +18,18 @@ struct DropinArgs {
   const float* C_r;
   const float* C_th;
   const float* Dp;       // [d]
-  const float* h_re;     // [b, d, n]
+  const float* h_re;     // [b, d, n] state before tile t0
   const float* h_im;
   float* y;              // [b, d, L] or null (states only)
-  float* nh_re;          // [b, d, n] or null
+  float* nh_re;          // [b, d, n] or null: state after tile t1 - 1 (may be the same buffer as h_*)
   float* nh_im;
   const u4* xp;          // rows of x as matrix operands: [d nb][ks][piece][64 lanes]
-  int b, d, n, L, ks;    // ks = ceil(d / 32)
+  const u4* up;          // tiles of u, prefix-summed along the tile, as matrix operands: [b][tile - up_t0][KS][piece][64 lanes]
+  int up_b0, up_t0, up_nt;   // up holds the batch elements from up_b0 on and the tiles up_t0 .. up_t0 + up_nt - 1
+  int b, d, n, L, ks;    // b: batch elements of this launch; ks = ceil(d / 32)
   int nb;                // blocks of 16 states per channel: 1, 2 or 4 (>= ceil(n / 16))
+  int b0;                // first batch element of this launch (tensors are indexed by b0 + ...)
+  int t0, t1;            // tiles of 16 timesteps of this launch (forward kernel; the backward kernel has its own)
 };
 
 struct DropinBwdArgs {

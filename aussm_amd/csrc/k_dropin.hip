@@ -39,6 +39,13 @@ static void launch_bwd(const DropinBwdArgs& a, hipStream_t s) {
 
 int dropin_channels_per_workgroup(int ks) { return ks > 8 ? 4 : DROPIN_NW; }
 
+// the compiled size of the contraction (steps of 32) that serves ceil(d / 32) = ks
+int dropin_compiled_ks(int ks) { return ks <= 4 ? (ks < 1 ? 1 : ks) : ks <= 6 ? 6 : ks <= 8 ? 8 : ks <= 12 ? 12 : 16; }
+
+void run_dropin_uprep(const float* u, u4* up, int d, int L, int ks, int b0, int bg, int t0, int nt, hipStream_t s) {
+  hipLaunchKernelGGL(dropin_uprep_kernel, dim3((unsigned)(bg * nt)), dim3(256), 0, s, u, up, d, L, dropin_compiled_ks(ks), b0, t0, nt);
+}
+
 // compiled sizes of the contraction over r, in steps of 32: the smallest one >= ceil(d / 32) runs
 #define DROPIN_KS_DISPATCH(LAUNCH, ks)          \
   if (ks <= 1) LAUNCH<1>(a, s);                 \

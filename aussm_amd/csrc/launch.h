@@ -43,6 +43,8 @@ int run_px_bwd(const UniBwdArgs& a, const u4* img, int in_dtype, hipStream_t s);
 // ---- k_dropin.hip: the reference's 12-input operator as fused kernels
 void run_dropin_xprep(const float* x, u4* xp, int d, int n, int ks, int nb, hipStream_t s);
 int dropin_channels_per_workgroup(int ks);
+int dropin_compiled_ks(int ks);
+void run_dropin_uprep(const float* u, u4* up, int d, int L, int ks, int b0, int bg, int t0, int nt, hipStream_t s);
 int run_dropin_fwd(const DropinArgs& a, hipStream_t s);
 int run_dropin_bwd(const DropinBwdArgs& a, hipStream_t s);
 void run_fill(const FillArgs& a, hipStream_t s);   // several buffers set (zero or a copy) in one launch

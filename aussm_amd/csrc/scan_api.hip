@@ -529,12 +529,25 @@ static int dropin_check(int b, int d, int n, int L) {
   return AUSSM_OK;
 }
 
+// floats of one prepared tile of u (all compiled steps of the contraction, three pieces, 64 lanes of 16 bytes)
+static size_t dropin_tile_floats(int d) { return (size_t)dropin_compiled_ks((d + 31) / 32) * 3 * 64 * 4; }
+// tiles per launch of the forward call: its prepared tiles of u (all batch elements) stay within the block budget
+static int dropin_fwd_chunk_tiles(int b, int d, int L) {
+  const int ntiles = (L + DT - 1) / DT;
+  size_t tmax = (size_t)DROPIN_BLOCK_FLOATS / ((size_t)b * dropin_tile_floats(d));
+  if (tmax < 1) tmax = 1;
+  const size_t nc = ((size_t)ntiles + tmax - 1) / tmax;
+  return (int)(((size_t)ntiles + nc - 1) / nc);
+}
+
 size_t aussm_ssm_adaptive_unitary_workspace_floats(int b, int d, int n, int L, int backward) {
   if (dropin_check(b, d, n, L) != AUSSM_OK) return 0;
   size_t f = dropin_xp_floats(d, n);
   if (backward) {
     const DropinBlocks k = dropin_blocks(b, d, n, L);
-    f += 2 * round4((size_t)b * d * n) + (size_t)k.bg * k.ct * DT * d * n;
+    f += 2 * round4((size_t)b * d * n) + (size_t)k.bg * k.ct * DT * d * n + (size_t)k.bg * k.ct * dropin_tile_floats(d);
+  } else {
+    f += (size_t)b * dropin_fwd_chunk_tiles(b, d, L) * dropin_tile_floats(d);
   }
   return f;
 }
@@ -550,11 +563,24 @@ int aussm_ssm_adaptive_unitary_fwd(const float* u, const float* dt, const float*
     return AUSSM_E_NULL;
   if (misaligned(workspace, 16)) return AUSSM_E_ALIGN;
   hipStream_t s = (hipStream_t)stream;
-  const int ks = (d + 31) / 32, nb = dropin_state_blocks(n);
-  run_dropin_xprep(x, (u4*)workspace, d, n, ks, nb, s);
-  DropinArgs a{u, dt, z, x_bias, B_r, B_theta, C_r, C_theta, D, h_re, h_im, y, nh_re, nh_im, (const u4*)workspace,
-               b, d, n, L, ks, nb};
-  return run_dropin_fwd(a, s);
+  const int ks = (d + 31) / 32, nb = dropin_state_blocks(n), ntiles = (L + DT - 1) / DT;
+  const int ct = dropin_fwd_chunk_tiles(b, d, L);
+  u4* xp = (u4*)workspace;
+  u4* up = (u4*)(workspace + dropin_xp_floats(d, n));
+  run_dropin_xprep(x, xp, d, n, ks, nb, s);
+  // the sequence in chunks of ct tiles (one chunk unless it is long): prepared tiles of u for the chunk, then the
+  // scan over it, the state handed from chunk to chunk in the output buffers
+  for (int t0 = 0; t0 < ntiles; t0 += ct) {
+    const int t1 = t0 + ct < ntiles ? t0 + ct : ntiles;
+    run_dropin_uprep(u, up, d, L, ks, 0, b, t0, t1 - t0, s);
+    DropinArgs a{};
+    a.u = u; a.dt = dt; a.z = z; a.x_bias = x_bias; a.B_r = B_r; a.B_th = B_theta; a.C_r = C_r; a.C_th = C_theta;
+    a.Dp = D; a.h_re = t0 ? nh_re : h_re; a.h_im = t0 ? nh_im : h_im; a.y = y; a.nh_re = nh_re; a.nh_im = nh_im;
+    a.xp = xp; a.up = up; a.up_b0 = 0; a.up_t0 = t0; a.up_nt = t1 - t0;
+    a.b = b; a.d = d; a.n = n; a.L = L; a.ks = ks; a.nb = nb; a.b0 = 0; a.t0 = t0; a.t1 = t1;
+    if (int e = run_dropin_fwd(a, s)) return e;
+  }
+  return AUSSM_OK;
 }
 
 int aussm_ssm_adaptive_unitary_bwd(const float* grad_y, const float* grad_nh_re, const float* grad_nh_im,
@@ -580,18 +606,19 @@ int aussm_ssm_adaptive_unitary_bwd(const float* grad_y, const float* grad_nh_re,
   float* hc_re = workspace + dropin_xp_floats(d, n);
   float* hc_im = hc_re + round4(nstate);
   float* dth = hc_im + round4(nstate);
+  u4* up = (u4*)(dth + (size_t)blk.bg * ct * DT * d * n);
   run_dropin_xprep(x, xp, d, n, ks, nb, s);
-  DropinArgs f{u, dt, z, x_bias, B_r, B_theta, C_r, C_theta, D, h_re, h_im, nullptr, hc_re, hc_im, xp, b, d, n, L, ks, nb};
+  DropinArgs f{};
+  f.u = u; f.dt = dt; f.z = z; f.x_bias = x_bias; f.B_r = B_r; f.B_th = B_theta; f.C_r = C_r; f.C_th = C_theta;
+  f.Dp = D; f.xp = xp; f.up = up; f.d = d; f.n = n; f.L = L; f.ks = ks; f.nb = nb;
   FillArgs fa{};
   auto fill = [&](float* dst, const float* src, size_t cnt) {
     fa.dst[fa.count] = dst; fa.src[fa.count] = src; fa.n[fa.count] = cnt; ++fa.count;
   };
-  if (nh_re && nh_im) {
+  const bool have_end = nh_re && nh_im;
+  if (have_end) {
     fill(hc_re, nh_re, nstate);
     fill(hc_im, nh_im, nstate);
-  } else {
-    // the state at the end of the sequence: one forward sweep without outputs
-    if (int e = run_dropin_fwd(f, s)) return e;
   }
   fill(dh_re, grad_nh_re, nstate);                  // the adjoint of the state travels in the output buffers
   fill(dh_im, grad_nh_im, nstate);
@@ -604,35 +631,50 @@ int aussm_ssm_adaptive_unitary_bwd(const float* grad_y, const float* grad_nh_re,
   fill(dD, nullptr, d);
   run_fill(fa, s);
   const long dn = (long)d * n;
-  for (int b0 = 0; b0 < b; b0 += blk.bg)
-  for (int t1 = ntiles; t1 > 0; t1 -= ct) {
+  for (int b0 = 0; b0 < b; b0 += blk.bg) {
     const int bg = b - b0 < blk.bg ? b - b0 : blk.bg;
-    const int t0 = t1 - ct > 0 ? t1 - ct : 0;
-    const int l0 = t0 * DT, len = (t1 * DT < L ? t1 * DT : L) - l0;
-    DropinBwdArgs q{};
-    q.f = f;
-    q.f.nh_re = q.f.nh_im = nullptr;
-    q.gy = grad_y; q.hc_re = hc_re; q.hc_im = hc_im; q.dth = dth;
-    q.du = du; q.ddt = ddt; q.dz = dz; q.dxb = dx_bias;
-    q.dB_r = dB_r; q.dB_th = dB_theta; q.dC_r = dC_r; q.dC_th = dC_theta; q.dD = dD;
-    q.dh_re = dh_re; q.dh_im = dh_im; q.b0 = b0; q.bg = bg; q.t0 = t0; q.t1 = t1; q.lc = lc;
-    if (int e = run_dropin_bwd(q, s)) return e;
-    // grad_u[b, r, l0 + l] += sum_(i j) x[(i j), r] hat theta[b, (i j), l]
-    GemmArgs gu{};
-    gu.A = x; gu.sam = 1; gu.sak = d; gu.saz = 0;
-    gu.Bm = dth; gu.sbk = lc; gu.sbn = 1; gu.sbz = dn * lc;
-    gu.C = du + (size_t)b0 * d * L + l0; gu.scm = L; gu.scn = 1; gu.scz = (long)d * L;
-    gu.M = d; gu.N = len; gu.K = (int)dn; gu.Z = bg; gu.reduce_z = 0; gu.accumulate = 1;
-    gemm_slices(gu);
-    if (int e = run_split_gemm(gu, s)) return e;
-    // grad_x[(i j), r] += sum_b sum_l hat theta[b, (i j), l] u[b, r, l0 + l]
-    GemmArgs gx{};
-    gx.A = dth; gx.sam = lc; gx.sak = 1; gx.saz = dn * lc;
-    gx.Bm = u + (size_t)b0 * d * L + l0; gx.sbk = 1; gx.sbn = L; gx.sbz = (long)d * L;
-    gx.C = dx; gx.scm = d; gx.scn = 1; gx.scz = 0;
-    gx.M = (int)dn; gx.N = d; gx.K = len; gx.Z = bg; gx.reduce_z = 1; gx.accumulate = 1;
-    gemm_slices(gx);
-    if (int e = run_split_gemm(gx, s)) return e;
+    f.b = bg; f.b0 = b0; f.up_b0 = b0;
+    if (!have_end) {
+      // the state at the end of the sequence: a forward sweep without outputs over this group's chunks
+      for (int t0 = 0; t0 < ntiles; t0 += ct) {
+        const int t1 = t0 + ct < ntiles ? t0 + ct : ntiles;
+        run_dropin_uprep(u, up, d, L, ks, b0, bg, t0, t1 - t0, s);
+        DropinArgs a = f;
+        a.h_re = t0 ? hc_re : h_re; a.h_im = t0 ? hc_im : h_im; a.y = nullptr; a.nh_re = hc_re; a.nh_im = hc_im;
+        a.up_t0 = t0; a.up_nt = t1 - t0; a.t0 = t0; a.t1 = t1;
+        if (int e = run_dropin_fwd(a, s)) return e;
+      }
+    }
+    // the chunks in reverse: chunk c covers the tiles c ct .. (same cuts as the forward sweep above)
+    for (int t0 = ((ntiles - 1) / ct) * ct; t0 >= 0; t0 -= ct) {
+      const int t1 = t0 + ct < ntiles ? t0 + ct : ntiles;
+      const int l0 = t0 * DT, len = (t1 * DT < L ? t1 * DT : L) - l0;
+      run_dropin_uprep(u, up, d, L, ks, b0, bg, t0, t1 - t0, s);
+      DropinBwdArgs q{};
+      q.f = f;
+      q.f.up_t0 = t0; q.f.up_nt = t1 - t0;
+      q.gy = grad_y; q.hc_re = hc_re; q.hc_im = hc_im; q.dth = dth;
+      q.du = du; q.ddt = ddt; q.dz = dz; q.dxb = dx_bias;
+      q.dB_r = dB_r; q.dB_th = dB_theta; q.dC_r = dC_r; q.dC_th = dC_theta; q.dD = dD;
+      q.dh_re = dh_re; q.dh_im = dh_im; q.b0 = b0; q.bg = bg; q.t0 = t0; q.t1 = t1; q.lc = lc;
+      if (int e = run_dropin_bwd(q, s)) return e;
+      // grad_u[b, r, l0 + l] += sum_(i j) x[(i j), r] hat theta[b, (i j), l]
+      GemmArgs gu{};
+      gu.A = x; gu.sam = 1; gu.sak = d; gu.saz = 0;
+      gu.Bm = dth; gu.sbk = lc; gu.sbn = 1; gu.sbz = dn * lc;
+      gu.C = du + (size_t)b0 * d * L + l0; gu.scm = L; gu.scn = 1; gu.scz = (long)d * L;
+      gu.M = d; gu.N = len; gu.K = (int)dn; gu.Z = bg; gu.reduce_z = 0; gu.accumulate = 1;
+      gemm_slices(gu);
+      if (int e = run_split_gemm(gu, s)) return e;
+      // grad_x[(i j), r] += sum_b sum_l hat theta[b, (i j), l] u[b, r, l0 + l]
+      GemmArgs gx{};
+      gx.A = dth; gx.sam = lc; gx.sak = 1; gx.saz = dn * lc;
+      gx.Bm = u + (size_t)b0 * d * L + l0; gx.sbk = 1; gx.sbn = L; gx.sbz = (long)d * L;
+      gx.C = dx; gx.scm = d; gx.scn = 1; gx.scz = 0;
+      gx.M = (int)dn; gx.N = d; gx.K = len; gx.Z = bg; gx.reduce_z = 1; gx.accumulate = 1;
+      gemm_slices(gx);
+      if (int e = run_split_gemm(gx, s)) return e;
+    }
   }
   return AUSSM_OK;
 }
