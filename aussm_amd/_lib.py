@@ -53,7 +53,7 @@ EXPORTED = tuple(_SIGNATURES) + ("aussm_error_string", "aussm_unitary_aux_floats
                                  "aussm_ssm_adaptive_unitary_workspace_floats")
 
 
-OPT_UNITARY_FWD, OPT_UNITARY_BWD, OPT_SPLIT_CAP, OPT_GENERIC_NW, OPT_GENERIC_NT = range(5)
+OPT_UNITARY_FWD, OPT_UNITARY_BWD, OPT_SPLIT_CAP, OPT_GENERIC_NW, OPT_GENERIC_NT, OPT_BLOCK_KFLOATS = range(6)
 
 
 class AussmError(RuntimeError):
@@ -103,7 +103,7 @@ class options:
     """Context manager: library options (aussm_set_option) for the duration of a block, e.g.
     `with options(unitary_fwd=0, split_cap=0): ...`; the previous values come back on exit."""
     _KEYS = {"unitary_fwd": OPT_UNITARY_FWD, "unitary_bwd": OPT_UNITARY_BWD, "split_cap": OPT_SPLIT_CAP,
-             "generic_nw": OPT_GENERIC_NW, "generic_nt": OPT_GENERIC_NT}
+             "generic_nw": OPT_GENERIC_NW, "generic_nt": OPT_GENERIC_NT, "block_kfloats": OPT_BLOCK_KFLOATS}
 
     def __init__(self, **kw):
         self.kw = {self._KEYS[k]: (-1 if v is None else int(v)) for k, v in kw.items()}

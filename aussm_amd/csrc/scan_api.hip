@@ -480,9 +480,11 @@ static size_t dropin_xp_floats(int d, int n) { return (size_t)d * dropin_state_b
 // of 16 timesteps: the workspace holds the phase adjoints of one block (about 50 MiB at most).  bg is
 // what fills the chip with one workgroup per compute unit (fewer would idle units, more would only
 // shorten the blocks and repeat the per-launch set-up, the rows of x among it, more often).
-#ifndef DROPIN_BLOCK_FLOATS
-#define DROPIN_BLOCK_FLOATS (25u << 19)
-#endif
+// budget of a block (phase adjoints; prepared tiles of u), in floats
+static size_t dropin_block_floats() {
+  const int o = opt(AUSSM_OPT_BLOCK_KFLOATS);
+  return (size_t)(o > 0 ? o : 12800) << 10;
+}
 struct DropinBlocks { int bg, ct; };
 static DropinBlocks dropin_blocks(int b, int d, int n, int L) {
   const int nw = dropin_channels_per_workgroup((d + 31) / 32);
@@ -491,7 +493,7 @@ static DropinBlocks dropin_blocks(int b, int d, int n, int L) {
   if (bg > b) bg = b;
   const int ng = (b + bg - 1) / bg;
   bg = (b + ng - 1) / ng;
-  const size_t per_tile = (size_t)bg * d * n * DT, cap = (size_t)DROPIN_BLOCK_FLOATS;
+  const size_t per_tile = (size_t)bg * d * n * DT, cap = dropin_block_floats();
   const int ntiles = (L + DT - 1) / DT;
   size_t tmax = cap / per_tile;
   if (tmax < 1) tmax = 1;
@@ -534,7 +536,7 @@ static size_t dropin_tile_floats(int d) { return (size_t)dropin_compiled_ks((d +
 // tiles per launch of the forward call: its prepared tiles of u (all batch elements) stay within the block budget
 static int dropin_fwd_chunk_tiles(int b, int d, int L) {
   const int ntiles = (L + DT - 1) / DT;
-  size_t tmax = (size_t)DROPIN_BLOCK_FLOATS / ((size_t)b * dropin_tile_floats(d));
+  size_t tmax = dropin_block_floats() / ((size_t)b * dropin_tile_floats(d));
   if (tmax < 1) tmax = 1;
   const size_t nc = ((size_t)ntiles + tmax - 1) / tmax;
   return (int)(((size_t)ntiles + nc - 1) / nc);

@@ -71,6 +71,9 @@ const char* aussm_error_string(int code);
  *                          pieces everywhere, 6 prepared operands
  *   AUSSM_OPT_SPLIT_CAP    largest number of segments a launch may be split into along L
  *                          (0 or 1: never split)
+ *   AUSSM_OPT_BLOCK_KFLOATS   budget, in units of 1024 floats, of the blocks in which the fused operator calls
+ *                          (aussm_ssm_adaptive_unitary_fwd / _bwd) walk their problem (default 12800 = 50 MiB);
+ *                          workspace sizes follow it, so set it before asking for them
  *   AUSSM_OPT_GENERIC_NW / AUSSM_OPT_GENERIC_NT   states per wavefront / threads per workgroup of
  *                          the vector-ALU kernels (both must be set; one of the built pairs) */
 #define AUSSM_OPT_UNITARY_FWD 0
@@ -78,7 +81,8 @@ const char* aussm_error_string(int code);
 #define AUSSM_OPT_SPLIT_CAP 2
 #define AUSSM_OPT_GENERIC_NW 3
 #define AUSSM_OPT_GENERIC_NT 4
-#define AUSSM_OPT_COUNT 5
+#define AUSSM_OPT_BLOCK_KFLOATS 5
+#define AUSSM_OPT_COUNT 6
 int aussm_set_option(int key, int value);
 int aussm_get_option(int key);   /* -1 = unset */
 

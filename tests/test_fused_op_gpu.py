@@ -71,6 +71,34 @@ def test_fused_backward_matches_oracle_autograd(shape):
         _close(g_, w, "gradient wrt " + name)
 
 
+@pytest.mark.parametrize("kfloats", [16, 256])
+def test_small_blocks_walk_the_problem_in_many_launches(kfloats):
+    """A tiny block budget forces what long sequences and large batches get: the forward call in several chunks
+    along the sequence, the backward call in (batch group) x (chunk) blocks with the state and its adjoint handed
+    from launch to launch.  Same results as the oracle."""
+    from aussm_amd import ops, _lib  # noqa: F401
+    b, d, n, l = 5, 24, 16, 300
+    print(f"case fused small blocks kfloats={kfloats}", flush=True)
+    args = _inputs(b, d, n, l, seed=11, xscale=d ** -0.5)
+    g = torch.Generator().manual_seed(12)
+    grads = [torch.randn(b, d, l, generator=g, dtype=torch.float64), torch.randn(b, d, n, generator=g, dtype=torch.float64),
+             torch.randn(b, d, n, generator=g, dtype=torch.float64)]
+    leaves = [a.clone().requires_grad_(True) for a in args]
+    outs = O.adaptive_unitary_op_loop(*leaves)
+    want = torch.autograd.grad(outs, leaves, grads)
+    dev = [a.float().cuda() for a in args]
+    with _lib.options(block_kfloats=kfloats):
+        got_f = torch.ops.extension_cpp.ssm_adaptive_unitary(*dev)
+        got_b = torch.ops.extension_cpp.ssm_adaptive_backward_unitary(*[t.float().cuda() for t in grads], *dev)
+        got_s = torch.ops.aussm_amd.ssm_adaptive_backward_unitary_from_state(*[t.float().cuda() for t in grads], *dev,
+                                                                              got_f[1], got_f[2])
+    for w, g_, name in zip(outs, got_f, ("y", "next_hid_real", "next_hid_imag")):
+        _close(g_, w.detach(), name)
+    for w, g1, g2, name in zip(want, got_b, got_s, IN_NAMES):
+        _close(g1, w, "gradient wrt " + name)
+        _close(g2, w, "gradient (from state) wrt " + name)
+
+
 def test_backward_from_saved_state_equals_backward_from_inputs():
     """The autograd formula hands the forward call's end state to the backward kernels; the reference-shaped
     backward operator recomputes it.  Same gradients either way."""
