@@ -35,7 +35,8 @@ def _close(got, want, name, tol=1e-4):
 
 
 SHAPES = [(2, 8, 4, 256), (3, 20, 5, 48), (2, 37, 16, 45), (1, 70, 11, 130), (2, 16, 16, 14),
-          (2, 12, 64, 70), (2, 9, 24, 33), (1, 21, 40, 50)]          # more than 16 states: 4, 2 and 4 (3 padded) blocks per channel
+          (2, 12, 64, 70), (2, 9, 24, 33), (1, 21, 40, 50),          # more than 16 states: 4, 2 and 4 (3 padded) blocks per channel
+          (1, 300, 16, 35), (1, 512, 32, 20), (2, 160, 8, 1), (1, 100, 3, 17)]   # wide: one wavefront per SIMD above d = 256
 
 
 @pytest.mark.parametrize("shape", SHAPES)
