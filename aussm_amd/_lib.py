@@ -39,9 +39,9 @@ _SIGNATURES = {
     "aussm_static_init": [],
     "aussm_unitary_fwd_static": [_P] * 10 + [_I] * 6 + [_P],
     "aussm_complex_fwd": [_P] * 12 + [_I] * 6 + [_P],
-    "aussm_complex_bwd": [_P] * 19 + [_I] * 6 + [_P],
+    "aussm_complex_bwd": [_P] * 21 + [_I] * 6 + [_P],
     "aussm_real_fwd": [_P] * 8 + [_I] + [_P] * 4 + [_I] * 6 + [_P],
-    "aussm_real_bwd": [_P] * 9 + [_I] + [_P] * 9 + [_I] * 6 + [_P],
+    "aussm_real_bwd": [_P] * 9 + [_I] + [_P] * 11 + [_I] * 6 + [_P],
     "aussm_causal_conv1d_fwd": [_P] * 4 + [_I] * 4 + [_LL] * 2 + [_P],
     "aussm_causal_conv1d_bwd": [_P] * 6 + [_I] * 4 + [_LL] * 2 + [_P],
     "aussm_swap_last2": [_P] * 2 + [_I] * 3 + [_LL] * 2 + [_P],

@@ -405,7 +405,7 @@ int aussm_complex_bwd(const float* dy, const float* dhL, const void* u, const vo
                       const float* theta, const void* Bc, const void* Cc, const float* Dskip,
                       const float* h0, const float* hck,
                       float* du, float* ddelta, float* drho, float* dtheta, float* dB, float* dC,
-                      float* dD, float* dh0,
+                      float* dD, float* dh0, const float* z, float* dz,
                       int B, int D, int N, int L, int ck, int in_dtype, void* stream) {
   if (int e = check_common(B, D, N, L, ck, in_dtype)) return e;
   if (ck != REC_CK) return AUSSM_E_CK;
@@ -418,6 +418,8 @@ int aussm_complex_bwd(const float* dy, const float* dhL, const void* u, const vo
   a.dy = dy; a.dhL = dhL; a.u = u; a.delta = delta; a.theta = theta; a.rho = rho; a.Bm = Bc; a.Cm = Cc;
   a.Dskip = Dskip; a.h0 = h0; a.hck = hck;
   a.du = du; a.ddelta = ddelta; a.dtheta = dtheta; a.drho = drho; a.dB = dB; a.dC = dC; a.dD = dD; a.dh0 = dh0;
+  if ((z == nullptr) != (dz == nullptr)) return AUSSM_E_NULL;
+  a.z = z; a.dz = dz;
   a.B = B; a.D = D; a.N = N; a.L = L; a.nck = (L + ck - 1) / ck; a.ncg = (D + CH - 1) / CH;
   return run_rec_bwd(VAR_COMPLEX, a, in_dtype, (hipStream_t)stream);
 }
@@ -426,6 +428,7 @@ int aussm_real_bwd(const float* dy, const float* dhL, const void* u, const void*
                    const void* Bm, const void* Cm, const float* Dskip, const float* delta_bias,
                    int delta_softplus, const float* h0, const float* hck,
                    float* du, float* ddelta, float* dA, float* dB, float* dC, float* dD, float* dh0,
+                   const float* z, float* dz,
                    int B, int D, int N, int L, int ck, int in_dtype, void* stream) {
   if (int e = check_common(B, D, N, L, ck, in_dtype)) return e;
   if (ck != REC_CK) return AUSSM_E_CK;
@@ -434,6 +437,8 @@ int aussm_real_bwd(const float* dy, const float* dhL, const void* u, const void*
   a.dy = dy; a.dhL = dhL; a.u = u; a.delta = delta; a.A = A; a.Bm = Bm; a.Cm = Cm; a.Dskip = Dskip;
   a.delta_bias = delta_bias; a.delta_softplus = delta_softplus; a.h0 = h0; a.hck = hck;
   a.du = du; a.ddelta = ddelta; a.dA = dA; a.dB = dB; a.dC = dC; a.dD = dD; a.dh0 = dh0;
+  if ((z == nullptr) != (dz == nullptr)) return AUSSM_E_NULL;
+  a.z = z; a.dz = dz;
   a.B = B; a.D = D; a.N = N; a.L = L; a.nck = (L + ck - 1) / ck; a.ncg = (D + CH - 1) / CH;
   return run_rec_bwd(VAR_REAL, a, in_dtype, (hipStream_t)stream);
 }

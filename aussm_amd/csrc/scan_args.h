@@ -86,6 +86,8 @@ struct RecBwdArgs {
   float *dB, *dC;           // [B,N,L(,2)], accumulated into
   float* dD;                // [D] or null, accumulated into
   float* dh0;               // [B,D,N,C] or null
+  const float* z;           // [B,D,L] or null: the output was gated, y = y_pre silu(z); dy is the gradient of y
+  float* dz;                // [B,D,L] (with z)
   int B, D, N, L, nck, ncg, delta_softplus;
   // A launch handles the states nbase .. nbase + 15 (a workgroup's four wavefronts of up to four states);
   // larger N takes one launch per block of 16 states.  accum: a later block - the sums over the states

@@ -11,6 +11,9 @@
 //          dw_l    = sum_n Re(conj(B_l) g_l)
 //          complex: drho_l = sum_n Re(conj(g_l) p_l)     dtheta_l = -sum_n Im(conj(g_l) p_l)
 //          real:    x = g_l h_{l-1} a_l;  dA[d,n] += x delta_l;  ddelta_l = sum_n x A[d,n] + dw_l u_l
+// Gate: with z given the forward output was y = y_pre silu(z); dy is then scaled by silu(z) on the way in,
+// y_pre = sum_n Re(C h) + D u is recomputed with the states (a fourth sum over the states), and
+// dz = dy y_pre silu'(z) leaves with the other gradients.
 // The work decomposition, LDS staging, wide scalar loads of B_t/C_t and the lane-transpose
 // channel reduction are those of the unitary kernels.
 // Reference semantics: extension-cpp/extension_cpp/ops.py:270-291 (complex), :349-356 (real),
@@ -142,7 +145,7 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
 
   // ---- staging-side mapping (lanes run along time) and the two raw register sets
   const int col = tid % RT, row0 = tid / RT;
-  struct RawTile { Tin u[E], dl[E]; float th[E], rho[E], gy[E]; };
+  struct RawTile { Tin u[E], dl[E]; float th[E], rho[E], gy[E], zz[E]; };
   RawTile rdy, fly;
   float dsk[E], dbias[E], accD[E];
   size_t goff[E];
@@ -157,6 +160,7 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
     accD[k] = 0.f;
     rdy.u[k] = rdy.dl[k] = fly.u[k] = fly.dl[k] = Tin(0);
     rdy.th[k] = rdy.rho[k] = rdy.gy[k] = fly.th[k] = fly.rho[k] = fly.gy[k] = 0.f;
+    rdy.zz[k] = fly.zz[k] = 0.f;
   }
   auto load_tile = [&](RawTile& r, int l0) {
 #pragma unroll
@@ -166,13 +170,14 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
       r.u[k] = gu[o];
       r.dl[k] = gdl[o];
       r.gy[k] = p.dy[o];
+      if (p.z) r.zz[k] = p.z[o];
       if (VAR == VAR_COMPLEX) { r.th[k] = p.theta[o]; r.rho[k] = p.rho[o]; }
     }
   };
   auto collect_tile = [&](RawTile& r) {
 #pragma unroll
     for (int k = 0; k < E; ++k) {
-      touch_vgpr(r.u[k]); touch_vgpr(r.dl[k]); touch_vgpr(r.gy[k]);
+      touch_vgpr(r.u[k]); touch_vgpr(r.dl[k]); touch_vgpr(r.gy[k]); touch_vgpr(r.zz[k]);
       if (VAR == VAR_COMPLEX) { touch_vgpr(r.th[k]); touch_vgpr(r.rho[k]); }
     }
   };
@@ -190,12 +195,17 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
     const int l0 = it * RT;
 
     // ---- stage
-    float eu[E], edl[E], egy[E], eraw[E];
+    float eu[E], edl[E], egy[E], eraw[E], egz[E];       // egz: dy silu'(z), for dz
 #pragma unroll
     for (int k = 0; k < E; ++k) {
       const bool ok = rowok[k] && l0 + col < L;
       eu[k] = ok ? to_f32(rdy.u[k]) : 0.f;
       egy[k] = ok ? rdy.gy[k] : 0.f;
+      egz[k] = 0.f;
+      if (p.z) {                                           // uniform
+        egz[k] = egy[k] * dsiluf_(rdy.zz[k]);
+        egy[k] *= siluf_(rdy.zz[k]);
+      }
       float dl = ok ? to_f32(rdy.dl[k]) : 0.f;
       float4 rec;
       if (VAR == VAR_REAL) {
@@ -270,9 +280,9 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
           const float4 v = s_in[(g * TG + t) * TS + lane];
           r0[t] = v.x; r1[t] = v.y; r2[t] = v.z; r3[t] = v.w;
         }
-        float kacc[TG], xacc[TG], zacc[TG];
+        float kacc[TG], xacc[TG], zacc[TG], yacc[TG];
 #pragma unroll
-        for (int t = 0; t < TG; ++t) { kacc[t] = 0.f; xacc[t] = 0.f; zacc[t] = 0.f; }
+        for (int t = 0; t < TG; ++t) { kacc[t] = 0.f; xacc[t] = 0.f; zacc[t] = 0.f; yacc[t] = 0.f; }
         float vals[RED_COLS];
 #pragma unroll
         for (int j = 0; j < RED_COLS; ++j) vals[j] = 0.f;
@@ -293,6 +303,7 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
                 gr[k] = fmaf(cc[t], gy, gr[k]);
                 vals[slot * 16 + t] = w * gr[k];
                 vals[slot * 16 + 8 + t] = gy * hsr[tt][k];
+                yacc[t] = fmaf(cc[t], hsr[tt][k], yacc[t]);
                 kacc[t] = fmaf(bc[t], gr[k], kacc[t]);
                 const float hprev = (tt > 0) ? hsr[tt > 0 ? tt - 1 : 0][k] : st_rdy.r[k];
                 const float x = gr[k] * hprev * a;
@@ -314,6 +325,7 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
                 vals[2 * t + 1] = w * gi[k];
                 vals[2 * TG + 2 * t] = gy * hsr[tt][k];
                 vals[2 * TG + 2 * t + 1] = -gy * hsi[tt][k];
+                yacc[t] = fmaf(cr, hsr[tt][k], fmaf(-ci, hsi[tt][k], yacc[t]));
                 kacc[t] = fmaf(br, gr[k], kacc[t]);
                 kacc[t] = fmaf(bi, gi[k], kacc[t]);
                 const float pr = fmaf(-br, w, hsr[tt][k]);
@@ -338,7 +350,7 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
           }
         }
 #pragma unroll
-        for (int t = 0; t < TG; ++t) part[(g * TG + t) * TS + lane] = make_float4(kacc[t], xacc[t], zacc[t], 0.f);
+        for (int t = 0; t < TG; ++t) part[(g * TG + t) * TS + lane] = make_float4(kacc[t], xacc[t], zacc[t], yacc[t]);
       }
         };
     if (active) {
@@ -395,9 +407,9 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
 #pragma unroll
     for (int k = 0; k < E; ++k) {
       const int ll = l0 + col;
-      float kk = 0.f, xx = 0.f, zz = 0.f;
+      float kk = 0.f, xx = 0.f, zz = 0.f, yy = 0.f;
 #pragma unroll
-      for (int w = 0; w < NWV; ++w) { kk += pv[k][w].x; xx += pv[k][w].y; zz += pv[k][w].z; }
+      for (int w = 0; w < NWV; ++w) { kk += pv[k][w].x; xx += pv[k][w].y; zz += pv[k][w].z; yy += pv[k][w].w; }
       if (rowok[k] && ll < L) {
         const size_t o = goff[k] + ll;
         const bool acc = p.accum != 0;                   // uniform
@@ -410,6 +422,10 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
           p.ddelta[o] = acc ? fmaf(kk, eu[k], p.ddelta[o]) : kk * eu[k];
           p.dtheta[o] = acc ? p.dtheta[o] + xx : xx;
           p.drho[o] = acc ? p.drho[o] + zz : zz;
+        }
+        if (p.dz) {                                        // y_pre = sum over the states + D u (the latter once)
+          const float dzv = egz[k] * (acc ? yy : fmaf(dsk[k], eu[k], yy));
+          p.dz[o] = acc ? p.dz[o] + dzv : dzv;
         }
         accD[k] = fmaf(egy[k], eu[k], accD[k]);
       }

@@ -266,7 +266,7 @@ def complex_fwd_raw(u, delta, rho, theta, Bri, Cri, D=None, z=None, h0=None, wan
     return y, hL, hck
 
 
-def complex_bwd_raw(dy, dhL, u, delta, rho, theta, Bri, Cri, D, h0, hck, want_dD=True, want_dh0=False):
+def complex_bwd_raw(dy, dhL, u, delta, rho, theta, Bri, Cri, D, h0, hck, want_dD=True, want_dh0=False, z=None):
     lib = _lib.load()
     b, d, l = u.shape
     n = Bri.shape[1]
@@ -276,28 +276,31 @@ def complex_bwd_raw(dy, dhL, u, delta, rho, theta, Bri, Cri, D, h0, hck, want_dD
     dC = torch.zeros((b, n, l, 2), **f32)
     dD = torch.zeros((d,), **f32) if (want_dD and D is not None) else None
     dh0 = torch.empty((b, d, n, 2), **f32) if want_dh0 else None
+    dz = torch.empty((b, d, l), **f32) if z is not None else None
     check(lib.aussm_complex_bwd(ptr(dy), ptr(dhL), ptr(u), ptr(delta), ptr(rho), ptr(theta), ptr(Bri), ptr(Cri),
                                 ptr(D), ptr(h0), ptr(hck), ptr(du), ptr(ddelta), ptr(drho), ptr(dtheta), ptr(dB),
-                                ptr(dC), ptr(dD), ptr(dh0), b, d, n, l, REC_CK, _in_dtype(u), _stream()),
+                                ptr(dC), ptr(dD), ptr(dh0), ptr(z), ptr(dz), b, d, n, l, REC_CK, _in_dtype(u), _stream()),
           "aussm_complex_bwd")
-    return du, ddelta, drho, dtheta, dB, dC, dD, dh0
+    return du, ddelta, drho, dtheta, dB, dC, dD, dh0, dz
 
 
 class _ComplexScanFn(torch.autograd.Function):
+    """The gate z (optional) is applied by the forward kernel and differentiated by the backward kernel."""
+
     @staticmethod
-    def forward(ctx, u, delta, rho, theta, Bri, Cri, D, h0):
-        y, hL, hck = complex_fwd_raw(u, delta, rho, theta, Bri, Cri, D, None, h0, want_state=True, ck=REC_CK)
-        ctx.save_for_backward(u, delta, rho, theta, Bri, Cri, D, h0, hck)
+    def forward(ctx, u, delta, rho, theta, Bri, Cri, D, h0, z):
+        y, hL, hck = complex_fwd_raw(u, delta, rho, theta, Bri, Cri, D, z, h0, want_state=True, ck=REC_CK)
+        ctx.save_for_backward(u, delta, rho, theta, Bri, Cri, D, h0, hck, z)
         return y, hL
 
     @staticmethod
     def backward(ctx, dy, dhL):
-        u, delta, rho, theta, Bri, Cri, D, h0, hck = ctx.saved_tensors
+        u, delta, rho, theta, Bri, Cri, D, h0, hck, z = ctx.saved_tensors
         dhL = None if dhL is None else dhL.contiguous()
-        du, ddelta, drho, dtheta, dB, dC, dD, dh0 = complex_bwd_raw(
+        du, ddelta, drho, dtheta, dB, dC, dD, dh0, dz = complex_bwd_raw(
             dy.contiguous(), dhL, u, delta, rho, theta, Bri, Cri, D, h0, hck,
-            want_dD=D is not None and ctx.needs_input_grad[6], want_dh0=h0 is not None and ctx.needs_input_grad[7])
-        return (du.to(u.dtype), ddelta.to(delta.dtype), drho, dtheta, dB.to(Bri.dtype), dC.to(Cri.dtype), dD, dh0)
+            want_dD=D is not None and ctx.needs_input_grad[6], want_dh0=h0 is not None and ctx.needs_input_grad[7], z=z)
+        return (du.to(u.dtype), ddelta.to(delta.dtype), drho, dtheta, dB.to(Bri.dtype), dC.to(Cri.dtype), dD, dh0, dz)
 
 
 def complex_scan(u: Tensor, delta: Tensor, rho: Tensor, theta: Tensor, Bc: Tensor, Cc: Tensor,
@@ -326,9 +329,7 @@ def complex_scan(u: Tensor, delta: Tensor, rho: Tensor, theta: Tensor, Bc: Tenso
     if needs_grad:
         if n > REC_MAX_STATE:
             raise RuntimeError(f"the complex backward pass supports at most {REC_MAX_STATE} states per channel")
-        y, hL = _ComplexScanFn.apply(u, delta, rho, theta, Bri, Cri, D, h0r)
-        if z is not None:
-            y = y * F.silu(z)
+        y, hL = _ComplexScanFn.apply(u, delta, rho, theta, Bri, Cri, D, h0r, z)
     else:
         y, hL, _ = complex_fwd_raw(u, delta, rho, theta, Bri, Cri, D, z, h0r, want_state=return_last_state)
     if return_last_state:
@@ -355,7 +356,7 @@ def real_fwd_raw(u, delta, A, Bm, Cm, D=None, z=None, delta_bias=None, delta_sof
 
 
 def real_bwd_raw(dy, dhL, u, delta, A, Bm, Cm, D, delta_bias, delta_softplus, h0, hck, want_dD=True,
-                 want_dh0=False):
+                 want_dh0=False, z=None):
     lib = _lib.load()
     b, d, l = u.shape
     n = A.shape[1]
@@ -366,31 +367,34 @@ def real_bwd_raw(dy, dhL, u, delta, A, Bm, Cm, D, delta_bias, delta_softplus, h0
     dC = torch.zeros((b, n, l), **f32)
     dD = torch.zeros((d,), **f32) if (want_dD and D is not None) else None
     dh0 = torch.empty((b, d, n), **f32) if want_dh0 else None
+    dz = torch.empty((b, d, l), **f32) if z is not None else None
     check(lib.aussm_real_bwd(ptr(dy), ptr(dhL), ptr(u), ptr(delta), ptr(A), ptr(Bm), ptr(Cm), ptr(D),
                              ptr(delta_bias), int(bool(delta_softplus)), ptr(h0), ptr(hck), ptr(du), ptr(ddelta),
-                             ptr(dA), ptr(dB), ptr(dC), ptr(dD), ptr(dh0), b, d, n, l, REC_CK, _in_dtype(u),
-                             _stream()), "aussm_real_bwd")
-    return du, ddelta, dA, dB, dC, dD, dh0
+                             ptr(dA), ptr(dB), ptr(dC), ptr(dD), ptr(dh0), ptr(z), ptr(dz), b, d, n, l, REC_CK,
+                             _in_dtype(u), _stream()), "aussm_real_bwd")
+    return du, ddelta, dA, dB, dC, dD, dh0, dz
 
 
 class _RealScanFn(torch.autograd.Function):
+    """The gate z (optional) is applied by the forward kernel and differentiated by the backward kernel."""
+
     @staticmethod
-    def forward(ctx, u, delta, A, Bm, Cm, D, delta_bias, h0, delta_softplus):
-        y, hL, hck = real_fwd_raw(u, delta, A, Bm, Cm, D, None, delta_bias, delta_softplus, h0,
+    def forward(ctx, u, delta, A, Bm, Cm, D, delta_bias, h0, delta_softplus, z):
+        y, hL, hck = real_fwd_raw(u, delta, A, Bm, Cm, D, z, delta_bias, delta_softplus, h0,
                                   want_state=True, ck=REC_CK)
-        ctx.save_for_backward(u, delta, A, Bm, Cm, D, delta_bias, h0, hck)
+        ctx.save_for_backward(u, delta, A, Bm, Cm, D, delta_bias, h0, hck, z)
         ctx.delta_softplus = delta_softplus
         return y, hL
 
     @staticmethod
     def backward(ctx, dy, dhL):
-        u, delta, A, Bm, Cm, D, delta_bias, h0, hck = ctx.saved_tensors
+        u, delta, A, Bm, Cm, D, delta_bias, h0, hck, z = ctx.saved_tensors
         dhL = None if dhL is None else dhL.contiguous()
-        du, ddelta, dA, dB, dC, dD, dh0 = real_bwd_raw(
+        du, ddelta, dA, dB, dC, dD, dh0, dz = real_bwd_raw(
             dy.contiguous(), dhL, u, delta, A, Bm, Cm, D, delta_bias, ctx.delta_softplus, h0, hck,
-            want_dD=D is not None and ctx.needs_input_grad[5], want_dh0=h0 is not None and ctx.needs_input_grad[7])
+            want_dD=D is not None and ctx.needs_input_grad[5], want_dh0=h0 is not None and ctx.needs_input_grad[7], z=z)
         dbias = ddelta.sum(dim=(0, 2)) if (delta_bias is not None and ctx.needs_input_grad[6]) else None
-        return (du.to(u.dtype), ddelta.to(delta.dtype), dA, dB.to(Bm.dtype), dC.to(Cm.dtype), dD, dbias, dh0, None)
+        return (du.to(u.dtype), ddelta.to(delta.dtype), dA, dB.to(Bm.dtype), dC.to(Cm.dtype), dD, dbias, dh0, None, dz)
 
 
 def selective_scan_fn(u: Tensor, delta: Tensor, A: Tensor, B: Tensor, C: Tensor, D: Optional[Tensor] = None,
@@ -428,9 +432,7 @@ def selective_scan_fn(u: Tensor, delta: Tensor, A: Tensor, B: Tensor, C: Tensor,
     if needs_grad:
         if n > REC_MAX_STATE:
             raise RuntimeError(f"the S6 backward pass supports at most {REC_MAX_STATE} states per channel")
-        y, hL = _RealScanFn.apply(u, delta, A, Bm, Cm, D, delta_bias, h0, bool(delta_softplus))
-        if z is not None:
-            y = y * F.silu(z)
+        y, hL = _RealScanFn.apply(u, delta, A, Bm, Cm, D, delta_bias, h0, bool(delta_softplus), z)
     else:
         y, hL, _ = real_fwd_raw(u, delta, A, Bm, Cm, D, z, delta_bias, delta_softplus, h0,
                                 want_state=return_last_state)

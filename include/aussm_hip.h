@@ -207,12 +207,15 @@ int aussm_complex_fwd(const void* u, const void* delta, const float* rho, const 
                       const float* h0, float* y, float* hL, float* hck,
                       int B, int D, int N, int L, int ck, int in_dtype, void* stream);
 
+/* z / dz of the two backward calls below (both NULL, or both given): the forward call was gated with this z
+ * (y = y_pre silu(z)); dy is then the gradient of the gated y, the kernel applies the gate's derivative
+ * itself and writes dz = dy y_pre silu'(z).  N <= 64 (one launch per block of 16 states). */
 int aussm_complex_bwd(const float* dy, const float* dhL,
                       const void* u, const void* delta, const float* rho, const float* theta,
                       const void* Bc, const void* Cc, const float* Dskip,
                       const float* h0, const float* hck,
                       float* du, float* ddelta, float* drho, float* dtheta, float* dB, float* dC,
-                      float* dD, float* dh0,
+                      float* dD, float* dh0, const float* z, float* dz,
                       int B, int D, int N, int L, int ck, int in_dtype, void* stream);
 
 /* ---------------------------------------------------------------------------------------
@@ -237,7 +240,7 @@ int aussm_real_bwd(const float* dy, const float* dhL,
                    const float* delta_bias, int delta_softplus,
                    const float* h0, const float* hck,
                    float* du, float* ddelta, float* dA, float* dB, float* dC,
-                   float* dD, float* dh0,
+                   float* dD, float* dh0, const float* z, float* dz,
                    int B, int D, int N, int L, int ck, int in_dtype, void* stream);
 
 /* ---------------------------------------------------------------------------------------

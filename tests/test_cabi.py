@@ -94,7 +94,7 @@ def test_argument_checks_without_a_device():
     rc = lib.aussm_unitary_bwd_aux(*([one] * 17), 3, 1, 1, 32, 32, 0, 0, null)
     assert rc == -2
     # the recomputing backward kernels insist on their checkpoint interval and on the state limit of the library
-    args = [one] * 9 + [0] + [one] * 9
+    args = [one] * 9 + [0] + [one] * 11
     assert lib.aussm_real_bwd(*args, 1, 1, 1, 32, 32, 0, null) == -3
     assert lib.aussm_real_bwd(*args, 1, 1, 65, 32, 16, 0, null) == -2
     # the blocks' causal convolution: kernel length limit, overlapping rows, required pointers
