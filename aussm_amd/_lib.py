@@ -16,6 +16,7 @@ F32, BF16 = 0, 1
 TILE = 32
 AUX_PAD = 64          # floats between the per-(b,d,l) part of the auxiliary buffer and the segment states
 MAX_STATE = 64
+VAR_UNITARY, VAR_COMPLEX, VAR_REAL = 0, 1, 2   # variant codes of the C ABI
 
 _lib = None
 
@@ -38,10 +39,10 @@ _SIGNATURES = {
     "aussm_unitary_bwd_aux": [_P] * 17 + [_I] * 7 + [_P],
     "aussm_static_init": [],
     "aussm_unitary_fwd_static": [_P] * 10 + [_I] * 6 + [_P],
-    "aussm_complex_fwd": [_P] * 12 + [_I] * 6 + [_P],
-    "aussm_complex_bwd": [_P] * 21 + [_I] * 6 + [_P],
-    "aussm_real_fwd": [_P] * 8 + [_I] + [_P] * 4 + [_I] * 6 + [_P],
-    "aussm_real_bwd": [_P] * 9 + [_I] + [_P] * 11 + [_I] * 6 + [_P],
+    "aussm_complex_fwd": [_P] * 13 + [_I] * 6 + [_P],
+    "aussm_complex_bwd": [_P] * 22 + [_I] * 6 + [_P],
+    "aussm_real_fwd": [_P] * 8 + [_I] + [_P] * 5 + [_I] * 6 + [_P],
+    "aussm_real_bwd": [_P] * 9 + [_I] + [_P] * 12 + [_I] * 6 + [_P],
     "aussm_causal_conv1d_fwd": [_P] * 4 + [_I] * 4 + [_LL] * 2 + [_P],
     "aussm_causal_conv1d_bwd": [_P] * 6 + [_I] * 4 + [_LL] * 2 + [_P],
     "aussm_swap_last2": [_P] * 2 + [_I] * 3 + [_LL] * 2 + [_P],
@@ -50,7 +51,7 @@ _SIGNATURES = {
 }
 
 EXPORTED = tuple(_SIGNATURES) + ("aussm_error_string", "aussm_unitary_aux_floats",
-                                 "aussm_ssm_adaptive_unitary_workspace_floats")
+                                 "aussm_ssm_adaptive_unitary_workspace_floats", "aussm_scan_workspace_floats")
 
 
 OPT_UNITARY_FWD, OPT_UNITARY_BWD, OPT_SPLIT_CAP, OPT_GENERIC_NW, OPT_GENERIC_NT, OPT_BLOCK_KFLOATS = range(6)
@@ -82,6 +83,8 @@ def load() -> ctypes.CDLL:
     lib.aussm_unitary_aux_floats.restype = ctypes.c_size_t
     lib.aussm_ssm_adaptive_unitary_workspace_floats.argtypes = [_I, _I, _I, _I, _I]
     lib.aussm_ssm_adaptive_unitary_workspace_floats.restype = ctypes.c_size_t
+    lib.aussm_scan_workspace_floats.argtypes = [_I] * 7
+    lib.aussm_scan_workspace_floats.restype = ctypes.c_size_t
     lib.aussm_error_string.argtypes = [c_int]
     lib.aussm_error_string.restype = c_char_p
     _lib = lib

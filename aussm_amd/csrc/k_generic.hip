@@ -6,16 +6,21 @@
 #include "scan_bwd_recompute.h"
 #include "scan_bwd_unitary.h"
 #include "scan_fwd.h"
+#include "scan_seg_generic.h"
 
 namespace aussm {
 
 #define AUSSM_FWD_CASE(NW_, NT_)                                                                     \
   if (c.nw == NW_ && c.nt == NT_) {                                                                  \
-    hipLaunchKernelGGL((core_fwd_kernel<VAR, NW_, NT_, Tin>), grid, dim3(NT_), 0, s, a);             \
+    hipLaunchKernelGGL((core_fwd_kernel<VAR, NW_, NT_, Tin, Tbc>), grid, dim3(NT_), 0, s, a);        \
     return launch_status();                                                                          \
   }
 
-template <int VAR, typename Tin>
+// in_dtype of the launch functions below: 0 float, 1 bf16, 2 (complex and real scans only, which take no
+// bf16 B_t / C_t) u and delta bf16 with B_t / C_t already converted to float
+constexpr int IN_BF16_BC32 = 2;
+
+template <int VAR, typename Tin, typename Tbc>
 static int core_fwd_t(const FwdArgs& a, Cfg c, hipStream_t s) {
   const dim3 grid((unsigned)(a.B * a.ncg));
   AUSSM_FWD_CASE(1, 256) AUSSM_FWD_CASE(2, 256) AUSSM_FWD_CASE(4, 256) AUSSM_FWD_CASE(8, 256)
@@ -26,7 +31,13 @@ static int core_fwd_t(const FwdArgs& a, Cfg c, hipStream_t s) {
 
 template <int VAR>
 static int core_fwd_v(const FwdArgs& a, int in_dtype, Cfg c, hipStream_t s) {
-  return in_dtype == 1 ? core_fwd_t<VAR, bf16_t>(a, c, s) : core_fwd_t<VAR, float>(a, c, s);
+  if (in_dtype == 0) return core_fwd_t<VAR, float, float>(a, c, s);
+  if constexpr (VAR == VAR_UNITARY) {
+    if (in_dtype == 1) return core_fwd_t<VAR, bf16_t, bf16_t>(a, c, s);
+  } else {
+    if (in_dtype == IN_BF16_BC32) return core_fwd_t<VAR, bf16_t, float>(a, c, s);
+  }
+  return -2;
 }
 
 int run_core_fwd(int variant, const FwdArgs& a, int in_dtype, Cfg c, hipStream_t s) {
@@ -59,7 +70,7 @@ int run_unitary_bwd_generic(const UniBwdArgs& a, int in_dtype, Cfg c, hipStream_
 
 #define AUSSM_RBWD_CASE(NW_)                                                                         \
   if (nw == NW_) {                                                                                   \
-    hipLaunchKernelGGL((recompute_bwd_kernel<VAR, NW_, 256, Tin>), grid, dim3(256), 0, s, a);        \
+    hipLaunchKernelGGL((recompute_bwd_kernel<VAR, NW_, 256, Tin, float>), grid, dim3(256), 0, s, a); \
     done = true;                                                                                     \
   }
 
@@ -82,9 +93,34 @@ static int rec_bwd_t(const RecBwdArgs& args, hipStream_t s) {
 }
 
 int run_rec_bwd(int variant, const RecBwdArgs& a, int in_dtype, hipStream_t s) {
+  if (in_dtype != 0 && in_dtype != IN_BF16_BC32) return -2;      // B_t / C_t are float in every instance
   if (variant == VAR_COMPLEX)
-    return in_dtype == 1 ? rec_bwd_t<VAR_COMPLEX, bf16_t>(a, s) : rec_bwd_t<VAR_COMPLEX, float>(a, s);
-  return in_dtype == 1 ? rec_bwd_t<VAR_REAL, bf16_t>(a, s) : rec_bwd_t<VAR_REAL, float>(a, s);
+    return in_dtype ? rec_bwd_t<VAR_COMPLEX, bf16_t>(a, s) : rec_bwd_t<VAR_COMPLEX, float>(a, s);
+  return in_dtype ? rec_bwd_t<VAR_REAL, bf16_t>(a, s) : rec_bwd_t<VAR_REAL, float>(a, s);
+}
+
+void run_adjoint_seg(int variant, const AdjSegArgs& a, int in_dtype, unsigned grid, hipStream_t s) {
+  // (B_t / C_t are float in every instance; the complex kernel reads no u / delta at all)
+  if (variant == VAR_COMPLEX) {
+    hipLaunchKernelGGL((adjoint_seg_kernel<VAR_COMPLEX, float, float>), dim3(grid), dim3(256), 0, s, a);
+  } else {
+    if (in_dtype) hipLaunchKernelGGL((adjoint_seg_kernel<VAR_REAL, bf16_t, float>), dim3(grid), dim3(256), 0, s, a);
+    else hipLaunchKernelGGL((adjoint_seg_kernel<VAR_REAL, float, float>), dim3(grid), dim3(256), 0, s, a);
+  }
+}
+
+void run_bc_to_f32(const void* Bm, const void* Cm, float* oB, float* oC, size_t n, hipStream_t s) {
+  const size_t blocks = (n + 255) / 256;
+  hipLaunchKernelGGL(bc_to_f32_kernel, dim3((unsigned)(blocks < 2048 ? blocks : 2048)), dim3(256), 0, s,
+                     static_cast<const bf16_t*>(Bm), static_cast<const bf16_t*>(Cm), oB, oC, n);
+}
+
+void run_seg_carry_real(bool adjoint, float* seg, const float* ptot, const float* A, const float* first, float* last,
+                        int B, int D, int N, int ns, hipStream_t s) {
+  const size_t n = (size_t)B * D * N;
+  const dim3 grid((unsigned)((n + 255) / 256));
+  if (adjoint) hipLaunchKernelGGL(seg_carry_real_kernel<true>, grid, dim3(256), 0, s, seg, ptot, A, first, last, B, D, N, ns);
+  else hipLaunchKernelGGL(seg_carry_real_kernel<false>, grid, dim3(256), 0, s, seg, ptot, A, first, last, B, D, N, ns);
 }
 
 // marks an auxiliary buffer as NOT filled (a forward kernel that does not fill it ran)

@@ -19,10 +19,16 @@ inline int launch_status() {
 struct Cfg { int nw, nt; };
 
 // ---- k_generic.hip: vector-ALU scans, convolution, layout swap
+// in_dtype: 0 float, 1 bf16 (unitary only), 2 = u / delta bf16 and B_t / C_t float (complex and real only)
 int run_core_fwd(int variant, const FwdArgs& a, int in_dtype, Cfg c, hipStream_t s);
 int run_unitary_bwd_generic(const UniBwdArgs& a, int in_dtype, Cfg c, hipStream_t s);
 int run_rec_bwd(int variant, const RecBwdArgs& a, int in_dtype, hipStream_t s);
 void run_aux_invalidate(float* tag, hipStream_t s);
+// split of the complex / real scans along L: adjoint entering every segment, chain of the real scan's segments
+void run_adjoint_seg(int variant, const AdjSegArgs& a, int in_dtype, unsigned grid, hipStream_t s);
+void run_bc_to_f32(const void* Bm, const void* Cm, float* oB, float* oC, size_t n, hipStream_t s);   // bf16 -> float
+void run_seg_carry_real(bool adjoint, float* seg, const float* ptot, const float* A, const float* first, float* last,
+                        int B, int D, int N, int ns, hipStream_t s);
 int run_conv_fwd(const ConvArgs& a, hipStream_t s);
 int run_conv_bwd(const ConvArgs& a, hipStream_t s);
 int run_swap_last2(const SwapArgs& a, int B, hipStream_t s);

@@ -107,6 +107,42 @@ inline size_t round64(size_t n) { return (n + 63) & ~(size_t)63; }
 inline size_t seg_floats(int B, int D, int N, int L, int ns) {
   return ns > 1 ? round64((size_t)B * ns * seg_fine(L, ns) * D * (2 * N + 2)) : 0;
 }
+// The complex and the real scan split the same way (scan_seg_generic.h) when the call brings a workspace:
+// ns segments of ls steps (whole tiles and checkpoint blocks), the last one possibly shorter.
+constexpr int GSPLIT_MAX = 64;
+struct GSplit { int ns, ls; };
+inline GSplit generic_split(int B, int D, int L, int ck, bool use_cap) {
+  const long long wgs = (long long)B * ((D + CH - 1) / CH);
+  const int cap = use_cap ? opt(AUSSM_OPT_SPLIT_CAP) : -1;
+  if (wgs >= SPLIT_MIN_WGS || cap == 0 || cap == 1) return GSplit{1, L};
+  int want = (int)((SPLIT_TARGET_WGS + wgs - 1) / wgs);
+  if (want > GSPLIT_MAX) want = GSPLIT_MAX;
+  if (cap > 1 && want > cap) want = cap;
+  const int unit = ck > XT ? ck : XT;
+  int ls = ((L + want - 1) / want + unit - 1) / unit * unit;
+  if (ls < SPLIT_MIN_LEN) ls = (SPLIT_MIN_LEN + unit - 1) / unit * unit;
+  const int ns = (L + ls - 1) / ls;
+  return ns > 1 ? GSplit{ns, ls} : GSplit{1, L};
+}
+inline size_t generic_split_floats(int variant, int B, int D, int N, int L, int ck) {
+  const GSplit sp = generic_split(B, D, L, ck, false);
+  const int C = variant == VAR_REAL ? 1 : 2;
+  return sp.ns > 1 ? round64((size_t)B * sp.ns * D * (N * C + 2)) : 0;
+}
+// ... and their kernels take B_t / C_t as float: bf16 rows are converted once per call, behind the segments
+inline size_t generic_bc_floats(int variant, int B, int N, int L, int in_dtype) {
+  return in_dtype == AUSSM_BF16 ? round64((size_t)B * N * L * (variant == VAR_REAL ? 1 : 2)) : 0;
+}
+struct BcF32 { const void* Bm; const void* Cm; int in_dtype; };
+inline BcF32 generic_bc(int variant, const void* Bm, const void* Cm, float* ws, int B, int D, int N, int L, int ck,
+                        int in_dtype, hipStream_t s) {
+  if (in_dtype != AUSSM_BF16) return BcF32{Bm, Cm, 0};
+  const size_t n = generic_bc_floats(variant, B, N, L, in_dtype);
+  float* fB = ws + generic_split_floats(variant, B, D, N, L, ck);
+  run_bc_to_f32(Bm, Cm, fB, fB + n, (size_t)B * N * L * (variant == VAR_REAL ? 1 : 2), s);
+  return BcF32{fB, fB + n, 2};
+}
+
 // Workspace of the prepared operands: one image per (batch element, chunk), sized for the larger
 // (backward) image; a forward and a backward call each write their own images into it.
 inline size_t img_floats(int B, int N, int L, int ck) {
@@ -183,6 +219,54 @@ int launch_unitary_fwd(FwdArgs a, int in_dtype, hipStream_t s, AuxLayout ws) {
   return run_xdl_fwd(mode, a, in_dtype, s);
 }
 
+// Complex and real scans: with a workspace and few (batch, channel group) pairs, split along the sequence.
+int launch_generic_fwd(int variant, FwdArgs a, int in_dtype, float* ws, hipStream_t s) {
+  if (in_dtype == AUSSM_BF16 && !ws) return AUSSM_E_NULL;
+  if (misaligned(ws, 16)) return AUSSM_E_ALIGN;
+  const BcF32 bc = generic_bc(variant, a.Bm, a.Cm, ws, a.B, a.D, a.N, a.L, a.ck, in_dtype, s);
+  a.Bm = bc.Bm; a.Cm = bc.Cm; in_dtype = bc.in_dtype;
+  const Cfg cfg = pick_cfg(a.N, 8);
+  const GSplit sp = ws ? generic_split(a.B, a.D, a.L, a.ck, true) : GSplit{1, a.L};
+  if (sp.ns > 1) {
+    const int B = a.B, C = variant == VAR_REAL ? 1 : 2;
+    float* seg = ws;
+    float* ptot = seg + (size_t)B * sp.ns * a.D * a.N * C;
+    // 1. end state of every segment from a zero state (no outputs) and the product of its a_l
+    FwdArgs z = a;
+    z.B = B * sp.ns; z.L = sp.ls; z.ns = sp.ns;
+    z.y = nullptr; z.z = nullptr; z.Dskip = nullptr; z.h0 = nullptr; z.hL = seg; z.hck = nullptr; z.ptot = ptot;
+    if (int e = run_core_fwd(variant, z, in_dtype, cfg, s)) return e;
+    // 2. the state that enters every segment; the state after the last one is the call's hL
+    if (variant == VAR_COMPLEX) run_seg_carry_fwd(seg, ptot, a.h0, a.hL, B, a.D, a.N, sp.ns, s);
+    else run_seg_carry_real(false, seg, ptot, a.A, a.h0, a.hL, B, a.D, a.N, sp.ns, s);
+    // 3. the scan proper over (batch, segment) pairs
+    a.B = B * sp.ns; a.L = sp.ls; a.ns = sp.ns; a.h0 = seg; a.hL = nullptr;
+  }
+  return run_core_fwd(variant, a, in_dtype, cfg, s);
+}
+
+int launch_generic_bwd(int variant, RecBwdArgs a, int in_dtype, float* ws, hipStream_t s) {
+  if (in_dtype == AUSSM_BF16 && !ws) return AUSSM_E_NULL;
+  if (misaligned(ws, 16)) return AUSSM_E_ALIGN;
+  const BcF32 bc = generic_bc(variant, a.Bm, a.Cm, ws, a.B, a.D, a.N, a.L, REC_CK, in_dtype, s);
+  a.Bm = bc.Bm; a.Cm = bc.Cm; in_dtype = bc.in_dtype;
+  const GSplit sp = ws ? generic_split(a.B, a.D, a.L, REC_CK, true) : GSplit{1, a.L};
+  if (sp.ns > 1) {
+    const int B = a.B, C = variant == VAR_REAL ? 1 : 2;
+    float* seg = ws;
+    float* ptot = seg + (size_t)B * sp.ns * a.D * a.N * C;
+    AdjSegArgs g{};
+    g.dy = a.dy; g.z = a.z; g.delta = a.delta; g.theta = a.theta; g.rho = a.rho; g.A = a.A; g.Cm = a.Cm;
+    g.delta_bias = a.delta_bias; g.out = seg; g.ptot = ptot;
+    g.D = a.D; g.N = a.N; g.L = sp.ls; g.ld = a.L; g.ns = sp.ns; g.ncg = a.ncg; g.delta_softplus = a.delta_softplus;
+    run_adjoint_seg(variant, g, in_dtype, (unsigned)(B * sp.ns * a.ncg), s);
+    if (variant == VAR_COMPLEX) run_seg_carry_bwd(seg, ptot, a.dhL, a.dh0, B, a.D, a.N, sp.ns, s);
+    else run_seg_carry_real(true, seg, ptot, a.A, a.dhL, a.dh0, B, a.D, a.N, sp.ns, s);
+    a.B = B * sp.ns; a.L = sp.ls; a.ns = sp.ns; a.dhL = seg; a.dh0 = nullptr;
+  }
+  return run_rec_bwd(variant, a, in_dtype, s);
+}
+
 // ---- static workspace of aussm_unitary_fwd_static ---------------------------------------------
 // A file-scope device array: every GPU the library runs on holds its own copy at its own address
 // until the process ends.  In host code the array's NAME is only a handle for the runtime, not a
@@ -252,6 +336,12 @@ size_t aussm_unitary_aux_floats(int B, int D, int N, int L, int ck) {
   return (size_t)B * D * L + AUX_PAD + seg_floats(B, D, N, L, seg_capacity(B, D, N, L, ck)) + img_floats(B, N, L, ck);
 }
 
+size_t aussm_scan_workspace_floats(int variant, int B, int D, int N, int L, int ck, int in_dtype) {
+  if (B < 1 || D < 1 || N < 1 || L < 1 || (variant != VAR_COMPLEX && variant != VAR_REAL)) return 0;
+  if (ck != AUSSM_TILE / 2 && (ck < AUSSM_TILE || ck % AUSSM_TILE != 0)) return 0;
+  return generic_split_floats(variant, B, D, N, L, ck) + 2 * generic_bc_floats(variant, B, N, L, in_dtype);
+}
+
 int aussm_unitary_kernel_mode(int backward, int B, int D, int N, int L, int ck, int in_dtype, int urep, int have_aux) {
   if (check_common(B, D, N, L, ck, in_dtype) != AUSSM_OK || urep < 1) return 0;
   const bool have_img = have_aux && img_floats(B, N, L, ck) > 0;
@@ -313,7 +403,7 @@ int aussm_unitary_fwd_static(const void* u, const void* delta, const float* thet
 
 int aussm_complex_fwd(const void* u, const void* delta, const float* rho, const float* theta, const void* Bc,
                       const void* Cc, const float* Dskip, const float* z, const float* h0, float* y, float* hL,
-                      float* hck, int B, int D, int N, int L, int ck, int in_dtype, void* stream) {
+                      float* hck, float* workspace, int B, int D, int N, int L, int ck, int in_dtype, void* stream) {
   if (int e = check_common(B, D, N, L, ck, in_dtype)) return e;
   if (!u || !delta || !rho || !theta || !Bc || !Cc) return AUSSM_E_NULL;
   const size_t ca = in_dtype == AUSSM_BF16 ? 4 : 8;
@@ -323,12 +413,12 @@ int aussm_complex_fwd(const void* u, const void* delta, const float* rho, const 
   a.h0 = h0; a.y = y; a.hL = hL; a.hck = hck;
   a.B = B; a.D = D; a.N = N; a.L = L; a.ck = ck; a.nck = (L + ck - 1) / ck; a.ncg = (D + CH - 1) / CH;
   a.ld = L; a.ns = 1; a.hs = 1; a.ho = 0; a.urep = 1;
-  return run_core_fwd(VAR_COMPLEX, a, in_dtype, pick_cfg(a.N, 8), (hipStream_t)stream);
+  return launch_generic_fwd(VAR_COMPLEX, a, in_dtype, workspace, (hipStream_t)stream);
 }
 
 int aussm_real_fwd(const void* u, const void* delta, const float* A, const void* Bm, const void* Cm,
                    const float* Dskip, const float* z, const float* delta_bias, int delta_softplus,
-                   const float* h0, float* y, float* hL, float* hck,
+                   const float* h0, float* y, float* hL, float* hck, float* workspace,
                    int B, int D, int N, int L, int ck, int in_dtype, void* stream) {
   if (int e = check_common(B, D, N, L, ck, in_dtype)) return e;
   if (!u || !delta || !A || !Bm || !Cm) return AUSSM_E_NULL;
@@ -338,7 +428,7 @@ int aussm_real_fwd(const void* u, const void* delta, const float* A, const void*
   a.h0 = h0; a.y = y; a.hL = hL; a.hck = hck;
   a.B = B; a.D = D; a.N = N; a.L = L; a.ck = ck; a.nck = (L + ck - 1) / ck; a.ncg = (D + CH - 1) / CH;
   a.ld = L; a.ns = 1; a.hs = 1; a.ho = 0; a.urep = 1;
-  return run_core_fwd(VAR_REAL, a, in_dtype, pick_cfg(a.N, 8), (hipStream_t)stream);
+  return launch_generic_fwd(VAR_REAL, a, in_dtype, workspace, (hipStream_t)stream);
 }
 
 int aussm_unitary_bwd(const float* dy, const float* dhL, const void* u, const void* delta, const float* theta,
@@ -405,7 +495,7 @@ int aussm_complex_bwd(const float* dy, const float* dhL, const void* u, const vo
                       const float* theta, const void* Bc, const void* Cc, const float* Dskip,
                       const float* h0, const float* hck,
                       float* du, float* ddelta, float* drho, float* dtheta, float* dB, float* dC,
-                      float* dD, float* dh0, const float* z, float* dz,
+                      float* dD, float* dh0, const float* z, float* dz, float* workspace,
                       int B, int D, int N, int L, int ck, int in_dtype, void* stream) {
   if (int e = check_common(B, D, N, L, ck, in_dtype)) return e;
   if (ck != REC_CK) return AUSSM_E_CK;
@@ -421,14 +511,15 @@ int aussm_complex_bwd(const float* dy, const float* dhL, const void* u, const vo
   if ((z == nullptr) != (dz == nullptr)) return AUSSM_E_NULL;
   a.z = z; a.dz = dz;
   a.B = B; a.D = D; a.N = N; a.L = L; a.nck = (L + ck - 1) / ck; a.ncg = (D + CH - 1) / CH;
-  return run_rec_bwd(VAR_COMPLEX, a, in_dtype, (hipStream_t)stream);
+  a.ld = L; a.ns = 1;
+  return launch_generic_bwd(VAR_COMPLEX, a, in_dtype, workspace, (hipStream_t)stream);
 }
 
 int aussm_real_bwd(const float* dy, const float* dhL, const void* u, const void* delta, const float* A,
                    const void* Bm, const void* Cm, const float* Dskip, const float* delta_bias,
                    int delta_softplus, const float* h0, const float* hck,
                    float* du, float* ddelta, float* dA, float* dB, float* dC, float* dD, float* dh0,
-                   const float* z, float* dz,
+                   const float* z, float* dz, float* workspace,
                    int B, int D, int N, int L, int ck, int in_dtype, void* stream) {
   if (int e = check_common(B, D, N, L, ck, in_dtype)) return e;
   if (ck != REC_CK) return AUSSM_E_CK;
@@ -440,7 +531,8 @@ int aussm_real_bwd(const float* dy, const float* dhL, const void* u, const void*
   if ((z == nullptr) != (dz == nullptr)) return AUSSM_E_NULL;
   a.z = z; a.dz = dz;
   a.B = B; a.D = D; a.N = N; a.L = L; a.nck = (L + ck - 1) / ck; a.ncg = (D + CH - 1) / CH;
-  return run_rec_bwd(VAR_REAL, a, in_dtype, (hipStream_t)stream);
+  a.ld = L; a.ns = 1;
+  return launch_generic_bwd(VAR_REAL, a, in_dtype, workspace, (hipStream_t)stream);
 }
 
 int aussm_causal_conv1d_fwd(const float* x, const float* w, const float* bias, float* y,

@@ -36,10 +36,14 @@ struct FwdArgs {
   float* hL;                // [B,D,N,C] or null
   float* hck;               // [B,nck,N,C,D] or null
   float* aux;               // unitary, optional: Im(P_t S_t) [B,D,L] followed by a validity tag
+  float* ptot;              // vector-ALU kernels, optional: [B,D,2] product of the a_l of the call's L steps
+                            // (complex: re, im; real: the sum of delta after bias / softplus, 0)
   int B, D, N, L, ck, nck, ncg, delta_softplus;
-  int ld, ns;                // matrix-core unitary kernels: row stride of the [.., L] tensors and segments per
-                             // sequence (B then counts batch x segment pairs and L is the segment length)
-  int hs, ho;                // ... and h0 of pair b is entry b * hs + ho of the state array
+  int ld, ns;                // row stride of the [.., L] tensors and segments per sequence: B then counts
+                             // (batch, segment) pairs and L is the segment length.  The vector-ALU kernels take a
+                             // shorter last segment (ld not a multiple of L) and keep nck = checkpoints of a whole
+                             // sequence; h0 / hL / ptot are indexed by the pair
+  int hs, ho;                // matrix-core kernels: h0 of pair b is entry b * hs + ho of the state array
   int urep;                  // generic kernels: u and delta are [B / urep, D, L], shared by urep consecutive batch elements
 };
 
@@ -89,11 +93,30 @@ struct RecBwdArgs {
   const float* z;           // [B,D,L] or null: the output was gated, y = y_pre silu(z); dy is the gradient of y
   float* dz;                // [B,D,L] (with z)
   int B, D, N, L, nck, ncg, delta_softplus;
+  // Split along the sequence: ld = row stride of the [.., L] tensors (the whole sequence), ns segments per
+  // sequence, B counts (batch, segment) pairs, L is the segment length (a multiple of 16; the last segment may
+  // be shorter), nck the checkpoints of a whole sequence; dhL / dh0 are indexed by the pair, h0 by the batch element.
+  int ld, ns;
   // A launch handles the states nbase .. nbase + 15 (a workgroup's four wavefronts of up to four states);
   // larger N takes one launch per block of 16 states.  accum: a later block - the sums over the states
   // (du, ddelta, dtheta, drho) are added to what the earlier blocks wrote, and the terms that do not
   // depend on the state (the D skip, dD) are left out.
   int nbase, accum;
+};
+
+// Adjoint of the state entering a segment, from a zero adjoint at its end (complex and real scans)
+struct AdjSegArgs {
+  const float* dy;          // [B,D,ld]
+  const float* z;           // [B,D,ld] or null
+  const void* delta;        // [B,D,ld] Tin (real)
+  const float* theta;       // [B,D,ld] (complex)
+  const float* rho;         // [B,D,ld] (complex)
+  const float* A;           // [D,N] (real)
+  const void* Cm;           // [B,N,ld(,2)] Tin
+  const float* delta_bias;  // [D] or null (real)
+  float* out;               // [B*ns,D,N,C]
+  float* ptot;              // [B*ns,D,2]  as FwdArgs::ptot
+  int D, N, L, ld, ns, ncg, delta_softplus;   // L: segment length (the last one may be shorter)
 };
 
 struct SegArgs {

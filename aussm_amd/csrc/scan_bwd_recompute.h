@@ -67,7 +67,7 @@ __device__ __forceinline__ f32x8 ld_r8_tile(const Tin* p, size_t row, int t0, in
   else return ld_r8_safe(p, row, t0, L);
 }
 
-template <int VAR, int NW, int NT, typename Tin>
+template <int VAR, int NW, int NT, typename Tin, typename Tbc = Tin>
 __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
   static_assert(VAR == VAR_COMPLEX || VAR == VAR_REAL, "unitary has its own kernel");
   constexpr int C = (VAR == VAR_REAL) ? 1 : 2;
@@ -86,8 +86,13 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
 
   const int tid = threadIdx.x, lane = tid & 63, wave = wave_index();
   const int wg = xcd_remap(blockIdx.x, gridDim.x);
-  const int b = wg / p.ncg, d0 = (wg % p.ncg) * CH;
-  const int N = p.N, L = p.L, D = p.D;
+  // vb: (batch, segment) pair of a launch that is split along the sequence, else the batch element
+  const int vb = wg / p.ncg, d0 = (wg % p.ncg) * CH;
+  const int b = vb / p.ns, sg = vb - b * p.ns;
+  const int lbeg = sg * p.L, ld = p.ld;
+  const int tile0 = lbeg / RT;                              // index of the segment's first tile in the sequence
+  const int N = p.N, D = p.D;
+  const int L = (ld - lbeg < p.L) ? ld - lbeg : p.L;        // steps of this segment
   const int n0 = p.nbase + wave * NW;
   const bool active = n0 < N;
   const int nwa = (N - p.nbase + NW - 1) / NW;         // wavefronts of this launch that own existing states
@@ -96,11 +101,11 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
 
   const Tin* __restrict__ gu = static_cast<const Tin*>(p.u);
   const Tin* __restrict__ gdl = static_cast<const Tin*>(p.delta);
-  const Tin* __restrict__ gB = static_cast<const Tin*>(p.Bm);
-  const Tin* __restrict__ gC = static_cast<const Tin*>(p.Cm);
+  const Tbc* __restrict__ gB = static_cast<const Tbc*>(p.Bm);
+  const Tbc* __restrict__ gC = static_cast<const Tbc*>(p.Cm);
   float* red = s_red + wave * 64 * RED_RS;
   float4* part = s_part + wave * RT * TS;
-  const size_t row_base = ((size_t)b * N + n0) * L;
+  const size_t row_base = ((size_t)b * N + n0) * ld + lbeg;
 
   // ---- per-lane constants and accumulators
   float a2[NW], an[NW], dAacc[NW], gr[NW], gi[NW];
@@ -111,7 +116,7 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
     if (dok && n < N) {
       if (VAR == VAR_REAL) { an[k] = p.A[(size_t)d * N + n]; a2[k] = an[k] * LOG2E; }
       if (p.dhL) {
-        const size_t o = (((size_t)b * D + d) * N + n) * C;
+        const size_t o = (((size_t)vb * D + d) * N + n) * C;
         gr[k] = p.dhL[o];
         if (C == 2) gi[k] = p.dhL[o + 1];
       }
@@ -126,8 +131,8 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
       const int n = n0 + k;
       s.r[k] = 0.f; s.i[k] = 0.f;
       if (dok && n < N) {
-        if (it > 0) {
-          const size_t o = ((((size_t)b * p.nck + (it - 1)) * N + n) * C) * D + d;
+        if (tile0 + it > 0) {
+          const size_t o = ((((size_t)b * p.nck + (tile0 + it - 1)) * N + n) * C) * D + d;
           s.r[k] = p.hck[o];
           if (C == 2) s.i[k] = p.hck[o + D];
         } else if (p.h0) {
@@ -154,7 +159,7 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
   for (int k = 0; k < E; ++k) {
     const int dd = d0 + row0 + k * RSTEP;
     rowok[k] = dd < D;
-    goff[k] = ((size_t)b * D + (rowok[k] ? dd : 0)) * L;
+    goff[k] = ((size_t)b * D + (rowok[k] ? dd : 0)) * ld + lbeg;
     dsk[k] = (p.Dskip && rowok[k]) ? p.Dskip[dd] : 0.f;
     dbias[k] = (VAR == VAR_REAL && p.delta_bias && rowok[k]) ? p.delta_bias[dd] : 0.f;
     accD[k] = 0.f;
@@ -247,7 +252,7 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
         for (int k = 0; k < NW; ++k) {
           if (FULL || n0 + k < N) {                // wave-uniform; FULL: all NW states of the wavefront exist
             if constexpr (VAR == VAR_REAL) {
-              const f32x8 bc = ld_r8_tile<FULL>(gB, brow + (size_t)k * L - l0, l0 + g * TG, L);
+              const f32x8 bc = ld_r8_tile<FULL>(gB, brow + (size_t)k * ld - l0, l0 + g * TG, L);
 #pragma unroll
               for (int t = 0; t < TG; ++t) {
                 const float a = __builtin_amdgcn_exp2f(rx[t] * a2[k]);
@@ -255,7 +260,7 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
                 hsr[g * TG + t][k] = cr_[k];
               }
             } else {
-              const f32x16 bc = ld_c8_tile<FULL>(gB, brow + (size_t)k * L - l0, l0 + g * TG, L);
+              const f32x16 bc = ld_c8_tile<FULL>(gB, brow + (size_t)k * ld - l0, l0 + g * TG, L);
 #pragma unroll
               for (int t = 0; t < TG; ++t) {
                 const float nr = fmaf(rx[t], cr_[k], fmaf(-ry[t], ci_[k], bc[2 * t] * rz[t]));
@@ -290,8 +295,8 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
         for (int k = 0; k < NW; ++k) {
           if (FULL || n0 + k < N) {                // wave-uniform; FULL: all NW states of the wavefront exist
             if constexpr (VAR == VAR_REAL) {
-              const f32x8 bc = ld_r8_tile<FULL>(gB, brow + (size_t)k * L - l0, l0 + g * TG, L);
-              const f32x8 cc = ld_r8_tile<FULL>(gC, brow + (size_t)k * L - l0, l0 + g * TG, L);
+              const f32x8 bc = ld_r8_tile<FULL>(gB, brow + (size_t)k * ld - l0, l0 + g * TG, L);
+              const f32x8 cc = ld_r8_tile<FULL>(gC, brow + (size_t)k * ld - l0, l0 + g * TG, L);
               constexpr int VB = 0;                // filled below per row slot
               (void)VB;
               const int slot = (RPT == 2) ? (k & 1) : 0;
@@ -312,8 +317,8 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
                 gr[k] *= a;
               }
             } else {
-              const f32x16 bc = ld_c8_tile<FULL>(gB, brow + (size_t)k * L - l0, l0 + g * TG, L);
-              const f32x16 cc = ld_c8_tile<FULL>(gC, brow + (size_t)k * L - l0, l0 + g * TG, L);
+              const f32x16 bc = ld_c8_tile<FULL>(gB, brow + (size_t)k * ld - l0, l0 + g * TG, L);
+              const f32x16 cc = ld_c8_tile<FULL>(gC, brow + (size_t)k * ld - l0, l0 + g * TG, L);
 #pragma unroll
               for (int t = TG - 1; t >= 0; --t) {
                 const int tt = g * TG + t;
@@ -355,7 +360,7 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
         };
     if (active) {
       // (bf16 rows start at even element offsets when L is even: wide loads stay 4-byte aligned)
-      const bool full = (l0 + RT <= L) && (n0 + NW <= N) && (sizeof(Tin) == 4 || (L & 1) == 0);
+      const bool full = (l0 + RT <= L) && (n0 + NW <= N) && (sizeof(Tbc) == 4 || (ld & 1) == 0);
       if (full) tile_body(std::true_type{});
       else tile_body(std::false_type{});
     }
@@ -383,14 +388,14 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
             const int tt = t + (c & 7);
             float* dst = ((c >> 3) & 1) ? p.dC : p.dB;
             if (n0 + k < N && (RPT == 2 || c < 16) && tt < L)
-              atomicAdd(dst + row_base + (size_t)k * L + tt, rres[g * (NW / RPT) + j]);
+              atomicAdd(dst + row_base + (size_t)k * ld + tt, rres[g * (NW / RPT) + j]);
           } else {
             // columns: 16 floats of dB (re, im interleaved), then 16 of dC
             const int k = j;
             const int tt = t + ((c & 15) >> 1);
             float* dst = (c < 16) ? p.dB : p.dC;
             if (n0 + k < N && tt < L)
-              atomicAdd(dst + 2 * (row_base + (size_t)k * L + t) + (c & 15), rres[g * (NW / RPT) + j]);
+              atomicAdd(dst + 2 * (row_base + (size_t)k * ld + t) + (c & 15), rres[g * (NW / RPT) + j]);
           }
         }
       (void)brow;
@@ -439,7 +444,7 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
       const int n = n0 + k;
       if (n < N) {
         if (p.dh0) {
-          const size_t o = (((size_t)b * D + d) * N + n) * C;
+          const size_t o = (((size_t)vb * D + d) * N + n) * C;
           p.dh0[o] = gr[k];
           if (C == 2) p.dh0[o + 1] = gi[k];
         }

@@ -9,8 +9,10 @@
 namespace aussm {
 
 
-// VAR: variant.  NW: states per wavefront.  NT: threads per workgroup.  Tin: float or bf16_t.
-template <int VAR, int NW, int NT, typename Tin>
+// VAR: variant.  NW: states per wavefront.  NT: threads per workgroup.  Tin: float or bf16_t (u, delta).
+// Tbc: type of B_t / C_t (bf16 rows cost scalar-ALU conversions in the scan; the complex and real entry
+// points convert them to float once per call instead).
+template <int VAR, int NW, int NT, typename Tin, typename Tbc = Tin>
 __global__ __launch_bounds__(NT) void core_fwd_kernel(const FwdArgs p) {
   constexpr int C = (VAR == VAR_REAL) ? 1 : 2;   // floats per state
   constexpr int NWV = NT / 64;                   // wavefronts per workgroup
@@ -24,8 +26,13 @@ __global__ __launch_bounds__(NT) void core_fwd_kernel(const FwdArgs p) {
 
   const int tid = threadIdx.x, lane = tid & 63, wave = wave_index();
   const int wg = xcd_remap(blockIdx.x, gridDim.x);
-  const int b = wg / p.ncg, d0 = (wg % p.ncg) * CH;
-  const int N = p.N, L = p.L, D = p.D;
+  // vb: (batch, segment) pair of a launch that is split along the sequence (p.ns segments of p.L
+  // steps, the last one possibly shorter), else the batch element itself
+  const int vb = wg / p.ncg, d0 = (wg % p.ncg) * CH;
+  const int b = vb / p.ns, sg = vb - b * p.ns;
+  const int lbeg = sg * p.L, ld = p.ld;
+  const int N = p.N, D = p.D;
+  const int L = (ld - lbeg < p.L) ? ld - lbeg : p.L;      // steps of this segment
   const int n0 = wave * NW;
   const bool active = n0 < N;                    // wave-uniform
   const int nwa = (N + NW - 1) / NW;             // wavefronts that own states
@@ -34,11 +41,11 @@ __global__ __launch_bounds__(NT) void core_fwd_kernel(const FwdArgs p) {
 
   // u and delta may be shared by p.urep consecutive batch elements (tensors [B / urep, D, L]): every
   // address below is formed for batch element b, so their base steps back by the difference
-  const size_t uback = (size_t)(b - b / p.urep) * p.D * p.L;
+  const size_t uback = (size_t)(b - b / p.urep) * p.D * ld;
   const Tin* __restrict__ gu = static_cast<const Tin*>(p.u) - uback;
   const Tin* __restrict__ gdl = static_cast<const Tin*>(p.delta) - uback;
-  const Tin* __restrict__ gB = static_cast<const Tin*>(p.Bm);
-  const Tin* __restrict__ gC = static_cast<const Tin*>(p.Cm);
+  const Tbc* __restrict__ gB = static_cast<const Tbc*>(p.Bm);
+  const Tbc* __restrict__ gC = static_cast<const Tbc*>(p.Cm);
 
   // ---- scan-side state (lane == channel)
   float hr[NW], hi[NW], a2[NW];
@@ -48,7 +55,7 @@ __global__ __launch_bounds__(NT) void core_fwd_kernel(const FwdArgs p) {
     hr[k] = 0.f; hi[k] = 0.f; a2[k] = 0.f;
     if (dok && n < N) {
       if (p.h0) {
-        const size_t o = (((size_t)b * D + d) * N + n) * C;
+        const size_t o = (((size_t)vb * D + d) * N + n) * C;
         hr[k] = p.h0[o];
         if (C == 2) hi[k] = p.h0[o + C - 1];
       }
@@ -76,7 +83,7 @@ __global__ __launch_bounds__(NT) void core_fwd_kernel(const FwdArgs p) {
     inrow[k] = srow[k] < CH;                     // this thread has a row in this pass
     const int dd = d0 + srow[k];
     rowok[k] = inrow[k] && dd < D;
-    goff[k] = ((size_t)b * D + (rowok[k] ? dd : 0)) * L;
+    goff[k] = ((size_t)b * D + (rowok[k] ? dd : 0)) * ld + lbeg;
     dsk[k] = (p.Dskip && rowok[k]) ? p.Dskip[dd] : 0.f;
     dbias[k] = (VAR == VAR_REAL && p.delta_bias && rowok[k]) ? p.delta_bias[dd] : 0.f;
     rdy.u[k].zero(); rdy.dl[k].zero(); rdy.th[k].zero(); rdy.rho[k].zero(); rdy.z[k].zero();
@@ -84,7 +91,7 @@ __global__ __launch_bounds__(NT) void core_fwd_kernel(const FwdArgs p) {
   }
   // 16-byte accesses need every row start (L % 4 == 0) and every tensor base aligned
   auto al = [](const void* q, size_t a) { return q == nullptr || (reinterpret_cast<uintptr_t>(q) % a) == 0; };
-  const bool vec = (L % 4 == 0) && al(p.u, 4 * sizeof(Tin)) && al(p.delta, 4 * sizeof(Tin)) && al(p.theta, 16) &&
+  const bool vec = (ld % 4 == 0) && (L % 4 == 0) && al(p.u, 4 * sizeof(Tin)) && al(p.delta, 4 * sizeof(Tin)) && al(p.theta, 16) &&
                    al(p.rho, 16) && al(p.z, 16) && al(p.y, 16);
 
   auto load_tile = [&](RawTile& r, int l0) {
@@ -124,17 +131,23 @@ __global__ __launch_bounds__(NT) void core_fwd_kernel(const FwdArgs p) {
   // the scalar cache and pay the full memory latency.  Instead the lines of the NEXT tile are
   // touched here, a whole tile ahead, while the vector ALUs are busy with the staging maths.
   constexpr bool WARM = NW <= 4;
-  constexpr int RB = (int)sizeof(Tin) * C;
+  constexpr int RB = (int)sizeof(Tbc) * C;
   const bool full_group = active && n0 + NW <= N;
   TileWarm<WARM ? NW : 1, RB> warm;
+  const size_t bc_row = ((size_t)b * N + n0) * ld + lbeg;   // B_t / C_t: row n0, first step of the segment
   if (WARM && full_group && T <= L) {
-    warm.issue(gB, gC, ((size_t)b * N + n0) * L, L);
+    warm.issue(gB, gC, bc_row, ld);
     warm.retire();
   }
 
+  // product of the a_l over the segment (complex) or sum of the step sizes (real), kept by wavefront 0
+  // of a launch that wants it (a split launch chains its segments with it)
+  const bool want_tot = p.ptot != nullptr && wave == 0;   // wave-uniform
+  float fr = (VAR == VAR_REAL) ? 0.f : 1.f, fi = 0.f;
+
   for (int l0 = 0; l0 < L; l0 += T) {
     const bool warm_next = WARM && full_group && l0 + 2 * T <= L;
-    if (warm_next) warm.issue(gB, gC, ((size_t)b * N + n0) * L + l0 + T, L);
+    if (warm_next) warm.issue(gB, gC, bc_row + l0 + T, ld);
     // ---- stage: convert this tile once per (channel, t) and transpose into LDS
     float yin[PASS][4], gate[PASS][4];
 #pragma unroll
@@ -165,11 +178,11 @@ __global__ __launch_bounds__(NT) void core_fwd_kernel(const FwdArgs p) {
 
     // ---- scan: lane == channel, sequential over the tile's timesteps
     const int tmax = (L - l0 < T) ? (L - l0) : T;
-    const size_t brow = ((size_t)b * N + n0) * L + l0;
+    const size_t brow = bc_row + l0;
     // fast path: a full tile and a full group of states.  (bf16 real rows need an even offset
     // so that the 8-element scalar load is 4-byte aligned.)
     const bool fast = tmax == T && n0 + NW <= N &&
-                      !(VAR == VAR_REAL && sizeof(Tin) == 2 && (L & 1));
+                      !(VAR == VAR_REAL && sizeof(Tbc) == 2 && (ld & 1));
     float mr[NW], mi[NW];                        // state after the first half of the tile
 #pragma unroll
     for (int k = 0; k < NW; ++k) { mr[k] = 0.f; mi[k] = 0.f; }
@@ -192,6 +205,10 @@ __global__ __launch_bounds__(NT) void core_fwd_kernel(const FwdArgs p) {
           float yacc[TG], nx[TG], ny[TG];
 #pragma unroll
           for (int t = 0; t < TG; ++t) yacc[t] = 0.f;
+          if (want_tot) {
+#pragma unroll
+            for (int t = 0; t < TG; ++t) fr += rx[t];
+          }
 #pragma unroll
           for (int k = 0; k < NW; ++k) {
             const f32x8 bc = bn, cc = cn;
@@ -199,8 +216,8 @@ __global__ __launch_bounds__(NT) void core_fwd_kernel(const FwdArgs p) {
             touch_uniform(cc[0]);
             sched_fence();
             if (k + 1 < NW) {
-              bn = ld_r8(gB, brow + (size_t)(k + 1) * L + g * TG);
-              cn = ld_r8(gC, brow + (size_t)(k + 1) * L + g * TG);
+              bn = ld_r8(gB, brow + (size_t)(k + 1) * ld + g * TG);
+              cn = ld_r8(gC, brow + (size_t)(k + 1) * ld + g * TG);
             } else if (g + 1 < T / TG) {
               bn = ld_r8(gB, brow + (g + 1) * TG);
               cn = ld_r8(gC, brow + (g + 1) * TG);
@@ -237,6 +254,14 @@ __global__ __launch_bounds__(NT) void core_fwd_kernel(const FwdArgs p) {
           float yacc[TG], nx[TG], ny[TG], nz[TG];
 #pragma unroll
           for (int t = 0; t < TG; ++t) yacc[t] = 0.f;
+          if (want_tot) {
+#pragma unroll
+            for (int t = 0; t < TG; ++t) {
+              const float nr = fmaf(fr, rx[t], -fi * ry[t]);
+              fi = fmaf(fr, ry[t], fi * rx[t]);
+              fr = nr;
+            }
+          }
 #pragma unroll
           for (int k = 0; k < NW; ++k) {
             const f32x16 bc = bn, cc = cn;
@@ -244,8 +269,8 @@ __global__ __launch_bounds__(NT) void core_fwd_kernel(const FwdArgs p) {
             touch_uniform(cc[0]);
             sched_fence();
             if (k + 1 < NW) {
-              bn = ld_c8(gB, brow + (size_t)(k + 1) * L + g * TG);
-              cn = ld_c8(gC, brow + (size_t)(k + 1) * L + g * TG);
+              bn = ld_c8(gB, brow + (size_t)(k + 1) * ld + g * TG);
+              cn = ld_c8(gC, brow + (size_t)(k + 1) * ld + g * TG);
             } else if (g + 1 < T / TG) {
               bn = ld_c8(gB, brow + (g + 1) * TG);
               cn = ld_c8(gC, brow + (g + 1) * TG);
@@ -283,10 +308,19 @@ __global__ __launch_bounds__(NT) void core_fwd_kernel(const FwdArgs p) {
       for (int t = 0; t < tmax; ++t) {
         const float4 v = s_in[t * TS + lane];
         float yacc = 0.f;
+        if (want_tot) {
+          if (VAR == VAR_REAL) {
+            fr += v.x;
+          } else {
+            const float nr = fmaf(fr, v.x, -fi * v.y);
+            fi = fmaf(fr, v.y, fi * v.x);
+            fr = nr;
+          }
+        }
 #pragma unroll
         for (int k = 0; k < NW; ++k) {
           if (n0 + k < N) {                      // wave-uniform
-            const size_t bi = brow + (size_t)k * L + t;
+            const size_t bi = brow + (size_t)k * ld + t;
             if (VAR == VAR_REAL) {
               const float bv = ld_r(gB, bi), cv = ld_r(gC, bi);
               const float a = __builtin_amdgcn_exp2f(v.x * a2[k]);
@@ -355,7 +389,7 @@ __global__ __launch_bounds__(NT) void core_fwd_kernel(const FwdArgs p) {
         for (int k = 0; k < NW; ++k) {
           const int n = n0 + k;
           if (n < N) {
-            const size_t o = ((((size_t)b * p.nck + kb) * N + n) * C) * D + d;
+            const size_t o = ((((size_t)b * p.nck + sg * (p.L / p.ck) + kb) * N + n) * C) * D + d;
             p.hck[o] = xr[k];
             if (C == 2) p.hck[o + D] = xi[k];
           }
@@ -373,12 +407,16 @@ __global__ __launch_bounds__(NT) void core_fwd_kernel(const FwdArgs p) {
     // every wavefront has finished this epilogue.
   }
 
+  if (want_tot && dok) {
+    p.ptot[((size_t)vb * D + d) * 2] = fr;
+    p.ptot[((size_t)vb * D + d) * 2 + 1] = fi;
+  }
   if (p.hL && active && dok) {
 #pragma unroll
     for (int k = 0; k < NW; ++k) {
       const int n = n0 + k;
       if (n < N) {
-        const size_t o = (((size_t)b * D + d) * N + n) * C;
+        const size_t o = (((size_t)vb * D + d) * N + n) * C;
         p.hL[o] = hr[k];
         if (C == 2) p.hL[o + 1] = hi[k];
       }

@@ -253,6 +253,15 @@ REC_CK = 16          # checkpoint interval the recomputing backward kernels (com
 REC_MAX_STATE = _lib.MAX_STATE   # largest state size those kernels take (16 states per launch, one launch per block)
 
 
+def _scan_workspace(variant: int, u: Tensor, n: int, ck: int) -> Optional[Tensor]:
+    """Workspace of a complex / real call for inputs shaped like u (aussm_scan_workspace_floats): segment
+    states that let a call with few (batch, channel group) pairs split along the sequence, and the float
+    copies of bfloat16 B_t / C_t.  None when the call needs neither."""
+    b, d, l = u.shape
+    floats = _lib.load().aussm_scan_workspace_floats(variant, b, d, n, l, ck, _in_dtype(u))
+    return torch.empty((floats,), device=u.device, dtype=torch.float32) if floats else None
+
+
 def complex_fwd_raw(u, delta, rho, theta, Bri, Cri, D=None, z=None, h0=None, want_state=False, ck=0):
     lib = _lib.load()
     b, d, l = u.shape
@@ -260,9 +269,10 @@ def complex_fwd_raw(u, delta, rho, theta, Bri, Cri, D=None, z=None, h0=None, wan
     y = torch.empty((b, d, l), device=u.device, dtype=torch.float32)
     hL = torch.empty((b, d, n, 2), device=u.device, dtype=torch.float32) if want_state else None
     hck = torch.empty((b, num_checkpoints(l, ck), n, 2, d), device=u.device, dtype=torch.float32) if ck else None
+    ws = _scan_workspace(_lib.VAR_COMPLEX, u, n, ck or _lib.TILE)
     check(lib.aussm_complex_fwd(ptr(u), ptr(delta), ptr(rho), ptr(theta), ptr(Bri), ptr(Cri), ptr(D), ptr(z),
-                                ptr(h0), ptr(y), ptr(hL), ptr(hck), b, d, n, l, ck or _lib.TILE, _in_dtype(u),
-                                _stream()), "aussm_complex_fwd")
+                                ptr(h0), ptr(y), ptr(hL), ptr(hck), ptr(ws), b, d, n, l, ck or _lib.TILE,
+                                _in_dtype(u), _stream()), "aussm_complex_fwd")
     return y, hL, hck
 
 
@@ -277,10 +287,11 @@ def complex_bwd_raw(dy, dhL, u, delta, rho, theta, Bri, Cri, D, h0, hck, want_dD
     dD = torch.zeros((d,), **f32) if (want_dD and D is not None) else None
     dh0 = torch.empty((b, d, n, 2), **f32) if want_dh0 else None
     dz = torch.empty((b, d, l), **f32) if z is not None else None
+    ws = _scan_workspace(_lib.VAR_COMPLEX, u, n, REC_CK)
     check(lib.aussm_complex_bwd(ptr(dy), ptr(dhL), ptr(u), ptr(delta), ptr(rho), ptr(theta), ptr(Bri), ptr(Cri),
                                 ptr(D), ptr(h0), ptr(hck), ptr(du), ptr(ddelta), ptr(drho), ptr(dtheta), ptr(dB),
-                                ptr(dC), ptr(dD), ptr(dh0), ptr(z), ptr(dz), b, d, n, l, REC_CK, _in_dtype(u), _stream()),
-          "aussm_complex_bwd")
+                                ptr(dC), ptr(dD), ptr(dh0), ptr(z), ptr(dz), ptr(ws), b, d, n, l, REC_CK,
+                                _in_dtype(u), _stream()), "aussm_complex_bwd")
     return du, ddelta, drho, dtheta, dB, dC, dD, dh0, dz
 
 
@@ -349,8 +360,9 @@ def real_fwd_raw(u, delta, A, Bm, Cm, D=None, z=None, delta_bias=None, delta_sof
     y = torch.empty((b, d, l), device=u.device, dtype=torch.float32)
     hL = torch.empty((b, d, n), device=u.device, dtype=torch.float32) if want_state else None
     hck = torch.empty((b, num_checkpoints(l, ck), n, 1, d), device=u.device, dtype=torch.float32) if ck else None
+    ws = _scan_workspace(_lib.VAR_REAL, u, n, ck or _lib.TILE)
     check(lib.aussm_real_fwd(ptr(u), ptr(delta), ptr(A), ptr(Bm), ptr(Cm), ptr(D), ptr(z), ptr(delta_bias),
-                             int(bool(delta_softplus)), ptr(h0), ptr(y), ptr(hL), ptr(hck), b, d, n, l,
+                             int(bool(delta_softplus)), ptr(h0), ptr(y), ptr(hL), ptr(hck), ptr(ws), b, d, n, l,
                              ck or _lib.TILE, _in_dtype(u), _stream()), "aussm_real_fwd")
     return y, hL, hck
 
@@ -368,9 +380,10 @@ def real_bwd_raw(dy, dhL, u, delta, A, Bm, Cm, D, delta_bias, delta_softplus, h0
     dD = torch.zeros((d,), **f32) if (want_dD and D is not None) else None
     dh0 = torch.empty((b, d, n), **f32) if want_dh0 else None
     dz = torch.empty((b, d, l), **f32) if z is not None else None
+    ws = _scan_workspace(_lib.VAR_REAL, u, n, REC_CK)
     check(lib.aussm_real_bwd(ptr(dy), ptr(dhL), ptr(u), ptr(delta), ptr(A), ptr(Bm), ptr(Cm), ptr(D),
                              ptr(delta_bias), int(bool(delta_softplus)), ptr(h0), ptr(hck), ptr(du), ptr(ddelta),
-                             ptr(dA), ptr(dB), ptr(dC), ptr(dD), ptr(dh0), ptr(z), ptr(dz), b, d, n, l, REC_CK,
+                             ptr(dA), ptr(dB), ptr(dC), ptr(dD), ptr(dh0), ptr(z), ptr(dz), ptr(ws), b, d, n, l, REC_CK,
                              _in_dtype(u), _stream()), "aussm_real_bwd")
     return du, ddelta, dA, dB, dC, dD, dh0, dz
 

@@ -201,10 +201,25 @@ int aussm_unitary_fwd_static(const void* u, const void* delta, const float* thet
  * Replaces extension-cpp/extension_cpp/ops.py:270-291 (loop) and the semantics of
  * extension-cpp/extension_cpp/csrc/cuda/ssm_adaptive_complex.cu:181-293 / :358-660.
  * The backward pass needs hck written with ck == aussm_bwd_checkpoint_interval(1).
+ *
+ * workspace (complex and real scans, forward and backward): aussm_scan_workspace_floats() floats of
+ * device memory, 16-byte aligned, contents irrelevant on entry; may be NULL for float inputs, required
+ * (AUSSM_E_NULL otherwise) for bf16 inputs, whose B_t / C_t rows the call first converts to float in it
+ * (the scan consumes them as wave-uniform scalar operands; converting them there costs a scalar
+ * instruction per value).  With it, a call with fewer
+ * than 129 (batch, group of 64 channels) pairs is split along the sequence into up to 64 segments of
+ * at least 128 steps that run side by side (end state / adjoint of every segment from zero, a chain
+ * over the segments, then the scan proper from the true incoming states), so that short batches of
+ * long sequences fill the chip; results equal the unsplit call's up to fp32 rounding.  The function
+ * answers 0 when the call needs none (pass NULL then).  No counterpart in the reference: its
+ * complex kernel walks the sequence chunk after chunk inside one thread block
+ * (ssm_adaptive_complex.cu:228-292, chunk size :313-321).
  * ------------------------------------------------------------------------------------- */
+size_t aussm_scan_workspace_floats(int variant, int B, int D, int N, int L, int ck, int in_dtype);
+
 int aussm_complex_fwd(const void* u, const void* delta, const float* rho, const float* theta,
                       const void* Bc, const void* Cc, const float* Dskip, const float* z,
-                      const float* h0, float* y, float* hL, float* hck,
+                      const float* h0, float* y, float* hL, float* hck, float* workspace,
                       int B, int D, int N, int L, int ck, int in_dtype, void* stream);
 
 /* z / dz of the two backward calls below (both NULL, or both given): the forward call was gated with this z
@@ -215,7 +230,7 @@ int aussm_complex_bwd(const float* dy, const float* dhL,
                       const void* Bc, const void* Cc, const float* Dskip,
                       const float* h0, const float* hck,
                       float* du, float* ddelta, float* drho, float* dtheta, float* dB, float* dC,
-                      float* dD, float* dh0, const float* z, float* dz,
+                      float* dD, float* dh0, const float* z, float* dz, float* workspace,
                       int B, int D, int N, int L, int ck, int in_dtype, void* stream);
 
 /* ---------------------------------------------------------------------------------------
@@ -231,7 +246,7 @@ int aussm_complex_bwd(const float* dy, const float* dhL,
 int aussm_real_fwd(const void* u, const void* delta, const float* A,
                    const void* Bm, const void* Cm, const float* Dskip, const float* z,
                    const float* delta_bias, int delta_softplus,
-                   const float* h0, float* y, float* hL, float* hck,
+                   const float* h0, float* y, float* hL, float* hck, float* workspace,
                    int B, int D, int N, int L, int ck, int in_dtype, void* stream);
 
 int aussm_real_bwd(const float* dy, const float* dhL,
@@ -240,7 +255,7 @@ int aussm_real_bwd(const float* dy, const float* dhL,
                    const float* delta_bias, int delta_softplus,
                    const float* h0, const float* hck,
                    float* du, float* ddelta, float* dA, float* dB, float* dC,
-                   float* dD, float* dh0, const float* z, float* dz,
+                   float* dD, float* dh0, const float* z, float* dz, float* workspace,
                    int B, int D, int N, int L, int ck, int in_dtype, void* stream);
 
 /* ---------------------------------------------------------------------------------------

@@ -94,9 +94,18 @@ def test_argument_checks_without_a_device():
     rc = lib.aussm_unitary_bwd_aux(*([one] * 17), 3, 1, 1, 32, 32, 0, 0, null)
     assert rc == -2
     # the recomputing backward kernels insist on their checkpoint interval and on the state limit of the library
-    args = [one] * 9 + [0] + [one] * 11
+    args = [one] * 9 + [0] + [one] * 11 + [null]          # ..., z, dz, workspace
     assert lib.aussm_real_bwd(*args, 1, 1, 1, 32, 32, 0, null) == -3
     assert lib.aussm_real_bwd(*args, 1, 1, 65, 32, 16, 0, null) == -2
+    # workspace for the split of the complex / real scans along the sequence: none for full launches
+    lib.aussm_scan_workspace_floats.restype = ctypes.c_size_t
+    assert lib.aussm_scan_workspace_floats(2, 32, 512, 16, 2048, 16, 0) == 0
+    assert lib.aussm_scan_workspace_floats(0, 4, 256, 16, 16384, 16, 0) == 0       # the unitary scan has its own
+    assert lib.aussm_scan_workspace_floats(2, 4, 256, 16, 16384, 16, 0) >= 4 * 16 * 256 * 18
+    assert lib.aussm_scan_workspace_floats(1, 4, 256, 16, 16384, 16, 0) >= 4 * 16 * 256 * 34
+    # bf16 inputs: float copies of B_t and C_t, and no call without the workspace that holds them
+    assert lib.aussm_scan_workspace_floats(1, 32, 512, 16, 2048, 16, 1) == 2 * 32 * 16 * 2048 * 2
+    assert lib.aussm_real_bwd(*args, 1, 1, 1, 32, 16, 1, null) == -1
     # the blocks' causal convolution: kernel length limit, overlapping rows, required pointers
     assert lib.aussm_causal_conv1d_fwd(one, one, null, one, 1, 8, 4, 9, 32, 4, null) == -2
     assert lib.aussm_causal_conv1d_fwd(one, one, null, one, 1, 8, 4, 4, 32, 3, null) == -2      # row stride < D

@@ -31,6 +31,11 @@ SHAPES = [
     (2, 40, 64, 50),          # more than 16 states: the backward pass takes one launch per block of 16
     (1, 70, 24, 33),
     (2, 20, 37, 40),
+    # few (batch, channel group) pairs and at least 256 steps: the launch is split along the sequence
+    # (segments of 128 steps here; the last one ragged, a single step in (3, 130, 4, 257) above)
+    (2, 70, 16, 600),
+    (1, 40, 64, 300),
+    (1, 33, 2, 513),
 ]
 
 
@@ -196,3 +201,53 @@ def test_random_shapes_and_input_types(seed):
         tol = 2e-2 if (lowp and k in low) else ATOL
         scale = max(1.0, float(want.abs().max()))
         torch.testing.assert_close(g.cpu() / scale, want / scale, atol=tol, rtol=tol, msg=lambda m, k=k: f"d{k}: {m}")
+
+
+@pytest.mark.parametrize("variant", ["complex", "real"])
+@pytest.mark.parametrize("lowp", [False, True])
+def test_split_along_sequence_matches_unsplit(variant, lowp):
+    """12 (batch, channel group) pairs of 4136 steps run as 22 segments side by side; the same call with the
+    split switched off is the comparison (itself checked against the oracle above at small sizes).  Outputs,
+    final state and every gradient, gate and initial state included, float32 and bfloat16 inputs."""
+    from aussm_amd import _lib, scan
+    B, D, N, L = 4, 192, 16, 4136
+    lib = _lib.load()
+    assert lib.aussm_scan_workspace_floats(_lib.VAR_COMPLEX if variant == "complex" else _lib.VAR_REAL, B, D, N, L, 16, 0) > 0
+    p = O.make_core_inputs(B, D, N, L, seed=11, variant=variant, gate=True)
+    names = (["u", "delta", "A", "Bm", "Cm", "Dskip", "z"] if variant == "real"
+             else ["u", "delta", "rho", "theta", "Bc", "Cc", "Dskip", "z"])
+    low = ("u", "delta", "Bm", "Cm", "Bc", "Cc")
+    h0, dhL = _h0(B, D, N, variant == "complex", 5), _h0(B, D, N, variant == "complex", 6)
+
+    def run():
+        lv = {}
+        for k in names:
+            t = p[k].clone().cuda()
+            if lowp and k in low:
+                t = (torch.view_as_real(t).contiguous() if t.is_complex() else t).to(torch.bfloat16)
+            lv[k] = t.requires_grad_(True)
+        h = h0.clone().cuda().requires_grad_(True)
+        if variant == "real":
+            y, hL = scan.selective_scan_fn(lv["u"], lv["delta"], lv["A"], lv["Bm"], lv["Cm"], lv["Dskip"], z=lv["z"],
+                                           return_last_state=True, h0=h)
+        else:
+            y, hL = scan.complex_scan(lv["u"], lv["delta"], lv["rho"], lv["theta"], lv["Bc"], lv["Cc"], lv["Dskip"],
+                                      lv["z"], h, return_last_state=True)
+        ((y * p["dy"].cuda()).sum() + (hL * dhL.cuda().conj()).real.sum()).backward()
+        torch.cuda.synchronize()
+        out = {k: v.grad.float() for k, v in lv.items()}
+        out["h0"] = h.grad
+        out["y"], out["hL"] = y.detach(), hL.detach()
+        return out
+
+    print(f"case split vs unsplit {variant} bf16={lowp} B={B} D={D} N={N} L={L}", flush=True)
+    got = run()
+    with _lib.options(split_cap=0):
+        want = run()
+    for k in want:
+        w, g = want[k], got[k]
+        if w.is_complex():
+            w, g = torch.view_as_real(w), torch.view_as_real(g)
+        tol = 2e-2 if (lowp and k in low) else ATOL
+        scale = max(1.0, float(w.abs().max()))
+        torch.testing.assert_close(g / scale, w / scale, atol=tol, rtol=tol, msg=lambda m, k=k: f"{k}: {m}")
