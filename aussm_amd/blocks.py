@@ -169,9 +169,8 @@ class SSMauBlock(nn.Module):
         elif args.cuda:
             self.optimized_SSMa_function = lambda **kw: ops.ssm_adaptive_interface(**kw, unitary=True)
         else:
-            raise NotImplementedError(
-                "cuda=False selects the reference's pure-PyTorch scan, which this package does not ship; "
-                "pass scan_impl=... to use another implementation")
+            # the reference's pure-PyTorch form (aussm.py:842-843): same name, same signature, HIP kernels
+            self.optimized_SSMa_function = ops.reference_ssm_adaptive_unitary_optimized_polar
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         (b, l, d) = x.shape

@@ -600,13 +600,20 @@ static DropinBlocks dropin_blocks(int b, int d, int n, int L) {
 // How a GEMM launch is cut: about three workgroups per compute unit.  Without reduce_z every z is a
 // slice of its own and k is cut (at least four steps per slice); with reduce_z the z are dealt to the
 // slices first and k is cut only when there are too few z.
+#ifdef AUSSM_TUNE
+#include <cstdlib>
+static long tune_target() { const char* e = getenv("GT"); return e ? atol(e) : 768; }
+#define GEMM_TARGET tune_target()
+#else
+#define GEMM_TARGET 768
+#endif
 static void gemm_slices(GemmArgs& g) {
   const long tiles = (long)((g.M + 127) / 128) * ((g.N + 63) / 64);
   const int nk = (g.K + 31) / 32;
   long zs = 1;                                   // slices of z
   g.zper = 1;
   if (g.reduce_z) {
-    zs = (768 + tiles - 1) / tiles;
+    zs = (GEMM_TARGET + tiles - 1) / tiles;
     if (zs > g.Z) zs = g.Z;
     if (zs < 1) zs = 1;
     g.zper = (int)((g.Z + zs - 1) / zs);
@@ -614,7 +621,7 @@ static void gemm_slices(GemmArgs& g) {
   } else {
     zs = g.Z;
   }
-  long s = (768 + tiles * zs - 1) / (tiles * zs);
+  long s = (GEMM_TARGET + tiles * zs - 1) / (tiles * zs);
   if (s > nk / 4) s = nk / 4;
   if (s < 1) s = 1;
   while (s > 1 && zs * s > 65535) --s;

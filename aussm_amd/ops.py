@@ -26,7 +26,7 @@ BLAS GEMM, and the sum over j is taken afterwards.
 """
 from __future__ import annotations
 
-from typing import Tuple
+from typing import Optional, Tuple
 
 import torch
 import torch.nn.functional as F
@@ -35,7 +35,8 @@ from torch import Tensor
 from . import _lib as L
 from . import scan
 
-__all__ = ["ssm_adaptive_unitary", "ssm_adaptive_interface", "pad_to_multiple_of"]
+__all__ = ["ssm_adaptive_unitary", "ssm_adaptive_interface", "pad_to_multiple_of",
+           "reference_ssm_adaptive_unitary_optimized_polar"]
 
 _NS = "extension_cpp"
 _FWD_SCHEMA = ("ssm_adaptive_unitary(Tensor u, Tensor dt, Tensor x, Tensor x_bias, Tensor B_r, Tensor B_theta, "
@@ -263,3 +264,24 @@ def ssm_adaptive_interface(u: Tensor, dt: Tensor, x: Tensor, x_bias: Tensor, B: 
                          z[:, :, s:e].contiguous(), h_r, h_i)
         outs.append(y)
     return outs[0] if len(outs) == 1 else torch.cat(outs, dim=-1)
+
+
+def reference_ssm_adaptive_unitary_optimized_polar(u: Tensor, dt: Tensor, x: Tensor, x_bias: Tensor, B: Tensor,
+                                                   C: Tensor, D: Tensor, z: Optional[Tensor] = None,
+                                                   diagnostic: bool = False, z_prod: bool = True, binary: bool = False,
+                                                   no_graded_rotation: bool = False, unitary: bool = True) -> Tensor:
+    """The callable `SSMauBlock(cuda=False)` selects in the reference (aussm.py:842-843; ops.py:614-769):
+    there a pure-PyTorch cumulative-sum form of the same operator.  Here the name and signature are kept
+    and the default case - constant complex B, C of shape (n,), gate on, graded rotation - runs on the
+    same fused HIP kernels as ssm_adaptive_interface (one launch sequence, any length); there is no eager
+    or CPU path behind it.  The research switches of the reference (diagnostic outputs, binary or ungraded
+    rotations, time-varying B / C phases, no gate) are not implemented and raise."""
+    if diagnostic or binary or no_graded_rotation or not unitary or not z_prod:
+        raise NotImplementedError("only the default form (unitary, graded rotation, gated, no diagnostics) is implemented")
+    if B.dim() != 1 or C.dim() != 1:
+        raise NotImplementedError("time-varying B / C phases are not implemented by the fused operator")
+    if z is None:
+        raise ValueError("z is required (z_prod=True)")
+    if not u.is_cuda:
+        raise RuntimeError("scan inputs must be on the GPU (no CPU implementation is shipped)")
+    return ssm_adaptive_interface(u, dt, x, x_bias, B, C, D, z, unitary=True, max_parallel_length=max(1, u.shape[-1]))

@@ -112,3 +112,32 @@ def test_dispatcher_operators_pass_opcheck():
     nh = list(torch.ops.extension_cpp.ssm_adaptive_unitary(*args)[1:])
     torch.library.opcheck(torch.ops.aussm_amd.ssm_adaptive_backward_unitary_from_state.default,
                           tuple(grads + args + nh), atol=1e-4, rtol=1e-4)
+
+
+def test_polar_callable_of_the_blocks():
+    """`reference_ssm_adaptive_unitary_optimized_polar`, the callable the reference's SSMauBlock(cuda=False)
+    selects (aussm.py:842-843), keeps name and signature and runs the default case on the HIP kernels;
+    the research switches raise."""
+    from aussm_amd import blocks, ops
+    args = O.make_adaptive_inputs(l=37)
+    print("case drop-in polar callable l=37", flush=True)
+    expected = O.adaptive_unitary_polar(*args)
+    dev = _cuda(args)
+    got = ops.reference_ssm_adaptive_unitary_optimized_polar(*dev)
+    torch.testing.assert_close(got.cpu(), expected, atol=7e-5, rtol=5e-5)
+    kw = dict(zip(["u", "dt", "x", "x_bias", "B", "C", "D", "z"], dev))
+    torch.testing.assert_close(ops.reference_ssm_adaptive_unitary_optimized_polar(**kw).cpu(), expected, atol=7e-5, rtol=5e-5)
+    for flag in ("diagnostic", "binary", "no_graded_rotation"):
+        with pytest.raises(NotImplementedError):
+            ops.reference_ssm_adaptive_unitary_optimized_polar(*dev, **{flag: True})
+    with pytest.raises(NotImplementedError):
+        ops.reference_ssm_adaptive_unitary_optimized_polar(*dev, unitary=False)
+    with pytest.raises(RuntimeError):
+        ops.reference_ssm_adaptive_unitary_optimized_polar(*args)          # CPU tensors: nothing is shipped for them
+    # the block built with cuda=False goes through it and agrees with the cuda=True block
+    torch.manual_seed(3)
+    a = blocks.SSMauBlock(blocks.ModelArgsSSMau(d_model=16, d_state=4, cuda=False)).cuda()
+    torch.manual_seed(3)
+    b = blocks.SSMauBlock(blocks.ModelArgsSSMau(d_model=16, d_state=4, cuda=True)).cuda()
+    xin = torch.randn(2, 40, 16, device="cuda")
+    torch.testing.assert_close(a(xin), b(xin), atol=1e-5, rtol=1e-5)
