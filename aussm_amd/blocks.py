@@ -38,6 +38,14 @@ def _causal_conv(conv1d: nn.Conv1d, x: torch.Tensor, l: int) -> torch.Tensor:
     return conv1d(x.transpose(1, 2))[:, :, :l].transpose(1, 2)
 
 
+def _swap_act(x: torch.Tensor, act: str, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """`_swap(act(x + bias))` in one pass on the GPU (the elementwise step rides on the layout change)."""
+    if x.is_cuda and x.dtype == torch.float32:
+        return conv.swap_last2(x, act=act, bias=bias)
+    v = x if bias is None else x + bias
+    return _swap(F.silu(v) if act == "silu" else F.softplus(v))
+
+
 def _swap(x: torch.Tensor) -> torch.Tensor:
     """Contiguous copy with the last two dimensions swapped: (b, l, d) <-> (b, d, l), the
     `rearrange` calls around the scans (ai-modules/wavesAI/model/aussm.py:760-803, :861-900)."""
@@ -130,10 +138,9 @@ class MambaBlock(nn.Module):
         x_proj = self.x_proj(x)
         dt, B, C = x_proj.split([self.args.dt_rank, self.args.d_state, self.args.d_state], dim=-1)
         dt = self.dt_proj(dt)
-        x = F.silu(x)
         A = -torch.exp(self.A_log.float())
         y = self.scan_impl(
-            _swap(x),
+            _swap_act(x, "silu"),                       # x = F.silu(x), aussm.py:787
             _swap(dt),
             A.contiguous(),
             _swap(B),
@@ -185,14 +192,13 @@ class SSMauBlock(nn.Module):
         b, l, d_in = x.shape
         n = self.args.d_state
         dt = self.dt_proj(self.x_proj(x))
-        dt = dt + self.dt_proj.bias.float()
-        dt = F.softplus(dt)
+        # dt = softplus(dt + self.dt_proj.bias) of aussm.py:879-880 happens inside the layout change below
         # "(n dstate1) dstate -> dstate1 n dstate"
         x_param = self.xA_proj.weight.view(n, d_in, d_in).permute(1, 0, 2)
         x_bias = self.xA_proj.bias.view(n, d_in).t()
         self.ssm_args = {
             "u": _swap(x),
-            "dt": _swap(dt),
+            "dt": _swap_act(dt, "softplus", self.dt_proj.bias.float()),
             "x": x_param.contiguous() * (1 / math.sqrt(self.args.d_model)),
             "x_bias": x_bias.contiguous(),
             "B": self.B.contiguous(),

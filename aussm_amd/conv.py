@@ -93,11 +93,54 @@ def _swap_last2(x: Tensor) -> Tensor:
     return y
 
 
-def swap_last2(x: Tensor) -> Tensor:
+_ACTS = {"silu": 1, "softplus": 2}
+
+
+class _SwapActFn(torch.autograd.Function):
+    """swap_last2 with the elementwise step done in the same pass, both directions."""
+
+    @staticmethod
+    def forward(ctx, x, bias, act):
+        lib = _lib.load()
+        b, r, c = x.shape
+        xr = _rows(x)
+        bs = None if bias is None else bias.float().contiguous()
+        y = torch.empty((b, c, r), device=x.device, dtype=torch.float32)
+        check(lib.aussm_swap_last2_act(ptr(xr), ptr(bs), None, ptr(y), b, r, c, xr.stride(0), xr.stride(1), 0, 0,
+                                       act, 0, _stream()), "aussm_swap_last2_act")
+        ctx.save_for_backward(xr, bs)
+        ctx.act = act
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        lib = _lib.load()
+        xr, bs = ctx.saved_tensors
+        b, r, c = xr.shape
+        dy = dy.float().contiguous()                    # (b, c, r)
+        dx = torch.empty((b, r, c), device=dy.device, dtype=torch.float32)
+        check(lib.aussm_swap_last2_act(ptr(dy), ptr(bs), ptr(xr), ptr(dx), b, c, r, dy.stride(0), dy.stride(1),
+                                       xr.stride(0), xr.stride(1), ctx.act, 1, _stream()), "aussm_swap_last2_act")
+        dbias = dx.sum((0, 1)) if (bs is not None and ctx.needs_input_grad[1]) else None
+        return dx, dbias, None
+
+
+def swap_last2(x: Tensor, act: Optional[str] = None, bias: Optional[Tensor] = None) -> Tensor:
     """Contiguous (b, c, r) copy of x (b, r, c) on the GPU: `x.transpose(1, 2).contiguous()` between
-    the blocks' (b, l, d) activations and the scans' (b, d, l) tensors, through LDS tiles."""
+    the blocks' (b, l, d) activations and the scans' (b, d, l) tensors, through LDS tiles.
+    act ("silu" or "softplus") with an optional per-channel bias (c,): the copy holds
+    act(x + bias) instead, computed (and differentiated) in the same pass."""
     if x.dim() != 3 or not x.is_cuda:
         raise ValueError("swap_last2 expects a (b, r, c) tensor on the GPU")
-    if x.shape[0] > 65535:
-        return x.transpose(1, 2).contiguous()
-    return _SwapLast2Fn.apply(x)
+    if act is None:
+        if bias is not None:
+            raise ValueError("a bias needs an activation")
+        if x.shape[0] > 65535:
+            return x.transpose(1, 2).contiguous()
+        return _SwapLast2Fn.apply(x)
+    if act not in _ACTS:
+        raise ValueError(f"unknown activation {act!r}")
+    if x.shape[0] > 65535 or x.dtype != torch.float32:
+        v = x if bias is None else x + bias
+        return (torch.nn.functional.silu(v) if act == "silu" else torch.nn.functional.softplus(v)).transpose(1, 2).contiguous()
+    return _SwapActFn.apply(x, bias, _ACTS[act])

@@ -512,9 +512,9 @@ __global__ __launch_bounds__(256) void fill_kernel(const FillArgs a) {
 // one row as 16-byte vectors (VEC; rows need not be 16-byte aligned) - a wavefront request covers 16
 // cache lines.  Otherwise both are contiguous along m / n and a 16-lane row of the wavefront
 // fetches 16 neighbouring rows' values of one k.
-template <bool K1, bool VEC>
+template <bool K1, bool VEC, int NP>
 __global__ __launch_bounds__(256) void split_gemm_kernel(const GemmArgs p) {
-  __shared__ u4 s_a[8 * 3 * 64], s_b[4 * 3 * 64];
+  __shared__ u4 s_a[8 * NP * 64], s_b[4 * NP * 64];
   const int tid = threadIdx.x, lane = tid & 63, wave = wave_index();
   const int m0 = blockIdx.x * 128, n0 = blockIdx.y * 64;
   const int zs = blockIdx.z / p.ksplit, ksl = blockIdx.z % p.ksplit;
@@ -533,7 +533,7 @@ __global__ __launch_bounds__(256) void split_gemm_kernel(const GemmArgs p) {
   // ... and where they go in LDS: [16-row tile][piece][16 g + (row + 4 g) % 16], g = kq / 8.  The rotation by
   // 4 g keeps the 16-byte writes of the K1 mapping (four neighbouring lanes = the four g of one row) and the
   // reads (16 neighbouring lanes = 16 rows of one g) both free of bank conflicts.
-  const int slot = (ra >> 4) * 192 + (kq >> 3) * 16 + ((ra + (kq >> 1)) & 15);
+  const int slot = (ra >> 4) * (NP * 64) + (kq >> 3) * 16 + ((ra + (kq >> 1)) & 15);
   const int rslot = (lane & 48) + ((lane + (lane >> 4) * 4) & 15);       // the record of (row lane % 16, g lane / 16)
   // uniform bases, 32-bit per-thread offsets (a z-slice of either operand is below 2^31 elements)
   const unsigned sak = (unsigned)p.sak, sbk = (unsigned)p.sbk;
@@ -585,33 +585,35 @@ __global__ __launch_bounds__(256) void split_gemm_kernel(const GemmArgs p) {
       }
     }
   };
+  // (requesting the values two steps ahead, with a second register set, was measured: the registers cost a
+  // wavefront per SIMD and the launch got 25 % slower - the other wavefronts hide the latency better)
   if (nit > 0) fetch(0);
   for (int step = 0; step < nit; ++step) {
-    u4 pa[2][3], pb[3];
-    split8<3>(sk, va[0], pa[0]);
-    split8<3>(sk, va[1], pa[1]);
-    split8<3>(sk, vb, pb);
+    u4 pa[2][NP], pb[NP];
+    split8<NP>(sk, va[0], pa[0]);
+    split8<NP>(sk, va[1], pa[1]);
+    split8<NP>(sk, vb, pb);
     __syncthreads();
 #pragma unroll
-    for (int c = 0; c < 3; ++c) {
+    for (int c = 0; c < NP; ++c) {
       s_a[slot + c * 64] = pa[0][c];
-      s_a[slot + 4 * 192 + c * 64] = pa[1][c];
+      s_a[slot + 4 * (NP * 64) + c * 64] = pa[1][c];
       s_b[slot + c * 64] = pb[c];
     }
     __syncthreads();
     if (step + 1 < nit) fetch(step + 1);      // in flight during the products
-    u4 rb[2][3];
+    u4 rb[2][NP];
 #pragma unroll
     for (int f = 0; f < 2; ++f)
 #pragma unroll
-      for (int c = 0; c < 3; ++c) rb[f][c] = s_b[((wn + f) * 3 + c) * 64 + rslot];
+      for (int c = 0; c < NP; ++c) rb[f][c] = s_b[((wn + f) * NP + c) * 64 + rslot];
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      u4 rA[3];
+      u4 rA[NP];
 #pragma unroll
-      for (int c = 0; c < 3; ++c) rA[c] = s_a[((wm + e) * 3 + c) * 64 + rslot];
+      for (int c = 0; c < NP; ++c) rA[c] = s_a[((wm + e) * NP + c) * 64 + rslot];
 #pragma unroll
-      for (int f = 0; f < 2; ++f) acc[e][f] = xmm<3>(rA, rb[f], acc[e][f]);
+      for (int f = 0; f < 2; ++f) acc[e][f] = xmm<NP>(rA, rb[f], acc[e][f]);
     }
   }
   // result tile (e, f): lane (column = lane % 16, rows 4 (lane / 16) + a)

@@ -3,13 +3,21 @@
 // (`rearrange(x, 'b l d -> b d l')` and back, ai-modules/wavesAI/model/aussm.py:760-803 and
 // :861-900).  32 x 32 tiles through LDS, so both the reads and the writes are full lines; the
 // input may be a column slice of a wider tensor (row stride xs_r >= C), the output is contiguous.
+// Optionally the elementwise step the blocks apply on the way is done in the same pass: silu on the
+// convolution output that feeds the S6 scan (aussm.py:787), softplus(dt + bias) in front of the
+// adaptive-unitary operator (aussm.py:878-880), and their derivatives on the way back.
 #pragma once
 #include <hip/hip_runtime.h>
 
 #include "scan_args.h"
+#include "scan_common.h"
 
 namespace aussm {
 
+__device__ __forceinline__ float swap_act(int act, float v) { return act == 1 ? siluf_(v) : softplusf_(v); }
+__device__ __forceinline__ float swap_dact(int act, float v) {
+  return act == 1 ? dsiluf_(v) : (v > 20.0f ? 1.0f : sigmoidf_(v));
+}
 
 __global__ __launch_bounds__(256) void swap_last2_kernel(const SwapArgs p) {
   __shared__ float tile[32][33];
@@ -20,13 +28,22 @@ __global__ __launch_bounds__(256) void swap_last2_kernel(const SwapArgs p) {
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const int r = r0 + ty + 8 * j, c = c0 + tx;
-    if (r < p.R && c < p.C) tile[ty + 8 * j][tx] = xb[(size_t)r * p.xs_r + c];
+    if (r < p.R && c < p.C) {
+      float v = xb[(size_t)r * p.xs_r + c];
+      if (p.act && !p.deriv) v = swap_act(p.act, v + (p.bias ? p.bias[c] : 0.0f));
+      tile[ty + 8 * j][tx] = v;
+    }
   }
   __syncthreads();
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const int c = c0 + ty + 8 * j, r = r0 + tx;
-    if (c < p.C && r < p.R) yb[(size_t)c * p.R + r] = tile[tx][ty + 8 * j];
+    if (c < p.C && r < p.R) {
+      float v = tile[tx][ty + 8 * j];
+      if (p.act && p.deriv)
+        v *= swap_dact(p.act, p.pre[(size_t)b * p.ps_b + (size_t)c * p.ps_r + r] + (p.bias ? p.bias[r] : 0.0f));
+      yb[(size_t)c * p.R + r] = v;
+    }
   }
 }
 

@@ -564,7 +564,22 @@ int aussm_swap_last2(const float* x, float* y, int B, int R, int C, long long xs
   if (B < 1 || R < 1 || C < 1 || B > 65535 || xs_r < C || xs_b < (long long)R * xs_r - (xs_r - C)) return AUSSM_E_SHAPE;
   if ((R + 31) / 32 > 65535) return AUSSM_E_SHAPE;
   if (!x || !y) return AUSSM_E_NULL;
-  SwapArgs a{x, y, xs_b, xs_r, R, C};
+  SwapArgs a{};
+  a.x = x; a.y = y; a.xs_b = xs_b; a.xs_r = xs_r; a.R = R; a.C = C;
+  return run_swap_last2(a, B, (hipStream_t)stream);
+}
+
+int aussm_swap_last2_act(const float* x, const float* bias, const float* pre, float* y, int B, int R, int C,
+                         long long xs_b, long long xs_r, long long ps_b, long long ps_r, int act, int deriv,
+                         void* stream) {
+  if (B < 1 || R < 1 || C < 1 || B > 65535 || xs_r < C || xs_b < (long long)R * xs_r - (xs_r - C)) return AUSSM_E_SHAPE;
+  if ((R + 31) / 32 > 65535 || act < 1 || act > 2) return AUSSM_E_SHAPE;
+  if (!x || !y || (deriv && !pre)) return AUSSM_E_NULL;
+  // pre has the output's shape (B, C, R): rows of R elements that do not overlap
+  if (deriv && (ps_r < R || ps_b < (long long)C * ps_r - (ps_r - R))) return AUSSM_E_SHAPE;
+  SwapArgs a{};
+  a.x = x; a.y = y; a.xs_b = xs_b; a.xs_r = xs_r; a.R = R; a.C = C;
+  a.bias = bias; a.pre = deriv ? pre : nullptr; a.ps_b = ps_b; a.ps_r = ps_r; a.act = act; a.deriv = deriv ? 1 : 0;
   return run_swap_last2(a, B, (hipStream_t)stream);
 }
 
@@ -600,13 +615,7 @@ static DropinBlocks dropin_blocks(int b, int d, int n, int L) {
 // How a GEMM launch is cut: about three workgroups per compute unit.  Without reduce_z every z is a
 // slice of its own and k is cut (at least four steps per slice); with reduce_z the z are dealt to the
 // slices first and k is cut only when there are too few z.
-#ifdef AUSSM_TUNE
-#include <cstdlib>
-static long tune_target() { const char* e = getenv("GT"); return e ? atol(e) : 768; }
-#define GEMM_TARGET tune_target()
-#else
-#define GEMM_TARGET 768
-#endif
+constexpr long GEMM_TARGET = 768;     // workgroups per launch aimed at (measured: 512 +4 %, 1024 +5 %, 256 +22 % of the backward call)
 static void gemm_slices(GemmArgs& g) {
   const long tiles = (long)((g.M + 127) / 128) * ((g.N + 63) / 64);
   const int nk = (g.K + 31) / 32;

@@ -168,6 +168,14 @@ struct SwapArgs {
   float* y;            // [B, C, R] contiguous
   long long xs_b, xs_r;
   int R, C;
+  // optional activation fused into the swap (act: 0 none, 1 silu, 2 softplus with torch's threshold 20)
+  //   forward (deriv 0):  y[b, c, r] = f(x[b, r, c] + bias[c])
+  //   gradient (deriv 1): y[b, c, r] = x[b, r, c] * f'(pre[b, c, r] + bias[r])   (x is the incoming gradient
+  //                       in the forward output's layout, pre the forward input, y its gradient)
+  const float* bias;   // per channel, or null
+  const float* pre;    // deriv: element (b, c, r) at pre[b * ps_b + c * ps_r + r]
+  long long ps_b, ps_r;
+  int act, deriv;
 };
 
 }  // namespace aussm

@@ -283,6 +283,18 @@ int aussm_causal_conv1d_bwd(const float* dy, const float* x, const float* w,
 int aussm_swap_last2(const float* x, float* y, int B, int R, int C,
                      long long xs_b, long long xs_r, void* stream);
 
+/* The same layout change with the elementwise step the blocks apply on the way done in the same pass:
+ * act 1 = silu (`x = F.silu(x)` on the convolution output that feeds the S6 scan, aussm.py:787),
+ * act 2 = softplus with threshold 20 (`dt = F.softplus(dt + self.dt_proj.bias)`, aussm.py:878-880).
+ *   deriv == 0:  y[b, c, r] = f(x[b, r, c] + bias[c])                 bias (C) may be NULL
+ *   deriv != 0:  y[b, c, r] = x[b, r, c] * f'(pre[b, c, r] + bias[r])  bias (R) may be NULL
+ * the second form is the gradient: x is the gradient w.r.t. the first form's output (in that output's
+ * layout), pre the first form's input (element (b, c, r) at pre[b*ps_b + c*ps_r + r]), y the gradient
+ * w.r.t. that input.  The gradient of bias is the sum of y over b and c (left to the caller). */
+int aussm_swap_last2_act(const float* x, const float* bias, const float* pre, float* y, int B, int R, int C,
+                         long long xs_b, long long xs_r, long long ps_b, long long ps_r, int act, int deriv,
+                         void* stream);
+
 /* ---------------------------------------------------------------------------------------
  * The reference's custom operator itself, as two calls: what
  *   torch.ops.extension_cpp.ssm_adaptive_unitary           (12 tensors -> y, next_hid_real, next_hid_imag)

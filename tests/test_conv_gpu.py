@@ -68,3 +68,34 @@ def test_swap_last2_matches_transpose(b, r, c, sliced):
     want = torch.zeros_like(wide)
     (want[:, :, c:] if sliced else want[:, :, :c]).copy_(dy.transpose(1, 2))
     assert torch.equal(gx, want)
+
+
+@pytest.mark.parametrize("b,r,c,sliced", [(2, 37, 70, False), (3, 720, 256, True), (1, 1, 5, False), (2, 33, 31, True)])
+@pytest.mark.parametrize("act,with_bias", [("silu", False), ("softplus", True), ("softplus", False)])
+def test_swap_last2_with_activation(b, r, c, sliced, act, with_bias):
+    """The layout change with silu / softplus(x + bias) done in the same pass, against torch's own
+    elementwise functions in float64 (values and the gradients of x and bias); large arguments
+    exercise softplus' linear branch (threshold 20)."""
+    import torch.nn.functional as F
+    from aussm_amd import conv
+    g = torch.Generator().manual_seed(7 * r + c)
+    wide = (torch.randn(b, r, 2 * c, generator=g) * 12).cuda().requires_grad_(True)
+    bias = torch.randn(c, generator=g).cuda().requires_grad_(True) if with_bias else None
+    x = wide[:, :, c:] if sliced else wide[:, :, :c]
+    print(f"case swap+{act} b={b} r={r} c={c} sliced={sliced} bias={with_bias}", flush=True)
+    y = conv.swap_last2(x, act=act, bias=bias)
+    assert y.is_contiguous() and y.shape == (b, c, r)
+    dy = torch.randn(b, c, r, generator=g).cuda()
+    grads = torch.autograd.grad(y, [wide] + ([bias] if with_bias else []), dy)
+    wide64 = wide.detach().double().requires_grad_(True)
+    bias64 = bias.detach().double().requires_grad_(True) if with_bias else None
+    x64 = wide64[:, :, c:] if sliced else wide64[:, :, :c]
+    v = x64 if bias64 is None else x64 + bias64
+    y64 = (F.silu(v) if act == "silu" else F.softplus(v)).transpose(1, 2)
+    want = torch.autograd.grad(y64, [wide64] + ([bias64] if with_bias else []), dy.double())
+    torch.testing.assert_close(y.double(), y64, atol=1e-5, rtol=1e-5)
+    for a, w in zip(grads, want):
+        scale = max(1.0, float(w.abs().max()))
+        torch.testing.assert_close(a.double() / scale, w / scale, atol=1e-5, rtol=1e-5)
+    with pytest.raises(ValueError):
+        conv.swap_last2(x, act="tanh")
