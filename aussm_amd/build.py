@@ -80,29 +80,31 @@ def build(verbose: bool = True, asm_dir: str | None = None, only=None, extra=())
 
 # ---- listing check of the kernels that track their own loads ------------------------------------
 #
-# The kernels of scan_px.h issue some global loads as hand-written instructions and wait for them
-# by count, so that the compiler neither sees a load nor places a wait.  Two things the compiler is
+# The kernels of scan_px.h (and the prefetch of scan_bwd_xdl.h, into accumulation registers) issue some
+# global loads as hand-written instructions and wait for them by count, so that the compiler neither
+# sees a load nor places a wait.  Two things the compiler is
 # then free to do would silently break them, and both are visible in the assembly it emits:
 #   * spilling vector registers (a register that is the destination of a load in flight would be
 #     saved before the data has arrived);
 #   * touching a load's destination registers between the load and the wait that retires it
 #     (copying them, or - when it considers the value dead - reusing them for something else,
 #     which the landing data then overwrites).
-# check_px_listing() compiles k_px.hip to assembly and looks for both in every kernel of the unit.
+# check_px_listing() compiles k_px.hip and k_xdl.hip to assembly and looks for both in every kernel
+# of the two units.
 
 def scan_listing(text: str):
-    """Findings [(line number, instruction)] of one kernel listing: vector registers touched while
-    they are the destination of a hand-written (ASMSTART ... ASMEND) global load that no
+    """Findings [(line number, instruction)] of one kernel listing: vector or accumulation registers
+    touched while they are the destination of a hand-written (ASMSTART ... ASMEND) global load that no
     s_waitcnt vmcnt has retired yet.  The scan follows the file order, not the control flow."""
     import re
 
     def regs(tok):
         out = set()
-        for m in re.finditer(r"\bv\[(\d+):(\d+)\]|\bv(\d+)\b", tok):
+        for m in re.finditer(r"\b([va])\[(\d+):(\d+)\]|\b([va])(\d+)\b", tok):
             if m.group(1):
-                out.update(range(int(m.group(1)), int(m.group(2)) + 1))
+                out.update((m.group(1), r) for r in range(int(m.group(2)), int(m.group(3)) + 1))
             else:
-                out.add(int(m.group(3)))
+                out.add((m.group(4), int(m.group(5))))
         return out
 
     inflight, in_asm, found = {}, False, []
@@ -135,15 +137,16 @@ def scan_listing(text: str):
     return found
 
 
-def check_px_listing(verbose: bool = True) -> None:
-    """Raises RuntimeError if a kernel of k_px.hip spills vector registers or touches registers
-    with a load in flight."""
+def check_unit_listing(unit: str, verbose: bool = True) -> int:
+    """Raises RuntimeError if a kernel of the unit touches registers that are the destination of a
+    hand-written load in flight, or spills vector registers while such loads land in vector registers;
+    returns the number of kernel listings checked."""
     import re
     import tempfile
     hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
     with tempfile.TemporaryDirectory() as tmp:
-        out = os.path.join(tmp, "k_px.s")
-        cmd = [hipcc] + HIPCC_FLAGS + ["-S", "--cuda-device-only", os.path.join(CSRC, "k_px.hip"), "-o", out]
+        out = os.path.join(tmp, os.path.splitext(unit)[0] + ".s")
+        cmd = [hipcc] + HIPCC_FLAGS + ["-S", "--cuda-device-only", os.path.join(CSRC, unit), "-o", out]
         if verbose:
             print(" ".join(cmd), flush=True)
         subprocess.run(cmd, check=True, cwd=tmp)
@@ -151,17 +154,30 @@ def check_px_listing(verbose: bool = True) -> None:
     problems = []
     kernels = re.findall(r"^(_ZN5aussm\w+):[^\n]*\n(.*?)s_endpgm", text, flags=re.S | re.M)
     if not kernels:
-        raise RuntimeError("no kernels found in the listing of k_px.hip")
+        raise RuntimeError(f"no kernels found in the listing of {unit}")
+    by_hand, by_hand_v = set(), set()    # kernels with hand-written loads; ... whose destinations are v registers
     for name, body in kernels:
+        if re.search(r"ASMSTART\s*\n\s*global_load", body):
+            by_hand.add(name)
+        if re.search(r"ASMSTART\s*\n\s*global_load_dwordx[24]\s+v", body):
+            by_hand_v.add(name)
         for ln, ins in scan_listing(body):
             problems.append(f"{name}: line {ln}: `{ins.strip()}` touches registers with a load in flight")
     for name, count in re.findall(r"^\s*\.name:\s+(_ZN5aussm\w+)\n(?:.*\n)*?\s*\.vgpr_spill_count:\s+(\d+)", text, flags=re.M):
-        if "_px_" in name and int(count):
+        # (a spilled v register cannot be the accumulation-register destination of a load in flight)
+        if name in by_hand_v and int(count):
             problems.append(f"{name}: {count} vector registers spilled")
     if problems:
-        raise RuntimeError("k_px.hip: " + "; ".join(problems))
+        raise RuntimeError(f"{unit}: " + "; ".join(problems))
     if verbose:
-        print(f"k_px.hip: {len(kernels)} kernel listings checked", flush=True)
+        print(f"{unit}: {len(kernels)} kernel listings checked, {len(by_hand)} of them with hand-written loads", flush=True)
+    return len(kernels)
+
+
+def check_px_listing(verbose: bool = True) -> None:
+    """The listing check over the two units whose kernels issue loads by hand."""
+    for unit in ("k_px.hip", "k_xdl.hip"):
+        check_unit_listing(unit, verbose)
 
 
 if __name__ == "__main__":

@@ -1,6 +1,7 @@
-"""The compiler-dependent assumptions of the kernels that track their own loads (scan_px.h), checked on
-the assembly hipcc emits for them (no GPU needed): no vector register spilled, no register touched
-while it is the destination of a load in flight.  Plus the scanner itself on hand-made listings."""
+"""The compiler-dependent assumptions of the kernels that track their own loads (scan_px.h, and the
+prefetch into accumulation registers of scan_bwd_xdl.h), checked on the assembly hipcc emits for them
+(no GPU needed): no register touched while it is the destination of a load in flight, no vector register
+spilled where loads land in vector registers.  Plus the scanner itself on hand-made listings."""
 from aussm_amd import build
 
 
@@ -39,6 +40,17 @@ COUNTED = """
 	v_mov_b32_e32 v20, v2
 	v_mov_b32_e32 v21, v12
 """
+# the same for a prefetch into accumulation registers: copied out before the wait
+ACC_BAD = """
+	;;#ASMSTART
+	global_load_dwordx4 a[4:7], v[8:9], off
+	;;#ASMEND
+	v_accvgpr_read_b32 v30, a5
+	;;#ASMSTART
+	s_waitcnt vmcnt(0)
+	;;#ASMEND
+	v_accvgpr_read_b32 v31, a6
+"""
 
 
 def test_scanner_on_hand_made_listings():
@@ -46,7 +58,9 @@ def test_scanner_on_hand_made_listings():
     assert [ln for ln, _ in build.scan_listing(BAD)] == [5, 6]
     found = build.scan_listing(COUNTED)
     assert len(found) == 1 and "v21" in found[0][1]
+    found = build.scan_listing(ACC_BAD)
+    assert len(found) == 1 and "a5" in found[0][1]
 
 
-def test_px_kernels_keep_loads_in_flight_intact():
+def test_kernels_keep_loads_in_flight_intact():
     build.check_px_listing(verbose=False)
