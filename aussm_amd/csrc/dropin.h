@@ -502,34 +502,40 @@ __global__ __launch_bounds__(256) void fill_kernel(const FillArgs a) {
 // ---- fp32-accurate GEMM on the bf16 matrix cores, operands in fp32 with arbitrary strides -------
 //     C_z[m][n] (+)= sum_k A_z(m, k) B_z(k, n)           z = 0 .. Z-1
 //     C[m][n]    += sum_z sum_k A_z(m, k) B_z(k, n)      (reduce_z)
-// Workgroup tile 128 x 64, four wavefronts of 64 x 32 each, 32 of k per step, one workgroup per
-// (tile, slice of z, slice of k): zper consecutive z per workgroup (1 unless reduce_z) and ksplit slices
-// of k.  With more than one slice per element of C the results are summed into C with atomics (C holds
-// the addend beforehand).  Both operands are split into three bf16 pieces while
-// they are staged in LDS; the values of the next step are requested before the products of the
-// current one.
+// Workgroup tile 128 x (64 TNH), four wavefronts of 64 x (32 TNH) each, 32 of k per step, one workgroup
+// per (tile, slice of z, slice of k): zper consecutive z per workgroup (1 unless reduce_z) and ksplit
+// slices of k.  With more than one slice per element of C the results are summed into C with atomics (C
+// holds the addend beforehand).  Both operands are split into NP bf16 pieces while they are staged in
+// LDS; the values of the next step are requested before the products of the current one.
+// TNH = 2 (128 x 128 tiles: two thirds of the operand traffic per product, two wavefronts per SIMD instead
+// of four) was measured at the same speed as TNH = 1 on the backward call of the fused operator, as was
+// starting each workgroup's walk over the steps at a different point; the launcher uses TNH = 1.
 // K1: both operands are contiguous along k.  Then four neighbouring lanes fetch the 32 values of
 // one row as 16-byte vectors (VEC; rows need not be 16-byte aligned) - a wavefront request covers 16
 // cache lines.  Otherwise both are contiguous along m / n and a 16-lane row of the wavefront
 // fetches 16 neighbouring rows' values of one k.
-template <bool K1, bool VEC, int NP>
+// Rows of a tile that lie past M or N are fetched from the last valid row instead (row m of A only
+// reaches row m of C, which is not stored then), so only the last, partial step along k takes the
+// bounds-checked loads.
+template <bool K1, bool VEC, int NP, int TNH>
 __global__ __launch_bounds__(256) void split_gemm_kernel(const GemmArgs p) {
-  __shared__ u4 s_a[8 * NP * 64], s_b[4 * NP * 64];
+  constexpr int TN = 64 * TNH;         // columns of the workgroup tile
+  constexpr int EN = 2 * TNH;          // 16-wide column tiles per wavefront
+  __shared__ u4 s_a[8 * NP * 64], s_b[4 * TNH * NP * 64];
   const int tid = threadIdx.x, lane = tid & 63, wave = wave_index();
-  const int m0 = blockIdx.x * 128, n0 = blockIdx.y * 64;
+  const int m0 = blockIdx.x * 128, n0 = blockIdx.y * TN;
   const int zs = blockIdx.z / p.ksplit, ksl = blockIdx.z % p.ksplit;
   const int z_lo = zs * p.zper, z_hi = z_lo + p.zper < p.Z ? z_lo + p.zper : p.Z;
-  const int wm = (wave >> 1) * 4, wn = (wave & 1) * 2;       // this wavefront's first 16-wide tiles
+  const int wm = (wave >> 1) * 4, wn = (wave & 1) * EN;      // this wavefront's first 16-wide tiles
   const SplitK sk = make_splitk();
-  f4 acc[4][2];
+  f4 acc[4][EN];
 #pragma unroll
   for (int e = 0; e < 4; ++e)
 #pragma unroll
-    for (int f = 0; f < 2; ++f) acc[e][f] = f4{0, 0, 0, 0};
-  // the three records this thread stages: rows ra, ra + 64 of the A tile and row rb of the B tile, k slots kq ..
+    for (int f = 0; f < EN; ++f) acc[e][f] = f4{0, 0, 0, 0};
+  // the records this thread stages: rows ra, ra + 64 of the A tile and rows ra + 64 h of the B tile, k slots kq ..
   const int ra = K1 ? tid >> 2 : wave * 16 + (lane & 15);
   const int kq = 8 * (K1 ? tid & 3 : lane >> 4);
-  const int ma = m0 + ra, mb = ma + 64, nb = n0 + ra;
   // ... and where they go in LDS: [16-row tile][piece][16 g + (row + 4 g) % 16], g = kq / 8.  The rotation by
   // 4 g keeps the 16-byte writes of the K1 mapping (four neighbouring lanes = the four g of one row) and the
   // reads (16 neighbouring lanes = 16 rows of one g) both free of bank conflicts.
@@ -537,74 +543,94 @@ __global__ __launch_bounds__(256) void split_gemm_kernel(const GemmArgs p) {
   const int rslot = (lane & 48) + ((lane + (lane >> 4) * 4) & 15);       // the record of (row lane % 16, g lane / 16)
   // uniform bases, 32-bit per-thread offsets (a z-slice of either operand is below 2^31 elements)
   const unsigned sak = (unsigned)p.sak, sbk = (unsigned)p.sbk;
-  const unsigned oa0 = (unsigned)ma * (unsigned)p.sam + (unsigned)kq * sak;
-  const unsigned oa1 = (unsigned)mb * (unsigned)p.sam + (unsigned)kq * sak;
-  const unsigned ob0 = (unsigned)nb * (unsigned)p.sbn + (unsigned)kq * sbk;
+  unsigned oa[2], ob[TNH];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int m = m0 + ra + 64 * h;
+    oa[h] = (unsigned)(m < p.M ? m : p.M - 1) * (unsigned)p.sam + (unsigned)kq * sak;
+  }
+#pragma unroll
+  for (int h = 0; h < TNH; ++h) {
+    const int n = n0 + ra + 64 * h;
+    ob[h] = (unsigned)(n < p.N ? n : p.N - 1) * (unsigned)p.sbn + (unsigned)kq * sbk;
+  }
   const int nk = (p.K + 31) / 32, per = (nk + p.ksplit - 1) / p.ksplit;
   const int it0 = ksl * per, it1 = it0 + per < nk ? it0 + per : nk;
   const int nit = it1 > it0 ? (it1 - it0) * (z_hi - z_lo) : 0;      // steps of this workgroup: (z, k step) pairs
-  const bool inside = m0 + 128 <= p.M && n0 + 64 <= p.N;      // uniform over the workgroup
-  float va[2][8], vb[8];
-  auto fetch = [&](int step) {
-    const int z = z_lo + step / (it1 - it0), it = it0 + step % (it1 - it0);
+  float va[2][8], vb[TNH][8];
+  int fz = z_lo, fit = it0;                   // (z, k step) of the next fetch: steps are fetched in order
+  auto fetch = [&]() {
+    const int z = fz, it = fit;
+    if (++fit == it1) { fit = it0; ++fz; }
     const float* __restrict__ Az = p.A + z * p.saz;
     const float* __restrict__ Bz = p.Bm + z * p.sbz;
     const unsigned ka = (unsigned)(it * 32) * sak, kb = (unsigned)(it * 32) * sbk;
-    if (inside && it * 32 + 32 <= p.K) {
+    if (it * 32 + 32 <= p.K) {
       if constexpr (K1 && VEC) {
         // 16-byte loads that are only known to be 4-byte aligned (rows start anywhere when the row length is
         // not a multiple of four): the memory pipeline takes them, the type tells the compiler so
         typedef float f4u __attribute__((ext_vector_type(4), aligned(4)));
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-          const f4u x0 = *reinterpret_cast<const f4u*>(Az + (oa0 + ka + 4 * h));
-          const f4u x1 = *reinterpret_cast<const f4u*>(Az + (oa1 + ka + 4 * h));
-          const f4u x2 = *reinterpret_cast<const f4u*>(Bz + (ob0 + kb + 4 * h));
+        for (int q = 0; q < 2; ++q) {
 #pragma unroll
-          for (int c = 0; c < 4; ++c) {
-            va[0][4 * h + c] = x0[c];
-            va[1][4 * h + c] = x1[c];
-            vb[4 * h + c] = x2[c];
+          for (int h = 0; h < 2; ++h) {
+            const f4u x = *reinterpret_cast<const f4u*>(Az + (oa[h] + ka + 4 * q));
+#pragma unroll
+            for (int c = 0; c < 4; ++c) va[h][4 * q + c] = x[c];
+          }
+#pragma unroll
+          for (int h = 0; h < TNH; ++h) {
+            const f4u x = *reinterpret_cast<const f4u*>(Bz + (ob[h] + kb + 4 * q));
+#pragma unroll
+            for (int c = 0; c < 4; ++c) vb[h][4 * q + c] = x[c];
           }
         }
       } else {
 #pragma unroll
         for (int c = 0; c < 8; ++c) {
-          va[0][c] = Az[oa0 + ka + (unsigned)c * sak];
-          va[1][c] = Az[oa1 + ka + (unsigned)c * sak];
-          vb[c] = Bz[ob0 + kb + (unsigned)c * sbk];
+#pragma unroll
+          for (int h = 0; h < 2; ++h) va[h][c] = Az[oa[h] + ka + (unsigned)c * sak];
+#pragma unroll
+          for (int h = 0; h < TNH; ++h) vb[h][c] = Bz[ob[h] + kb + (unsigned)c * sbk];
         }
       }
     } else {
 #pragma unroll
       for (int c = 0; c < 8; ++c) {
         const bool kok = it * 32 + kq + c < p.K;
-        va[0][c] = (ma < p.M && kok) ? Az[oa0 + ka + (unsigned)c * sak] : 0.0f;
-        va[1][c] = (mb < p.M && kok) ? Az[oa1 + ka + (unsigned)c * sak] : 0.0f;
-        vb[c] = (nb < p.N && kok) ? Bz[ob0 + kb + (unsigned)c * sbk] : 0.0f;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) va[h][c] = kok ? Az[oa[h] + ka + (unsigned)c * sak] : 0.0f;
+#pragma unroll
+        for (int h = 0; h < TNH; ++h) vb[h][c] = kok ? Bz[ob[h] + kb + (unsigned)c * sbk] : 0.0f;
       }
     }
   };
-  // (requesting the values two steps ahead, with a second register set, was measured: the registers cost a
-  // wavefront per SIMD and the launch got 25 % slower - the other wavefronts hide the latency better)
-  if (nit > 0) fetch(0);
+  // (Cycle marks inside this loop, four wavefronts per SIMD: per step the 48 matrix instructions of a wavefront
+  // and their LDS reads take about 1.3-1.5 k cycles, splitting the next operands and getting them into LDS
+  // 2.4-3.0 k, issuing the loads after them 0.6-0.8 k; the loads have always landed when they are asked for and
+  // each barrier costs about 100 cycles.  The loop is bound by vector-instruction issue - the split, the address
+  // arithmetic - not by memory: requesting the values two steps ahead with a second register set made the
+  // launch 25 % slower, the registers cost a wavefront per SIMD.)
+  if (nit > 0) fetch();
   for (int step = 0; step < nit; ++step) {
-    u4 pa[2][NP], pb[NP];
-    split8<NP>(sk, va[0], pa[0]);
-    split8<NP>(sk, va[1], pa[1]);
-    split8<NP>(sk, vb, pb);
+    u4 pa[2][NP], pb[TNH][NP];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) split8<NP>(sk, va[h], pa[h]);
+#pragma unroll
+    for (int h = 0; h < TNH; ++h) split8<NP>(sk, vb[h], pb[h]);
     __syncthreads();
 #pragma unroll
     for (int c = 0; c < NP; ++c) {
-      s_a[slot + c * 64] = pa[0][c];
-      s_a[slot + 4 * (NP * 64) + c * 64] = pa[1][c];
-      s_b[slot + c * 64] = pb[c];
+#pragma unroll
+      for (int h = 0; h < 2; ++h) s_a[slot + 4 * h * (NP * 64) + c * 64] = pa[h][c];
+#pragma unroll
+      for (int h = 0; h < TNH; ++h) s_b[slot + 4 * h * (NP * 64) + c * 64] = pb[h][c];
     }
     __syncthreads();
-    if (step + 1 < nit) fetch(step + 1);      // in flight during the products
-    u4 rb[2][NP];
+    if (step + 1 < nit) fetch();              // in flight during the products
+    u4 rb[EN][NP];
 #pragma unroll
-    for (int f = 0; f < 2; ++f)
+    for (int f = 0; f < EN; ++f)
 #pragma unroll
       for (int c = 0; c < NP; ++c) rb[f][c] = s_b[((wn + f) * NP + c) * 64 + rslot];
 #pragma unroll
@@ -613,21 +639,33 @@ __global__ __launch_bounds__(256) void split_gemm_kernel(const GemmArgs p) {
 #pragma unroll
       for (int c = 0; c < NP; ++c) rA[c] = s_a[((wm + e) * NP + c) * 64 + rslot];
 #pragma unroll
-      for (int f = 0; f < 2; ++f) acc[e][f] = xmm<NP>(rA, rb[f], acc[e][f]);
+      for (int f = 0; f < EN; ++f) acc[e][f] = xmm<NP>(rA, rb[f], acc[e][f]);
     }
   }
   // result tile (e, f): lane (column = lane % 16, rows 4 (lane / 16) + a)
   float* __restrict__ C = p.C + (p.reduce_z ? 0 : z_lo * p.scz);
   const bool atomic = p.ksplit > 1 || (p.reduce_z && p.zper < p.Z);
+  // element offsets inside a z-slice of C fit 32 bits (checked by the caller)
+  const unsigned scm = (unsigned)p.scm, scn = (unsigned)p.scn;
+  const int mr = m0 + wm * 16 + 4 * (lane >> 4), nc = n0 + wn * 16 + (lane & 15);
+  const unsigned o0 = (unsigned)mr * scm + (unsigned)nc * scn;
+  if (atomic && m0 + 128 <= p.M && n0 + TN <= p.N) {       // uniform: a whole tile, summed into C
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+#pragma unroll
+      for (int f = 0; f < EN; ++f)
+#pragma unroll
+        for (int a = 0; a < 4; ++a) atomicAdd(C + (o0 + (unsigned)(16 * e + a) * scm + (unsigned)(16 * f) * scn), acc[e][f][a]);
+    return;
+  }
 #pragma unroll
   for (int e = 0; e < 4; ++e)
 #pragma unroll
-    for (int f = 0; f < 2; ++f)
+    for (int f = 0; f < EN; ++f)
 #pragma unroll
       for (int a = 0; a < 4; ++a) {
-        const int m = m0 + (wm + e) * 16 + 4 * (lane >> 4) + a, nn = n0 + (wn + f) * 16 + (lane & 15);
-        if (m < p.M && nn < p.N) {
-          float* c = C + m * p.scm + nn * p.scn;
+        if (mr + 16 * e + a < p.M && nc + 16 * f < p.N) {
+          float* c = C + (o0 + (unsigned)(16 * e + a) * scm + (unsigned)(16 * f) * scn);
           if (atomic) atomicAdd(c, acc[e][f][a]);
           else *c = p.accumulate ? *c + acc[e][f][a] : acc[e][f][a];
         }

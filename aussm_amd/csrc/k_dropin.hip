@@ -73,11 +73,9 @@ int run_split_gemm(const GemmArgs& a, hipStream_t s) {
   if (gz > 65535) return -2;
   const dim3 grid((unsigned)((a.M + 127) / 128), (unsigned)((a.N + 63) / 64), (unsigned)gz);
   const bool k1 = a.sak == 1 && a.sbk == 1;
-#ifndef AUSSM_GEMM_NP
-#define AUSSM_GEMM_NP 3
-#endif
-  if (k1) hipLaunchKernelGGL((split_gemm_kernel<true, true, AUSSM_GEMM_NP>), grid, dim3(256), 0, s, a);
-  else hipLaunchKernelGGL((split_gemm_kernel<false, false, AUSSM_GEMM_NP>), grid, dim3(256), 0, s, a);
+  constexpr int NP = 3;               // bf16 pieces per operand: fp32-accurate products
+  if (k1) hipLaunchKernelGGL((split_gemm_kernel<true, true, NP, 1>), grid, dim3(256), 0, s, a);
+  else hipLaunchKernelGGL((split_gemm_kernel<false, false, NP, 1>), grid, dim3(256), 0, s, a);
   return launch_status();
 }
 

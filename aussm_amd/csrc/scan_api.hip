@@ -618,11 +618,12 @@ static DropinBlocks dropin_blocks(int b, int d, int n, int L) {
 constexpr long GEMM_TARGET = 768;     // workgroups per launch aimed at (measured: 512 +4 %, 1024 +5 %, 256 +22 % of the backward call)
 static void gemm_slices(GemmArgs& g) {
   const long tiles = (long)((g.M + 127) / 128) * ((g.N + 63) / 64);
+  const long target = GEMM_TARGET;
   const int nk = (g.K + 31) / 32;
   long zs = 1;                                   // slices of z
   g.zper = 1;
   if (g.reduce_z) {
-    zs = (GEMM_TARGET + tiles - 1) / tiles;
+    zs = (target + tiles - 1) / tiles;
     if (zs > g.Z) zs = g.Z;
     if (zs < 1) zs = 1;
     g.zper = (int)((g.Z + zs - 1) / zs);
@@ -630,7 +631,7 @@ static void gemm_slices(GemmArgs& g) {
   } else {
     zs = g.Z;
   }
-  long s = (GEMM_TARGET + tiles * zs - 1) / (tiles * zs);
+  long s = (target + tiles * zs - 1) / (tiles * zs);
   if (s > nk / 4) s = nk / 4;
   if (s < 1) s = 1;
   while (s > 1 && zs * s > 65535) --s;
