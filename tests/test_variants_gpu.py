@@ -235,7 +235,7 @@ def test_split_along_sequence_matches_unsplit(variant, lowp):
                                       lv["z"], h, return_last_state=True)
         ((y * p["dy"].cuda()).sum() + (hL * dhL.cuda().conj()).real.sum()).backward()
         torch.cuda.synchronize()
-        out = {k: v.grad.float() for k, v in lv.items()}
+        out = {k: (v.grad if v.grad.is_complex() else v.grad.float()) for k, v in lv.items()}
         out["h0"] = h.grad
         out["y"], out["hL"] = y.detach(), hL.detach()
         return out
@@ -251,3 +251,56 @@ def test_split_along_sequence_matches_unsplit(variant, lowp):
         tol = 2e-2 if (lowp and k in low) else ATOL
         scale = max(1.0, float(w.abs().max()))
         torch.testing.assert_close(g / scale, w / scale, atol=tol, rtol=tol, msg=lambda m, k=k: f"{k}: {m}")
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_split_random_shapes_match_unsplit(seed):
+    """Seeded sweep of calls that split along the sequence (few batch x channel-group pairs, ragged lengths,
+    1 to 64 states, gate / initial state / softplus and bias present or not) against the same call with the
+    split switched off: outputs, final state and every gradient."""
+    import random
+    from aussm_amd import _lib, scan
+    r = random.Random(900 + seed)
+    variant = r.choice(["real", "complex"])
+    B, D = r.randint(1, 3), r.choice([r.randint(1, 64), r.randint(65, 200)])
+    N = r.choice([1, 3, 8, 16, 17, 33, 64])
+    L = r.choice([r.randint(257, 700), 128 * r.randint(2, 6), 4 * r.randint(65, 300)])
+    gate, with_h0, softplus = r.random() < 0.5, r.random() < 0.5, r.random() < 0.5
+    p = O.make_core_inputs(B, D, N, L, seed=seed, variant=variant, gate=gate)
+    names = (["u", "delta", "A", "Bm", "Cm", "Dskip"] if variant == "real"
+             else ["u", "delta", "rho", "theta", "Bc", "Cc", "Dskip"]) + (["z"] if gate else [])
+    h0 = _h0(B, D, N, variant == "complex", 7) if with_h0 else None
+    dhL = _h0(B, D, N, variant == "complex", 8)
+    bias = torch.randn(D, generator=torch.Generator().manual_seed(seed)) if variant == "real" and softplus else None
+
+    def run():
+        lv = {k: p[k].clone().cuda().requires_grad_(True) for k in names}
+        h = h0.clone().cuda().requires_grad_(True) if with_h0 else None
+        if variant == "real":
+            y, hL = scan.selective_scan_fn(lv["u"], lv["delta"], lv["A"], lv["Bm"], lv["Cm"], lv["Dskip"], z=lv.get("z"),
+                                           delta_bias=None if bias is None else bias.cuda(), delta_softplus=softplus,
+                                           return_last_state=True, h0=h)
+        else:
+            y, hL = scan.complex_scan(lv["u"], lv["delta"], lv["rho"], lv["theta"], lv["Bc"], lv["Cc"], lv["Dskip"],
+                                      lv.get("z"), h, return_last_state=True)
+        ((y * p["dy"].cuda()).sum() + (hL * dhL.cuda().conj()).real.sum()).backward()
+        torch.cuda.synchronize()
+        out = {k: v.grad for k, v in lv.items()}
+        if with_h0:
+            out["h0"] = h.grad
+        out["y"], out["hL"] = y.detach(), hL.detach()
+        return out
+
+    print(f"case split sweep seed={seed} {variant} B={B} D={D} N={N} L={L} gate={gate} h0={with_h0} softplus={softplus}",
+          flush=True)
+    vcode = _lib.VAR_COMPLEX if variant == "complex" else _lib.VAR_REAL
+    assert _lib.load().aussm_scan_workspace_floats(vcode, B, D, N, L, 16, 0) > 0
+    got = run()
+    with _lib.options(split_cap=0):
+        want = run()
+    for k in want:
+        w, g = want[k], got[k]
+        if w.is_complex():
+            w, g = torch.view_as_real(w), torch.view_as_real(g)
+        scale = max(1.0, float(w.abs().max()))
+        torch.testing.assert_close(g / scale, w / scale, atol=ATOL, rtol=RTOL, msg=lambda m, k=k: f"{k}: {m}")
