@@ -123,9 +123,16 @@ void run_seg_carry_real(bool adjoint, float* seg, const float* ptot, const float
   else hipLaunchKernelGGL(seg_carry_real_kernel<false>, grid, dim3(256), 0, s, seg, ptot, A, first, last, B, D, N, ns);
 }
 
-// marks an auxiliary buffer as NOT filled (a forward kernel that does not fill it ran)
-__global__ void aux_invalidate_kernel(float* tag) { *tag = 0.0f; }
-void run_aux_invalidate(float* tag, hipStream_t s) { hipLaunchKernelGGL(aux_invalidate_kernel, dim3(1), dim3(1), 0, s, tag); }
+// marks an auxiliary buffer as NOT filled (a forward kernel that does not fill it ran) and / or the
+// operand images behind it as not belonging to the call's tensors
+__global__ void aux_invalidate_kernel(float* tag, int first, int last) {
+  if ((int)threadIdx.x >= first && (int)threadIdx.x <= last) tag[threadIdx.x] = 0.0f;
+}
+void run_aux_invalidate(float* tag, bool fill_tag, bool images_tag, hipStream_t s) {
+  if (!fill_tag && !images_tag) return;
+  hipLaunchKernelGGL(aux_invalidate_kernel, dim3(1), dim3(64), 0, s, tag, fill_tag ? 0 : AUX_IMG_FP,
+                     images_tag ? AUX_IMG_FP + 7 : 0);
+}
 
 int run_conv_fwd(const ConvArgs& a, hipStream_t s) {
   const size_t rows = (size_t)a.B * a.L;

@@ -10,14 +10,14 @@ void run_px_prep(const PrepArgs& a, int B, int in_dtype, hipStream_t s) {
   else hipLaunchKernelGGL(unitary_px_prep_kernel<float>, grid, dim3(256), 0, s, a);
 }
 
-int run_px_fwd(const FwdArgs& a, const u4* img, int in_dtype, hipStream_t s) {
+int run_px_fwd(const FwdArgs& a, const u4* img, const ImgNote& note, int in_dtype, hipStream_t s) {
   const dim3 grid((unsigned)(a.B * a.ncg));
   if (in_dtype == 1) {
-    if (a.z) hipLaunchKernelGGL((unitary_fwd_px_kernel<true, bf16_t>), grid, dim3(512), 0, s, a, img);
-    else hipLaunchKernelGGL((unitary_fwd_px_kernel<false, bf16_t>), grid, dim3(512), 0, s, a, img);
+    if (a.z) hipLaunchKernelGGL((unitary_fwd_px_kernel<true, bf16_t>), grid, dim3(512), 0, s, a, img, note);
+    else hipLaunchKernelGGL((unitary_fwd_px_kernel<false, bf16_t>), grid, dim3(512), 0, s, a, img, note);
   } else {
-    if (a.z) hipLaunchKernelGGL((unitary_fwd_px_kernel<true, float>), grid, dim3(512), 0, s, a, img);
-    else hipLaunchKernelGGL((unitary_fwd_px_kernel<false, float>), grid, dim3(512), 0, s, a, img);
+    if (a.z) hipLaunchKernelGGL((unitary_fwd_px_kernel<true, float>), grid, dim3(512), 0, s, a, img, note);
+    else hipLaunchKernelGGL((unitary_fwd_px_kernel<false, float>), grid, dim3(512), 0, s, a, img, note);
   }
   return launch_status();
 }

@@ -23,7 +23,7 @@ struct Cfg { int nw, nt; };
 int run_core_fwd(int variant, const FwdArgs& a, int in_dtype, Cfg c, hipStream_t s);
 int run_unitary_bwd_generic(const UniBwdArgs& a, int in_dtype, Cfg c, hipStream_t s);
 int run_rec_bwd(int variant, const RecBwdArgs& a, int in_dtype, hipStream_t s);
-void run_aux_invalidate(float* tag, hipStream_t s);
+void run_aux_invalidate(float* tag, bool fill_tag, bool images_tag, hipStream_t s);   // clears tag(s) in the buffer's pad
 // split of the complex / real scans along L: adjoint entering every segment, chain of the real scan's segments
 void run_adjoint_seg(int variant, const AdjSegArgs& a, int in_dtype, unsigned grid, hipStream_t s);
 void run_bc_to_f32(const void* Bm, const void* Cm, float* oB, float* oC, size_t n, hipStream_t s);   // bf16 -> float
@@ -43,7 +43,7 @@ void run_seg_carry_bwd(float* seg, const float* ptot, const float* dhL, float* d
 
 // ---- k_px.hip: matrix-core unitary scans on operands prepared by a pre-pass
 void run_px_prep(const PrepArgs& a, int B, int in_dtype, hipStream_t s);
-int run_px_fwd(const FwdArgs& a, const u4* img, int in_dtype, hipStream_t s);
+int run_px_fwd(const FwdArgs& a, const u4* img, const ImgNote& note, int in_dtype, hipStream_t s);
 int run_px_bwd(const UniBwdArgs& a, const u4* img, int in_dtype, hipStream_t s);
 
 // ---- k_dropin.hip: the reference's 12-input operator as fused kernels

@@ -14,7 +14,8 @@ namespace {
 
 // Process-wide options (aussm_set_option): kernel selection for comparisons and tuning.  They are
 // plain atomics read once per call; -1 means "let the launcher decide".
-std::atomic<int> g_opt[AUSSM_OPT_COUNT] = {{-1}, {-1}, {-1}, {-1}, {-1}};
+std::atomic<int> g_opt[AUSSM_OPT_COUNT] = {{-1}, {-1}, {-1}, {-1}, {-1}, {-1}};
+static_assert(AUSSM_OPT_COUNT == 6, "one initialiser per option");
 inline int opt(int key) { return g_opt[key].load(std::memory_order_relaxed); }
 
 // ---- configuration of the vector-ALU kernels --------------------------------------------------
@@ -62,7 +63,7 @@ inline bool misaligned(const void* p, size_t a) { return p && (reinterpret_cast<
 // The matrix-core kernels cost the same for every N <= 16 while the vector-ALU ones scale with N:
 // measured, the crossover is between N = 4 (vector ALU 15 % faster) and N = 8 (matrix 30 % faster).
 constexpr int MATRIX_MIN_STATE = 6;
-constexpr int DEFAULT_FWD_MODE = 3, DEFAULT_BWD_MODE = 6;   // (6 falls back to 3 where the call brings no workspace)
+constexpr int DEFAULT_FWD_MODE = 6, DEFAULT_BWD_MODE = 6;   // (6 falls back to 3 where the call brings no workspace)
 inline int kernel_mode(int key, int dflt, int N) {
   const int e = opt(key);
   if (e >= 0) return e;                        // an explicit choice is honoured for every N <= 16
@@ -143,21 +144,24 @@ inline BcF32 generic_bc(int variant, const void* Bm, const void* Cm, float* ws, 
   return BcF32{fB, fB + n, 2};
 }
 
-// Workspace of the prepared operands: one image per (batch element, chunk), sized for the larger
-// (backward) image; a forward and a backward call each write their own images into it.
+// Workspace of the prepared operands: per (batch element, chunk) one backward image and, behind
+// all of those, one forward image.  The forward call of a training step writes both (one pre-pass);
+// a backward call whose auxiliary buffer does not hold the images of its own tensors writes its own.
+// The size does not depend on the option table: a buffer sized under one set of options fits every other.
+inline size_t img_chunks(int B, int L) { return (size_t)B * ((L + XT - 1) / XT); }
 inline size_t img_floats(int B, int N, int L, int ck) {
   if (!matrix_shape(N, L, ck)) return 0;
-  // (below MATRIX_MIN_STATE only when the prepared-operand kernels have been asked for explicitly)
-  if (N < MATRIX_MIN_STATE && opt(AUSSM_OPT_UNITARY_FWD) != 6 && opt(AUSSM_OPT_UNITARY_BWD) != 6) return 0;
-  return (size_t)B * ((L + XT - 1) / XT) * PXB_REC * 4;
+  return img_chunks(B, L) * (PXB_REC + PXF_REC) * 4;
 }
-// Layout of the auxiliary buffer: [B*D*L floats Im(P S)] [AUX_PAD] [segment states] [images]
-struct AuxLayout { float* seg; u4* img; };
+// Layout of the auxiliary buffer: [B*D*L floats Im(P S)] [AUX_PAD] [segment states] [backward images] [forward images]
+struct AuxLayout { float* seg; u4* img; u4* fimg; uint32_t* stamp; };
 inline AuxLayout aux_layout(float* aux, int B, int D, int N, int L, int ck) {
-  if (!aux) return AuxLayout{nullptr, nullptr};
-  float* seg = aux + (size_t)B * D * L + AUX_PAD;
-  float* img = seg + seg_floats(B, D, N, L, seg_capacity(B, D, N, L, ck));
-  return AuxLayout{seg, img_floats(B, N, L, ck) ? reinterpret_cast<u4*>(img) : nullptr};
+  if (!aux) return AuxLayout{nullptr, nullptr, nullptr, nullptr};
+  float* pad = aux + (size_t)B * D * L;
+  float* seg = pad + AUX_PAD;
+  u4* img = reinterpret_cast<u4*>(seg + seg_floats(B, D, N, L, seg_capacity(B, D, N, L, ck)));
+  if (!img_floats(B, N, L, ck)) return AuxLayout{seg, nullptr, nullptr, nullptr};
+  return AuxLayout{seg, img, img + img_chunks(B, L) * PXB_REC, reinterpret_cast<uint32_t*>(pad) + AUX_IMG_FP};
 }
 
 // Kernel family of a call whose tensors are 16-byte aligned: 0 vector ALU, 2 / 3 / 5 matrix-core kernels
@@ -191,9 +195,10 @@ inline int mfma_fwd_mode(const FwdArgs& a, int in_dtype, bool have_img) {
 int launch_unitary_fwd(FwdArgs a, int in_dtype, hipStream_t s, AuxLayout ws) {
   const int mode = mfma_fwd_mode(a, in_dtype, ws.img != nullptr);
   // Im(P S) is only worth writing when a backward call can follow (it needs the checkpoints too);
-  // a call that does not fill the buffer marks it as not filled
+  // a call that does not fill the buffer marks it as not filled, and a call that does not prepare
+  // images clears the note about the ones behind the buffer
   const bool fill = a.aux && a.hck && mode >= 2;
-  if (a.aux && !fill) run_aux_invalidate(a.aux + (size_t)a.B * a.D * a.L, s);
+  if (a.aux) run_aux_invalidate(a.aux + (size_t)a.B * a.D * a.L, !fill, mode != 6 && ws.stamp, s);
   if (!fill) a.aux = nullptr;
   if (!mode) return run_core_fwd(VAR_UNITARY, a, in_dtype, pick_cfg(a.N, 8), s);
   const int B = a.B, L = a.L;
@@ -212,9 +217,13 @@ int launch_unitary_fwd(FwdArgs a, int in_dtype, hipStream_t s, AuxLayout ws) {
     }
   }
   if (mode == 6) {
-    PrepArgs pa{a.Bm, a.Cm, ws.img, nullptr, a.N, L, (L + XT - 1) / XT};
+    // one pre-pass for the step: the backward call that follows finds its images too (it needs the
+    // checkpoints, so a call without them is not followed by one)
+    const bool with_bwd = a.hck != nullptr;
+    PrepArgs pa{a.Bm, a.Cm, ws.fimg, with_bwd ? ws.img : nullptr, a.N, L, (L + XT - 1) / XT, nullptr, ImgStamp{}};
     run_px_prep(pa, B, in_dtype, s);
-    return run_px_fwd(a, ws.img, in_dtype, s);
+    const ImgNote note{ws.stamp, img_stamp(a.Bm, a.Cm, B, a.N, L, in_dtype, with_bwd)};
+    return run_px_fwd(a, ws.fimg, note, in_dtype, s);
   }
   return run_xdl_fwd(mode, a, in_dtype, s);
 }
@@ -398,7 +407,7 @@ int aussm_unitary_fwd_static(const void* u, const void* delta, const float* thet
   a.ld = L; a.ns = 1; a.hs = 1; a.ho = 0; a.urep = 1;
   // (every segment state the scan reads is written earlier in the same call: nothing in the
   // scratch has to start at zero)
-  return launch_unitary_fwd(a, in_dtype, (hipStream_t)stream, AuxLayout{scratch, nullptr});
+  return launch_unitary_fwd(a, in_dtype, (hipStream_t)stream, AuxLayout{scratch, nullptr, nullptr, nullptr});
 }
 
 int aussm_complex_fwd(const void* u, const void* delta, const float* rho, const float* theta, const void* Bc,
@@ -479,7 +488,8 @@ int aussm_unitary_bwd_aux(const float* dy, const float* dhL, const void* u, cons
       // The prepared-operand kernel needs Im(P S) from the forward call in the auxiliary buffer; its
       // workgroups leave at once if the buffer's tag says it is not there, and the kernel that
       // recomputes it (launched behind, leaving at once in the opposite case) does the work.
-      PrepArgs pa{Bc, Cc, nullptr, ws.img, N, L, (L + XT - 1) / XT};
+      // (the pre-pass leaves at once when the forward call of these tensors has left the images)
+      PrepArgs pa{Bc, Cc, nullptr, ws.img, N, L, (L + XT - 1) / XT, ws.stamp, img_stamp(Bc, Cc, B, N, L, in_dtype, true)};
       run_px_prep(pa, B, in_dtype, s);
       a.tag_mode = 1;
       if (int e = run_px_bwd(a, ws.img, in_dtype, s)) return e;
@@ -593,19 +603,22 @@ static size_t dropin_xp_floats(int d, int n) { return (size_t)d * dropin_state_b
 // what fills the chip with one workgroup per compute unit (fewer would idle units, more would only
 // shorten the blocks and repeat the per-launch set-up, the rows of x among it, more often).
 // budget of a block (phase adjoints; prepared tiles of u), in floats
-static size_t dropin_block_floats() {
+// (the option can only lower it: the workspace query sizes for the full budget, so a buffer obtained under
+// one setting of the option holds what a call under any other setting uses)
+constexpr int DROPIN_BLOCK_KFLOATS = 12800;
+static size_t dropin_block_floats(bool largest) {
   const int o = opt(AUSSM_OPT_BLOCK_KFLOATS);
-  return (size_t)(o > 0 ? o : 12800) << 10;
+  return (size_t)(!largest && o > 0 && o < DROPIN_BLOCK_KFLOATS ? o : DROPIN_BLOCK_KFLOATS) << 10;
 }
 struct DropinBlocks { int bg, ct; };
-static DropinBlocks dropin_blocks(int b, int d, int n, int L) {
+static DropinBlocks dropin_blocks(int b, int d, int n, int L, bool largest = false) {
   const int nw = dropin_channels_per_workgroup((d + 31) / 32);
   const int wgs_per_b = (d * dropin_state_blocks(n) + nw - 1) / nw;
   int bg = (256 + wgs_per_b - 1) / wgs_per_b;
   if (bg > b) bg = b;
   const int ng = (b + bg - 1) / bg;
   bg = (b + ng - 1) / ng;
-  const size_t per_tile = (size_t)bg * d * n * DT, cap = dropin_block_floats();
+  const size_t per_tile = (size_t)bg * d * n * DT, cap = dropin_block_floats(largest);
   const int ntiles = (L + DT - 1) / DT;
   size_t tmax = cap / per_tile;
   if (tmax < 1) tmax = 1;
@@ -648,9 +661,9 @@ static int dropin_check(int b, int d, int n, int L) {
 // floats of one prepared tile of u (all compiled steps of the contraction, three pieces, 64 lanes of 16 bytes)
 static size_t dropin_tile_floats(int d) { return (size_t)dropin_compiled_ks((d + 31) / 32) * 3 * 64 * 4; }
 // tiles per launch of the forward call: its prepared tiles of u (all batch elements) stay within the block budget
-static int dropin_fwd_chunk_tiles(int b, int d, int L) {
+static int dropin_fwd_chunk_tiles(int b, int d, int L, bool largest = false) {
   const int ntiles = (L + DT - 1) / DT;
-  size_t tmax = dropin_block_floats() / ((size_t)b * dropin_tile_floats(d));
+  size_t tmax = dropin_block_floats(largest) / ((size_t)b * dropin_tile_floats(d));
   if (tmax < 1) tmax = 1;
   const size_t nc = ((size_t)ntiles + tmax - 1) / tmax;
   return (int)(((size_t)ntiles + nc - 1) / nc);
@@ -660,10 +673,10 @@ size_t aussm_ssm_adaptive_unitary_workspace_floats(int b, int d, int n, int L, i
   if (dropin_check(b, d, n, L) != AUSSM_OK) return 0;
   size_t f = dropin_xp_floats(d, n);
   if (backward) {
-    const DropinBlocks k = dropin_blocks(b, d, n, L);
+    const DropinBlocks k = dropin_blocks(b, d, n, L, true);
     f += 2 * round4((size_t)b * d * n) + (size_t)k.bg * k.ct * DT * d * n + (size_t)k.bg * k.ct * dropin_tile_floats(d);
   } else {
-    f += (size_t)b * dropin_fwd_chunk_tiles(b, d, L) * dropin_tile_floats(d);
+    f += (size_t)b * dropin_fwd_chunk_tiles(b, d, L, true) * dropin_tile_floats(d);
   }
   return f;
 }

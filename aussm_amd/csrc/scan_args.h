@@ -15,8 +15,12 @@ enum { VAR_UNITARY = 0, VAR_COMPLEX = 1, VAR_REAL = 2 };
 
 // The optional auxiliary buffer of the unitary scan holds B*D*L floats followed by AUX_PAD floats;
 // the first of those is AUX_TAG when a forward kernel has filled the buffer, anything else if not.
+// Words AUX_IMG_FP .. + 7 of the pad describe the operand images behind it (ImgStamp below): written
+// by the forward kernel that ran on freshly prepared images, cleared by every other forward call.
 constexpr uint32_t AUX_TAG = 0x4f484950u;
+constexpr uint32_t IMG_TAG = 0x494d4147u;
 constexpr int AUX_PAD = 64;
+constexpr int AUX_IMG_FP = 8;
 
 typedef uint32_t u4 __attribute__((ext_vector_type(4)));
 
@@ -138,13 +142,29 @@ constexpr int PXB_A = 4 * PX_NP * XN * 4;                   // backward: bt_r, b
 constexpr int PXB_B = 3 * PX_NP * XT * 4;                   //           bs, g_r, g_i
 constexpr int PXB_REC = PXB_A + PXB_B;                      // 1920 records = 30 KiB
 
+// What a set of images was made from.  A backward call recomputes its images unless the stamp in
+// the auxiliary buffer equals the stamp of its own arguments: same tensors (addresses), same
+// shape and input type, backward images present.
+struct ImgStamp { uint32_t w[8]; };
+inline ImgStamp img_stamp(const void* Bm, const void* Cm, int B, int N, int L, int in_dtype, bool with_bwd) {
+  const uint64_t b = (uint64_t)(uintptr_t)Bm, c = (uint64_t)(uintptr_t)Cm;
+  return ImgStamp{{IMG_TAG, (uint32_t)B, (uint32_t)N, (uint32_t)L, (uint32_t)in_dtype | (with_bwd ? 0x100u : 0u),
+                   (uint32_t)b ^ (uint32_t)(b >> 32) * 0x9e3779b1u, (uint32_t)c ^ (uint32_t)(c >> 32) * 0x9e3779b1u,
+                   (uint32_t)(b >> 4) + (uint32_t)(c >> 4) * 31u}};
+}
+
 struct PrepArgs {
   const void* Bm;       // [B, N, ld, 2] Tin
   const void* Cm;
   u4* fimg;             // [B, nch, PXF_REC] or null
   u4* bimg;             // [B, nch, PXB_REC] or null
   int N, ld, nch;       // nch = ceil(ld / 32) chunks per batch element
+  const uint32_t* have; // or null: the launch has nothing to do if these eight words equal `want`
+  ImgStamp want;
 };
+
+// Where a forward kernel that ran on freshly prepared images records what they were made from
+struct ImgNote { uint32_t* dst; ImgStamp stamp; };
 
 constexpr int CONV_MAX_K = 8;
 constexpr int CONV_ROWS = 128;   // (b, l) rows per workgroup of the weight-gradient kernel

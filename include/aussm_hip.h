@@ -63,17 +63,20 @@ const char* aussm_error_string(int code);
  * No reference counterpart (the reference fixes its launch table at compile time,
  * extension-cpp/extension_cpp/csrc/cuda/ssm_adaptive_unitary_forward.cu:215-266).
  *   AUSSM_OPT_UNITARY_FWD  forward kernel of the unitary scan: 0 vector ALU, 2 / 3 matrix cores on
- *                          two- / three-piece operands (3 = fp32-accurate, the default choice
- *                          where the shape allows), 6 matrix cores on operands prepared once per
- *                          batch element by a pre-pass
+ *                          two- / three-piece operands built inside the scan kernel (3 = fp32-accurate,
+ *                          the choice where the shape allows and the call has no auxiliary buffer),
+ *                          6 matrix cores on three-piece operands prepared once per batch element by a
+ *                          pre-pass (the default for calls with an auxiliary buffer)
  *   AUSSM_OPT_UNITARY_BWD  backward kernel: 0 vector ALU, 2 two-piece operands, 3 three pieces
  *                          along the sequence and two in the sums over the channel, 5 three
  *                          pieces everywhere, 6 prepared operands
  *   AUSSM_OPT_SPLIT_CAP    largest number of segments a launch may be split into along L
  *                          (0 or 1: never split)
  *   AUSSM_OPT_BLOCK_KFLOATS   budget, in units of 1024 floats, of the blocks in which the fused operator calls
- *                          (aussm_ssm_adaptive_unitary_fwd / _bwd) walk their problem (default 12800 = 50 MiB);
- *                          workspace sizes follow it, so set it before asking for them
+ *                          (aussm_ssm_adaptive_unitary_fwd / _bwd) walk their problem (default and largest
+ *                          value 12800 = 50 MiB; the option can only lower it)
+ * Workspace and auxiliary-buffer sizes do not depend on any option: a buffer sized by the query
+ * functions below holds what a call of that shape uses under every setting.
  *   AUSSM_OPT_GENERIC_NW / AUSSM_OPT_GENERIC_NT   states per wavefront / threads per workgroup of
  *                          the vector-ALU kernels (both must be set; one of the built pairs) */
 #define AUSSM_OPT_UNITARY_FWD 0
@@ -130,12 +133,20 @@ int aussm_unitary_bwd(const float* dy, const float* dhL,
 
 /* Variants of the two calls above with an optional auxiliary buffer (NULL allowed; then they are
  * the calls above).  `aux` holds aussm_unitary_aux_floats(B, D, N, L, ck) floats, 16-byte aligned,
- * sized with the arguments of the calls it is passed to.  Two uses, both internal:
+ * sized with the arguments of the calls it is passed to.  Three uses, all internal:
  *  - the forward call may leave per-(b,d,l) intermediate results in it (Im(P_t S_t), the term of
  *    the phase gradient that needs the forward states) together with a validity tag; the backward
  *    call given the same buffer then skips recomputing them.  A forward kernel that does not fill
  *    the buffer clears the tag, so a backward call never consumes stale contents: handing over
  *    `aux` is always safe and only ever a speed-up;
+ *  - the matrix-core kernels run on operands prepared from Bc and Cc by a pre-pass (split into bf16
+ *    pieces, in the record orders the products need); they live at the end of the buffer.  A forward
+ *    call that is given hck (a backward call can follow) prepares the backward call's operands in
+ *    the same pre-pass and notes, behind the validity tag, what they were made from: the addresses
+ *    of Bc and Cc, B, N, L and in_dtype.  A backward call whose arguments match that note uses them;
+ *    any other backward call prepares its own.  So the contract for reusing one buffer is the
+ *    autograd one: between a forward call and the backward call that is handed its buffer, Bc and
+ *    Cc must not be modified in place, and no other call may be given the buffer;
  *  - a launch with few (batch, channel) pairs and a long sequence is split along L over more
  *    workgroups (per-segment end states from a zero start, a short chain over the segments, then
  *    the scan of every segment from its true incoming state - the two-level scan of
@@ -182,8 +193,9 @@ int aussm_unitary_bwd_aux(const float* dy, const float* dhL,
  * The one workspace such a call uses - the segment states of a launch with few (batch, channel)
  * pairs that is split along L, see above - lives in a device array of AUSSM_STATIC_SCRATCH_BYTES
  * inside the library, which every GPU the library runs on holds from the first use to the end of
- * the process.  Same arguments, results and kernel choice as aussm_unitary_fwd_aux with a buffer
- * sized for (B, D, N, L, ck); a call whose segment states do not fit returns AUSSM_E_SCRATCH.
+ * the process.  Same arguments and results (to rounding) as aussm_unitary_fwd_aux with a buffer
+ * sized for (B, D, N, L, ck); it runs the kernels that build their operands themselves, since it
+ * has no room for prepared ones.  A call whose segment states do not fit returns AUSSM_E_SCRATCH.
  * All calls on one GPU share that GPU's array: calls that overlap there (different streams,
  * different threads) race; calls in one stream are ordered and safe.  Nothing in the array has
  * to start at zero (every state read is written earlier in the same call).

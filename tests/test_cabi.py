@@ -64,8 +64,9 @@ def test_argument_checks_without_a_device():
                                1, 1, 1, 32, 32, 0, null)
     assert rc == -5
     # the auxiliary buffer: size query, alignment check, NULL accepted like the plain entry points
-    # per-(b,d,l) part + tag, then one 30 KiB image of prepared operands per (batch element, 32-step chunk)
-    img = lambda b, l: b * ((l + 31) // 32) * 1920 * 4
+    # per-(b,d,l) part + tag, then per (batch element, 32-step chunk) one 30 KiB image of prepared operands for the
+    # backward pass and one of 24 KiB for the forward pass
+    img = lambda b, l: b * ((l + 31) // 32) * (1920 + 1536) * 4
     assert lib.aussm_unitary_aux_floats(32, 512, 16, 2048, 256) == 32 * 512 * 2048 + 64 + img(32, 2048)
     assert lib.aussm_unitary_aux_floats(0, 1, 1, 1, 32) == 0
     # few (batch, channel) pairs and a long sequence: room for the states of 64 segments of 256 steps
@@ -73,7 +74,15 @@ def test_argument_checks_without_a_device():
                                                                     + img(4, 16384))
     # ... which needs whole checkpoint blocks per segment, and states the matrix-core kernels serve
     assert lib.aussm_unitary_aux_floats(4, 256, 16, 16384 + 4, 256) == 4 * 256 * (16384 + 4) + 64 + img(4, 16388)
-    assert lib.aussm_unitary_aux_floats(4, 256, 4, 16384, 256) == 4 * 256 * 16384 + 64
+    # (sizes do not depend on the option table: below the state size the matrix-core kernels take by default the images
+    # are still provided for, because an option can ask for those kernels)
+    assert lib.aussm_unitary_aux_floats(4, 256, 4, 16384, 256) == 4 * 256 * 16384 + 64 + img(4, 16384)
+    assert lib.aussm_unitary_aux_floats(4, 256, 32, 16384, 256) == 4 * 256 * 16384 + 64
+    lib.aussm_ssm_adaptive_unitary_workspace_floats.restype = ctypes.c_size_t
+    w0 = lib.aussm_ssm_adaptive_unitary_workspace_floats(32, 256, 16, 720, 1)
+    assert lib.aussm_set_option(5, 64) == 0 and lib.aussm_ssm_adaptive_unitary_workspace_floats(32, 256, 16, 720, 1) == w0
+    assert lib.aussm_set_option(5, 1 << 20) == 0 and lib.aussm_ssm_adaptive_unitary_workspace_floats(32, 256, 16, 720, 1) == w0
+    assert lib.aussm_set_option(5, -1) == 0
     # options: unset by default, settable, restorable
     assert lib.aussm_get_option(0) == -1 and lib.aussm_set_option(0, 3) == 0 and lib.aussm_get_option(0) == 3
     assert lib.aussm_set_option(0, -1) == 0 and lib.aussm_get_option(0) == -1 and lib.aussm_set_option(99, 1) == -2
