@@ -3,10 +3,13 @@
     python -m aussm_amd.build                 # compile every translation unit and link
     python -m aussm_amd.build --only k_px     # recompile one unit (the others' objects must exist) and relink
     python -m aussm_amd.build --asm DIR       # also keep the compiler's gfx950 assembly in DIR
-    python -m aussm_amd.build --experimental  # also build the measured-and-dropped alternative kernels
     python -m aussm_amd.build --check         # compile k_px.hip to assembly and check its listings (below)
 
 hipcc cross-compiles without a GPU, so this runs on a CPU-only machine.
+
+The kernels of k_px.hip and k_xdl.hip track some of their loads by hand (see check_unit_listing):
+they were validated with the compiler named in VALIDATED_HIPCC, every build checks their listings,
+and a build with another compiler says so.
 """
 from __future__ import annotations
 
@@ -37,6 +40,20 @@ HIPCC_FLAGS = [
 ]
 
 
+# `hipcc --version` line ("HIP version: ...") of the compiler the hand-tracked loads were validated with
+VALIDATED_HIPCC = "HIP version: 7.2.26015-fc0010cf6a"
+# units whose kernels issue loads as hand-written instructions: their listings are checked by every build
+HAND_TRACKED = ("k_px.hip", "k_xdl.hip")
+
+
+def hipcc_version(hipcc: str) -> str:
+    out = subprocess.run([hipcc, "--version"], capture_output=True, text=True).stdout
+    for line in out.splitlines():
+        if line.startswith("HIP version"):
+            return line.strip()
+    return out.strip().splitlines()[0] if out.strip() else "unknown"
+
+
 def lib_path() -> str:
     return os.path.join(LIBDIR, LIBNAME)
 
@@ -64,9 +81,27 @@ def build(verbose: bool = True, asm_dir: str | None = None, only=None, extra=())
     os.makedirs(LIBDIR, exist_ok=True)
     if asm_dir:
         os.makedirs(asm_dir, exist_ok=True)
+    ver = hipcc_version(hipcc)
+    if ver != VALIDATED_HIPCC:
+        print(f"aussm_amd.build: WARNING: compiling with `{ver}`; the kernels that track their loads by hand were "
+              f"validated with `{VALIDATED_HIPCC}` (their listings are checked below)", file=sys.stderr, flush=True)
+    if only:
+        # the argument blocks in the headers are shared by every unit: an object older than a header would be
+        # linked against kernels with another layout of their arguments
+        newest = max(os.path.getmtime(os.path.join(CSRC, f)) for f in os.listdir(CSRC) if f.endswith(".h"))
+        incl = os.path.getmtime(os.path.join(os.path.dirname(HERE), "include", "aussm_hip.h"))
+        stale = [s for s in SOURCES if os.path.splitext(s)[0] not in only and os.path.exists(_obj(s))
+                 and os.path.getmtime(_obj(s)) < max(newest, incl)]
+        if stale:
+            print(f"aussm_amd.build: a header is newer than the objects of {stale}: rebuilding every unit", flush=True)
+            only = None
     todo = [s for s in SOURCES if not only or os.path.splitext(s)[0] in only or not os.path.exists(_obj(s))]
-    with ThreadPoolExecutor(max_workers=min(len(todo), 8) or 1) as ex:
-        for f in [ex.submit(_compile, hipcc, s, verbose, asm_dir, extra) for s in todo]:
+    # the listings of the hand-tracked units among them are checked alongside (same compiler, same flags);
+    # a finding fails the build before the library is put in place
+    with ThreadPoolExecutor(max_workers=8) as ex:
+        jobs = [ex.submit(_compile, hipcc, s, verbose, asm_dir, extra) for s in todo]
+        jobs += [ex.submit(check_unit_listing, u, verbose) for u in HAND_TRACKED if u in todo]
+        for f in jobs:
             f.result()
     out = lib_path()
     tmp = out + ".tmp"
@@ -95,7 +130,10 @@ def build(verbose: bool = True, asm_dir: str | None = None, only=None, extra=())
 def scan_listing(text: str):
     """Findings [(line number, instruction)] of one kernel listing: vector or accumulation registers
     touched while they are the destination of a hand-written (ASMSTART ... ASMEND) global load that no
-    s_waitcnt vmcnt has retired yet.  The scan follows the file order, not the control flow."""
+    s_waitcnt vmcnt has retired yet.  The scan follows the file order; at a branch back to an earlier
+    label (a loop's back-edge) with loads still in flight it also walks the loop body once more from
+    that label with those loads in flight, so a load issued at the end of an iteration and retired at
+    the top of the next is followed across the edge."""
     import re
 
     def regs(tok):
@@ -107,34 +145,53 @@ def scan_listing(text: str):
                 out.add((m.group(4), int(m.group(5))))
         return out
 
-    inflight, in_asm, found = {}, False, []
-    for i, line in enumerate(text.split("\n")):
-        s = line.strip()
-        if "ASMSTART" in s:
-            in_asm = True
-            continue
-        if "ASMEND" in s:
-            in_asm = False
-            continue
-        if not s or s[0] in ";.":
-            continue
-        ins = s.split(";")[0]
-        if ins.startswith("s_waitcnt") and "vmcnt" in ins:
-            k = int(re.search(r"vmcnt\((\d+)\)", ins).group(1))
-            issued = sorted(set(inflight.values()))
-            keep = set(issued[len(issued) - k:]) if k > 0 else set()
-            inflight = {r: ln for r, ln in inflight.items() if ln in keep}
-            continue
-        if in_asm and re.match(r"global_load_dwordx[24] ", ins):
-            ops = ins.split(None, 1)[1].split(",")
-            if any(r in inflight for r in regs(ops[1])):
+    lines = text.split("\n")
+    labels = {}
+    for i, line in enumerate(lines):
+        m = re.match(r"^(\.LBB\w+):", line.strip())
+        if m:
+            labels[m.group(1)] = i
+
+    found = []
+
+    def walk(start, end, inflight, follow):
+        in_asm = False
+        for i in range(start, end):
+            s = lines[i].strip()
+            if "ASMSTART" in s:
+                in_asm = True
+                continue
+            if "ASMEND" in s:
+                in_asm = False
+                continue
+            if not s or s[0] in ";.":
+                continue
+            ins = s.split(";")[0]
+            if ins.startswith("s_waitcnt") and "vmcnt" in ins:
+                k = int(re.search(r"vmcnt\((\d+)\)", ins).group(1))
+                issued = sorted(set(inflight.values()))
+                keep = set(issued[len(issued) - k:]) if k > 0 else set()
+                inflight = {r: ln for r, ln in inflight.items() if ln in keep}
+                if not follow and not inflight:
+                    return
+                continue
+            if in_asm and re.match(r"global_load_dwordx[24] ", ins):
+                ops = ins.split(None, 1)[1].split(",")
+                if any(r in inflight for r in regs(ops[1])):
+                    found.append((i + 1, ins))
+                for r in regs(ops[0]):
+                    inflight[r] = i + 1
+                continue
+            if any(r in inflight for r in regs(ins)):
                 found.append((i + 1, ins))
-            for r in regs(ops[0]):
-                inflight[r] = i + 1
-            continue
-        if any(r in inflight for r in regs(ins)):
-            found.append((i + 1, ins))
-    return found
+            if follow and inflight and ins.startswith("s_cbranch"):
+                tgt = ins.split()[-1]
+                if tgt in labels and labels[tgt] < i:
+                    # (loads carried over the edge are older than anything the body issues: line numbers below it)
+                    walk(labels[tgt], i, {r: ln - len(lines) for r, ln in inflight.items()}, False)
+
+    walk(0, len(lines), {}, True)
+    return sorted(set(found))
 
 
 def check_unit_listing(unit: str, verbose: bool = True) -> int:
@@ -176,7 +233,7 @@ def check_unit_listing(unit: str, verbose: bool = True) -> int:
 
 def check_px_listing(verbose: bool = True) -> None:
     """The listing check over the two units whose kernels issue loads by hand."""
-    for unit in ("k_px.hip", "k_xdl.hip"):
+    for unit in HAND_TRACKED:
         check_unit_listing(unit, verbose)
 
 
@@ -186,7 +243,5 @@ if __name__ == "__main__":
         check_px_listing()
         sys.exit(0)
     only = [argv[i + 1] for i, a in enumerate(argv) if a == "--only"]
-    extra = ["-DAUSSM_EXPERIMENTAL_KERNELS"] if "--experimental" in argv else []
-    build(asm_dir=os.path.abspath(argv[argv.index("--asm") + 1]) if "--asm" in argv else None, only=only or None,
-          extra=extra)
+    build(asm_dir=os.path.abspath(argv[argv.index("--asm") + 1]) if "--asm" in argv else None, only=only or None)
     print("built", lib_path())

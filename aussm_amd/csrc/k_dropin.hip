@@ -4,18 +4,20 @@
 
 namespace aussm {
 
-void run_dropin_xprep(const float* x, u4* xp, int d, int n, int ks, int nb, hipStream_t s) {
+int run_dropin_xprep(const float* x, u4* xp, int d, int n, int ks, int nb, hipStream_t s) {
   const size_t total = (size_t)d * nb * ks * 64;
   hipLaunchKernelGGL(dropin_xprep_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, x, xp, d, n, ks, nb);
+  return launch_status();
 }
 
-void run_fill(const FillArgs& a, hipStream_t s) {
+int run_fill(const FillArgs& a, hipStream_t s) {
   size_t most = 0;
   for (int i = 0; i < a.count; ++i) most = a.n[i] > most ? a.n[i] : most;
-  if (!a.count || !most) return;
+  if (!a.count || !most) return 0;
   size_t blocks = (most + 255) / 256;
   if (blocks > 4096) blocks = 4096;
   hipLaunchKernelGGL(fill_kernel, dim3((unsigned)blocks, (unsigned)a.count), dim3(256), 0, s, a);
+  return launch_status();
 }
 
 #ifndef DROPIN_NW_
@@ -42,8 +44,9 @@ int dropin_channels_per_workgroup(int ks) { return ks > 8 ? 4 : DROPIN_NW; }
 // the compiled size of the contraction (steps of 32) that serves ceil(d / 32) = ks
 int dropin_compiled_ks(int ks) { return ks <= 4 ? (ks < 1 ? 1 : ks) : ks <= 6 ? 6 : ks <= 8 ? 8 : ks <= 12 ? 12 : 16; }
 
-void run_dropin_uprep(const float* u, u4* up, int d, int L, int ks, int b0, int bg, int t0, int nt, hipStream_t s) {
+int run_dropin_uprep(const float* u, u4* up, int d, int L, int ks, int b0, int bg, int t0, int nt, hipStream_t s) {
   hipLaunchKernelGGL(dropin_uprep_kernel, dim3((unsigned)(bg * nt)), dim3(256), 0, s, u, up, d, L, dropin_compiled_ks(ks), b0, t0, nt);
+  return launch_status();
 }
 
 // compiled sizes of the contraction over r, in steps of 32: the smallest one >= ceil(d / 32) runs

@@ -99,7 +99,7 @@ int run_rec_bwd(int variant, const RecBwdArgs& a, int in_dtype, hipStream_t s) {
   return in_dtype ? rec_bwd_t<VAR_REAL, bf16_t>(a, s) : rec_bwd_t<VAR_REAL, float>(a, s);
 }
 
-void run_adjoint_seg(int variant, const AdjSegArgs& a, int in_dtype, unsigned grid, hipStream_t s) {
+int run_adjoint_seg(int variant, const AdjSegArgs& a, int in_dtype, unsigned grid, hipStream_t s) {
   // (B_t / C_t are float in every instance; the complex kernel reads no u / delta at all)
   if (variant == VAR_COMPLEX) {
     hipLaunchKernelGGL((adjoint_seg_kernel<VAR_COMPLEX, float, float>), dim3(grid), dim3(256), 0, s, a);
@@ -107,20 +107,23 @@ void run_adjoint_seg(int variant, const AdjSegArgs& a, int in_dtype, unsigned gr
     if (in_dtype) hipLaunchKernelGGL((adjoint_seg_kernel<VAR_REAL, bf16_t, float>), dim3(grid), dim3(256), 0, s, a);
     else hipLaunchKernelGGL((adjoint_seg_kernel<VAR_REAL, float, float>), dim3(grid), dim3(256), 0, s, a);
   }
+  return launch_status();
 }
 
-void run_bc_to_f32(const void* Bm, const void* Cm, float* oB, float* oC, size_t n, hipStream_t s) {
+int run_bc_to_f32(const void* Bm, const void* Cm, float* oB, float* oC, size_t n, hipStream_t s) {
   const size_t blocks = (n + 255) / 256;
   hipLaunchKernelGGL(bc_to_f32_kernel, dim3((unsigned)(blocks < 2048 ? blocks : 2048)), dim3(256), 0, s,
                      static_cast<const bf16_t*>(Bm), static_cast<const bf16_t*>(Cm), oB, oC, n);
+  return launch_status();
 }
 
-void run_seg_carry_real(bool adjoint, float* seg, const float* ptot, const float* A, const float* first, float* last,
+int run_seg_carry_real(bool adjoint, float* seg, const float* ptot, const float* A, const float* first, float* last,
                         int B, int D, int N, int ns, hipStream_t s) {
   const size_t n = (size_t)B * D * N;
   const dim3 grid((unsigned)((n + 255) / 256));
   if (adjoint) hipLaunchKernelGGL(seg_carry_real_kernel<true>, grid, dim3(256), 0, s, seg, ptot, A, first, last, B, D, N, ns);
   else hipLaunchKernelGGL(seg_carry_real_kernel<false>, grid, dim3(256), 0, s, seg, ptot, A, first, last, B, D, N, ns);
+  return launch_status();
 }
 
 // marks an auxiliary buffer as NOT filled (a forward kernel that does not fill it ran) and / or the
@@ -128,10 +131,11 @@ void run_seg_carry_real(bool adjoint, float* seg, const float* ptot, const float
 __global__ void aux_invalidate_kernel(float* tag, int first, int last) {
   if ((int)threadIdx.x >= first && (int)threadIdx.x <= last) tag[threadIdx.x] = 0.0f;
 }
-void run_aux_invalidate(float* tag, bool fill_tag, bool images_tag, hipStream_t s) {
-  if (!fill_tag && !images_tag) return;
+int run_aux_invalidate(float* tag, bool fill_tag, bool images_tag, hipStream_t s) {
+  if (!fill_tag && !images_tag) return 0;
   hipLaunchKernelGGL(aux_invalidate_kernel, dim3(1), dim3(64), 0, s, tag, fill_tag ? 0 : AUX_IMG_FP,
                      images_tag ? AUX_IMG_FP + 7 : 0);
+  return launch_status();
 }
 
 int run_conv_fwd(const ConvArgs& a, hipStream_t s) {

@@ -4,10 +4,11 @@
 
 namespace aussm {
 
-void run_px_prep(const PrepArgs& a, int B, int in_dtype, hipStream_t s) {
+int run_px_prep(const PrepArgs& a, int B, int in_dtype, hipStream_t s) {
   const dim3 grid((unsigned)(B * a.nch));
   if (in_dtype == 1) hipLaunchKernelGGL(unitary_px_prep_kernel<bf16_t>, grid, dim3(256), 0, s, a);
   else hipLaunchKernelGGL(unitary_px_prep_kernel<float>, grid, dim3(256), 0, s, a);
+  return launch_status();
 }
 
 int run_px_fwd(const FwdArgs& a, const u4* img, const ImgNote& note, int in_dtype, hipStream_t s) {

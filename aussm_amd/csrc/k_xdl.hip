@@ -4,24 +4,11 @@
 #include "scan_bwd_xdl.h"
 #include "scan_fwd_xdl.h"
 #include "scan_seg_xdl.h"
-#ifdef AUSSM_EXPERIMENTAL_KERNELS
-#include "scan_fwd_mfma.h"
-#include "scan_fwd_xdl2.h"
-#endif
 
 namespace aussm {
 
 int run_xdl_fwd(int mode, const FwdArgs& a, int in_dtype, hipStream_t s) {
   const dim3 grid((unsigned)(a.B * a.ncg));
-#ifdef AUSSM_EXPERIMENTAL_KERNELS
-  if (mode == 1) {
-    if (a.z) hipLaunchKernelGGL(unitary_fwd_mfma_kernel<true>, grid, dim3(256), 0, s, a);
-    else hipLaunchKernelGGL(unitary_fwd_mfma_kernel<false>, grid, dim3(256), 0, s, a);
-  } else if (mode == 4) {
-    if (a.z) hipLaunchKernelGGL((unitary_fwd_xdl2_kernel<3, true>), grid, dim3(512), 0, s, a);
-    else hipLaunchKernelGGL((unitary_fwd_xdl2_kernel<3, false>), grid, dim3(512), 0, s, a);
-  } else
-#endif
   if (in_dtype == 1) {
     if (a.z) hipLaunchKernelGGL((unitary_fwd_xdl_kernel<3, true, bf16_t>), grid, dim3(256), 0, s, a);
     else hipLaunchKernelGGL((unitary_fwd_xdl_kernel<3, false, bf16_t>), grid, dim3(256), 0, s, a);
@@ -44,7 +31,7 @@ int run_xdl_bwd(int mode, const UniBwdArgs& a, int in_dtype, hipStream_t s) {
   return launch_status();
 }
 
-void run_seg_state(bool adjoint, const SegArgs& a, int in_dtype, unsigned grid, hipStream_t s) {
+int run_seg_state(bool adjoint, const SegArgs& a, int in_dtype, unsigned grid, hipStream_t s) {
   if (adjoint) {
     if (in_dtype == 1) hipLaunchKernelGGL((unitary_seg_state_kernel<3, true, bf16_t>), dim3(grid), dim3(256), 0, s, a);
     else hipLaunchKernelGGL((unitary_seg_state_kernel<3, true>), dim3(grid), dim3(256), 0, s, a);
@@ -52,16 +39,19 @@ void run_seg_state(bool adjoint, const SegArgs& a, int in_dtype, unsigned grid, 
     if (in_dtype == 1) hipLaunchKernelGGL((unitary_seg_state_kernel<3, false, bf16_t>), dim3(grid), dim3(256), 0, s, a);
     else hipLaunchKernelGGL((unitary_seg_state_kernel<3, false>), dim3(grid), dim3(256), 0, s, a);
   }
+  return launch_status();
 }
 
-void run_seg_carry_fwd(float* seg, const float* ptot, const float* h0, float* hL, int B, int D, int N, int nf, hipStream_t s) {
+int run_seg_carry_fwd(float* seg, const float* ptot, const float* h0, float* hL, int B, int D, int N, int nf, hipStream_t s) {
   const size_t nst = (size_t)B * D * N;
   hipLaunchKernelGGL(seg_carry_fwd_kernel, dim3((unsigned)((nst + 255) / 256)), dim3(256), 0, s, seg, ptot, h0, hL, B, D, N, nf);
+  return launch_status();
 }
 
-void run_seg_carry_bwd(float* seg, const float* ptot, const float* dhL, float* dh0, int B, int D, int N, int nf, hipStream_t s) {
+int run_seg_carry_bwd(float* seg, const float* ptot, const float* dhL, float* dh0, int B, int D, int N, int nf, hipStream_t s) {
   const size_t nst = (size_t)B * D * N;
   hipLaunchKernelGGL(seg_carry_bwd_kernel, dim3((unsigned)((nst + 255) / 256)), dim3(256), 0, s, seg, ptot, dhL, dh0, B, D, N, nf);
+  return launch_status();
 }
 
 }  // namespace aussm

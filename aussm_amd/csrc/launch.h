@@ -23,11 +23,11 @@ struct Cfg { int nw, nt; };
 int run_core_fwd(int variant, const FwdArgs& a, int in_dtype, Cfg c, hipStream_t s);
 int run_unitary_bwd_generic(const UniBwdArgs& a, int in_dtype, Cfg c, hipStream_t s);
 int run_rec_bwd(int variant, const RecBwdArgs& a, int in_dtype, hipStream_t s);
-void run_aux_invalidate(float* tag, bool fill_tag, bool images_tag, hipStream_t s);   // clears tag(s) in the buffer's pad
+int run_aux_invalidate(float* tag, bool fill_tag, bool images_tag, hipStream_t s);   // clears tag(s) in the buffer's pad
 // split of the complex / real scans along L: adjoint entering every segment, chain of the real scan's segments
-void run_adjoint_seg(int variant, const AdjSegArgs& a, int in_dtype, unsigned grid, hipStream_t s);
-void run_bc_to_f32(const void* Bm, const void* Cm, float* oB, float* oC, size_t n, hipStream_t s);   // bf16 -> float
-void run_seg_carry_real(bool adjoint, float* seg, const float* ptot, const float* A, const float* first, float* last,
+int run_adjoint_seg(int variant, const AdjSegArgs& a, int in_dtype, unsigned grid, hipStream_t s);
+int run_bc_to_f32(const void* Bm, const void* Cm, float* oB, float* oC, size_t n, hipStream_t s);   // bf16 -> float
+int run_seg_carry_real(bool adjoint, float* seg, const float* ptot, const float* A, const float* first, float* last,
                         int B, int D, int N, int ns, hipStream_t s);
 int run_conv_fwd(const ConvArgs& a, hipStream_t s);
 int run_conv_bwd(const ConvArgs& a, hipStream_t s);
@@ -37,23 +37,23 @@ int run_swap_last2(const SwapArgs& a, int B, hipStream_t s);
 // kernels of the split along L.  mode: operand pieces (2, 3; backward also 5 = three everywhere).
 int run_xdl_fwd(int mode, const FwdArgs& a, int in_dtype, hipStream_t s);
 int run_xdl_bwd(int mode, const UniBwdArgs& a, int in_dtype, hipStream_t s);
-void run_seg_state(bool adjoint, const SegArgs& a, int in_dtype, unsigned grid, hipStream_t s);
-void run_seg_carry_fwd(float* seg, const float* ptot, const float* h0, float* hL, int B, int D, int N, int nf, hipStream_t s);
-void run_seg_carry_bwd(float* seg, const float* ptot, const float* dhL, float* dh0, int B, int D, int N, int nf, hipStream_t s);
+int run_seg_state(bool adjoint, const SegArgs& a, int in_dtype, unsigned grid, hipStream_t s);
+int run_seg_carry_fwd(float* seg, const float* ptot, const float* h0, float* hL, int B, int D, int N, int nf, hipStream_t s);
+int run_seg_carry_bwd(float* seg, const float* ptot, const float* dhL, float* dh0, int B, int D, int N, int nf, hipStream_t s);
 
 // ---- k_px.hip: matrix-core unitary scans on operands prepared by a pre-pass
-void run_px_prep(const PrepArgs& a, int B, int in_dtype, hipStream_t s);
+int run_px_prep(const PrepArgs& a, int B, int in_dtype, hipStream_t s);
 int run_px_fwd(const FwdArgs& a, const u4* img, const ImgNote& note, int in_dtype, hipStream_t s);
 int run_px_bwd(const UniBwdArgs& a, const u4* img, int in_dtype, hipStream_t s);
 
 // ---- k_dropin.hip: the reference's 12-input operator as fused kernels
-void run_dropin_xprep(const float* x, u4* xp, int d, int n, int ks, int nb, hipStream_t s);
+int run_dropin_xprep(const float* x, u4* xp, int d, int n, int ks, int nb, hipStream_t s);
 int dropin_channels_per_workgroup(int ks);
 int dropin_compiled_ks(int ks);
-void run_dropin_uprep(const float* u, u4* up, int d, int L, int ks, int b0, int bg, int t0, int nt, hipStream_t s);
+int run_dropin_uprep(const float* u, u4* up, int d, int L, int ks, int b0, int bg, int t0, int nt, hipStream_t s);
 int run_dropin_fwd(const DropinArgs& a, hipStream_t s);
 int run_dropin_bwd(const DropinBwdArgs& a, hipStream_t s);
-void run_fill(const FillArgs& a, hipStream_t s);   // several buffers set (zero or a copy) in one launch
+int run_fill(const FillArgs& a, hipStream_t s);   // several buffers set (zero or a copy) in one launch
 int run_split_gemm(const GemmArgs& a, hipStream_t s);
 
 }  // namespace aussm

@@ -55,8 +55,7 @@ inline bool misaligned(const void* p, size_t a) { return p && (reinterpret_cast<
 // vector-ALU kernels.  aussm_set_option(AUSSM_OPT_UNITARY_FWD, m) selects the forward kernel for
 // comparisons: 0 vector ALU, 2 / 3 bf16 matrix instructions on two- / three-piece operands built
 // inside the scan kernel, 6 three-piece operands prepared by a pre-pass, two wavefronts per SIMD
-// (the default when the call brings the workspace for them, i.e. an auxiliary buffer; builds with
-// AUSSM_EXPERIMENTAL_KERNELS also know 1 = fp32 matrix instructions and 4).
+// (the default when the call brings the workspace for them, i.e. an auxiliary buffer).
 // AUSSM_OPT_UNITARY_BWD: 0 vector ALU, 2 two pieces everywhere, 3 three pieces along the sequence
 // and two in the sums over the channel (dB, dC), 5 three pieces everywhere, 6 prepared operands.
 //
@@ -134,14 +133,14 @@ inline size_t generic_split_floats(int variant, int B, int D, int N, int L, int 
 inline size_t generic_bc_floats(int variant, int B, int N, int L, int in_dtype) {
   return in_dtype == AUSSM_BF16 ? round64((size_t)B * N * L * (variant == VAR_REAL ? 1 : 2)) : 0;
 }
-struct BcF32 { const void* Bm; const void* Cm; int in_dtype; };
+struct BcF32 { const void* Bm; const void* Cm; int in_dtype; int err; };
 inline BcF32 generic_bc(int variant, const void* Bm, const void* Cm, float* ws, int B, int D, int N, int L, int ck,
                         int in_dtype, hipStream_t s) {
-  if (in_dtype != AUSSM_BF16) return BcF32{Bm, Cm, 0};
+  if (in_dtype != AUSSM_BF16) return BcF32{Bm, Cm, 0, 0};
   const size_t n = generic_bc_floats(variant, B, N, L, in_dtype);
   float* fB = ws + generic_split_floats(variant, B, D, N, L, ck);
-  run_bc_to_f32(Bm, Cm, fB, fB + n, (size_t)B * N * L * (variant == VAR_REAL ? 1 : 2), s);
-  return BcF32{fB, fB + n, 2};
+  const int err = run_bc_to_f32(Bm, Cm, fB, fB + n, (size_t)B * N * L * (variant == VAR_REAL ? 1 : 2), s);
+  return BcF32{fB, fB + n, 2, err};
 }
 
 // Workspace of the prepared operands: per (batch element, chunk) one backward image and, behind
@@ -198,7 +197,8 @@ int launch_unitary_fwd(FwdArgs a, int in_dtype, hipStream_t s, AuxLayout ws) {
   // a call that does not fill the buffer marks it as not filled, and a call that does not prepare
   // images clears the note about the ones behind the buffer
   const bool fill = a.aux && a.hck && mode >= 2;
-  if (a.aux) run_aux_invalidate(a.aux + (size_t)a.B * a.D * a.L, !fill, mode != 6 && ws.stamp, s);
+  if (a.aux)
+    if (int e = run_aux_invalidate(a.aux + (size_t)a.B * a.D * a.L, !fill, mode != 6 && ws.stamp, s)) return e;
   if (!fill) a.aux = nullptr;
   if (!mode) return run_core_fwd(VAR_UNITARY, a, in_dtype, pick_cfg(a.N, 8), s);
   const int B = a.B, L = a.L;
@@ -211,8 +211,8 @@ int launch_unitary_fwd(FwdArgs a, int in_dtype, hipStream_t s, AuxLayout ws) {
       float* seg = ws.seg;
       float* ptot = seg + (size_t)B * nf * a.D * a.N * 2;
       SegArgs sa{a.delta, a.u, a.theta, a.Bm, seg, ptot, a.D, a.N, Ls / r, L, nf, a.ncg};
-      run_seg_state(false, sa, in_dtype, (unsigned)(B * nf * a.ncg), s);
-      run_seg_carry_fwd(seg, ptot, a.h0, a.hL, B, a.D, a.N, nf, s);
+      if (int e = run_seg_state(false, sa, in_dtype, (unsigned)(B * nf * a.ncg), s)) return e;
+      if (int e = run_seg_carry_fwd(seg, ptot, a.h0, a.hL, B, a.D, a.N, nf, s)) return e;
       a.B = B * ns; a.L = Ls; a.ns = ns; a.nck = Ls / a.ck; a.h0 = seg; a.hL = nullptr; a.hs = r; a.ho = 0;
     }
   }
@@ -221,7 +221,7 @@ int launch_unitary_fwd(FwdArgs a, int in_dtype, hipStream_t s, AuxLayout ws) {
     // checkpoints, so a call without them is not followed by one)
     const bool with_bwd = a.hck != nullptr;
     PrepArgs pa{a.Bm, a.Cm, ws.fimg, with_bwd ? ws.img : nullptr, a.N, L, (L + XT - 1) / XT, nullptr, ImgStamp{}};
-    run_px_prep(pa, B, in_dtype, s);
+    if (int e = run_px_prep(pa, B, in_dtype, s)) return e;
     const ImgNote note{ws.stamp, img_stamp(a.Bm, a.Cm, B, a.N, L, in_dtype, with_bwd)};
     return run_px_fwd(a, ws.fimg, note, in_dtype, s);
   }
@@ -233,6 +233,7 @@ int launch_generic_fwd(int variant, FwdArgs a, int in_dtype, float* ws, hipStrea
   if (in_dtype == AUSSM_BF16 && !ws) return AUSSM_E_NULL;
   if (misaligned(ws, 16)) return AUSSM_E_ALIGN;
   const BcF32 bc = generic_bc(variant, a.Bm, a.Cm, ws, a.B, a.D, a.N, a.L, a.ck, in_dtype, s);
+  if (bc.err) return bc.err;
   a.Bm = bc.Bm; a.Cm = bc.Cm; in_dtype = bc.in_dtype;
   const Cfg cfg = pick_cfg(a.N, 8);
   const GSplit sp = ws ? generic_split(a.B, a.D, a.L, a.ck, true) : GSplit{1, a.L};
@@ -246,8 +247,9 @@ int launch_generic_fwd(int variant, FwdArgs a, int in_dtype, float* ws, hipStrea
     z.y = nullptr; z.z = nullptr; z.Dskip = nullptr; z.h0 = nullptr; z.hL = seg; z.hck = nullptr; z.ptot = ptot;
     if (int e = run_core_fwd(variant, z, in_dtype, cfg, s)) return e;
     // 2. the state that enters every segment; the state after the last one is the call's hL
-    if (variant == VAR_COMPLEX) run_seg_carry_fwd(seg, ptot, a.h0, a.hL, B, a.D, a.N, sp.ns, s);
-    else run_seg_carry_real(false, seg, ptot, a.A, a.h0, a.hL, B, a.D, a.N, sp.ns, s);
+    if (int e = variant == VAR_COMPLEX ? run_seg_carry_fwd(seg, ptot, a.h0, a.hL, B, a.D, a.N, sp.ns, s)
+                                       : run_seg_carry_real(false, seg, ptot, a.A, a.h0, a.hL, B, a.D, a.N, sp.ns, s))
+      return e;
     // 3. the scan proper over (batch, segment) pairs
     a.B = B * sp.ns; a.L = sp.ls; a.ns = sp.ns; a.h0 = seg; a.hL = nullptr;
   }
@@ -258,6 +260,7 @@ int launch_generic_bwd(int variant, RecBwdArgs a, int in_dtype, float* ws, hipSt
   if (in_dtype == AUSSM_BF16 && !ws) return AUSSM_E_NULL;
   if (misaligned(ws, 16)) return AUSSM_E_ALIGN;
   const BcF32 bc = generic_bc(variant, a.Bm, a.Cm, ws, a.B, a.D, a.N, a.L, REC_CK, in_dtype, s);
+  if (bc.err) return bc.err;
   a.Bm = bc.Bm; a.Cm = bc.Cm; in_dtype = bc.in_dtype;
   const GSplit sp = ws ? generic_split(a.B, a.D, a.L, REC_CK, true) : GSplit{1, a.L};
   if (sp.ns > 1) {
@@ -268,9 +271,10 @@ int launch_generic_bwd(int variant, RecBwdArgs a, int in_dtype, float* ws, hipSt
     g.dy = a.dy; g.z = a.z; g.delta = a.delta; g.theta = a.theta; g.rho = a.rho; g.A = a.A; g.Cm = a.Cm;
     g.delta_bias = a.delta_bias; g.out = seg; g.ptot = ptot;
     g.D = a.D; g.N = a.N; g.L = sp.ls; g.ld = a.L; g.ns = sp.ns; g.ncg = a.ncg; g.delta_softplus = a.delta_softplus;
-    run_adjoint_seg(variant, g, in_dtype, (unsigned)(B * sp.ns * a.ncg), s);
-    if (variant == VAR_COMPLEX) run_seg_carry_bwd(seg, ptot, a.dhL, a.dh0, B, a.D, a.N, sp.ns, s);
-    else run_seg_carry_real(true, seg, ptot, a.A, a.dhL, a.dh0, B, a.D, a.N, sp.ns, s);
+    if (int e = run_adjoint_seg(variant, g, in_dtype, (unsigned)(B * sp.ns * a.ncg), s)) return e;
+    if (int e = variant == VAR_COMPLEX ? run_seg_carry_bwd(seg, ptot, a.dhL, a.dh0, B, a.D, a.N, sp.ns, s)
+                                       : run_seg_carry_real(true, seg, ptot, a.A, a.dhL, a.dh0, B, a.D, a.N, sp.ns, s))
+      return e;
     a.B = B * sp.ns; a.L = sp.ls; a.ns = sp.ns; a.dhL = seg; a.dh0 = nullptr;
   }
   return run_rec_bwd(variant, a, in_dtype, s);
@@ -378,6 +382,7 @@ int aussm_unitary_fwd_aux(const void* u, const void* delta, const float* theta, 
   a.h0 = h0; a.y = y; a.hL = hL; a.hck = hck; a.aux = aux;
   a.B = B; a.D = D; a.N = N; a.L = L; a.ck = ck; a.nck = (L + ck - 1) / ck; a.ncg = (D + CH - 1) / CH;
   a.ld = L; a.ns = 1; a.hs = 1; a.ho = 0; a.urep = urep;
+  a.auxtag = aux_tag(u, delta, theta, Bc, Cc, B, D, N, L, in_dtype);
   return launch_unitary_fwd(a, in_dtype, (hipStream_t)stream, aux_layout(aux, B, D, N, L, ck));
 }
 
@@ -466,6 +471,7 @@ int aussm_unitary_bwd_aux(const float* dy, const float* dhL, const void* u, cons
   a.B = B; a.D = D; a.N = N; a.L = L; a.ck = ck; a.nck = (L + ck - 1) / ck; a.ncg = (D + CH - 1) / CH;
   a.ld = L; a.ns = 1; a.hs = 1; a.ho = 0; a.urep = 1;
   a.urep = urep;
+  a.auxtag = aux_tag(u, delta, theta, Bc, Cc, B, D, N, L, in_dtype);
   const AuxLayout ws = aux_layout(aux, B, D, N, L, ck);
   const int mode = bwd_mode_for(B, D, N, L, ck, urep, ws.img != nullptr);
   if (mode > 0 &&
@@ -479,8 +485,8 @@ int aussm_unitary_bwd_aux(const float* dy, const float* dhL, const void* u, cons
       float* seg = ws.seg;
       float* ptot = seg + (size_t)B * nf * D * N * 2;
       SegArgs sa{dy, nullptr, theta, Cc, seg, ptot, D, N, Ls / r, L, nf, a.ncg};
-      run_seg_state(true, sa, in_dtype, (unsigned)(B * nf * a.ncg), s);
-      run_seg_carry_bwd(seg, ptot, dhL, dh0, B, D, N, nf, s);
+      if (int e = run_seg_state(true, sa, in_dtype, (unsigned)(B * nf * a.ncg), s)) return e;
+      if (int e = run_seg_carry_bwd(seg, ptot, dhL, dh0, B, D, N, nf, s)) return e;
       // a segment of the scan ends where its last fine segment ends
       a.B = B * ns; a.L = Ls; a.ns = ns; a.nck = Ls / ck; a.dhL = seg; a.dh0 = nullptr; a.hs = r; a.ho = r - 1;
     }
@@ -490,7 +496,7 @@ int aussm_unitary_bwd_aux(const float* dy, const float* dhL, const void* u, cons
       // recomputes it (launched behind, leaving at once in the opposite case) does the work.
       // (the pre-pass leaves at once when the forward call of these tensors has left the images)
       PrepArgs pa{Bc, Cc, nullptr, ws.img, N, L, (L + XT - 1) / XT, ws.stamp, img_stamp(Bc, Cc, B, N, L, in_dtype, true)};
-      run_px_prep(pa, B, in_dtype, s);
+      if (int e = run_px_prep(pa, B, in_dtype, s)) return e;
       a.tag_mode = 1;
       if (int e = run_px_bwd(a, ws.img, in_dtype, s)) return e;
       a.tag_mode = 2;
@@ -696,12 +702,12 @@ int aussm_ssm_adaptive_unitary_fwd(const float* u, const float* dt, const float*
   const int ct = dropin_fwd_chunk_tiles(b, d, L);
   u4* xp = (u4*)workspace;
   u4* up = (u4*)(workspace + dropin_xp_floats(d, n));
-  run_dropin_xprep(x, xp, d, n, ks, nb, s);
+  if (int e = run_dropin_xprep(x, xp, d, n, ks, nb, s)) return e;
   // the sequence in chunks of ct tiles (one chunk unless it is long): prepared tiles of u for the chunk, then the
   // scan over it, the state handed from chunk to chunk in the output buffers
   for (int t0 = 0; t0 < ntiles; t0 += ct) {
     const int t1 = t0 + ct < ntiles ? t0 + ct : ntiles;
-    run_dropin_uprep(u, up, d, L, ks, 0, b, t0, t1 - t0, s);
+    if (int e = run_dropin_uprep(u, up, d, L, ks, 0, b, t0, t1 - t0, s)) return e;
     DropinArgs a{};
     a.u = u; a.dt = dt; a.z = z; a.x_bias = x_bias; a.B_r = B_r; a.B_th = B_theta; a.C_r = C_r; a.C_th = C_theta;
     a.Dp = D; a.h_re = t0 ? nh_re : h_re; a.h_im = t0 ? nh_im : h_im; a.y = y; a.nh_re = nh_re; a.nh_im = nh_im;
@@ -736,7 +742,7 @@ int aussm_ssm_adaptive_unitary_bwd(const float* grad_y, const float* grad_nh_re,
   float* hc_im = hc_re + round4(nstate);
   float* dth = hc_im + round4(nstate);
   u4* up = (u4*)(dth + (size_t)blk.bg * ct * DT * d * n);
-  run_dropin_xprep(x, xp, d, n, ks, nb, s);
+  if (int e = run_dropin_xprep(x, xp, d, n, ks, nb, s)) return e;
   DropinArgs f{};
   f.u = u; f.dt = dt; f.z = z; f.x_bias = x_bias; f.B_r = B_r; f.B_th = B_theta; f.C_r = C_r; f.C_th = C_theta;
   f.Dp = D; f.xp = xp; f.up = up; f.d = d; f.n = n; f.L = L; f.ks = ks; f.nb = nb;
@@ -758,7 +764,7 @@ int aussm_ssm_adaptive_unitary_bwd(const float* grad_y, const float* grad_nh_re,
   fill(dC_r, nullptr, n);
   fill(dC_theta, nullptr, n);
   fill(dD, nullptr, d);
-  run_fill(fa, s);
+  if (int e = run_fill(fa, s)) return e;
   const long dn = (long)d * n;
   for (int b0 = 0; b0 < b; b0 += blk.bg) {
     const int bg = b - b0 < blk.bg ? b - b0 : blk.bg;
@@ -767,7 +773,7 @@ int aussm_ssm_adaptive_unitary_bwd(const float* grad_y, const float* grad_nh_re,
       // the state at the end of the sequence: a forward sweep without outputs over this group's chunks
       for (int t0 = 0; t0 < ntiles; t0 += ct) {
         const int t1 = t0 + ct < ntiles ? t0 + ct : ntiles;
-        run_dropin_uprep(u, up, d, L, ks, b0, bg, t0, t1 - t0, s);
+        if (int e = run_dropin_uprep(u, up, d, L, ks, b0, bg, t0, t1 - t0, s)) return e;
         DropinArgs a = f;
         a.h_re = t0 ? hc_re : h_re; a.h_im = t0 ? hc_im : h_im; a.y = nullptr; a.nh_re = hc_re; a.nh_im = hc_im;
         a.up_t0 = t0; a.up_nt = t1 - t0; a.t0 = t0; a.t1 = t1;
@@ -778,7 +784,7 @@ int aussm_ssm_adaptive_unitary_bwd(const float* grad_y, const float* grad_nh_re,
     for (int t0 = ((ntiles - 1) / ct) * ct; t0 >= 0; t0 -= ct) {
       const int t1 = t0 + ct < ntiles ? t0 + ct : ntiles;
       const int l0 = t0 * DT, len = (t1 * DT < L ? t1 * DT : L) - l0;
-      run_dropin_uprep(u, up, d, L, ks, b0, bg, t0, t1 - t0, s);
+      if (int e = run_dropin_uprep(u, up, d, L, ks, b0, bg, t0, t1 - t0, s)) return e;
       DropinBwdArgs q{};
       q.f = f;
       q.f.up_t0 = t0; q.f.up_nt = t1 - t0;

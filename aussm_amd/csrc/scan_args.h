@@ -14,7 +14,8 @@ constexpr int XN = 16;        // state rows of the matrix tiles (N is zero-padde
 enum { VAR_UNITARY = 0, VAR_COMPLEX = 1, VAR_REAL = 2 };
 
 // The optional auxiliary buffer of the unitary scan holds B*D*L floats followed by AUX_PAD floats;
-// the first of those is AUX_TAG when a forward kernel has filled the buffer, anything else if not.
+// the first of those is the call's aux_tag() when a forward kernel has filled the buffer, anything
+// else if not: a backward call consumes the contents only when its own arguments give the same tag.
 // Words AUX_IMG_FP .. + 7 of the pad describe the operand images behind it (ImgStamp below): written
 // by the forward kernel that ran on freshly prepared images, cleared by every other forward call.
 constexpr uint32_t AUX_TAG = 0x4f484950u;
@@ -23,6 +24,18 @@ constexpr int AUX_PAD = 64;
 constexpr int AUX_IMG_FP = 8;
 
 typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+
+// What the per-(b,d,l) part of an auxiliary buffer was computed from: the tensors (addresses), the shape
+// and the input type.  Never zero (zero is what an invalidated buffer holds).
+inline uint32_t aux_tag(const void* u, const void* delta, const void* theta, const void* Bm, const void* Cm,
+                        int B, int D, int N, int L, int in_dtype) {
+  uint64_t h = AUX_TAG;
+  const uint64_t v[] = {(uint64_t)(uintptr_t)u, (uint64_t)(uintptr_t)delta, (uint64_t)(uintptr_t)theta,
+                        (uint64_t)(uintptr_t)Bm, (uint64_t)(uintptr_t)Cm, (uint64_t)B, (uint64_t)D, (uint64_t)N,
+                        (uint64_t)L, (uint64_t)in_dtype};
+  for (uint64_t x : v) h = (h ^ x) * 0x9e3779b97f4a7c15ull + (h >> 29);
+  return (uint32_t)(h >> 32) | 1u;
+}
 
 struct FwdArgs {
   const void* u;            // [B,D,L]  Tin
@@ -49,6 +62,7 @@ struct FwdArgs {
                              // sequence; h0 / hL / ptot are indexed by the pair
   int hs, ho;                // matrix-core kernels: h0 of pair b is entry b * hs + ho of the state array
   int urep;                  // generic kernels: u and delta are [B / urep, D, L], shared by urep consecutive batch elements
+  uint32_t auxtag;           // what a kernel that fills aux writes behind it (aux_tag of the call)
 };
 
 struct UniBwdArgs {
@@ -72,6 +86,7 @@ struct UniBwdArgs {
   int urep;             // generic kernel: u and delta are [B / urep, D, L], shared by urep consecutive batch elements
   int tag_mode;         // matrix-core kernels: 0 use the auxiliary buffer if its tag is valid; 1 leave at once
                         // unless it is; 2 leave at once if it is
+  uint32_t auxtag;      // the tag a forward call of the same arguments leaves behind aux (aux_tag)
 };
 
 struct RecBwdArgs {

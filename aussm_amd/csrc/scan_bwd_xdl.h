@@ -180,7 +180,7 @@ __global__ __launch_bounds__(256) void unitary_bwd_xdl_kernel(const UniBwdArgs p
   constexpr int NPA = sizeof(Tin) == 2 ? 1 : NP, NPAC = sizeof(Tin) == 2 ? 1 : NPC;
   // Im(P_t S_t) left by the forward kernel (if it filled the buffer): saves recomputing S here
   const bool use_phi = p.aux != nullptr &&
-      __builtin_amdgcn_readfirstlane(__float_as_uint(p.aux[(size_t)p.B * D * L])) == AUX_TAG;
+      __builtin_amdgcn_readfirstlane(__float_as_uint(p.aux[(size_t)p.B * D * L])) == p.auxtag;
   if (p.tag_mode == 2 && use_phi) return;      // the kernel that needs the buffer's contents has done the work
   // (always a valid address: the load below is unconditional, its result unused without the tag)
   const float* __restrict__ gph = use_phi ? p.aux + row : gth;

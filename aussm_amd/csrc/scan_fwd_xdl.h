@@ -725,7 +725,7 @@ __global__ __launch_bounds__(256) void unitary_fwd_xdl_kernel(const FwdArgs p) {
     step(c + 1, inB, inA, P1, P0);
   }
 
-  if (p.aux && blockIdx.x == 0 && tid == 0) p.aux[(size_t)p.B * D * L] = __uint_as_float(AUX_TAG);
+  if (p.aux && blockIdx.x == 0 && tid == 0) p.aux[(size_t)p.B * D * L] = __uint_as_float(p.auxtag);
   if (p.hL && dok) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {

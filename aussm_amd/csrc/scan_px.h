@@ -240,15 +240,6 @@ __device__ __forceinline__ void cs_i_from_r(const u4 (&a)[NP], u4 (&o)[NP]) {
   for (int q = 0; q < NP; ++q) o[q] = u4{a[q][2] ^ 0x80008000u, a[q][3] ^ 0x80008000u, a[q][0], a[q][1]};
 }
 
-// Development aid (-DAUSSM_PX_TIMING): lane 0 of wavefronts 0 and 4 of workgroup 0 records the
-// shader clock at marked points of every interval into the hL buffer (which is then not an output).
-#ifdef AUSSM_PX_TIMING
-#define PX_MARK(k) do { if (blockIdx.x == 0 && cg == 0 && lane == 0 && i < 70 && i >= 0) \
-    reinterpret_cast<long long*>(p.hL)[(hf * 70 + i) * 8 + (k)] = clock64(); } while (0)
-#else
-#define PX_MARK(k) do { } while (0)
-#endif
-
 // Requires what unitary_fwd_xdl_kernel requires, and the forward images of the call's B_t / C_t.
 // img: [B / ns batch elements][ceil(ld / 32)] images.
 template <bool GATED, typename Tin = float>
@@ -446,12 +437,10 @@ __global__ __launch_bounds__(512) void unitary_fwd_px_kernel(const FwdArgs p, co
   // run on zero input and zero phase: the state passes through unchanged, nothing is stored.
   auto phase_a = [&](int c) {
     const int i = c;
-    PX_MARK(0);
     // (the phase B before it issued the input loads of its gather after the image loads)
     img_store(i + 2, i + 1, std::integral_constant<int, N_IN>{});
     flush_out();
     img_load(i + 3, i + 2);
-    PX_MARK(1);
     float vr[8], vi[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
@@ -465,7 +454,6 @@ __global__ __launch_bounds__(512) void unitary_fwd_px_kernel(const FwdArgs p, co
     split8<NP>(sk, vi, Vi);
     // rotation over the whole chunk: the element (st 1, g 3, i 3) is timestep 31
     const float cT = __shfl(cs[7], 48 + dl), sT = __shfl(sn[7], 48 + dl);
-    PX_MARK(2);
     // ---- Z = B^T V  (four independent accumulation chains)
     f4 z0 = {0, 0, 0, 0}, z1 = {0, 0, 0, 0}, z2 = {0, 0, 0, 0}, z3 = {0, 0, 0, 0};
     {
@@ -488,7 +476,6 @@ __global__ __launch_bounds__(512) void unitary_fwd_px_kernel(const FwdArgs p, co
             z3 = xdl(b_i[k], Vr[s - k], z3);
           }
     }
-    PX_MARK(3);
     // ---- carry: H_{c+1} = P_T (H_c + Z)
     Hr = s_h[c & 1][cg][0][lane];
     Hi = s_h[c & 1][cg][1][lane];
@@ -508,19 +495,15 @@ __global__ __launch_bounds__(512) void unitary_fwd_px_kernel(const FwdArgs p, co
       for (int k = 0; k < 4; ++k)
         if (4 * g + k < N) { hp[(size_t)k * 2 * D] = nr[k]; hp[(size_t)k * 2 * D + D] = ni[k]; }
     }
-    PX_MARK(4);
     lds_barrier();
-    PX_MARK(6);
   };
 
   // ---- phase B of chunk c (interval i = c + 1): S = C.H + G.V, outputs; then the gather of chunk c + 2
   auto phase_b = [&](int c) {
     const int i = c + 1;
-    PX_MARK(0);
     // (the phase A before it issued nothing after the image loads but, now and then, checkpoint stores)
     img_store(i + 2, i + 1, std::integral_constant<int, 0>{});
     img_load(i + 3, i + 2);
-    PX_MARK(1);
     const u4* sb_ = s_b[c % 3];
     u4 hk[NP];
     {
@@ -558,7 +541,6 @@ __global__ __launch_bounds__(512) void unitary_fwd_px_kernel(const FwdArgs p, co
       Sr[tt] = a0 + a2;
       Si[tt] = a1 + a3;
     }
-    PX_MARK(3);
     // ---- outputs: rows 16 tt + 4 g + k of channel dl are this lane's own timesteps.  They are
     // stored at the start of this wavefront's next interval: a store issued here would still be
     // in flight at the wait that ends the interval (loads and stores share one counter).
@@ -575,12 +557,9 @@ __global__ __launch_bounds__(512) void unitary_fwd_px_kernel(const FwdArgs p, co
       }
     }
     out_l0 = c * XT;
-    PX_MARK(4);
     // (younger than the inputs it collects: the image loads of this interval)
     gather(c + 2, c + 4, std::integral_constant<int, N_IMG>{});
-    PX_MARK(5);
     lds_barrier();
-    PX_MARK(6);
   };
   // an interval in which this wavefront has no chunk: it still takes part in the image loads
   auto idle = [&](int i) {
@@ -611,10 +590,9 @@ __global__ __launch_bounds__(512) void unitary_fwd_px_kernel(const FwdArgs p, co
   in_landed(in, std::integral_constant<int, 0>{});
 
   flush_out();
-  if (p.aux && blockIdx.x == 0 && tid == 0) p.aux[(size_t)(p.B / p.ns) * D * p.ld] = __uint_as_float(AUX_TAG);
+  if (p.aux && blockIdx.x == 0 && tid == 0) p.aux[(size_t)(p.B / p.ns) * D * p.ld] = __uint_as_float(p.auxtag);
   // (the pre-pass that wrote the images has finished: this kernel read them)
   if (note.dst && blockIdx.x == 0 && tid < 8) note.dst[tid] = note.stamp.w[tid];
-#ifndef AUSSM_PX_TIMING
   if (p.hL && dok && hf == 0) {
     const f4 hr = s_h[0][cg][0][lane], hi = s_h[0][cg][1][lane];    // state after the last (possibly padding) chunk
 #pragma unroll
@@ -627,7 +605,6 @@ __global__ __launch_bounds__(512) void unitary_fwd_px_kernel(const FwdArgs p, co
       }
     }
   }
-#endif
 }
 
 
@@ -661,13 +638,6 @@ constexpr int PXB_ND = 4 * PXB_NS * 4;
 constexpr int PXB_RS = 68;                 // row stride of the dB / dC shares (64 floats + pad)
 static_assert(4 * PXB_ND <= PXB_WS, "the scratch is reused");
 
-#ifdef AUSSM_PX_TIMING
-#define PXB_MARK(k) do { if (blockIdx.x == 0 && cg == 0 && lane == 0 && i_ < 40) \
-    reinterpret_cast<long long*>(p.dh0)[(hf * 40 + i_) * 12 + (k)] = clock64(); } while (0)
-#else
-#define PXB_MARK(k) do { } while (0)
-#endif
-
 template <int NPC, typename Tin = float>
 __global__ __launch_bounds__(512) void unitary_bwd_px_kernel(const UniBwdArgs p, const u4* __restrict__ img) {
   constexpr int NP = PX_NP;
@@ -695,7 +665,7 @@ __global__ __launch_bounds__(512) void unitary_bwd_px_kernel(const UniBwdArgs p,
   const size_t row = ((size_t)bb * D + dc) * p.ld + so;
   const size_t tagpos = (size_t)(p.B / p.ns) * D * p.ld;
   if (p.tag_mode == 1 &&
-      __builtin_amdgcn_readfirstlane(__float_as_uint(p.aux[tagpos])) != AUX_TAG)
+      __builtin_amdgcn_readfirstlane(__float_as_uint(p.aux[tagpos])) != p.auxtag)
     return;
   // (the launcher only takes this kernel for tensors below 4 GiB: 32-bit byte offsets per lane)
   const uint32_t rowf = (uint32_t)(row * 4), rowt = (uint32_t)(row * sizeof(Tin));
@@ -829,8 +799,6 @@ __global__ __launch_bounds__(512) void unitary_bwd_px_kernel(const UniBwdArgs p,
   // ---- phase A of chunk index r
   auto phase_a = [&](int r) {
     const int c = nchunks - 1 - r;
-    const int i_ = r;
-    PXB_MARK(0);
     // A chunk that starts a checkpoint block hands the stored state on instead of the recomputed
     // one (this stops the drift of the backward recomputation).  Plain loads, once per block.
     const bool ck_here = c > 0 && c % ck_chunks == 0;     // (uniform)
@@ -843,7 +811,6 @@ __global__ __launch_bounds__(512) void unitary_bwd_px_kernel(const UniBwdArgs p,
         if (n < N) { ckv[i] = cp[(size_t)n * 2 * D]; ckv[4 + i] = cp[(size_t)n * 2 * D + D]; }
       }
     }
-    PXB_MARK(1);
     u4 Vr[NP], Vi[NP], Qr[NP], Qi[NP];
     float vr[8], vi[8];
     {
@@ -859,7 +826,6 @@ __global__ __launch_bounds__(512) void unitary_bwd_px_kernel(const UniBwdArgs p,
       split8<NP>(sk, vr, Vr); split8<NP>(sk, vi, Vi); split8<NP>(sk, qr, Qr); split8<NP>(sk, qi, Qi);
     }
     const float cT = __shfl(cs[7], 48 + dl), sT = __shfl(sn[7], 48 + dl);
-    PXB_MARK(2);
     // ---- Z = B^T V, then W = conj(C)^T Q  (four independent accumulation chains each; one after
     // the other so that only one set of operand records is live at a time)
     f4 z0 = {0, 0, 0, 0}, z1 = z0, z2 = z0, z3 = z0, w0 = z0, w1 = z0, w2 = z0, w3 = z0;
@@ -904,7 +870,6 @@ __global__ __launch_bounds__(512) void unitary_bwd_px_kernel(const UniBwdArgs p,
           }
     }
     __builtin_amdgcn_sched_barrier(0);
-    PXB_MARK(3);
     // (here rather than at the start of the interval, where every wavefront of the workgroup has
     // memory operations to issue)
     flush_acc(r);
@@ -934,7 +899,6 @@ __global__ __launch_bounds__(512) void unitary_bwd_px_kernel(const UniBwdArgs p,
     s_x[cg][2][lane] = nAr;
     s_x[cg][3][lane] = nAi;
     __builtin_amdgcn_sched_barrier(0);
-    PXB_MARK(4);
     const u4* sb_ = s_b[r & 1];
     // ---- gV = sum_n conj(B_s[n]) J[n] + sum_{t>=s} conj(G[t,s]) Q_t   (one set of operand records live at a time)
     f4 gVr[2], gVi[2];
@@ -981,7 +945,6 @@ __global__ __launch_bounds__(512) void unitary_bwd_px_kernel(const UniBwdArgs p,
       }
     }
     __builtin_amdgcn_sched_barrier(0);
-    PXB_MARK(5);
     // ---- per-element results
     {
       float dw[8], gth[8];
@@ -1026,17 +989,13 @@ __global__ __launch_bounds__(512) void unitary_bwd_px_kernel(const UniBwdArgs p,
         }
       }
     }
-    PXB_MARK(6);
     lds_barrier();                 // (the shares of dB / dC of the interval before have been read)
     lds_barrier();
-    PXB_MARK(7);
   };
 
   // ---- phase B of chunk index r
   auto phase_b = [&](int r) {
     const int c = nchunks - 1 - r;
-    const int i_ = r + 1;
-    PXB_MARK(0);
     // ---- this wavefront's loads: the images of the next interval, the inputs of its next chunk
     img_load(r + 2, r + 2);
     const u4* sa_ = s_a[r % 3];
@@ -1104,7 +1063,6 @@ __global__ __launch_bounds__(512) void unitary_bwd_px_kernel(const UniBwdArgs p,
     }
     __builtin_amdgcn_sched_barrier(0);
     in_load(r + 2);                // (not at the start of the interval, where every wavefront has loads to issue)
-    PXB_MARK(1);
     // One output tile at a time: (dC, timesteps 16 tile ..), then (dB, ...).  The closing product
     // takes M with rows = the tile's timesteps and the other time index in the K slots: two 16 x 16
     // blocks of M side by side (the second one is zero above the block diagonal).
@@ -1166,13 +1124,9 @@ __global__ __launch_bounds__(512) void unitary_bwd_px_kernel(const UniBwdArgs p,
       __builtin_amdgcn_sched_barrier(0);
     };
     close_tile(true, 0);
-    PXB_MARK(3);
     close_tile(true, 1);
-    PXB_MARK(4);
     close_tile(false, 0);
-    PXB_MARK(5);
     close_tile(false, 1);
-    PXB_MARK(6);
     // ---- the one wait for this wavefront's loads: they were issued at the start of the phase, and
     // nothing else of it is in flight (the stores of the phase A before are an interval old)
     all_landed();
@@ -1189,7 +1143,6 @@ __global__ __launch_bounds__(512) void unitary_bwd_px_kernel(const UniBwdArgs p,
       }
     }
     lds_barrier();
-    PXB_MARK(7);
   };
   // an interval in which this wavefront has no chunk
   auto idle = [&](int i) { flush_acc(i); lds_barrier(); lds_barrier(); };
@@ -1246,7 +1199,6 @@ __global__ __launch_bounds__(512) void unitary_bwd_px_kernel(const UniBwdArgs p,
     flush_acc(2 * npairs + 1);          // (what the second half accumulated in the last interval)
   }
 
-#ifndef AUSSM_PX_TIMING
   if (p.dh0 && dok && hf == 0) {
     const f4 ar = s_x[cg][2][lane], ai = s_x[cg][3][lane];
 #pragma unroll
@@ -1259,7 +1211,6 @@ __global__ __launch_bounds__(512) void unitary_bwd_px_kernel(const UniBwdArgs p,
       }
     }
   }
-#endif
   if (p.dD && dok) {
     accD += __shfl_xor(accD, 16);
     accD += __shfl_xor(accD, 32);

@@ -120,6 +120,12 @@ def scaling(args):
     del warm
     for b, d, n in shapes:
         for system in systems:
+            # one-off costs of a system's first use (code objects of its backward kernels loaded on first launch, the
+            # autograd engine's thread, first allocations) stay out of the timed repetitions of its first point
+            try:
+                point(system, b, d, n, lengths[0])
+            except RuntimeError:
+                pass
             for l in lengths:
                 try:
                     rec = point(system, b, d, n, l)

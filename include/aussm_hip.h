@@ -135,10 +135,12 @@ int aussm_unitary_bwd(const float* dy, const float* dhL,
  * the calls above).  `aux` holds aussm_unitary_aux_floats(B, D, N, L, ck) floats, 16-byte aligned,
  * sized with the arguments of the calls it is passed to.  Three uses, all internal:
  *  - the forward call may leave per-(b,d,l) intermediate results in it (Im(P_t S_t), the term of
- *    the phase gradient that needs the forward states) together with a validity tag; the backward
- *    call given the same buffer then skips recomputing them.  A forward kernel that does not fill
- *    the buffer clears the tag, so a backward call never consumes stale contents: handing over
- *    `aux` is always safe and only ever a speed-up;
+ *    the phase gradient that needs the forward states) together with a tag formed from the call's
+ *    tensor addresses (u, delta, theta, Bc, Cc), B, D, N, L and in_dtype; a backward call given the
+ *    same buffer AND the same tensors skips recomputing them.  A forward kernel that does not fill
+ *    the buffer clears the tag, and a backward call whose arguments give another tag recomputes,
+ *    so handing over `aux` is safe and only ever a speed-up - as long as the tensors are not
+ *    modified in place between the two calls (the tag knows addresses, not contents);
  *  - the matrix-core kernels run on operands prepared from Bc and Cc by a pre-pass (split into bf16
  *    pieces, in the record orders the products need); they live at the end of the buffer.  A forward
  *    call that is given hck (a backward call can follow) prepares the backward call's operands in
@@ -312,7 +314,7 @@ int aussm_swap_last2_act(const float* x, const float* bias, const float* pre, fl
  *   torch.ops.extension_cpp.ssm_adaptive_unitary           (12 tensors -> y, next_hid_real, next_hid_imag)
  *   torch.ops.extension_cpp.ssm_adaptive_backward_unitary  (3 + 12 tensors -> 12 gradients)
  * bind to - extension-cpp/extension_cpp/csrc/cuda/ssm_adaptive_unitary_forward.cu:184-286 and
- * ssm_adaptive_unitary_backward.cu:333-497, Python side extension-cpp/extension_cpp/ops.py:97-154.
+ * ssm_adaptive_unitary_backward.cu:493-617, Python side extension-cpp/extension_cpp/ops.py:97-154.
  * Arguments in the operator's order; all tensors fp32 and contiguous:
  *   u, dt, z (b, d, L);  x (d, n, d);  x_bias (d, n);  B_r, B_theta, C_r, C_theta (n);  D (d);
  *   h_re, h_im (b, d, n) the state before the first step;  y (b, d, L);  nh_* (b, d, n).

@@ -51,9 +51,30 @@ ACC_BAD = """
 	;;#ASMEND
 	v_accvgpr_read_b32 v31, a6
 """
+# a load issued at the end of a loop body and retired at the top of the next iteration: the register is
+# touched between the loop's label and the wait, which only the walk over the back-edge sees
+LOOP_BAD = """
+.LBB0_1:
+	v_mov_b32_e32 v40, v2
+	;;#ASMSTART
+	s_waitcnt vmcnt(0)
+	;;#ASMEND
+	v_mov_b32_e32 v41, v3
+	;;#ASMSTART
+	global_load_dwordx4 v[2:5], v[8:9], off
+	;;#ASMEND
+	s_cbranch_scc1 .LBB0_1
+	;;#ASMSTART
+	s_waitcnt vmcnt(0)
+	;;#ASMEND
+"""
+LOOP_GOOD = LOOP_BAD.replace("v_mov_b32_e32 v40, v2", "v_mov_b32_e32 v40, v9")
 
 
 def test_scanner_on_hand_made_listings():
+    found = build.scan_listing(LOOP_BAD)
+    assert len(found) == 1 and "v40" in found[0][1]
+    assert build.scan_listing(LOOP_GOOD) == []
     assert build.scan_listing(GOOD) == []
     assert [ln for ln, _ in build.scan_listing(BAD)] == [5, 6]
     found = build.scan_listing(COUNTED)
