@@ -36,7 +36,8 @@ from . import _lib as L
 from . import scan
 
 __all__ = ["ssm_adaptive_unitary", "ssm_adaptive_interface", "pad_to_multiple_of",
-           "reference_ssm_adaptive_unitary_optimized_polar"]
+           "reference_ssm_adaptive_unitary_optimized_polar", "reference_ssm_adaptive_preal",
+           "reference_ssm_adaptive_preal_optimized"]
 
 _NS = "extension_cpp"
 _FWD_SCHEMA = ("ssm_adaptive_unitary(Tensor u, Tensor dt, Tensor x, Tensor x_bias, Tensor B_r, Tensor B_theta, "
@@ -285,3 +286,54 @@ def reference_ssm_adaptive_unitary_optimized_polar(u: Tensor, dt: Tensor, x: Ten
     if not u.is_cuda:
         raise RuntimeError("scan inputs must be on the GPU (no CPU implementation is shipped)")
     return ssm_adaptive_interface(u, dt, x, x_bias, B, C, D, z, unitary=True, max_parallel_length=max(1, u.shape[-1]))
+
+
+# ---- the positive-real adaptive scan of the reference's pure-PyTorch file -------------------------------------
+# Upstream it has no reachable kernel (ssm_adaptive_interface raises for unitary=False, ops.py:86-87, as this
+# package's does) and no caller in the models; the two callables keep their names and signatures and run the
+# recurrence on the HIP scan kernels.  The decay exp(x.u) differs per (channel, state) pair, so every pair is one
+# channel with a single state of the complex scan (log-modulus = the contracted decay, phase 0): the launch
+# covers d n channels, the products with B_t in front of it and with C_t behind it are elementwise torch, and
+# autograd runs through the scan's own backward kernels.
+
+def _preal_scan(log_a: Tensor, w: Tensor, B: Tensor, C: Tensor) -> Tensor:
+    """sum_j C_l[b,j] h_l[b,i,j] with h_l = exp(log_a_l) h_{l-1} + w_l[b,i] B_l[b,j], h_0 = 0.
+    log_a: (b, d, n, l); w: (b, d, l); B, C: (b, n, l) real."""
+    b, d, n, l = log_a.shape
+    inp = (w[:, :, None, :] * B[:, None, :, :]).reshape(b, d * n, l)
+    one = torch.ones((b, d * n, l), device=w.device, dtype=torch.float32)
+    unit = torch.ones((b, 1, l), device=w.device, dtype=torch.complex64)
+    h = scan.complex_scan(inp, one, log_a.reshape(b, d * n, l).contiguous(), torch.zeros_like(one), unit, unit)
+    return (h.view(b, d, n, l) * C[:, None, :, :]).sum(2)
+
+
+def _preal_check(u, dt, x, B, C, D, z):
+    for name, t in (("u", u), ("dt", dt), ("x", x), ("B", B), ("C", C), ("D", D), ("z", z)):
+        if t.dtype != torch.float32:
+            raise RuntimeError(f"expected {name} to be float32, got {t.dtype}")
+        if not t.is_cuda:
+            raise RuntimeError("scan inputs must be on the GPU (no CPU implementation is shipped)")
+    if x.dim() != 3:
+        raise RuntimeError("x must be (d, n, d)")
+
+
+def reference_ssm_adaptive_preal(u: Tensor, dt: Tensor, x: Tensor, B: Tensor, C: Tensor, D: Tensor, z: Tensor) -> Tensor:
+    """Name, signature and arithmetic of extension-cpp/extension_cpp/ops.py:300-357:
+    h_l = exp(x.u_l) h_{l-1} + dt_l B_l silu(u_l),  y_l = (sum_j C_l h_l + D silu(u_l)) silu(z_l), from a zero state.
+    u, dt, z: (b, d, l); x: (d, n, d); B, C: (b, n, l) real; D: (d,)."""
+    _preal_check(u, dt, x, B, C, D, z)
+    log_a = torch.einsum("ijr,brl->bijl", x, u)
+    us = F.silu(u)
+    y = _preal_scan(log_a, dt * us, B, C)
+    return (y + us * D[None, :, None]) * F.silu(z)
+
+
+def reference_ssm_adaptive_preal_optimized(u: Tensor, dt: Tensor, x: Tensor, x_bias: Tensor, B: Tensor, C: Tensor,
+                                           D: Tensor, z: Tensor) -> Tensor:
+    """Name, signature and arithmetic of extension-cpp/extension_cpp/ops.py:465-510: the decay is
+    exp((x.u_l + x_bias) dt_l) and the raw input enters (no silu).  Upstream evaluates it with cumulative sums
+    of exp(-G), which overflow on long sequences; here it is the recurrence itself."""
+    _preal_check(u, dt, x, B, C, D, z)
+    log_a = (torch.einsum("ijr,brl->bijl", x, u) + x_bias[None, :, :, None]) * dt[:, :, None, :]
+    y = _preal_scan(log_a, dt * u, B, C)
+    return (y + u * D[None, :, None]) * F.silu(z)

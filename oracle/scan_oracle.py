@@ -34,6 +34,11 @@ Pinning status (which independent check fixes each function):
                          brute-force scalar loop                       pinned
   causal_conv1d_bld      torch's conv1d called exactly as the reference's blocks
                          call it; explicit causal sum in Python loops  pinned
+  adaptive_preal_loop    brute-force scalar loop; with the decay scaled by
+                         the step size it agrees with the reference's own
+                         cumulative-sum formulation restated beside it
+                         (adaptive_preal_cumsum); float64 gradcheck    pinned
+  adaptive_preal_cumsum  same pair                                     pinned
 """
 from __future__ import annotations
 
@@ -256,6 +261,51 @@ def reference_unitary_phase_loop(u: Tensor, dt: Tensor, x: Tensor, x_bias: Tenso
         h = a[:, :, :, t] * h + (dt[:, :, t] * u[:, :, t])[:, :, None] * Bc[:, None, :, t]
         ys.append((h * Cc[:, None, :, t]).sum(-1).real)
     y = torch.stack(ys, dim=-1)
+    return (y + u * D[None, :, None]) * F.silu(z)
+
+
+# --------------------------------------------------------------------------
+# Positive-real adaptive scan of the reference's pure-PyTorch file (no kernel
+# of the reference is reachable for it; extension_cpp/ops.py:86-87 raises).
+# --------------------------------------------------------------------------
+
+def adaptive_preal_loop(u: Tensor, dt: Tensor, x: Tensor, B: Tensor, C: Tensor, D: Tensor, z: Tensor,
+                        x_bias: Optional[Tensor] = None, step_scaled: bool = False) -> Tensor:
+    """Real adaptive scan whose decay is contracted from the input,
+        log a_l[b,i,j] = sum_r x[i,j,r] u_l[b,r]           (+ x_bias[i,j], times dt_l[b,i] if step_scaled)
+        h_l = a_l h_{l-1} + dt_l[b,i] B_l[b,j] v_l[b,i],   y_l = (sum_j C_l[b,j] h_l + D_i v_l) silu(z_l),  h_0 = 0.
+    step_scaled=False restates reference_ssm_adaptive_preal (extension-cpp/extension_cpp/ops.py:300-357):
+    no bias, and the input enters through v = silu(u) (ops.py:333) while the decay sees the raw u (ops.py:331).
+    step_scaled=True restates the recurrence behind reference_ssm_adaptive_preal_optimized (ops.py:465-510):
+    log a = (x.u + x_bias) dt (ops.py:491-493) and v = u, the raw input (no silu there).
+    u, dt, z: (b, d, l); x: (d, n, d); B, C: (b, n, l) real; D: (d,)."""
+    b, d, l = u.shape
+    log_a = torch.einsum("ijr,brl->bijl", x, u)
+    if x_bias is not None:
+        log_a = log_a + x_bias[None, :, :, None]
+    if step_scaled:
+        log_a = log_a * dt[:, :, None, :]
+    v = u if step_scaled else F.silu(u)
+    a = torch.exp(log_a)                                                 # (b, d, n, l)
+    w = dt * v
+    h = torch.zeros(b, d, x.shape[1], dtype=u.dtype)
+    ys = []
+    for t in range(l):
+        h = a[:, :, :, t] * h + w[:, :, t, None] * B[:, None, :, t]
+        ys.append((h * C[:, None, :, t]).sum(-1))
+    y = torch.stack(ys, dim=-1)
+    return (y + v * D[None, :, None]) * F.silu(z)
+
+
+def adaptive_preal_cumsum(u: Tensor, dt: Tensor, x: Tensor, x_bias: Tensor, B: Tensor, C: Tensor, D: Tensor,
+                          z: Tensor) -> Tensor:
+    """The cumulative-sum formulation the reference writes for the step-scaled form
+    (extension-cpp/extension_cpp/ops.py:491-503): G = cumsum(log a), y = sum_j C exp(G) cumsum(exp(-G) dt B u).
+    Independent of the recurrence above (and overflow-prone for long sequences, as upstream)."""
+    log_a = (torch.einsum("ijr,brl->bijl", x, u) + x_bias[None, :, :, None]) * dt[:, :, None, :]
+    G = torch.cumsum(log_a, dim=-1)
+    inner = torch.cumsum(torch.exp(-G) * (dt * u)[:, :, None, :] * B[:, None, :, :], dim=-1)
+    y = (C[:, None, :, :] * torch.exp(G) * inner).sum(2)
     return (y + u * D[None, :, None]) * F.silu(z)
 
 
