@@ -74,26 +74,34 @@ def _check_op_inputs(args) -> Tuple[int, int, int, int]:
     return b, d, n, l
 
 
-def _composite(u, dt, x, x_bias, B_r, B_theta, C_r, C_theta, D, z, h_r, h_i):
-    """The operator as differentiable torch ops around ONE core-scan launch."""
-    b, d, n, l = _check_op_inputs((u, dt, x, x_bias, B_r, B_theta, C_r, C_theta, D, z, h_r, h_i))
+def _composite_scan(u, dt, x, x_bias, Bt, Ct, D, z, h_r, h_i):
+    """Differentiable torch ops around ONE core-scan launch.  Bt, Ct: complex (n,) constants or (b, n, l)
+    time-varying; z None: no gate."""
+    b, d, l = u.shape
+    n = x.shape[1]
     # phase projection: theta[b, j, i, l]  (state index before channel so that (b, j) is a batch)
     xm = x.permute(1, 0, 2).reshape(n * d, d)                          # (j i) x r
     # one strided-batched GEMM straight into (b, (j i), l); the 2-D x 3-D form of matmul goes through
     # transposed copies of the whole phase tensor
     theta = torch.baddbmm(x_bias.t().reshape(1, n * d, 1), xm.unsqueeze(0).expand(b, n * d, d), u).view(b, n, d, l)
     us = F.silu(u)
-    Bt = torch.polar(B_r, B_theta)                                     # (n,)
-    Ct = torch.polar(C_r, C_theta)
-    row = lambda c: c[None, :, None].expand(b, n, l).reshape(b * n, 1, l)
+    row = lambda c: (c[None, :, None].expand(b, n, l) if c.dim() == 1 else c).reshape(b * n, 1, l)
     h0 = torch.complex(h_r, h_i).permute(0, 2, 1).reshape(b * n, d, 1)
     # us, dt stay (b, d, l): each of their batch elements serves the n consecutive (batch, state) pairs
     y, hL = scan.unitary_scan(us, dt.contiguous(), theta.reshape(b * n, d, l), row(Bt), row(Ct), None, None, h0,
                               return_last_state=True)
     y = y.view(b, n, d, l).sum(dim=1)
-    y = (y + us * D[None, :, None]) * F.silu(z)
+    y = y + us * D[None, :, None]
+    if z is not None:
+        y = y * F.silu(z)
     hL = hL.view(b, n, d).permute(0, 2, 1)
     return y, hL.real.contiguous(), hL.imag.contiguous()
+
+
+def _composite(u, dt, x, x_bias, B_r, B_theta, C_r, C_theta, D, z, h_r, h_i):
+    """The operator as differentiable torch ops around ONE core-scan launch."""
+    _check_op_inputs((u, dt, x, x_bias, B_r, B_theta, C_r, C_theta, D, z, h_r, h_i))
+    return _composite_scan(u, dt, x, x_bias, torch.polar(B_r, B_theta), torch.polar(C_r, C_theta), D, z, h_r, h_i)
 
 
 # ---- dispatcher ops -------------------------------------------------------------------------
@@ -273,19 +281,35 @@ def reference_ssm_adaptive_unitary_optimized_polar(u: Tensor, dt: Tensor, x: Ten
                                                    no_graded_rotation: bool = False, unitary: bool = True) -> Tensor:
     """The callable `SSMauBlock(cuda=False)` selects in the reference (aussm.py:842-843; ops.py:614-769):
     there a pure-PyTorch cumulative-sum form of the same operator.  Here the name and signature are kept
-    and the default case - constant complex B, C of shape (n,), gate on, graded rotation - runs on the
-    same fused HIP kernels as ssm_adaptive_interface (one launch sequence, any length); there is no eager
-    or CPU path behind it.  The research switches of the reference (diagnostic outputs, binary or ungraded
-    rotations, time-varying B / C phases, no gate) are not implemented and raise."""
-    if diagnostic or binary or no_graded_rotation or not unitary or not z_prod:
-        raise NotImplementedError("only the default form (unitary, graded rotation, gated, no diagnostics) is implemented")
-    if B.dim() != 1 or C.dim() != 1:
-        raise NotImplementedError("time-varying B / C phases are not implemented by the fused operator")
-    if z is None:
+    and every case runs on the HIP kernels; there is no eager or CPU path behind it.
+      * constant complex B, C of shape (n,) with the gate (the default, what the blocks call): the fused
+        kernels of ssm_adaptive_interface, one launch sequence, any length;
+      * B and / or C given as real phases of shape (b, n, l) (unit modulus, ops.py:721-723, :745-746), or
+        z_prod=False (no gate, ops.py:759-761): the composite route - phase projection by BLAS, one core-scan
+        launch with every (batch, state) pair as a batch element.
+    The remaining research switches of the reference (diagnostic outputs, binary or ungraded rotations) replace
+    the rotation by sign functions and return (b, l, d, n) intermediates; they are not implemented and raise."""
+    if diagnostic or binary or no_graded_rotation or not unitary:
+        raise NotImplementedError("diagnostic outputs and binary / ungraded rotations are not implemented")
+    if z_prod and z is None:
         raise ValueError("z is required (z_prod=True)")
     if not u.is_cuda:
         raise RuntimeError("scan inputs must be on the GPU (no CPU implementation is shipped)")
-    return ssm_adaptive_interface(u, dt, x, x_bias, B, C, D, z, unitary=True, max_parallel_length=max(1, u.shape[-1]))
+    if B.dim() == 1 and C.dim() == 1 and z_prod:
+        return ssm_adaptive_interface(u, dt, x, x_bias, B, C, D, z, unitary=True, max_parallel_length=max(1, u.shape[-1]))
+    b, d, l = u.shape
+    n = x.shape[1]
+
+    def coefficient(c, name):
+        if c.dim() == 1:                                   # radius = softplus(real part), phase = imaginary part
+            return torch.polar(F.softplus(c.real), c.imag)
+        if c.is_complex() or tuple(c.shape) != (b, n, l):
+            raise RuntimeError(f"expected {name} complex of shape ({n},) or real phases of shape {(b, n, l)}")
+        return torch.polar(torch.ones_like(c), c)
+    zero = torch.zeros((b, d, n), device=u.device, dtype=torch.float32)
+    y, _, _ = _composite_scan(u.contiguous(), dt, x, x_bias, coefficient(B, "B"), coefficient(C, "C"), D,
+                              z if z_prod else None, zero, zero)
+    return y
 
 
 # ---- the positive-real adaptive scan of the reference's pure-PyTorch file -------------------------------------

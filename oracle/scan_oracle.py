@@ -219,19 +219,26 @@ def adaptive_unitary_loop(u: Tensor, dt: Tensor, x: Tensor, x_bias: Tensor, Bp: 
 
 def adaptive_unitary_polar(u: Tensor, dt: Tensor, x: Tensor, x_bias: Tensor, Bp: Tensor, Cp: Tensor,
                            D: Tensor, z: Optional[Tensor] = None) -> Tensor:
-    """Cumulative-sum ("polar") formulation with constant complex Bp, Cp (n,).
+    """Cumulative-sum ("polar") formulation.
 
-    Restates extension-cpp/extension_cpp/ops.py:661-764 for the branch the
-    reference's tests use (constant B and C, binary=False, z_prod=True):
+    Restates extension-cpp/extension_cpp/ops.py:661-764 (binary=False):
         G = cumsum(theta) mod 2 pi
         re = cumsum(B_r cos(B_theta - G) dt silu(u)), im likewise with sin
-        y  = sum_j C_r (cos(C_theta + G) re - sin(C_theta + G) im) + silu(u) D
-    This is a formulation independent of the recurrence in
-    adaptive_unitary_loop; the two must agree.
+        y  = sum_j C_r (cos(C_theta + G) re - sin(C_theta + G) im) + silu(u) D      (* silu(z) if z is given)
+    Bp, Cp: constant complex (n,) - radius softplus(real part), phase the imaginary part (ops.py:705-706,
+    :737-738), the branch the reference's tests use - or real phases (b, n, l) of unit-modulus time-varying
+    coefficients (ops.py:721-723, :745-746).  z None is the reference's z_prod=False.
+    This is a formulation independent of the recurrence in adaptive_unitary_loop; the two must agree.
     """
     theta = adaptive_phase(u, x, x_bias).permute(0, 3, 1, 2)             # (b, l, d, n)
     G = torch.cumsum(theta, dim=1) % (2 * math.pi)
-    B_r, B_th, C_r, C_th = polar_params(Bp, Cp)
+
+    def polar_of(c):
+        if c.dim() == 1:
+            return F.softplus(c.real), c.imag
+        return torch.ones_like(c).permute(0, 2, 1)[:, :, None, :], c.permute(0, 2, 1)[:, :, None, :]   # (b, l, 1, n)
+    B_r, B_th = polar_of(Bp)
+    C_r, C_th = polar_of(Cp)
     us = F.silu(u).permute(0, 2, 1)                                      # (b, l, d)
     dtl = dt.permute(0, 2, 1)
     amp = (dtl * us)[..., None]

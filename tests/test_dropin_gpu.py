@@ -134,6 +134,27 @@ def test_polar_callable_of_the_blocks():
         ops.reference_ssm_adaptive_unitary_optimized_polar(*dev, unitary=False)
     with pytest.raises(RuntimeError):
         ops.reference_ssm_adaptive_unitary_optimized_polar(*args)          # CPU tensors: nothing is shipped for them
+    # time-varying unit-modulus B / C given as phases (b, n, l), and the ungated form (z_prod=False): the
+    # reference's other branches (ops.py:721-723, :745-746, :759-761), outputs and gradients against the
+    # float64 cumulative-sum oracle
+    u, dt, x, xb, Bp, Cp, D, z = args
+    b, n, l = u.shape[0], x.shape[1], u.shape[2]
+    g = torch.Generator().manual_seed(8)
+    Bph, Cph = torch.randn(b, n, l, generator=g), torch.randn(b, n, l, generator=g)
+    for Bx, Cx, zp in ((Bph, Cph, True), (Bph, Cp, True), (Bp, Cph, False), (Bp, Cp, False)):
+        def run(fn, dev, dtype):
+            cast = lambda t: (t.to(torch.complex128 if dtype == torch.float64 else torch.complex64) if t.is_complex() else t.to(dtype))
+            lv = [cast(t).clone().to(dev).requires_grad_(True) for t in (u, dt, x, xb, Bx, Cx, D, z)]
+            y = fn(*lv)
+            (y * y).sum().backward()
+            return y.detach().cpu().double(), [(torch.view_as_real(t.grad) if t.grad.is_complex() else t.grad).cpu().double()
+                                                for t in (lv if zp else lv[:-1])]
+        want, gw = run(lambda *a: O.adaptive_unitary_polar(*a[:7], a[7] if zp else None), "cpu", torch.float64)
+        got, gg = run(lambda *a: ops.reference_ssm_adaptive_unitary_optimized_polar(*a, z_prod=zp), "cuda", torch.float32)
+        torch.testing.assert_close(got, want, atol=1e-4, rtol=1e-4)
+        for a_, w_ in zip(gg, gw):
+            sc = max(1.0, float(w_.abs().max()))
+            torch.testing.assert_close(a_ / sc, w_ / sc, atol=1e-4, rtol=1e-4)
     # the block built with cuda=False goes through it and agrees with the cuda=True block
     torch.manual_seed(3)
     a = blocks.SSMauBlock(blocks.ModelArgsSSMau(d_model=16, d_state=4, cuda=False)).cuda()

@@ -321,3 +321,26 @@ def test_gradcheck_adaptive_preal():
     p = _preal_inputs(1, 2, 2, 4, seed=14)
     leaves = [p[k].clone().requires_grad_(True) for k in ("u", "dt", "x", "B", "C", "D", "z")]
     assert torch.autograd.gradcheck(lambda *a: O.adaptive_preal_loop(*a), leaves, atol=1e-6, rtol=1e-5)
+
+
+def test_polar_with_time_varying_phases_bruteforce():
+    """The cumulative-sum formulation with B, C given as phases (b, n, l) and without the gate (the reference's
+    other branches, ops.py:721-723, :745-746, :759-761) against scalar complex loops: the contraction sees the raw
+    input, the recurrence silu(u), the coefficients are unit-modulus."""
+    g = torch.Generator().manual_seed(21)
+    b, d, n, l = 2, 3, 2, 5
+    r = lambda *s: torch.randn(*s, generator=g, dtype=torch.float64)
+    u, dt, x, xb, Bph, Cph, D = r(b, d, l), r(b, d, l), r(d, n, d), r(d, n), r(b, n, l), r(b, n, l), r(d)
+    y = O.adaptive_unitary_polar(u, dt, x, xb, Bph, Cph, D, None)
+    for ib in range(b):
+        for i in range(d):
+            h = [0j] * n
+            for t in range(l):
+                acc = 0.0
+                us = _silu(float(u[ib, i, t]))
+                for j in range(n):
+                    th = sum(float(x[i, j, q]) * float(u[ib, q, t]) for q in range(d)) + float(xb[i, j])
+                    h[j] = cmath.exp(1j * th) * h[j] + float(dt[ib, i, t]) * us * cmath.exp(1j * float(Bph[ib, j, t]))
+                    acc += (cmath.exp(1j * float(Cph[ib, j, t])) * h[j]).real
+                val = acc + us * float(D[i])
+                assert abs(val - float(y[ib, i, t])) < 1e-10
