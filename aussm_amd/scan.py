@@ -36,16 +36,25 @@ Tensor = torch.Tensor
 # so a long interval is enough; the complex and real backward passes recompute every tile from
 # its checkpoint and need one per tile.
 UNITARY_CK = 256
+# ... and where the launch is not split along L nothing ties the interval to a segment length: measured
+# against the float64 oracle the gradients do not change between an interval of 256 and one checkpoint at
+# the end of 2048 or 8192 steps (the reverse recurrence is norm-preserving), so such a call keeps a
+# checkpoint every UNITARY_CK_LONG steps only
+UNITARY_CK_LONG = 4096
 
 
 def unitary_ck(b: int, d: int, n: int, l: int) -> int:
     """Checkpoint interval of the unitary scan for a shape: UNITARY_CK, or half of it where that
     lets a launch with few (batch, channel) pairs be split into more segments along L (a segment
-    is a whole number of checkpoint blocks)."""
+    is a whole number of checkpoint blocks); calls that are not split at all checkpoint every
+    UNITARY_CK_LONG steps (one checkpoint, at the end, for shorter sequences)."""
     lib = _lib.load()
     half = UNITARY_CK // 2
-    if lib.aussm_unitary_split_segments(b, d, n, l, half) > lib.aussm_unitary_split_segments(b, d, n, l, UNITARY_CK):
+    s_half, s_full = (lib.aussm_unitary_split_segments(b, d, n, l, ck) for ck in (half, UNITARY_CK))
+    if s_half > s_full:
         return half
+    if s_full <= 1:
+        return min(UNITARY_CK_LONG, -(-l // _lib.TILE) * _lib.TILE)
     return UNITARY_CK
 TILE_CK = _lib.TILE
 

@@ -187,9 +187,9 @@ def main():
          "Dskip": rn(D), "dy": rn(B, D, L)}
     Bri = torch.view_as_real(p["Bc"]).contiguous()
     Cri = torch.view_as_real(p["Cc"]).contiguous()
-    ck = scan.UNITARY_CK
+    ck = scan.unitary_ck(B, D, N, L)                       # what the autograd wrapper uses for this shape
 
-    aux = scan.unitary_aux(p["u"], N, scan.UNITARY_CK)      # what the autograd wrapper hands from forward to backward
+    aux = scan.unitary_aux(p["u"], N, ck)                    # what the autograd wrapper hands from forward to backward
 
     def step():
         y, _, hck = scan.unitary_fwd_raw(p["u"], p["delta"], p["theta"], Bri, Cri, p["Dskip"], None, None,
