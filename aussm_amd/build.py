@@ -130,10 +130,12 @@ def build(verbose: bool = True, asm_dir: str | None = None, only=None, extra=())
 def scan_listing(text: str):
     """Findings [(line number, instruction)] of one kernel listing: vector or accumulation registers
     touched while they are the destination of a hand-written (ASMSTART ... ASMEND) global load that no
-    s_waitcnt vmcnt has retired yet.  The scan follows the file order; at a branch back to an earlier
-    label (a loop's back-edge) with loads still in flight it also walks the loop body once more from
-    that label with those loads in flight, so a load issued at the end of an iteration and retired at
-    the top of the next is followed across the edge."""
+    s_waitcnt vmcnt has retired yet.  The scan follows the file order; at a branch back to a loop header
+    (a label the compiler marks "Loop Header") with loads still in flight it also walks the loop body once
+    more from that label with those loads in flight, so a load issued at the end of an iteration and retired
+    at the top of the next is followed across the edge.  (Blocks the compiler places out of line, behind the
+    loop, also branch back to earlier labels; those are not back-edges and the state the file order has
+    there is not the state of their entry, so they are not followed.)"""
     import re
 
     def regs(tok):
@@ -148,8 +150,8 @@ def scan_listing(text: str):
     lines = text.split("\n")
     labels = {}
     for i, line in enumerate(lines):
-        m = re.match(r"^(\.LBB\w+):", line.strip())
-        if m:
+        m = re.match(r"^(\.LBB\w+):(.*)", line.strip())
+        if m and ("Loop Header" in m.group(2) or "Loop Header" not in text):
             labels[m.group(1)] = i
 
     found = []

@@ -342,9 +342,9 @@ __global__ __launch_bounds__(512) void unitary_fwd_px_kernel(const FwdArgs p, co
   f4 Hr = {0, 0, 0, 0}, Hi = {0, 0, 0, 0};           // H_c: lane (dl, g) holds n = 4 g + i of channel dl
   In in;
 
-  // Gather: the loaded inputs of chunk c become masked values and running phases; the same
-  // registers are then refilled with the inputs of chunk cn (clamped).
-  auto gather = [&](int c, int cn, auto kc) {
+  // Gather: the loaded inputs of chunk c become masked values and running phases (the registers are
+  // refilled with the inputs of the chunk after it at the start of the wavefront's next phase A).
+  auto gather = [&](int c, auto kc) {
     in_landed(in, kc);
     float th[2][4];
     bool big = false;
@@ -365,7 +365,6 @@ __global__ __launch_bounds__(512) void unitary_fwd_px_kernel(const FwdArgs p, co
       asm volatile("" : "+v"(un[e]), "+v"(w[e]), "+v"(th[e >> 2][e & 3]));
       if (GATED) asm volatile("" : "+v"(zn[e]));
     }
-    in_load(in, cn);
     // large phases are first reduced to (-pi, pi] so that the running sums stay small enough for
     // sincos_small and for fp32 sums of 32 terms (rare, uniform branch)
     if (__builtin_expect(__any(big), 0)) {
@@ -414,7 +413,7 @@ __global__ __launch_bounds__(512) void unitary_fwd_px_kernel(const FwdArgs p, co
   img_store(1, 0, std::integral_constant<int, 0>{});
   img_load(2, 1);                                   // collected in interval 0
   in_load(in, hf);
-  gather(hf, hf + 2, std::integral_constant<int, 0>{});
+  gather(hf, std::integral_constant<int, 0>{});
   __syncthreads();
 
   const int ck_chunks = p.ck / XT;
@@ -437,10 +436,13 @@ __global__ __launch_bounds__(512) void unitary_fwd_px_kernel(const FwdArgs p, co
   // run on zero input and zero phase: the state passes through unchanged, nothing is stored.
   auto phase_a = [&](int c) {
     const int i = c;
-    // (the phase B before it issued the input loads of its gather after the image loads)
-    img_store(i + 2, i + 1, std::integral_constant<int, N_IN>{});
+    // (nothing of the phase B before it is in flight but its image loads: it collected its inputs at its end)
+    img_store(i + 2, i + 1, std::integral_constant<int, 0>{});
     flush_out();
     img_load(i + 3, i + 2);
+    // the inputs of this wavefront's next chunk: behind the image loads, so that the wait for those at the start
+    // of the next phase can leave them in flight - they are collected at that phase's end, two intervals from here
+    in_load(in, c + 2);
     float vr[8], vi[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
@@ -501,8 +503,9 @@ __global__ __launch_bounds__(512) void unitary_fwd_px_kernel(const FwdArgs p, co
   // ---- phase B of chunk c (interval i = c + 1): S = C.H + G.V, outputs; then the gather of chunk c + 2
   auto phase_b = [&](int c) {
     const int i = c + 1;
-    // (the phase A before it issued nothing after the image loads but, now and then, checkpoint stores)
-    img_store(i + 2, i + 1, std::integral_constant<int, 0>{});
+    // (behind the image loads it collects, the phase A before it issued the input loads and, now and then,
+    // checkpoint stores: a wait that leaves only the input loads in flight is the safe side of both cases)
+    img_store(i + 2, i + 1, std::integral_constant<int, N_IN>{});
     img_load(i + 3, i + 2);
     const u4* sb_ = s_b[c % 3];
     u4 hk[NP];
@@ -558,7 +561,7 @@ __global__ __launch_bounds__(512) void unitary_fwd_px_kernel(const FwdArgs p, co
     }
     out_l0 = c * XT;
     // (younger than the inputs it collects: the image loads of this interval)
-    gather(c + 2, c + 4, std::integral_constant<int, N_IMG>{});
+    gather(c + 2, std::integral_constant<int, N_IMG>{});
     lds_barrier();
   };
   // an interval in which this wavefront has no chunk: it still takes part in the image loads
@@ -570,9 +573,11 @@ __global__ __launch_bounds__(512) void unitary_fwd_px_kernel(const FwdArgs p, co
   };
 
   // Vector-memory operations of a wavefront are issued in this order.  Phase A: the stores of the
-  // previous phase B, then the image loads.  Phase B: the image loads, then (at its end) the input
-  // loads of the gather.  Every load is collected one interval (images) or two (inputs) after it
-  // was issued, by a wait that leaves the known number of younger operations in flight.  The
+  // previous phase B, the image loads, the input loads of the wavefront's next chunk (and, now and then,
+  // checkpoint stores at its end).  Phase B: the image loads.  Every load is collected one interval (images)
+  // or two (inputs) after it was issued, and every wait is for the OLDEST loads in flight: the counter
+  // retires in order, so a wait for a younger load would drain the input loads long before they are needed
+  // (they used to be issued at the end of phase B, in front of the next image loads: 4 % slower).  The
   // loop body is straight-line code on purpose: a join of two paths would make the compiler move
   // live registers, loads in flight included.
   const int npairs = (nchunks + 1) / 2;               // chunks per wavefront (the last may be past the end)
