@@ -250,6 +250,17 @@ __device__ __forceinline__ void sincos_small(float x, float* sn, float* cs) {
   *cs = ((q + 1) & 2) ? -c1 : c1;
 }
 
+// The same through the hardware's sine and cosine (arguments in revolutions): the argument is first reduced
+// to a remainder of at most half a turn in two steps, as above, so what the units see is accurate to a rounding.
+__device__ __forceinline__ void sincos_small_hw(float x, float* sn, float* cs) {
+  const float kf = rintf(x * 0.159154943091895336f);
+  float r = fmaf(-kf, 6.283185482025146484375f, x);
+  r = fmaf(-kf, -1.74845560007449e-7f, r);
+  const float t = r * 0.159154943091895336f;
+  *sn = __builtin_amdgcn_sinf(t);
+  *cs = __builtin_amdgcn_cosf(t);
+}
+
 __device__ __forceinline__ void touch4(const f4& v) { touch_vgpr(v[0]); touch_vgpr(v[1]); touch_vgpr(v[2]); touch_vgpr(v[3]); }
 
 // Sum `v` over the lanes of each aligned group of 32 lanes; result valid in every lane.

@@ -446,7 +446,7 @@ __global__ __launch_bounds__(512) void unitary_fwd_px_kernel(const FwdArgs p, co
     float vr[8], vi[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      sincos_small(ph[e], &sn[e], &cs[e]);
+      sincos_small_hw(ph[e], &sn[e], &cs[e]);
       vr[e] = cs[e] * w[e];
       vi[e] = -sn[e] * w[e];
       uu[e] = un[e];
@@ -796,7 +796,7 @@ __global__ __launch_bounds__(512) void unitary_bwd_px_kernel(const UniBwdArgs p,
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       const float ph = th[e >> 2][e & 3] + ((e >> 2) ? off_b : off_a);
-      sincos_small(ph, &sn[e], &cs[e]);
+      sincos_small_hw(ph, &sn[e], &cs[e]);
       accD = fmaf(dy[e], uu[e], accD);
     }
   };
