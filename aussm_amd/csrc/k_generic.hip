@@ -126,6 +126,77 @@ int run_seg_carry_real(bool adjoint, float* seg, const float* ptot, const float*
   return launch_status();
 }
 
+// ---- what the memory system gives for the scans' access pattern (no arithmetic to speak of): o1 = a + b c,
+// o2 = 2 o1 over [rows, L] tensors.  PATTERN 0: every thread streams consecutive 16-byte pieces (a plain
+// elementwise kernel).  PATTERN 1: what the matrix-core scan kernels do - a workgroup owns 64 rows, its eight
+// wavefronts are four groups of 16 rows times two halves that take the 32-step chunks in turn, and one load or
+// store instruction of a wavefront covers 16 rows x 64 bytes (the two halves of a 128-byte line in two
+// consecutive instructions), loads running two chunks ahead of their use.
+template <int PATTERN, bool WRITE>
+__global__ __launch_bounds__(512) void hbm_probe_kernel(const float* __restrict__ a, const float* __restrict__ b,
+                                                        const float* __restrict__ c, float* __restrict__ o1,
+                                                        float* __restrict__ o2, int rows, int L) {
+  typedef float v4 __attribute__((ext_vector_type(4)));
+  v4 acc = {0, 0, 0, 0};
+  if (PATTERN == 0) {
+    const size_t n4 = (size_t)rows * L / 4;
+    for (size_t i = (size_t)blockIdx.x * 512 + threadIdx.x; i < n4; i += (size_t)gridDim.x * 512) {
+      const v4 x = reinterpret_cast<const v4*>(a)[i] + reinterpret_cast<const v4*>(b)[i] * reinterpret_cast<const v4*>(c)[i];
+      if (WRITE) { reinterpret_cast<v4*>(o1)[i] = x; reinterpret_cast<v4*>(o2)[i] = x + x; } else acc += x;
+    }
+  } else {
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, cg = w & 3, hf = w >> 2;
+    const int dl = lane & 15, g = lane >> 4;
+    const size_t row = (size_t)blockIdx.x * 64 + cg * 16 + dl;
+    const int nch = L / 64;                       // chunks of this half (L is a multiple of 64)
+    auto at = [&](int u, int st) -> size_t { return row * L + (size_t)(2 * u + hf) * 32 + 16 * st + 4 * g; };
+    v4 buf[2][2][3];
+#pragma unroll
+    for (int q = 0; q < 2; ++q)
+#pragma unroll
+      for (int st = 0; st < 2; ++st) {
+        const size_t o = at(q < nch ? q : nch - 1, st);
+        buf[q][st][0] = *reinterpret_cast<const v4*>(a + o);
+        buf[q][st][1] = *reinterpret_cast<const v4*>(b + o);
+        buf[q][st][2] = *reinterpret_cast<const v4*>(c + o);
+      }
+    for (int u = 0; u < nch; u += 2) {
+#pragma unroll
+      for (int q = 0; q < 2; ++q) {
+        if (u + q >= nch) break;
+#pragma unroll
+        for (int st = 0; st < 2; ++st) {
+          const v4 x = buf[q][st][0] + buf[q][st][1] * buf[q][st][2];
+          const size_t o = at(u + q, st);
+          if (WRITE) { *reinterpret_cast<v4*>(o1 + o) = x; *reinterpret_cast<v4*>(o2 + o) = x + x; } else acc += x;
+        }
+        const int un = u + q + 2 < nch ? u + q + 2 : u + q;
+#pragma unroll
+        for (int st = 0; st < 2; ++st) {
+          const size_t o = at(un, st);
+          buf[q][st][0] = *reinterpret_cast<const v4*>(a + o);
+          buf[q][st][1] = *reinterpret_cast<const v4*>(b + o);
+          buf[q][st][2] = *reinterpret_cast<const v4*>(c + o);
+        }
+      }
+    }
+  }
+  // (keeps the loads of the read-only form alive; never true for finite data)
+  if (!WRITE && acc[0] + acc[1] + acc[2] + acc[3] == 1.2345678e38f) o1[0] = acc[0];
+}
+int run_hbm_probe(const float* a, const float* b, const float* c, float* o1, float* o2, int rows, int L, int pattern,
+                  int write, hipStream_t s) {
+  if (pattern == 0) {
+    if (write) hipLaunchKernelGGL((hbm_probe_kernel<0, true>), dim3(2048), dim3(512), 0, s, a, b, c, o1, o2, rows, L);
+    else hipLaunchKernelGGL((hbm_probe_kernel<0, false>), dim3(2048), dim3(512), 0, s, a, b, c, o1, o2, rows, L);
+  } else {
+    const dim3 grid((unsigned)(rows / 64));
+    if (write) hipLaunchKernelGGL((hbm_probe_kernel<1, true>), grid, dim3(512), 0, s, a, b, c, o1, o2, rows, L);
+    else hipLaunchKernelGGL((hbm_probe_kernel<1, false>), grid, dim3(512), 0, s, a, b, c, o1, o2, rows, L);
+  }
+  return launch_status();
+}
+
 // marks an auxiliary buffer as NOT filled (a forward kernel that does not fill it ran) and / or the
 // operand images behind it as not belonging to the call's tensors
 __global__ void aux_invalidate_kernel(float* tag, int first, int last) {

@@ -6,8 +6,13 @@ namespace aussm {
 
 int run_px_prep(const PrepArgs& a, int B, int in_dtype, hipStream_t s) {
   const dim3 grid((unsigned)(B * a.nch));
-  if (in_dtype == 1) hipLaunchKernelGGL(unitary_px_prep_kernel<bf16_t>, grid, dim3(256), 0, s, a);
-  else hipLaunchKernelGGL(unitary_px_prep_kernel<float>, grid, dim3(256), 0, s, a);
+  if (a.have) {
+    if (in_dtype == 1) hipLaunchKernelGGL((unitary_px_prep_kernel<bf16_t, true>), grid, dim3(256), 0, s, a);
+    else hipLaunchKernelGGL((unitary_px_prep_kernel<float, true>), grid, dim3(256), 0, s, a);
+  } else {
+    if (in_dtype == 1) hipLaunchKernelGGL((unitary_px_prep_kernel<bf16_t, false>), grid, dim3(256), 0, s, a);
+    else hipLaunchKernelGGL((unitary_px_prep_kernel<float, false>), grid, dim3(256), 0, s, a);
+  }
   return launch_status();
 }
 

@@ -29,6 +29,8 @@ int run_adjoint_seg(int variant, const AdjSegArgs& a, int in_dtype, unsigned gri
 int run_bc_to_f32(const void* Bm, const void* Cm, float* oB, float* oC, size_t n, hipStream_t s);   // bf16 -> float
 int run_seg_carry_real(bool adjoint, float* seg, const float* ptot, const float* A, const float* first, float* last,
                         int B, int D, int N, int ns, hipStream_t s);
+int run_hbm_probe(const float* a, const float* b, const float* c, float* o1, float* o2, int rows, int L, int pattern,
+                  int write, hipStream_t s);
 int run_conv_fwd(const ConvArgs& a, hipStream_t s);
 int run_conv_bwd(const ConvArgs& a, hipStream_t s);
 int run_swap_last2(const SwapArgs& a, int B, hipStream_t s);

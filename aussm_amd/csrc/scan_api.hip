@@ -361,6 +361,15 @@ int aussm_unitary_kernel_mode(int backward, int B, int D, int N, int L, int ck, 
   return backward ? bwd_mode_for(B, D, N, L, ck, urep, have_img) : fwd_mode_for(N, L, ck, in_dtype, urep, have_img);
 }
 
+int aussm_hbm_probe(const float* a, const float* b, const float* c, float* o1, float* o2, int rows, int L,
+                    int pattern, int write, void* stream) {
+  if (rows < 64 || rows % 64 != 0 || L < 64 || L % 64 != 0 || (pattern != 0 && pattern != 1)) return AUSSM_E_SHAPE;
+  if (!a || !b || !c || !o1 || (write && !o2)) return AUSSM_E_NULL;
+  if (misaligned(a, 16) || misaligned(b, 16) || misaligned(c, 16) || misaligned(o1, 16) || misaligned(o2, 16))
+    return AUSSM_E_ALIGN;
+  return run_hbm_probe(a, b, c, o1, o2, rows, L, pattern, write, (hipStream_t)stream);
+}
+
 int aussm_unitary_fwd(const void* u, const void* delta, const float* theta, const void* Bc, const void* Cc,
                       const float* Dskip, const float* z, const float* h0, float* y, float* hL, float* hck,
                       int B, int D, int N, int L, int ck, int in_dtype, void* stream) {

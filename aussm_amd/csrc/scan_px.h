@@ -28,15 +28,17 @@
 
 namespace aussm {
 
-// One workgroup (256 threads) per (batch element, chunk).
-template <typename Tin>
+// One workgroup (256 threads) per (batch element, chunk).  CHECK: the launch of a backward call, which has
+// nothing to do when the forward call of the same tensors has left the images (its own instance, so that a
+// profile tells the two launches of a training step apart).
+template <typename Tin, bool CHECK>
 __global__ __launch_bounds__(256) void unitary_px_prep_kernel(const PrepArgs p) {
   constexpr int NP = PX_NP;
   __shared__ XbBC<NP> s_bc;
   __shared__ XbG<NP> s_g;
 
   // the images a forward call left behind are still those of these tensors: nothing to do
-  if (p.have) {
+  if (CHECK && p.have) {
     bool same = true;
 #pragma unroll
     for (int i = 0; i < 8; ++i) same &= __builtin_amdgcn_readfirstlane(p.have[i]) == p.want.w[i];

@@ -162,10 +162,13 @@ def unitary_bwd_raw(dy, dhL, u, delta, theta, Bri, Cri, D, hck, ck, want_dD=True
     n = Bri.shape[1]
     f32 = dict(device=u.device, dtype=torch.float32)
     du, ddelta, dtheta = (torch.empty((b, d, l), **f32) for _ in range(3))
-    # accumulated into with atomics by the kernel: start from zero
-    dB = torch.zeros((b, n, l, 2), **f32)
-    dC = torch.zeros((b, n, l, 2), **f32)
-    dD = torch.zeros((d,), **f32) if (want_dD and D is not None) else None
+    # accumulated into with atomics by the kernel: start from zero (one allocation, one fill launch; the pad keeps
+    # every view 16-byte aligned)
+    nbc = b * n * l * 2
+    pad = (nbc + 3) // 4 * 4
+    acc = torch.zeros((2 * pad + d,), **f32)
+    dB, dC = acc[:nbc].view(b, n, l, 2), acc[pad:pad + nbc].view(b, n, l, 2)
+    dD = acc[2 * pad:2 * pad + d] if (want_dD and D is not None) else None
     dh0 = torch.empty((b, d, n, 2), **f32) if want_dh0 else None
     check(lib.aussm_unitary_bwd_aux(ptr(dy), ptr(dhL), ptr(u), ptr(delta), ptr(theta), ptr(Bri), ptr(Cri), ptr(D),
                                     ptr(hck), ptr(aux), ptr(du), ptr(ddelta), ptr(dtheta), ptr(dB), ptr(dC), ptr(dD),

@@ -14,8 +14,9 @@ resident in HBM.  Prints ONE JSON line.
   value          (b,d,l) samples per second over forward+backward (B*D*L / step time)
   roofline       dominant kernel (the backward scan): algorithmic bytes (28E + 32S + 4D,
                  E = B*D*L, S = B*N*L) / the average duration of one backward call (the scan kernel
-                 and, for the prepared-operand kernel, its light operand pre-pass), measured here
-                 with HIP events on the launch stream, against the 8 TB/s HBM peak.  "traffic" is
+                 and the two launches around it that leave at once in a training step), measured here
+                 with HIP events on the launch stream, against the 8 TB/s HBM peak.  The operand
+                 pre-pass of the step runs inside the forward call, whose figures carry it.  "traffic" is
                  the HBM bytes per call from rocprofv3 FETCH_SIZE / WRITE_SIZE passes over this same
                  script, scaled by what the counters read for the 256 MiB device copy that
                  --copy-probe adds to the run.  It is read from profiles/traffic.json, which
@@ -45,11 +46,13 @@ HBM_PEAK_GBS = 8000.0
 SHAPE = dict(B=32, D=512, N=16, L=2048)
 TRAFFIC_JSON = os.path.join(ROOT, "profiles", "traffic.json")
 # kernels of one call, by the kernel family the library reports (aussm_unitary_kernel_mode)
+# (family 6: the forward call's pre-pass prepares the operands of both directions; the backward call's instance of
+# it - <float, true> - finds them and leaves at once, as does the recomputing kernel launched behind the scan kernel)
 FWD_KERNELS = {0: ["core_fwd_kernel<0"], 2: ["unitary_fwd_xdl_kernel<2"], 3: ["unitary_fwd_xdl_kernel<3"],
-               6: ["unitary_px_prep_kernel", "unitary_fwd_px_kernel"]}
+               6: ["unitary_px_prep_kernel<float, false", "unitary_fwd_px_kernel"]}
 BWD_KERNELS = {0: ["unitary_bwd_kernel"], 2: ["unitary_bwd_xdl_kernel<2"], 3: ["unitary_bwd_xdl_kernel<3, 2"],
                5: ["unitary_bwd_xdl_kernel<3, 3"],
-               6: ["unitary_px_prep_kernel", "unitary_bwd_px_kernel", "unitary_bwd_xdl_kernel<3, 2"]}
+               6: ["unitary_bwd_px_kernel", "unitary_px_prep_kernel<float, true", "unitary_bwd_xdl_kernel<3, 2"]}
 
 
 def source_digest() -> str:
@@ -144,6 +147,44 @@ def cpu_baseline(B_sample: int):
     }
 
 
+def hbm_probe(rows: int, L: int, dev) -> None:
+    """Rates of aussm_hbm_probe over [rows, L] float tensors: three read and two written (the mix of a scan call), and
+    read only, for a plain streaming kernel and for the scan kernels' pattern.  HIP events, median of 15 launches
+    after 300 ms of load."""
+    import torch
+    from aussm_amd import scan
+    lib = scan._lib.load()
+    ptr, stream = scan.ptr, scan._stream()
+    a, b, c = (torch.randn(rows, L, device=dev) for _ in range(3))
+    o1, o2 = torch.empty_like(a), torch.empty_like(a)
+
+    def launch(pattern, write):
+        scan.check(lib.aussm_hbm_probe(ptr(a), ptr(b), ptr(c), ptr(o1), ptr(o2), rows, L, pattern, write, stream), "probe")
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < 0.3:
+        launch(0, 1)
+        torch.cuda.synchronize()
+    out = {"probe": "o1 = a + b c, o2 = 2 o1 over [rows, L] float tensors", "rows": rows, "L": L, "unit": "GB/s",
+           "hbm_peak": HBM_PEAK_GBS}
+    for pattern, pname in ((0, "stream"), (1, "scan_pattern")):
+        for write, wname in ((1, "3_read_2_written"), (0, "3_read")):
+            ts = []
+            for _ in range(15):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                launch(pattern, write)
+                e1.record()
+                torch.cuda.synchronize()
+                ts.append(e0.elapsed_time(e1) * 1e-3)
+            nbytes = (5 if write else 3) * rows * L * 4
+            out[f"{pname}_{wname}"] = round(nbytes / sorted(ts)[7] / 1e9, 1)
+    launch(1, 1)
+    torch.cuda.synchronize()
+    want = a.double() + b.double() * c.double()          # (the kernel fuses the multiply and the add)
+    assert (o1.double() - want).abs().max() < 1e-5 and (o2.double() - 2 * want).abs().max() < 2e-5, "probe kernel wrote something else"
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -157,6 +198,9 @@ def main():
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one 256 MiB device-to-device copy (calibrates FETCH_SIZE / WRITE_SIZE under rocprofv3)")
     ap.add_argument("--shape", default=None, help="B,D,N,L instead of the headline shape (no recorded traffic figure then)")
+    ap.add_argument("--hbm-probe", action="store_true",
+                    help="instead of the benchmark: what the memory system delivers for a plain streaming kernel and for "
+                         "the scan kernels' access pattern at this shape (aussm_hbm_probe), one JSON line")
     args = ap.parse_args()
     headline = args.shape is None
     if not headline:
@@ -177,6 +221,9 @@ def main():
     B, D, N, L = SHAPE["B"], SHAPE["D"], SHAPE["N"], SHAPE["L"]
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.hbm_probe:
+        hbm_probe(B * D, L, dev)
+        return
     # synthetic inputs with the benchmark contract's value distributions, generated on the device (the CPU oracle is only
     # used by the cpu_baseline leg): u ~ N(0,1), delta = softplus(N(0,1)), theta ~ N(0, 0.5), B_t and C_t complex
     # with parts ~ N(0, 1/sqrt(N)), D ~ N(0,1), dy ~ N(0,1)
@@ -281,7 +328,7 @@ def main():
         "fwd_bwd_algorithmic_GBps": (bytes_fwd + bytes_bwd) / ((t_fwd + t_bwd) * 1e-6) / 1e9,
         "fwd_bwd_frac_of_hbm_peak": (bytes_fwd + bytes_bwd) / ((t_fwd + t_bwd) * 1e-6) / 1e9 / HBM_PEAK_GBS,
         "kernels_us": {"unitary_fwd": t_fwd, "unitary_bwd": t_bwd},
-        "roofline": {"bound": "hbm", "kernel": " + ".join(BWD_KERNELS[bmode][:2 if bmode == 6 else 1]) + " (one backward call)",
+        "roofline": {"bound": "hbm", "kernel": BWD_KERNELS[bmode][0] + " (one backward call)",
                      "achieved": ach, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": ach / HBM_PEAK_GBS, "traffic": traffic_bwd, "traffic_source": note_bwd,
                      "algorithmic_bytes": bytes_bwd,

@@ -350,6 +350,19 @@ int aussm_ssm_adaptive_unitary_bwd(const float* grad_y, const float* grad_nh_re,
                                    float* dC_r, float* dC_theta, float* dD, float* dz, float* dh_re, float* dh_im,
                                    float* workspace, int b, int d, int n, int L, void* stream);
 
+/* ---------------------------------------------------------------------------------------
+ * Measurement aid: what the memory system delivers for the scan kernels' access pattern, with
+ * next to no arithmetic: o1 = a + b * c and o2 = 2 * o1 over [rows, L] float tensors (three
+ * tensors read, two written when write != 0; read only, nothing but o1[0] possibly written,
+ * when write == 0).  pattern 0: a plain streaming elementwise kernel; pattern 1: the matrix-core
+ * scans' pattern (a workgroup owns 64 rows and walks them in 32-step chunks; one load or store
+ * instruction of a wavefront covers 16 rows x 64 bytes; loads two chunks ahead).  rows and L are
+ * multiples of 64.  `bench.py --hbm-probe` times both at the headline shape; the rates bound what
+ * a scan kernel with this layout of work can reach.  No counterpart in the reference.
+ * ------------------------------------------------------------------------------------- */
+int aussm_hbm_probe(const float* a, const float* b, const float* c, float* o1, float* o2, int rows, int L,
+                    int pattern, int write, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

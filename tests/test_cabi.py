@@ -129,3 +129,24 @@ def test_python_layer_fails_loudly_without_library(monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "missing.so"))
     with pytest.raises(_lib.AussmError):
         _lib.load()
+
+
+@pytest.mark.gpu
+def test_hbm_probe_computes_what_it_says():
+    """The measurement aid of `bench.py --hbm-probe`: both access patterns write o1 = a + b c and o2 = 2 o1."""
+    import torch
+    from aussm_amd import _lib, scan
+    lib = _lib.load()
+    rows, L = 128, 192
+    a, b, c = (torch.randn(rows, L, device="cuda") for _ in range(3))
+    want = a.double() + b.double() * c.double()
+    for pattern in (0, 1):
+        o1, o2 = torch.zeros_like(a), torch.zeros_like(a)
+        print(f"case hbm probe pattern {pattern}", flush=True)
+        _lib.check(lib.aussm_hbm_probe(_lib.ptr(a), _lib.ptr(b), _lib.ptr(c), _lib.ptr(o1), _lib.ptr(o2), rows, L, pattern, 1,
+                                       scan._stream()), "aussm_hbm_probe")
+        torch.cuda.synchronize()
+        torch.testing.assert_close(o1.double(), want, atol=1e-5, rtol=1e-5)
+        torch.testing.assert_close(o2.double(), 2 * want, atol=2e-5, rtol=1e-5)
+    one = ctypes.c_void_p(256)
+    assert lib.aussm_hbm_probe(one, one, one, one, one, 100, 192, 0, 1, None) == -2      # rows not a multiple of 64
