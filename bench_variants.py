@@ -37,6 +37,7 @@ from __future__ import annotations
 
 import argparse
 import json
+import time
 import os
 import sys
 
@@ -136,6 +137,56 @@ def scaling(args):
                 torch.cuda.empty_cache()
 
 
+def fused_operator(args):
+    """Forward and backward operator calls at one shape, HIP events, with the roofline that bounds them: the phase
+    projection theta[b,i,j,l] = x[i,j,:] . u[b,:,l] and, backward, the two products with the phase adjoints
+    (grad_x, grad_u) are matrix work, 2 b d^2 n L flops each in fp32 terms; the kernels run every product as six
+    bf16 products on exactly split operands, so the fp32-equivalent rate is held against the fp32 matrix peak and the
+    bf16 rate (six times the flops) against the bf16 one."""
+    import torch
+    import aussm_amd.ops  # noqa: F401
+    b, d, n, L = (int(v) for v in args.fused.split(","))
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev).manual_seed(0)
+    rn = lambda *s: torch.randn(*s, generator=g, device=dev)
+    sp = torch.nn.functional.softplus
+    t = [rn(b, d, L), sp(rn(b, d, L)), rn(d, n, d) * d ** -0.5, rn(d, n), sp(rn(n)), rn(n), sp(rn(n)), rn(n), rn(d),
+         rn(b, d, L), rn(b, d, n), rn(b, d, n)]
+    grads = [rn(b, d, L), rn(b, d, n), rn(b, d, n)]
+    fwd = lambda: torch.ops.extension_cpp.ssm_adaptive_unitary(*t)
+    nh = list(fwd()[1:])
+    bwd = lambda: torch.ops.aussm_amd.ssm_adaptive_backward_unitary_from_state(*grads, *t, *nh)
+
+    def timed(fn):
+        t0 = time.perf_counter()
+        while time.perf_counter() - t0 < 0.2:
+            fn()
+            torch.cuda.synchronize()
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.reps)]
+        for s_, e_ in evs:
+            s_.record()
+            fn()
+            e_.record()
+        torch.cuda.synchronize()
+        return sum(s_.elapsed_time(e_) for s_, e_ in evs) / args.reps * 1e3
+    t_f, t_b = timed(fwd), timed(bwd)
+    unit = 2.0 * b * d * d * n * L
+
+    def roof(flops, us):
+        tf = flops / us / 1e6
+        return {"bound": "mfma", "achieved": round(tf, 1), "peak": 157.3, "unit": "TFLOP/s (fp32-equivalent)",
+                "frac": round(tf / 157.3, 4), "flops": flops,
+                "as_bf16_products": {"achieved": round(6 * tf, 1), "peak": 2500.0, "unit": "TFLOP/s", "frac": round(6 * tf / 2500.0, 4)}}
+    E = b * d * L
+    print(json.dumps({
+        "operator": "extension_cpp::ssm_adaptive_unitary (fused kernels)", "shape": {"b": b, "d": d, "n": n, "L": L},
+        "fwd_us": round(t_f, 1), "bwd_us": round(t_b, 1), "bwd_over_fwd": round(t_b / t_f, 2),
+        "roofline_fwd": roof(unit, t_f), "roofline_bwd": roof(3 * unit, t_b),
+        "algorithmic_bytes": {"fwd": 16 * E + 4 * d * n * d, "bwd": 32 * E + 8 * d * n * d},
+        "note": "backward flops: the phase projection again (the operator recomputes from its inputs) and the two products "
+                "with the phase adjoints; durations include output allocation and the workspace"}), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--reps", type=int, default=30)
@@ -148,6 +199,9 @@ def main():
     ap.add_argument("--bdn", action="append", help="b,d,n of the sweep (repeatable)")
     ap.add_argument("--lengths", default=None, help="comma-separated sequence lengths of the sweep")
     ap.add_argument("--systems", default="SSMau-hip,SSMau-hip-composite,mamba-hip")
+    ap.add_argument("--fused", default=None, metavar="b,d,n,L", nargs="?", const="32,256,16,720",
+                    help="time the fused operator (extension_cpp::ssm_adaptive_unitary and its backward operator) at a shape, "
+                         "default BASELINE configuration 4's, with its matrix-pipe roofline")
     args = ap.parse_args()
     B, D, N, L = (int(v) for v in args.shape.split(","))
 
@@ -161,6 +215,9 @@ def main():
     torch.cuda.set_device(dev)
     if args.scaling:
         scaling(args)
+        return
+    if args.fused:
+        fused_operator(args)
         return
 
     def timed(fn):
@@ -212,7 +269,7 @@ def main():
                 Bri = torch.view_as_real(p["Bc"]).to(dt).contiguous()
                 Cri = torch.view_as_real(p["Cc"]).to(dt).contiguous()
                 if variant == "unitary":
-                    ck = scan.UNITARY_CK
+                    ck = scan.unitary_ck(B, D, N, L)
                     aux = scan.unitary_aux(u, N, ck)
 
                     def fwd():
