@@ -85,7 +85,15 @@ static int rec_bwd_t(const RecBwdArgs& args, hipStream_t s) {
     const int left = args.N - nbase;
     const int nw = left <= 4 ? 1 : (left <= 8 ? 2 : 4);
     bool done = false;
-    AUSSM_RBWD_CASE(1) AUSSM_RBWD_CASE(2) AUSSM_RBWD_CASE(4)
+#ifndef AUSSM_REC_NARROW
+    // a full block of 16 states: eight wavefronts of two states, two wavefronts per SIMD (the gated complex scan
+    // needs a fourth partial sum per wavefront, which only fits with four wavefronts)
+    if (left > 8 && !(VAR == VAR_COMPLEX && a.z)) {
+      hipLaunchKernelGGL((recompute_bwd_kernel<VAR, 2, 512, Tin, float>), grid, dim3(512), 0, s, a);
+      done = true;
+    }
+#endif
+    if (!done) { AUSSM_RBWD_CASE(1) AUSSM_RBWD_CASE(2) AUSSM_RBWD_CASE(4) }
     if (!done) return -2;
     if (int e = launch_status()) return e;
   }

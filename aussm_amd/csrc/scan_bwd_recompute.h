@@ -67,6 +67,41 @@ __device__ __forceinline__ f32x8 ld_r8_tile(const Tin* p, size_t row, int t0, in
   else return ld_r8_safe(p, row, t0, L);
 }
 
+// Column sums of 16 products per lane (the workgroups of eight wavefronts: half the scratch per wavefront).
+// Lane (c = lane % 16, q = lane / 16) reads column c of the rows 16 (i / 4) + 4 q + i % 4, i = 0 .. 15: with a
+// row stride of 20 floats the two q of a 32-lane half are 16 banks apart, and the 16-byte row writes of
+// eight neighbouring lanes cover all banks.  finish() leaves the column's total in all four lanes.
+constexpr int RED16_RS = 20;
+struct LaneTranspose16 {
+  float v[16];
+  __device__ __forceinline__ void issue(const float (&vals)[16], float* red, int lane) {
+    float4* row = reinterpret_cast<float4*>(red + lane * RED16_RS);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) row[j] = make_float4(vals[4 * j], vals[4 * j + 1], vals[4 * j + 2], vals[4 * j + 3]);
+    __builtin_amdgcn_wave_barrier();
+    const float* colp = red + (4 * (lane >> 4)) * RED16_RS + (lane & 15);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) v[i] = colp[(16 * (i >> 2) + (i & 3)) * RED16_RS];
+    sched_fence();
+  }
+  __device__ __forceinline__ float finish() {
+#pragma unroll
+    for (int s = 8; s >= 1; s >>= 1)
+#pragma unroll
+      for (int i = 0; i < s; ++i) v[i] += v[i + s];
+    float t = v[0];
+    t += __shfl_xor(t, 16, 64);
+    t += __shfl_xor(t, 32, 64);
+    return t;
+  }
+};
+
+// Workgroups of four wavefronts (NT = 256) keep one slab of per-(timestep, channel) partial sums per
+// wavefront and reduce 32 products per lane transpose.  Workgroups of eight wavefronts (NT = 512, two
+// wavefronts per SIMD) fit with three planes of floats per wavefront instead of four-float records - complex:
+// (dw, dtheta, drho), real: (dw, ddelta, y_pre), so the gated complex scan stays with four wavefronts - and with
+// transposes of 16 products at a time.  (Adding the partial sums of two wavefronts into one slab with LDS float
+// atomics instead made the kernel 2.5 times slower: those run far below the rate of plain LDS writes.)
 template <int VAR, int NW, int NT, typename Tin, typename Tbc = Tin>
 __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
   static_assert(VAR == VAR_COMPLEX || VAR == VAR_REAL, "unitary has its own kernel");
@@ -77,12 +112,18 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
   constexpr int NGRP = RT / TG;
   // rows reduced per lane transpose: a complex row fills the 32 columns, two real rows do
   constexpr int RPT = (VAR == VAR_REAL && NW % 2 == 0) ? 2 : 1;
-  constexpr int NRES = NGRP * NW / RPT;
+  constexpr bool WIDE = NWV > 4;
+  // real scan, two states per wavefront: the decay factors of the recomputed tile stay in registers for the
+  // walk back (the exponential is a quarter-rate instruction; with more states per wavefront the registers are taken)
+  constexpr bool KEEP_A = VAR == VAR_REAL && NW <= 2;
+  constexpr int NRES = WIDE ? NGRP * NW * C : NGRP * NW / RPT;
+  constexpr int PLANE = RT * TS;                           // floats of one plane of a slab
   static_assert(E >= 1, "tile too small for this workgroup size");
 
   __shared__ float4 s_in[RT * TS];                         // complex (Re a, Im a, w, dy); real (delta, w, dy, -)
-  __shared__ float4 s_part[NWV * RT * TS];                 // per wavefront partial (dw, dtheta|ddelta, drho, -)
-  __shared__ __align__(16) float s_red[NWV * 64 * RED_RS]; // lane-transpose scratch
+  __shared__ float4 s_part[WIDE ? 1 : NWV * RT * TS];      // per wavefront partial (dw, dtheta|ddelta, drho, y_pre)
+  __shared__ float s_slab[WIDE ? NWV * 3 * PLANE : 1];     // WIDE: per wavefront, three of those sums as planes
+  __shared__ __align__(16) float s_red[NWV * 64 * (WIDE ? RED16_RS : RED_RS)]; // lane-transpose scratch
 
   const int tid = threadIdx.x, lane = tid & 63, wave = wave_index();
   const int wg = xcd_remap(blockIdx.x, gridDim.x);
@@ -103,8 +144,9 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
   const Tin* __restrict__ gdl = static_cast<const Tin*>(p.delta);
   const Tbc* __restrict__ gB = static_cast<const Tbc*>(p.Bm);
   const Tbc* __restrict__ gC = static_cast<const Tbc*>(p.Cm);
-  float* red = s_red + wave * 64 * RED_RS;
-  float4* part = s_part + wave * RT * TS;
+  float* red = s_red + wave * 64 * (WIDE ? RED16_RS : RED_RS);
+  float4* part = s_part + (WIDE ? 0 : wave * RT * TS);
+  float* slab = s_slab + (WIDE ? wave * 3 * PLANE : 0);
   const size_t row_base = ((size_t)b * N + n0) * ld + lbeg;
 
   // ---- per-lane constants and accumulators
@@ -258,6 +300,7 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
                 const float a = __builtin_amdgcn_exp2f(rx[t] * a2[k]);
                 cr_[k] = fmaf(a, cr_[k], bc[t] * ry[t]);
                 hsr[g * TG + t][k] = cr_[k];
+                if constexpr (KEEP_A) hsi[g * TG + t][k] = a;        // (the real scan has no imaginary parts to keep there)
               }
             } else {
               const f32x16 bc = ld_c8_tile<FULL>(gB, brow + (size_t)k * ld - l0, l0 + g * TG, L);
@@ -288,6 +331,8 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
         float kacc[TG], xacc[TG], zacc[TG], yacc[TG];
 #pragma unroll
         for (int t = 0; t < TG; ++t) { kacc[t] = 0.f; xacc[t] = 0.f; zacc[t] = 0.f; yacc[t] = 0.f; }
+        // products for the channel sums: [dB | dC] of TG steps; the narrow workgroups gather a complex row's 32
+        // (or two real rows' 2 x 16) per transpose, the wide ones 16 at a time (vals, then vals + 16)
         float vals[RED_COLS];
 #pragma unroll
         for (int j = 0; j < RED_COLS; ++j) vals[j] = 0.f;
@@ -297,14 +342,12 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
             if constexpr (VAR == VAR_REAL) {
               const f32x8 bc = ld_r8_tile<FULL>(gB, brow + (size_t)k * ld - l0, l0 + g * TG, L);
               const f32x8 cc = ld_r8_tile<FULL>(gC, brow + (size_t)k * ld - l0, l0 + g * TG, L);
-              constexpr int VB = 0;                // filled below per row slot
-              (void)VB;
-              const int slot = (RPT == 2) ? (k & 1) : 0;
+              const int slot = (!WIDE && RPT == 2) ? (k & 1) : 0;
 #pragma unroll
               for (int t = TG - 1; t >= 0; --t) {
                 const int tt = g * TG + t;
                 const float dlt = r0[t], w = r1[t], gy = r2[t];
-                const float a = __builtin_amdgcn_exp2f(dlt * a2[k]);
+                const float a = KEEP_A ? hsi[tt][k] : __builtin_amdgcn_exp2f(dlt * a2[k]);
                 gr[k] = fmaf(cc[t], gy, gr[k]);
                 vals[slot * 16 + t] = w * gr[k];
                 vals[slot * 16 + 8 + t] = gy * hsr[tt][k];
@@ -346,7 +389,19 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
             }
           }
           // channel reduction of this turn's (or row pair's) dB/dC products
-          if ((k % RPT) == RPT - 1) {
+          if constexpr (WIDE) {
+            float half[16];
+#pragma unroll
+            for (int h = 0; h < C; ++h) {
+#pragma unroll
+              for (int j = 0; j < 16; ++j) half[j] = vals[16 * h + j];
+              LaneTranspose16 xs;
+              xs.issue(half, red, lane);
+              rres[(g * NW + k) * C + h] = xs.finish();
+            }
+#pragma unroll
+            for (int j = 0; j < RED_COLS; ++j) vals[j] = 0.f;
+          } else if ((k % RPT) == RPT - 1) {
             LaneTranspose xs;
             xs.issue(vals, red, lane);
             rres[g * (NW / RPT) + k / RPT] = xs.finish();
@@ -354,8 +409,18 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
             for (int j = 0; j < RED_COLS; ++j) vals[j] = 0.f;
           }
         }
+        if constexpr (WIDE) {
 #pragma unroll
-        for (int t = 0; t < TG; ++t) part[(g * TG + t) * TS + lane] = make_float4(kacc[t], xacc[t], zacc[t], yacc[t]);
+          for (int t = 0; t < TG; ++t) {
+            float* q = slab + (g * TG + t) * TS + lane;
+            q[0] = kacc[t];
+            q[PLANE] = xacc[t];
+            q[2 * PLANE] = (VAR == VAR_COMPLEX) ? zacc[t] : yacc[t];
+          }
+        } else {
+#pragma unroll
+          for (int t = 0; t < TG; ++t) part[(g * TG + t) * TS + lane] = make_float4(kacc[t], xacc[t], zacc[t], yacc[t]);
+        }
       }
         };
     if (active) {
@@ -375,7 +440,26 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
     if (it > 1) load_start(st_fly, it - 2);
     sched_fence();
     if (active) {
-      const size_t brow = row_base + l0;
+      if constexpr (WIDE) {
+        // lanes 0 .. 15 hold the 16 columns: complex (dB | dC of a row: 8 steps x (re, im)), real (8 dB, 8 dC)
+        const int c = lane & 15;
+#pragma unroll
+        for (int g = 0; g < NGRP; ++g)
+#pragma unroll
+          for (int k = 0; k < NW; ++k)
+#pragma unroll
+            for (int h = 0; h < C; ++h) {
+              const int t = l0 + g * TG;
+              const float v = rres[(g * NW + k) * C + h];
+              if (VAR == VAR_REAL) {
+                float* dst = (c >> 3) ? p.dC : p.dB;
+                if (lane < 16 && n0 + k < N && t + (c & 7) < L) atomicAdd(dst + row_base + (size_t)k * ld + t + (c & 7), v);
+              } else {
+                float* dst = h ? p.dC : p.dB;
+                if (lane < 16 && n0 + k < N && t + (c >> 1) < L) atomicAdd(dst + 2 * (row_base + (size_t)k * ld + t) + c, v);
+              }
+            }
+      } else {
 #pragma unroll
       for (int g = 0; g < NGRP; ++g)
 #pragma unroll
@@ -398,23 +482,31 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
               atomicAdd(dst + 2 * (row_base + (size_t)k * ld + t) + (c & 15), rres[g * (NW / RPT) + j]);
           }
         }
-      (void)brow;
+      }
     }
 
     // ---- epilogue: channel-wise gradients, coalesced along time
-    float4 pv[E][NWV];
+    constexpr int NSLAB = NWV;
+    float4 pv[E][NSLAB];
 #pragma unroll
     for (int k = 0; k < E; ++k)
 #pragma unroll
-      for (int w = 0; w < NWV; ++w)
-        pv[k][w] = (w < nwa) ? s_part[(w * RT + col) * TS + row0 + k * RSTEP] : make_float4(0.f, 0.f, 0.f, 0.f);
+      for (int w = 0; w < NSLAB; ++w) {
+        if constexpr (WIDE) {
+          const float* q = s_slab + w * 3 * PLANE + col * TS + row0 + k * RSTEP;
+          pv[k][w] = (w < nwa) ? make_float4(q[0], q[PLANE], VAR == VAR_COMPLEX ? q[2 * PLANE] : 0.f, VAR == VAR_COMPLEX ? 0.f : q[2 * PLANE])
+                               : make_float4(0.f, 0.f, 0.f, 0.f);
+        } else {
+          pv[k][w] = (w < nwa) ? s_part[(w * RT + col) * TS + row0 + k * RSTEP] : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+      }
     sched_fence();
 #pragma unroll
     for (int k = 0; k < E; ++k) {
       const int ll = l0 + col;
       float kk = 0.f, xx = 0.f, zz = 0.f, yy = 0.f;
 #pragma unroll
-      for (int w = 0; w < NWV; ++w) { kk += pv[k][w].x; xx += pv[k][w].y; zz += pv[k][w].z; yy += pv[k][w].w; }
+      for (int w = 0; w < NSLAB; ++w) { kk += pv[k][w].x; xx += pv[k][w].y; zz += pv[k][w].z; yy += pv[k][w].w; }
       if (rowok[k] && ll < L) {
         const size_t o = goff[k] + ll;
         const bool acc = p.accum != 0;                   // uniform
