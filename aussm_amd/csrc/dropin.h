@@ -499,29 +499,62 @@ __global__ __launch_bounds__(256) void fill_kernel(const FillArgs a) {
   for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) dst[i] = src ? src[i] : 0.0f;
 }
 
-// ---- fp32-accurate GEMM on the bf16 matrix cores, operands in fp32 with arbitrary strides -------
+// ---- fp32-accurate GEMM on the bf16 matrix cores ------------------------------------------------
 //     C_z[m][n] (+)= sum_k A_z(m, k) B_z(k, n)           z = 0 .. Z-1
 //     C[m][n]    += sum_z sum_k A_z(m, k) B_z(k, n)      (reduce_z)
-// Workgroup tile 128 x (64 TNH), four wavefronts of 64 x (32 TNH) each, 32 of k per step, one workgroup
-// per (tile, slice of z, slice of k): zper consecutive z per workgroup (1 unless reduce_z) and ksplit
-// slices of k.  With more than one slice per element of C the results are summed into C with atomics (C
-// holds the addend beforehand).  Both operands are split into NP bf16 pieces while they are staged in
-// LDS; the values of the next step are requested before the products of the current one.
-// TNH = 2 (128 x 128 tiles: two thirds of the operand traffic per product, two wavefronts per SIMD instead
-// of four) was measured at the same speed as TNH = 1 on the backward call of the fused operator, as was
-// starting each workgroup's walk over the steps at a different point; the launcher uses TNH = 1.
-// K1: both operands are contiguous along k.  Then four neighbouring lanes fetch the 32 values of
-// one row as 16-byte vectors (VEC; rows need not be 16-byte aligned) - a wavefront request covers 16
-// cache lines.  Otherwise both are contiguous along m / n and a 16-lane row of the wavefront
-// fetches 16 neighbouring rows' values of one k.
-// Rows of a tile that lie past M or N are fetched from the last valid row instead (row m of A only
-// reaches row m of C, which is not stored then), so only the last, partial step along k takes the
-// bounds-checked loads.
-template <bool K1, bool VEC, int NP, int TNH>
+// Workgroup tile 128 x (64 TNH), four wavefronts of 64 x (32 TNH) each, 32 of k per step, one workgroup per (tile,
+// slice of z, slice of k): zper consecutive z per workgroup (1 unless reduce_z) and ksplit slices of k.  With more
+// than one slice per element of C the results are summed into C with atomics (C holds the addend beforehand).
+// A - the operand with the 128-row side of the tile - arrives split into three bf16 pieces in the order the
+// kernel keeps it in LDS (a pre-pass, gemm_aprep_kernel: the callers' A is small and used by every workgroup of
+// a column of tiles), so a step copies 24 KiB of records; B is fp32 with arbitrary strides and is split while
+// it is staged.  The values of the next step are requested before the products of the current one.
+// (Measured on the backward call of the fused operator, b = 32, d = 256, n = 16, L = 720, per launch of 12.4 GFLOP in
+// fp32 terms: with neither the matrix instructions nor the stores of C 60 us, the matrix instructions add about 25 us
+// and the stores - atomics, the launch is cut along k or z - about 25 us; 128 x 128 tiles (TNH = 2) take 84-97 us
+// against 99-102 us of 128 x 64.  Splitting A inside the loop, as B is, cost 5 % more.)
+// K1: B is contiguous along k.  Then four neighbouring lanes fetch the 32 values of one row as 16-byte
+// vectors (VEC; rows need not be 16-byte aligned) - a wavefront request covers 16 cache lines.  Otherwise it is
+// contiguous along n and a 16-lane row of the wavefront fetches 16 neighbouring rows' values of one k.
+// Rows of the B tile that lie past N are fetched from the last valid row instead (column n of B only reaches
+// column n of C, which is not stored then), so only the last, partial step along k takes the bounds-checked loads.
+// TR: the two operands change places in the matrix instruction, so that the lanes of a result register run
+// along m: for a C that is contiguous along m (the stores and atomics of a wavefront then cover whole lines).
+
+// Record slot of (row r of a 16-row tile, k group g = 8 values): 16 g + (r + 4 g) % 16.  The rotation keeps the
+// 16-byte writes of the K1 mapping (four neighbouring lanes = the four g of one row) and the reads (16
+// neighbouring lanes = 16 rows of one g) both free of bank conflicts.
+__device__ __forceinline__ int gemm_slot(int r, int g) { return 16 * g + ((r + 4 * g) & 15); }
+
+// A (fp32, strides sam / sak / saz) -> image: one thread per (z, 16-row tile, step, record)
+__global__ __launch_bounds__(256) void gemm_aprep_kernel(const float* __restrict__ A, u4* __restrict__ img, long sam, long sak, long saz,
+                                                         int M, int K, int m16, int nk, long total) {
+  const long idx = (long)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= total) return;
+  const int slot = (int)(idx & 63);
+  const long rest = idx >> 6;
+  const int it = (int)(rest % nk), mt = (int)((rest / nk) % m16);
+  const long z = rest / ((long)nk * m16);
+  const int g = slot >> 4, r = ((slot & 15) - 4 * g) & 15;
+  const int m = mt * 16 + r, k0 = it * 32 + 8 * g;
+  const SplitK sk = make_splitk();
+  float v[8];
+#pragma unroll
+  for (int q = 0; q < 8; ++q) v[q] = (m < M && k0 + q < K) ? A[z * saz + (long)m * sam + (long)(k0 + q) * sak] : 0.0f;
+  u4 pc[3];
+  split8<3>(sk, v, pc);
+#pragma unroll
+  for (int c = 0; c < 3; ++c) img[(rest * 3 + c) * 64 + slot] = pc[c];
+}
+
+template <bool K1, bool VEC, bool TR, int TNH>
 __global__ __launch_bounds__(256) void split_gemm_kernel(const GemmArgs p) {
+  constexpr int NP = 3;                // bf16 pieces per operand: fp32-accurate products
+  constexpr int AREC = 8 * NP * 64;    // records of the A tile of one step
+  constexpr int AQ = AREC / 256;       // ... per thread
   constexpr int TN = 64 * TNH;         // columns of the workgroup tile
   constexpr int EN = 2 * TNH;          // 16-wide column tiles per wavefront
-  __shared__ u4 s_a[8 * NP * 64], s_b[4 * TNH * NP * 64];
+  __shared__ u4 s_a[AREC], s_b[4 * TNH * NP * 64];
   const int tid = threadIdx.x, lane = tid & 63, wave = wave_index();
   const int m0 = blockIdx.x * 128, n0 = blockIdx.y * TN;
   const int zs = blockIdx.z / p.ksplit, ksl = blockIdx.z % p.ksplit;
@@ -533,129 +566,111 @@ __global__ __launch_bounds__(256) void split_gemm_kernel(const GemmArgs p) {
   for (int e = 0; e < 4; ++e)
 #pragma unroll
     for (int f = 0; f < EN; ++f) acc[e][f] = f4{0, 0, 0, 0};
-  // the records this thread stages: rows ra, ra + 64 of the A tile and rows ra + 64 h of the B tile, k slots kq ..
-  const int ra = K1 ? tid >> 2 : wave * 16 + (lane & 15);
+  // the record of B this thread stages: row rb of the tile, k slots kq ..
+  const int rb = K1 ? tid >> 2 : wave * 16 + (lane & 15);
   const int kq = 8 * (K1 ? tid & 3 : lane >> 4);
-  // ... and where they go in LDS: [16-row tile][piece][16 g + (row + 4 g) % 16], g = kq / 8.  The rotation by
-  // 4 g keeps the 16-byte writes of the K1 mapping (four neighbouring lanes = the four g of one row) and the
-  // reads (16 neighbouring lanes = 16 rows of one g) both free of bank conflicts.
-  const int slot = (ra >> 4) * (NP * 64) + (kq >> 3) * 16 + ((ra + (kq >> 1)) & 15);
-  const int rslot = (lane & 48) + ((lane + (lane >> 4) * 4) & 15);       // the record of (row lane % 16, g lane / 16)
-  // uniform bases, 32-bit per-thread offsets (a z-slice of either operand is below 2^31 elements)
-  const unsigned sak = (unsigned)p.sak, sbk = (unsigned)p.sbk;
-  unsigned oa[2], ob[TNH];
-#pragma unroll
-  for (int h = 0; h < 2; ++h) {
-    const int m = m0 + ra + 64 * h;
-    oa[h] = (unsigned)(m < p.M ? m : p.M - 1) * (unsigned)p.sam + (unsigned)kq * sak;
-  }
+  const int slot = (rb >> 4) * (NP * 64) + gemm_slot(rb & 15, kq >> 3);
+  const int rslot = gemm_slot(lane & 15, lane >> 4);       // the record of (row lane % 16, g lane / 16)
+  // uniform bases, 32-bit per-thread offsets (a z-slice of B is below 2^31 elements)
+  const unsigned sbk = (unsigned)p.sbk;
+  unsigned ob[TNH];
 #pragma unroll
   for (int h = 0; h < TNH; ++h) {
-    const int n = n0 + ra + 64 * h;
+    const int n = n0 + rb + 64 * h;
     ob[h] = (unsigned)(n < p.N ? n : p.N - 1) * (unsigned)p.sbn + (unsigned)kq * sbk;
   }
   const int nk = (p.K + 31) / 32, per = (nk + p.ksplit - 1) / p.ksplit;
   const int it0 = ksl * per, it1 = it0 + per < nk ? it0 + per : nk;
   const int nit = it1 > it0 ? (it1 - it0) * (z_hi - z_lo) : 0;      // steps of this workgroup: (z, k step) pairs
-  float va[2][8], vb[TNH][8];
+  // this thread's records of the A tile: record tid + 256 q of the tile = record (tid + 256 q) % 192 of row tile
+  // m0 / 16 + (tid + 256 q) / 192, whose steps lie nk * 192 records apart
+  unsigned oa[AQ];
+#pragma unroll
+  for (int q = 0; q < AQ; ++q) {
+    const int idx = tid + 256 * q, e = idx / (NP * 64);
+    oa[q] = (unsigned)(((m0 >> 4) + e) * nk) * (unsigned)(NP * 64) + (unsigned)(idx - e * (NP * 64));
+  }
+  u4 ia[AQ];
+  float vb[TNH][8];
   int fz = z_lo, fit = it0;                   // (z, k step) of the next fetch: steps are fetched in order
   auto fetch = [&]() {
     const int z = fz, it = fit;
     if (++fit == it1) { fit = it0; ++fz; }
-    const float* __restrict__ Az = p.A + z * p.saz;
+    const u4* __restrict__ Az = p.Aimg + z * p.simz + (size_t)it * (NP * 64);
+#pragma unroll
+    for (int q = 0; q < AQ; ++q) ia[q] = Az[oa[q]];
     const float* __restrict__ Bz = p.Bm + z * p.sbz;
-    const unsigned ka = (unsigned)(it * 32) * sak, kb = (unsigned)(it * 32) * sbk;
+    const unsigned kb = (unsigned)(it * 32) * sbk;
     if (it * 32 + 32 <= p.K) {
       if constexpr (K1 && VEC) {
         // 16-byte loads that are only known to be 4-byte aligned (rows start anywhere when the row length is
         // not a multiple of four): the memory pipeline takes them, the type tells the compiler so
         typedef float f4u __attribute__((ext_vector_type(4), aligned(4)));
 #pragma unroll
-        for (int q = 0; q < 2; ++q) {
-#pragma unroll
-          for (int h = 0; h < 2; ++h) {
-            const f4u x = *reinterpret_cast<const f4u*>(Az + (oa[h] + ka + 4 * q));
-#pragma unroll
-            for (int c = 0; c < 4; ++c) va[h][4 * q + c] = x[c];
-          }
+        for (int q = 0; q < 2; ++q)
 #pragma unroll
           for (int h = 0; h < TNH; ++h) {
             const f4u x = *reinterpret_cast<const f4u*>(Bz + (ob[h] + kb + 4 * q));
 #pragma unroll
             for (int c = 0; c < 4; ++c) vb[h][4 * q + c] = x[c];
           }
-        }
       } else {
 #pragma unroll
-        for (int c = 0; c < 8; ++c) {
-#pragma unroll
-          for (int h = 0; h < 2; ++h) va[h][c] = Az[oa[h] + ka + (unsigned)c * sak];
+        for (int c = 0; c < 8; ++c)
 #pragma unroll
           for (int h = 0; h < TNH; ++h) vb[h][c] = Bz[ob[h] + kb + (unsigned)c * sbk];
-        }
       }
     } else {
 #pragma unroll
-      for (int c = 0; c < 8; ++c) {
-        const bool kok = it * 32 + kq + c < p.K;
+      for (int c = 0; c < 8; ++c)
 #pragma unroll
-        for (int h = 0; h < 2; ++h) va[h][c] = kok ? Az[oa[h] + ka + (unsigned)c * sak] : 0.0f;
-#pragma unroll
-        for (int h = 0; h < TNH; ++h) vb[h][c] = kok ? Bz[ob[h] + kb + (unsigned)c * sbk] : 0.0f;
-      }
+        for (int h = 0; h < TNH; ++h) vb[h][c] = (it * 32 + kq + c < p.K) ? Bz[ob[h] + kb + (unsigned)c * sbk] : 0.0f;
     }
   };
-  // (Cycle marks inside this loop, four wavefronts per SIMD: per step the 48 matrix instructions of a wavefront
-  // and their LDS reads take about 1.3-1.5 k cycles, splitting the next operands and getting them into LDS
-  // 2.4-3.0 k, issuing the loads after them 0.6-0.8 k; the loads have always landed when they are asked for and
-  // each barrier costs about 100 cycles.  The loop is bound by vector-instruction issue - the split, the address
-  // arithmetic - not by memory: requesting the values two steps ahead with a second register set made the
-  // launch 25 % slower, the registers cost a wavefront per SIMD.)
   if (nit > 0) fetch();
   for (int step = 0; step < nit; ++step) {
-    u4 pa[2][NP], pb[TNH][NP];
-#pragma unroll
-    for (int h = 0; h < 2; ++h) split8<NP>(sk, va[h], pa[h]);
+    u4 pb[TNH][NP];
 #pragma unroll
     for (int h = 0; h < TNH; ++h) split8<NP>(sk, vb[h], pb[h]);
     __syncthreads();
 #pragma unroll
-    for (int c = 0; c < NP; ++c) {
+    for (int q = 0; q < AQ; ++q) s_a[tid + 256 * q] = ia[q];
 #pragma unroll
-      for (int h = 0; h < 2; ++h) s_a[slot + 4 * h * (NP * 64) + c * 64] = pa[h][c];
+    for (int c = 0; c < NP; ++c)
 #pragma unroll
       for (int h = 0; h < TNH; ++h) s_b[slot + 4 * h * (NP * 64) + c * 64] = pb[h][c];
-    }
     __syncthreads();
     if (step + 1 < nit) fetch();              // in flight during the products
-    u4 rb[EN][NP];
+    u4 rB[EN][NP];
 #pragma unroll
     for (int f = 0; f < EN; ++f)
 #pragma unroll
-      for (int c = 0; c < NP; ++c) rb[f][c] = s_b[((wn + f) * NP + c) * 64 + rslot];
+      for (int c = 0; c < NP; ++c) rB[f][c] = s_b[((wn + f) * NP + c) * 64 + rslot];
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       u4 rA[NP];
 #pragma unroll
       for (int c = 0; c < NP; ++c) rA[c] = s_a[((wm + e) * NP + c) * 64 + rslot];
 #pragma unroll
-      for (int f = 0; f < EN; ++f) acc[e][f] = xmm<NP>(rA, rb[f], acc[e][f]);
+      for (int f = 0; f < EN; ++f) acc[e][f] = TR ? xmm<NP>(rB[f], rA, acc[e][f]) : xmm<NP>(rA, rB[f], acc[e][f]);
     }
   }
-  // result tile (e, f): lane (column = lane % 16, rows 4 (lane / 16) + a)
+  // result tile (e, f), register a: row 16 e + 4 (lane / 16) + a, column 16 f + lane % 16 of the wavefront's block
+  // (TR: row 16 e + lane % 16, column 16 f + 4 (lane / 16) + a)
   float* __restrict__ C = p.C + (p.reduce_z ? 0 : z_lo * p.scz);
   const bool atomic = p.ksplit > 1 || (p.reduce_z && p.zper < p.Z);
   // element offsets inside a z-slice of C fit 32 bits (checked by the caller)
   const unsigned scm = (unsigned)p.scm, scn = (unsigned)p.scn;
-  const int mr = m0 + wm * 16 + 4 * (lane >> 4), nc = n0 + wn * 16 + (lane & 15);
+  const int mr = m0 + wm * 16 + (TR ? (lane & 15) : 4 * (lane >> 4)), nc = n0 + wn * 16 + (TR ? 4 * (lane >> 4) : (lane & 15));
   const unsigned o0 = (unsigned)mr * scm + (unsigned)nc * scn;
+  const unsigned sa = TR ? scn : scm;           // stride between the four registers of a result
   if (atomic && m0 + 128 <= p.M && n0 + TN <= p.N) {       // uniform: a whole tile, summed into C
 #pragma unroll
     for (int e = 0; e < 4; ++e)
 #pragma unroll
       for (int f = 0; f < EN; ++f)
 #pragma unroll
-        for (int a = 0; a < 4; ++a) atomicAdd(C + (o0 + (unsigned)(16 * e + a) * scm + (unsigned)(16 * f) * scn), acc[e][f][a]);
+        for (int a = 0; a < 4; ++a) atomicAdd(C + (o0 + (unsigned)(16 * e) * scm + (unsigned)(16 * f) * scn + (unsigned)a * sa), acc[e][f][a]);
     return;
   }
 #pragma unroll
@@ -664,8 +679,8 @@ __global__ __launch_bounds__(256) void split_gemm_kernel(const GemmArgs p) {
     for (int f = 0; f < EN; ++f)
 #pragma unroll
       for (int a = 0; a < 4; ++a) {
-        if (mr + 16 * e + a < p.M && nc + 16 * f < p.N) {
-          float* c = C + (o0 + (unsigned)(16 * e + a) * scm + (unsigned)(16 * f) * scn);
+        if (mr + 16 * e + (TR ? 0 : a) < p.M && nc + 16 * f + (TR ? a : 0) < p.N) {
+          float* c = C + (o0 + (unsigned)(16 * e) * scm + (unsigned)(16 * f) * scn + (unsigned)a * sa);
           if (atomic) atomicAdd(c, acc[e][f][a]);
           else *c = p.accumulate ? *c + acc[e][f][a] : acc[e][f][a];
         }

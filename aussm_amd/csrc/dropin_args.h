@@ -62,13 +62,16 @@ struct FillArgs {
   int count;
 };
 
+// A is a prepared image (gemm_aprep_kernel): [z][16-row tile][step of 32 along k][piece][64 records], the
+// row tiles padded to whole workgroup tiles of 128 rows, zeros past M and K.
 struct GemmArgs {
-  const float* A; const float* Bm; float* C;
-  long sam, sak, saz;     // element strides of A over m, k, z
-  long sbk, sbn, sbz;
+  const u4* Aimg; const float* Bm; float* C;
+  long simz;              // records between the images of consecutive z (0: one image for all)
+  long sbk, sbn, sbz;     // element strides of B over k, n, z
   long scm, scn, scz;
   int M, N, K, Z;
   int reduce_z, accumulate;
+  int tr;                 // results leave with the lanes along m (for C contiguous along m) instead of along n
   int ksplit;             // slices of k per (tile, slice of z)
   int zper;               // z per workgroup (summed inside it; 1 unless reduce_z)
 };

@@ -71,14 +71,27 @@ int run_dropin_bwd(const DropinBwdArgs& a, hipStream_t s) {
 }
 
 int run_split_gemm(const GemmArgs& a, hipStream_t s) {
-  if (a.ksplit < 1 || a.zper < 1 || (!a.reduce_z && a.zper != 1)) return -2;
+  if (a.ksplit < 1 || a.zper < 1 || (!a.reduce_z && a.zper != 1) || !a.Aimg) return -2;
   const long gz = (long)((a.Z + a.zper - 1) / a.zper) * a.ksplit;
   if (gz > 65535) return -2;
-  const dim3 grid((unsigned)((a.M + 127) / 128), (unsigned)((a.N + 63) / 64), (unsigned)gz);
-  const bool k1 = a.sak == 1 && a.sbk == 1;
-  constexpr int NP = 3;               // bf16 pieces per operand: fp32-accurate products
-  if (k1) hipLaunchKernelGGL((split_gemm_kernel<true, true, NP, 1>), grid, dim3(256), 0, s, a);
-  else hipLaunchKernelGGL((split_gemm_kernel<false, false, NP, 1>), grid, dim3(256), 0, s, a);
+  constexpr int TNH = GEMM_TILE_N / 64;
+  const dim3 grid((unsigned)((a.M + 127) / 128), (unsigned)((a.N + 64 * TNH - 1) / (64 * TNH)), (unsigned)gz);
+  const bool k1 = a.sbk == 1;
+  if (k1 && a.tr) hipLaunchKernelGGL((split_gemm_kernel<true, true, true, TNH>), grid, dim3(256), 0, s, a);
+  else if (k1) hipLaunchKernelGGL((split_gemm_kernel<true, true, false, TNH>), grid, dim3(256), 0, s, a);
+  else if (a.tr) hipLaunchKernelGGL((split_gemm_kernel<false, false, true, TNH>), grid, dim3(256), 0, s, a);
+  else hipLaunchKernelGGL((split_gemm_kernel<false, false, false, TNH>), grid, dim3(256), 0, s, a);
+  return launch_status();
+}
+
+// records of the image of an A with M rows and K columns (one z)
+size_t gemm_image_records(int M, int K) { return (size_t)8 * ((M + 127) / 128) * ((K + 31) / 32) * 3 * 64; }
+
+int run_gemm_aprep(const float* A, u4* img, long sam, long sak, long saz, int M, int K, int Z, hipStream_t s) {
+  const int m16 = 8 * ((M + 127) / 128), nk = (K + 31) / 32;
+  const long total = (long)Z * m16 * nk * 64;
+  if (total <= 0 || (total + 255) / 256 > 0x7fffffffL) return -2;
+  hipLaunchKernelGGL(gemm_aprep_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, A, img, sam, sak, saz, M, K, m16, nk, total);
   return launch_status();
 }
 

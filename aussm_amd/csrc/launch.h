@@ -56,6 +56,9 @@ int run_dropin_uprep(const float* u, u4* up, int d, int L, int ks, int b0, int b
 int run_dropin_fwd(const DropinArgs& a, hipStream_t s);
 int run_dropin_bwd(const DropinBwdArgs& a, hipStream_t s);
 int run_fill(const FillArgs& a, hipStream_t s);   // several buffers set (zero or a copy) in one launch
+constexpr int GEMM_TILE_M = 128, GEMM_TILE_N = 128;   // workgroup tile of run_split_gemm
 int run_split_gemm(const GemmArgs& a, hipStream_t s);
+size_t gemm_image_records(int M, int K);       // 16-byte records of the prepared image of an M x K operand
+int run_gemm_aprep(const float* A, u4* img, long sam, long sak, long saz, int M, int K, int Z, hipStream_t s);
 
 }  // namespace aussm

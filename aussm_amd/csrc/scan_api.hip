@@ -614,13 +614,15 @@ int aussm_swap_last2_act(const float* x, const float* bias, const float* pre, fl
 static int dropin_state_blocks(int n) { const int k = (n + 15) / 16; return k == 3 ? 4 : k; }
 static size_t dropin_xp_floats(int d, int n) { return (size_t)d * dropin_state_blocks(n) * ((d + 31) / 32) * 3 * 64 * 4; }
 // The backward call works through the (batch, sequence) plane in blocks of bg batch elements x ct tiles
-// of 16 timesteps: the workspace holds the phase adjoints of one block (about 50 MiB at most).  bg is
+// of 16 timesteps: the workspace holds the phase adjoints of one block (about 100 MiB at most:
+// at b = 32, d = 256, n = 16, L = 720 a block of 8 batch elements then spans the whole sequence, 1.39 ms per backward
+// call against 1.64 ms with 50 MiB blocks).  bg is
 // what fills the chip with one workgroup per compute unit (fewer would idle units, more would only
 // shorten the blocks and repeat the per-launch set-up, the rows of x among it, more often).
 // budget of a block (phase adjoints; prepared tiles of u), in floats
 // (the option can only lower it: the workspace query sizes for the full budget, so a buffer obtained under
 // one setting of the option holds what a call under any other setting uses)
-constexpr int DROPIN_BLOCK_KFLOATS = 12800;
+constexpr int DROPIN_BLOCK_KFLOATS = 25600;
 static size_t dropin_block_floats(bool largest) {
   const int o = opt(AUSSM_OPT_BLOCK_KFLOATS);
   return (size_t)(!largest && o > 0 && o < DROPIN_BLOCK_KFLOATS ? o : DROPIN_BLOCK_KFLOATS) << 10;
@@ -640,12 +642,12 @@ static DropinBlocks dropin_blocks(int b, int d, int n, int L, bool largest = fal
   const size_t nc = ((size_t)ntiles + tmax - 1) / tmax;
   return DropinBlocks{bg, (int)(((size_t)ntiles + nc - 1) / nc)};
 }
-// How a GEMM launch is cut: about three workgroups per compute unit.  Without reduce_z every z is a
+// How a GEMM launch is cut: about three workgroups of 128 x 128 per two compute units.  Without reduce_z every z is a
 // slice of its own and k is cut (at least four steps per slice); with reduce_z the z are dealt to the
 // slices first and k is cut only when there are too few z.
-constexpr long GEMM_TARGET = 768;     // workgroups per launch aimed at (measured: 512 +4 %, 1024 +5 %, 256 +22 % of the backward call)
+constexpr long GEMM_TARGET = 384;     // workgroups per launch aimed at (measured: 256 and 512 +9 % of the backward call)
 static void gemm_slices(GemmArgs& g) {
-  const long tiles = (long)((g.M + 127) / 128) * ((g.N + 63) / 64);
+  const long tiles = (long)((g.M + GEMM_TILE_M - 1) / GEMM_TILE_M) * ((g.N + GEMM_TILE_N - 1) / GEMM_TILE_N);
   const long target = GEMM_TARGET;
   const int nk = (g.K + 31) / 32;
   long zs = 1;                                   // slices of z
@@ -690,6 +692,8 @@ size_t aussm_ssm_adaptive_unitary_workspace_floats(int b, int d, int n, int L, i
   if (backward) {
     const DropinBlocks k = dropin_blocks(b, d, n, L, true);
     f += 2 * round4((size_t)b * d * n) + (size_t)k.bg * k.ct * DT * d * n + (size_t)k.bg * k.ct * dropin_tile_floats(d);
+    // prepared first operands of the two products with the phase adjoints: x transposed (once per call), u of a block
+    f += 4 * (gemm_image_records(d, d * n) + (size_t)k.bg * gemm_image_records(d, k.ct * DT));
   } else {
     f += (size_t)b * dropin_fwd_chunk_tiles(b, d, L, true) * dropin_tile_floats(d);
   }
@@ -751,7 +755,10 @@ int aussm_ssm_adaptive_unitary_bwd(const float* grad_y, const float* grad_nh_re,
   float* hc_im = hc_re + round4(nstate);
   float* dth = hc_im + round4(nstate);
   u4* up = (u4*)(dth + (size_t)blk.bg * ct * DT * d * n);
+  u4* xt = up + (size_t)blk.bg * ct * (dropin_tile_floats(d) / 4);     // image of A(r, (i j)) = x[(i j), r]
+  u4* ui = xt + gemm_image_records(d, d * n);                          // images of A_b(r, l) = u[b, r, l0 + l] of a block
   if (int e = run_dropin_xprep(x, xp, d, n, ks, nb, s)) return e;
+  if (int e = run_gemm_aprep(x, xt, 1, d, 0, d, d * n, 1, s)) return e;
   DropinArgs f{};
   f.u = u; f.dt = dt; f.z = z; f.x_bias = x_bias; f.B_r = B_r; f.B_th = B_theta; f.C_r = C_r; f.C_th = C_theta;
   f.Dp = D; f.xp = xp; f.up = up; f.d = d; f.n = n; f.L = L; f.ks = ks; f.nb = nb;
@@ -804,18 +811,19 @@ int aussm_ssm_adaptive_unitary_bwd(const float* grad_y, const float* grad_nh_re,
       if (int e = run_dropin_bwd(q, s)) return e;
       // grad_u[b, r, l0 + l] += sum_(i j) x[(i j), r] hat theta[b, (i j), l]
       GemmArgs gu{};
-      gu.A = x; gu.sam = 1; gu.sak = d; gu.saz = 0;
+      gu.Aimg = xt; gu.simz = 0;
       gu.Bm = dth; gu.sbk = lc; gu.sbn = 1; gu.sbz = dn * lc;
       gu.C = du + (size_t)b0 * d * L + l0; gu.scm = L; gu.scn = 1; gu.scz = (long)d * L;
-      gu.M = d; gu.N = len; gu.K = (int)dn; gu.Z = bg; gu.reduce_z = 0; gu.accumulate = 1;
+      gu.M = d; gu.N = len; gu.K = (int)dn; gu.Z = bg; gu.reduce_z = 0; gu.accumulate = 1; gu.tr = 0;
       gemm_slices(gu);
       if (int e = run_split_gemm(gu, s)) return e;
-      // grad_x[(i j), r] += sum_b sum_l hat theta[b, (i j), l] u[b, r, l0 + l]
+      // grad_x[(i j), r] += sum_b sum_l u[b, r, l0 + l] hat theta[b, (i j), l]: rows r, columns (i j), C contiguous along r
+      if (int e = run_gemm_aprep(u + (size_t)b0 * d * L + l0, ui, L, 1, (long)d * L, d, len, bg, s)) return e;
       GemmArgs gx{};
-      gx.A = dth; gx.sam = lc; gx.sak = 1; gx.saz = dn * lc;
-      gx.Bm = u + (size_t)b0 * d * L + l0; gx.sbk = 1; gx.sbn = L; gx.sbz = (long)d * L;
-      gx.C = dx; gx.scm = d; gx.scn = 1; gx.scz = 0;
-      gx.M = (int)dn; gx.N = d; gx.K = len; gx.Z = bg; gx.reduce_z = 1; gx.accumulate = 1;
+      gx.Aimg = ui; gx.simz = (long)gemm_image_records(d, len);
+      gx.Bm = dth; gx.sbk = 1; gx.sbn = lc; gx.sbz = dn * lc;
+      gx.C = dx; gx.scm = 1; gx.scn = d; gx.scz = 0;
+      gx.M = d; gx.N = (int)dn; gx.K = len; gx.Z = bg; gx.reduce_z = 1; gx.accumulate = 1; gx.tr = 1;
       gemm_slices(gx);
       if (int e = run_split_gemm(gx, s)) return e;
     }

@@ -74,7 +74,7 @@ const char* aussm_error_string(int code);
  *                          (0 or 1: never split)
  *   AUSSM_OPT_BLOCK_KFLOATS   budget, in units of 1024 floats, of the blocks in which the fused operator calls
  *                          (aussm_ssm_adaptive_unitary_fwd / _bwd) walk their problem (default and largest
- *                          value 12800 = 50 MiB; the option can only lower it)
+ *                          value 25600 = 100 MiB; the option can only lower it)
  * Workspace and auxiliary-buffer sizes do not depend on any option: a buffer sized by the query
  * functions below holds what a call of that shape uses under every setting.
  *   AUSSM_OPT_GENERIC_NW / AUSSM_OPT_GENERIC_NT   states per wavefront / threads per workgroup of

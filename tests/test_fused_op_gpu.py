@@ -141,8 +141,9 @@ def test_fused_matches_composite_at_training_shape():
     zeros = torch.zeros(b, d, n, device="cuda")
     inputs_bytes = sum(a.numel() * 4 for a in args)
     # The fused route never holds the phase tensor (b d n l floats = 377 MB here).  What a call allocates on top of
-    # its inputs - outputs and workspace - stays within the operator's input footprint for the forward call and
-    # within twice that for the backward call (twelve gradients the size of the inputs, plus the workspace).
+    # its inputs - outputs and workspace - stays within the operator's input footprint for the forward call; for the
+    # backward call within that (twelve gradients the size of the inputs) plus a workspace whose size does not grow
+    # with the sequence: one block of phase adjoints (100 MiB at most) and the prepared operands of its products.
     torch.cuda.synchronize()
     torch.cuda.reset_peak_memory_stats()
     base = torch.cuda.memory_allocated()
@@ -156,7 +157,7 @@ def test_fused_matches_composite_at_training_shape():
     peak_bwd = torch.cuda.max_memory_allocated() - base
     print(f"inputs {inputs_bytes / 1e6:.0f} MB, forward call +{peak_fwd / 1e6:.0f} MB, backward call +{peak_bwd / 1e6:.0f} MB", flush=True)
     assert peak_fwd <= inputs_bytes, (peak_fwd, inputs_bytes)
-    assert peak_bwd <= 2 * inputs_bytes, (peak_bwd, inputs_bytes)
+    assert peak_bwd <= inputs_bytes + 140 * 2 ** 20 and peak_bwd < b * d * n * l * 4, (peak_bwd, inputs_bytes)
     leaves = [a.clone().requires_grad_(True) for a in args]
     yc, hrc, hic = ops._composite(*leaves)
     want = torch.autograd.grad([yc], leaves, [gy], allow_unused=True)
