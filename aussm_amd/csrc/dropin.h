@@ -30,13 +30,10 @@ namespace aussm {
 
 
 // sin and cos of any argument without a branch: reduction by 2 pi in two fused steps (the result is as exact
-// as the fp32 argument itself), then the polynomial kernel for small arguments.  A branch here would cut the
-// four state groups of a lane into separate blocks that the scheduler cannot interleave.
+// as the fp32 argument itself), then the hardware sine and cosine of the reduced argument (sincos_small_hw).  A
+// branch here would cut the four state groups of a lane into separate blocks that the scheduler cannot interleave.
 __device__ __forceinline__ void sincos_any(float x, float* sn, float* cs) {
-  const float k = rintf(x * 0.15915494309189535f);
-  float r = fmaf(-k, 6.2831854820251465f, x);
-  r = fmaf(-k, -1.7484555e-07f, r);
-  sincos_small(r, sn, cs);
+  sincos_small_hw(x, sn, cs);
 }
 
 // silu and its derivative with the hardware reciprocal (1 ulp) instead of an IEEE division (ten instructions)
