@@ -506,10 +506,11 @@ __global__ __launch_bounds__(256) void fill_kernel(const FillArgs a) {
 // kernel keeps it in LDS (a pre-pass, gemm_aprep_kernel: the callers' A is small and used by every workgroup of
 // a column of tiles), so a step copies 24 KiB of records; B is fp32 with arbitrary strides and is split while
 // it is staged.  The values of the next step are requested before the products of the current one.
-// (Measured on the backward call of the fused operator, b = 32, d = 256, n = 16, L = 720, per launch of 12.4 GFLOP in
-// fp32 terms: with neither the matrix instructions nor the stores of C 60 us, the matrix instructions add about 25 us
-// and the stores - atomics, the launch is cut along k or z - about 25 us; 128 x 128 tiles (TNH = 2) take 84-97 us
-// against 99-102 us of 128 x 64.  Splitting A inside the loop, as B is, cost 5 % more.)
+// (Measured on the backward call of the fused operator, b = 32, d = 256, n = 16, L = 720.  Launches of 6.2 GFLOP in
+// fp32 terms with 128 x 64 tiles: 54-58 us; without the stores of C - atomics, the launch is cut along k or z -
+// 40-46 us; without the matrix instructions 41-43 us; with neither 30 us: operand traffic, LDS and the two barriers
+// of a step set the floor, the rest adds up.  Launches twice that size: 99-102 us with 128 x 64 tiles, 84-97 us
+// with 128 x 128 (TNH = 2).  Splitting A inside the loop, as B is, cost 5 % more.)
 // K1: B is contiguous along k.  Then four neighbouring lanes fetch the 32 values of one row as 16-byte
 // vectors (VEC; rows need not be 16-byte aligned) - a wavefront request covers 16 cache lines.  Otherwise it is
 // contiguous along n and a 16-lane row of the wavefront fetches 16 neighbouring rows' values of one k.
