@@ -31,6 +31,11 @@ SHAPES = [
     (2, 40, 64, 50),          # more than 16 states: the backward pass takes one launch per block of 16
     (1, 70, 24, 33),
     (2, 20, 37, 40),
+    # 9 to 15 states: the backward workgroups of eight wavefronts (two states each) are partly filled - whole
+    # wavefronts without states, and with an odd count one wavefront with a single state
+    (2, 70, 12, 100),
+    (1, 33, 9, 50),
+    (1, 20, 29, 300),
     # few (batch, channel group) pairs and at least 256 steps: the launch is split along the sequence
     # (segments of 128 steps here; the last one ragged, a single step in (3, 130, 4, 257) above)
     (2, 70, 16, 600),
