@@ -206,7 +206,7 @@ constexpr int SEG_BATCH = 16;
 
 // Chains the segments of one (batch, channel, state): on entry seg[k] holds Z_k, on return the
 // state that enters segment k; the state after the last segment goes to hL (if wanted).
-__global__ void seg_carry_fwd_kernel(float* __restrict__ seg, const float* __restrict__ ptot,
+__global__ __launch_bounds__(64) void seg_carry_fwd_kernel(float* __restrict__ seg, const float* __restrict__ ptot,
                                      const float* __restrict__ h0, float* __restrict__ hL,
                                      int B, int D, int N, int ns) {
   const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -240,7 +240,7 @@ __global__ void seg_carry_fwd_kernel(float* __restrict__ seg, const float* __res
 
 // The same for the adjoint, last segment first: on entry seg[k] holds Y_k, on return the adjoint
 // that enters segment k at its end; the adjoint of the initial state goes to dh0 (if wanted).
-__global__ void seg_carry_bwd_kernel(float* __restrict__ seg, const float* __restrict__ ptot,
+__global__ __launch_bounds__(64) void seg_carry_bwd_kernel(float* __restrict__ seg, const float* __restrict__ ptot,
                                      const float* __restrict__ dhL, float* __restrict__ dh0,
                                      int B, int D, int N, int ns) {
   const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
