@@ -108,8 +108,12 @@ int run_rec_bwd(int variant, const RecBwdArgs& a, int in_dtype, hipStream_t s) {
 }
 
 int run_adjoint_seg(int variant, const AdjSegArgs& a, int in_dtype, unsigned grid, hipStream_t s) {
-  // (B_t / C_t are float in every instance; the complex kernel reads no u / delta at all)
-  if (variant == VAR_COMPLEX) {
+  // (B_t / C_t are float in every instance of the complex and real scans; the complex kernel reads no u / delta
+  // at all.  The unitary scan runs the complex instance without rho, with C_t in the type of its inputs.)
+  if (variant == VAR_UNITARY) {
+    if (in_dtype == 1) hipLaunchKernelGGL((adjoint_seg_kernel<VAR_COMPLEX, float, bf16_t>), dim3(grid), dim3(256), 0, s, a);
+    else hipLaunchKernelGGL((adjoint_seg_kernel<VAR_COMPLEX, float, float>), dim3(grid), dim3(256), 0, s, a);
+  } else if (variant == VAR_COMPLEX) {
     hipLaunchKernelGGL((adjoint_seg_kernel<VAR_COMPLEX, float, float>), dim3(grid), dim3(256), 0, s, a);
   } else {
     if (in_dtype) hipLaunchKernelGGL((adjoint_seg_kernel<VAR_REAL, bf16_t, float>), dim3(grid), dim3(256), 0, s, a);

@@ -152,15 +152,24 @@ inline size_t img_floats(int B, int N, int L, int ck) {
   if (!matrix_shape(N, L, ck)) return 0;
   return img_chunks(B, L) * (PXB_REC + PXF_REC) * 4;
 }
-// Layout of the auxiliary buffer: [B*D*L floats Im(P S)] [AUX_PAD] [segment states] [backward images] [forward images]
-struct AuxLayout { float* seg; u4* img; u4* fimg; uint32_t* stamp; };
+// Layout of the auxiliary buffer: [B*D*L floats Im(P S)] [AUX_PAD] [segment states] [backward images] [forward images].
+// A shape that only the vector-ALU kernels serve (more than 16 states, a length that is not a multiple of 4, ...)
+// has no Im(P S) part and no images.  The segment area holds what either way of splitting a call along L
+// needs (the matrix-core kernels' fine segments or the vector-ALU kernels' segments), so a call of a shape
+// that could run on the matrix cores but does not (shared inputs, misaligned tensors, an option) can still split.
+inline size_t aux_im_floats(int B, int D, int N, int L, int ck) { return matrix_shape(N, L, ck) ? (size_t)B * D * L : 0; }
+inline size_t aux_seg_floats(int B, int D, int N, int L, int ck) {
+  const size_t m = seg_floats(B, D, N, L, seg_capacity(B, D, N, L, ck)), g = generic_split_floats(VAR_COMPLEX, B, D, N, L, ck);
+  return m > g ? m : g;
+}
+struct AuxLayout { float* seg; u4* img; u4* fimg; uint32_t* stamp; float* pad; float* gseg; };
 inline AuxLayout aux_layout(float* aux, int B, int D, int N, int L, int ck) {
-  if (!aux) return AuxLayout{nullptr, nullptr, nullptr, nullptr};
-  float* pad = aux + (size_t)B * D * L;
+  if (!aux) return AuxLayout{nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
+  float* pad = aux + aux_im_floats(B, D, N, L, ck);
   float* seg = pad + AUX_PAD;
-  u4* img = reinterpret_cast<u4*>(seg + seg_floats(B, D, N, L, seg_capacity(B, D, N, L, ck)));
-  if (!img_floats(B, N, L, ck)) return AuxLayout{seg, nullptr, nullptr, nullptr};
-  return AuxLayout{seg, img, img + img_chunks(B, L) * PXB_REC, reinterpret_cast<uint32_t*>(pad) + AUX_IMG_FP};
+  u4* img = reinterpret_cast<u4*>(seg + aux_seg_floats(B, D, N, L, ck));
+  if (!img_floats(B, N, L, ck)) return AuxLayout{seg, nullptr, nullptr, nullptr, pad, seg};
+  return AuxLayout{seg, img, img + img_chunks(B, L) * PXB_REC, reinterpret_cast<uint32_t*>(pad) + AUX_IMG_FP, pad, seg};
 }
 
 // Kernel family of a call whose tensors are 16-byte aligned: 0 vector ALU, 2 / 3 / 5 matrix-core kernels
@@ -198,9 +207,28 @@ int launch_unitary_fwd(FwdArgs a, int in_dtype, hipStream_t s, AuxLayout ws) {
   // images clears the note about the ones behind the buffer
   const bool fill = a.aux && a.hck && mode >= 2;
   if (a.aux)
-    if (int e = run_aux_invalidate(a.aux + (size_t)a.B * a.D * a.L, !fill, mode != 6 && ws.stamp, s)) return e;
+    if (int e = run_aux_invalidate(ws.pad, !fill, mode != 6 && ws.stamp, s)) return e;
   if (!fill) a.aux = nullptr;
-  if (!mode) return run_core_fwd(VAR_UNITARY, a, in_dtype, pick_cfg(a.N, 8), s);
+  if (!mode) {
+    // vector-ALU kernel; with a segment area and few (batch, channel group) pairs, split along the sequence
+    const Cfg cfg = pick_cfg(a.N, 8);
+    const GSplit sp = ws.gseg ? generic_split(a.B, a.D, a.L, a.ck, true) : GSplit{1, a.L};
+    if (sp.ns > 1) {
+      const int B = a.B;
+      float* seg = ws.gseg;
+      float* ptot = seg + (size_t)B * sp.ns * a.D * a.N * 2;
+      // 1. end state of every segment from a zero state (no outputs) and the product of its a_l
+      FwdArgs z = a;
+      z.B = B * sp.ns; z.L = sp.ls; z.ns = sp.ns;
+      z.y = nullptr; z.z = nullptr; z.Dskip = nullptr; z.h0 = nullptr; z.hL = seg; z.hck = nullptr; z.ptot = ptot;
+      if (int e = run_core_fwd(VAR_UNITARY, z, in_dtype, cfg, s)) return e;
+      // 2. the state that enters every segment; the state after the last one is the call's hL
+      if (int e = run_seg_carry_fwd(seg, ptot, a.h0, a.hL, B, a.D, a.N, sp.ns, s)) return e;
+      // 3. the scan proper over (batch, segment) pairs
+      a.B = B * sp.ns; a.L = sp.ls; a.ns = sp.ns; a.h0 = seg; a.hL = nullptr;
+    }
+    return run_core_fwd(VAR_UNITARY, a, in_dtype, cfg, s);
+  }
   const int B = a.B, L = a.L;
   if ((mode == 2 || mode == 3 || mode == 6) && ws.seg) {
     const int ns = seg_count(B, a.D, a.N, L, a.ck);
@@ -341,12 +369,19 @@ int aussm_num_checkpoints(int L, int ck) { return (L < 1 || ck < 1) ? 0 : (L + c
 int aussm_bwd_checkpoint_interval(int variant) { return variant == VAR_UNITARY ? 0 : REC_CK; }
 
 int aussm_unitary_split_segments(int B, int D, int N, int L, int ck) {
-  return (B < 1 || D < 1 || N < 1 || L < 1) ? 0 : seg_capacity(B, D, N, L, ck);
+  if (B < 1 || D < 1 || N < 1 || L < 1 || ck < 1) return 0;
+  int ns = seg_capacity(B, D, N, L, ck);
+  // shapes that the vector-ALU kernels serve by default split their way
+  if (!(matrix_shape(N, L, ck) && N >= MATRIX_MIN_STATE)) {
+    const int g = generic_split(B, D, L, ck, false).ns;
+    if (g > ns) ns = g;
+  }
+  return ns;
 }
 
 size_t aussm_unitary_aux_floats(int B, int D, int N, int L, int ck) {
   if (B < 1 || D < 1 || N < 1 || L < 1) return 0;
-  return (size_t)B * D * L + AUX_PAD + seg_floats(B, D, N, L, seg_capacity(B, D, N, L, ck)) + img_floats(B, N, L, ck);
+  return aux_im_floats(B, D, N, L, ck) + AUX_PAD + aux_seg_floats(B, D, N, L, ck) + img_floats(B, N, L, ck);
 }
 
 size_t aussm_scan_workspace_floats(int variant, int B, int D, int N, int L, int ck, int in_dtype) {
@@ -421,7 +456,8 @@ int aussm_unitary_fwd_static(const void* u, const void* delta, const float* thet
   a.ld = L; a.ns = 1; a.hs = 1; a.ho = 0; a.urep = 1;
   // (every segment state the scan reads is written earlier in the same call: nothing in the
   // scratch has to start at zero)
-  return launch_unitary_fwd(a, in_dtype, (hipStream_t)stream, AuxLayout{scratch, nullptr, nullptr, nullptr});
+  // (the vector-ALU kernels do not split here: no gseg)
+  return launch_unitary_fwd(a, in_dtype, (hipStream_t)stream, AuxLayout{scratch, nullptr, nullptr, nullptr, nullptr, nullptr});
 }
 
 int aussm_complex_fwd(const void* u, const void* delta, const float* rho, const float* theta, const void* Bc,
@@ -512,6 +548,18 @@ int aussm_unitary_bwd_aux(const float* dy, const float* dhL, const void* u, cons
       return run_xdl_bwd(3, a, in_dtype, s);
     }
     return run_xdl_bwd(mode, a, in_dtype, s);
+  }
+  // vector-ALU kernel; split along the sequence like the forward call
+  const GSplit sp = ws.gseg ? generic_split(B, D, L, ck, true) : GSplit{1, L};
+  if (sp.ns > 1) {
+    float* seg = ws.gseg;
+    float* ptot = seg + (size_t)B * sp.ns * D * N * 2;
+    AdjSegArgs g{};
+    g.dy = dy; g.theta = theta; g.Cm = Cc; g.out = seg; g.ptot = ptot;
+    g.D = D; g.N = N; g.L = sp.ls; g.ld = L; g.ns = sp.ns; g.ncg = a.ncg;
+    if (int e = run_adjoint_seg(VAR_UNITARY, g, in_dtype, (unsigned)(B * sp.ns * a.ncg), s)) return e;
+    if (int e = run_seg_carry_bwd(seg, ptot, dhL, dh0, B, D, N, sp.ns, s)) return e;
+    a.B = B * sp.ns; a.L = sp.ls; a.ns = sp.ns; a.dhL = seg; a.dh0 = nullptr;
   }
   return run_unitary_bwd_generic(a, in_dtype, pick_cfg(a.N, 8), s);
 }

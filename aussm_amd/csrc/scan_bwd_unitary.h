@@ -71,8 +71,13 @@ __global__ __launch_bounds__(NT) void unitary_bwd_kernel(const UniBwdArgs p) {
 
   const int tid = threadIdx.x, lane = tid & 63, wave = wave_index();
   const int wg = xcd_remap(blockIdx.x, gridDim.x);
-  const int b = wg / p.ncg, d0 = (wg % p.ncg) * CH;
-  const int N = p.N, L = p.L, D = p.D;
+  // vb: (batch, segment) pair of a launch that is split along the sequence (p.ns segments of p.L steps,
+  // the last one possibly shorter; p.ld = row stride of the [.., L] tensors), else the batch element
+  const int vb = wg / p.ncg, d0 = (wg % p.ncg) * CH;
+  const int b = vb / p.ns, sg = vb - b * p.ns;
+  const int lbeg = sg * p.L, ld = p.ld;
+  const int N = p.N, D = p.D;
+  const int L = (ld - lbeg < p.L) ? ld - lbeg : p.L;        // steps of this segment
   const int n0 = wave * NW;
   const bool active = n0 < N;
   const bool full_group = active && n0 + NW <= N;
@@ -82,7 +87,7 @@ __global__ __launch_bounds__(NT) void unitary_bwd_kernel(const UniBwdArgs p) {
 
   // u and delta may be shared by p.urep consecutive batch elements (tensors [B / urep, D, L]): every
   // address below is formed for batch element b, so their base steps back by the difference
-  const size_t uback = (size_t)(b - b / p.urep) * p.D * p.L;
+  const size_t uback = (size_t)(b - b / p.urep) * p.D * ld;
   const Tin* __restrict__ gu = static_cast<const Tin*>(p.u) - uback;
   const Tin* __restrict__ gdl = static_cast<const Tin*>(p.delta) - uback;
   const Tin* __restrict__ gB = static_cast<const Tin*>(p.Bm);
@@ -107,15 +112,16 @@ __global__ __launch_bounds__(NT) void unitary_bwd_kernel(const UniBwdArgs p) {
     }
   };
 
-  // ---- state h_L and adjoint g_L
+  // ---- state and adjoint at the end of the segment (checkpoints are numbered along the whole sequence, a
+  // segment is a whole number of checkpoint blocks, the sequence's last block may be shorter)
   float hr[NW], hi[NW], gr[NW], gi[NW];
-  load_ck(p.nck - 1, hr, hi);
+  load_ck((lbeg + L + p.ck - 1) / p.ck - 1, hr, hi);
 #pragma unroll
   for (int k = 0; k < NW; ++k) {
     const int n = n0 + k;
     gr[k] = 0.f; gi[k] = 0.f;
     if (p.dhL && dok && n < N) {
-      const size_t o = (((size_t)b * D + d) * N + n) * 2;
+      const size_t o = (((size_t)vb * D + d) * N + n) * 2;
       gr[k] = p.dhL[o]; gi[k] = p.dhL[o + 1];
     }
   }
@@ -134,7 +140,7 @@ __global__ __launch_bounds__(NT) void unitary_bwd_kernel(const UniBwdArgs p) {
   for (int k = 0; k < E; ++k) {
     const int dd = d0 + row0 + k * RSTEP;
     rowok[k] = dd < D;
-    goff[k] = ((size_t)b * D + (rowok[k] ? dd : 0)) * L;
+    goff[k] = ((size_t)b * D + (rowok[k] ? dd : 0)) * ld + lbeg;
     dsk[k] = (p.Dskip && rowok[k]) ? p.Dskip[dd] : 0.f;
     accD[k] = 0.f;
     fly.u[k] = fly.dl[k] = Tin(0);
@@ -166,10 +172,10 @@ __global__ __launch_bounds__(NT) void unitary_bwd_kernel(const UniBwdArgs p) {
   // scalar-cache warm-up of the B_t/C_t lines, one tile ahead of the scan (see the forward kernel)
   constexpr bool WARM = NW <= 4;
   constexpr int RB = (int)sizeof(Tin) * 2;
-  const size_t row_base = ((size_t)b * N + n0) * L;
+  const size_t row_base = ((size_t)b * N + n0) * ld + lbeg;
   TileWarm<WARM ? NW : 1, RB, TT> warm;
   if (WARM && full_group && ntiles * TT == L) {
-    warm.issue(gB, gC, row_base + (size_t)(ntiles - 1) * TT, L);
+    warm.issue(gB, gC, row_base + (size_t)(ntiles - 1) * TT, ld);
     warm.retire();
   }
 
@@ -177,7 +183,7 @@ __global__ __launch_bounds__(NT) void unitary_bwd_kernel(const UniBwdArgs p) {
     const int l0 = it * TT;
     const int tmax = (L - l0 < TT) ? (L - l0) : TT;
     const bool warm_next = WARM && full_group && it > 0;
-    if (warm_next) warm.issue(gB, gC, row_base + l0 - TT, L);
+    if (warm_next) warm.issue(gB, gC, row_base + l0 - TT, ld);
 
     // ---- stage
     float eu[E], edl[E], egy[E];
@@ -222,8 +228,8 @@ __global__ __launch_bounds__(NT) void unitary_bwd_kernel(const UniBwdArgs p) {
           touch_uniform(cc[0]);
           sched_fence();
           if (k + 1 < NW) {
-            bn = ld_c8(gB, brow + (size_t)(k + 1) * L + g * TG);
-            cn = ld_c8(gC, brow + (size_t)(k + 1) * L + g * TG);
+            bn = ld_c8(gB, brow + (size_t)(k + 1) * ld + g * TG);
+            cn = ld_c8(gC, brow + (size_t)(k + 1) * ld + g * TG);
           } else if (g > 0) {
             bn = ld_c8(gB, brow + (g - 1) * TG);
             cn = ld_c8(gC, brow + (g - 1) * TG);
@@ -282,7 +288,7 @@ __global__ __launch_bounds__(NT) void unitary_bwd_kernel(const UniBwdArgs p) {
         for (int k = 0; k < NW; ++k) {
           float2 bv = make_float2(0.f, 0.f), cv = make_float2(0.f, 0.f);
           const bool nok = n0 + k < N;
-          const size_t bi = brow + (size_t)k * L + t;
+          const size_t bi = brow + (size_t)k * ld + t;
           if (nok) { bv = ld_c(gB, bi); cv = ld_c(gC, bi); }
           gr[k] = fmaf(cv.x, gy, gr[k]);
           gi[k] = fmaf(-cv.y, gy, gi[k]);
@@ -324,7 +330,7 @@ __global__ __launch_bounds__(NT) void unitary_bwd_kernel(const UniBwdArgs p) {
     // (re-synchronise the regenerated state with the forward pass's checkpoint first, so that
     // its rare load is part of the same wait)
     if (active && l0 > 0 && (l0 % p.ck) == 0) {
-      load_ck(l0 / p.ck - 1, hr, hi);
+      load_ck((lbeg + l0) / p.ck - 1, hr, hi);
 #pragma unroll
       for (int k = 0; k < NW; ++k) { touch_vgpr(hr[k]); touch_vgpr(hi[k]); }
     }
@@ -337,7 +343,7 @@ __global__ __launch_bounds__(NT) void unitary_bwd_kernel(const UniBwdArgs p) {
       for (int g = 0; g < NGRP; ++g)
 #pragma unroll
         for (int k = 0; k < NW; ++k)
-          atomicAdd(red_dst + 2 * (brow + (size_t)k * L + g * TG) + red_off, rres[g * NW + k]);
+          atomicAdd(red_dst + 2 * (brow + (size_t)k * ld + g * TG) + red_off, rres[g * NW + k]);
     }
 
     // ---- epilogue: channel-wise gradients, coalesced along time
@@ -372,7 +378,7 @@ __global__ __launch_bounds__(NT) void unitary_bwd_kernel(const UniBwdArgs p) {
     for (int k = 0; k < NW; ++k) {
       const int n = n0 + k;
       if (n < N) {
-        const size_t o = (((size_t)b * D + d) * N + n) * 2;
+        const size_t o = (((size_t)vb * D + d) * N + n) * 2;
         p.dh0[o] = gr[k]; p.dh0[o + 1] = gi[k];
       }
     }

@@ -10,8 +10,12 @@
 //                at its end (the reverse recurrence alone - no states are needed for it), and q_k,
 //             2. the chain  g <- conj(q_k) g + Y_k, last segment first,
 //             3. recompute_bwd_kernel over the pairs, each from the adjoint that enters it at its end.
-// Reference semantics: the loops of extension-cpp/extension_cpp/ops.py:270-291 (complex) and :349-356
-// (real) are associative in exactly this way; the reference itself does not split.
+// The unitary scan on the vector-ALU kernels (more than 16 states, a length that is not a multiple of 4, ...)
+// splits the same way: core_fwd_kernel<VAR_UNITARY> for 1. and 3., the complex instance of adjoint_seg_kernel
+// without rho, the complex chains, and unitary_bwd_kernel over the pairs, which takes the state at the end of
+// each segment from the forward pass's checkpoints.
+// Reference semantics: the loops of extension-cpp/extension_cpp/ops.py:215-223 (unitary), :270-291 (complex)
+// and :349-356 (real) are associative in exactly this way; the reference itself does not split.
 #pragma once
 #include "scan_bwd_recompute.h"
 #include "scan_common.h"
@@ -25,7 +29,7 @@ constexpr int ADJ_NSW = 16;      // states per wavefront of adjoint_seg_kernel (
 // along time), two LDS buffers so that one barrier per tile is enough.
 template <int VAR, typename Tin, typename Tbc = Tin>
 __global__ __launch_bounds__(256) void adjoint_seg_kernel(const AdjSegArgs p) {
-  static_assert(VAR == VAR_COMPLEX || VAR == VAR_REAL, "the unitary scan has its own segment kernels");
+  static_assert(VAR == VAR_COMPLEX || VAR == VAR_REAL, "the unitary scan runs the complex instance without rho");
   constexpr int C = (VAR == VAR_REAL) ? 1 : 2;
   constexpr int E = CH * RT / 256;
   constexpr int RSTEP = 256 / RT;
@@ -83,7 +87,7 @@ __global__ __launch_bounds__(256) void adjoint_seg_kernel(const AdjSegArgs p) {
       } else {
         float sn, cs;
         fast_sincosf(ok ? p.theta[o] : 0.f, &sn, &cs);
-        const float r = expf(ok ? p.rho[o] : 0.f);
+        const float r = p.rho ? expf(ok ? p.rho[o] : 0.f) : 1.f;     // (no rho: the unitary scan, uniform)
         rec = make_float4(cs * r, sn * r, gy, 0.f);
       }
       buf[col * TS + row0 + k * RSTEP] = rec;

@@ -125,11 +125,12 @@ def unitary_aux(u, n: int, ck: int) -> Tensor:
 
 def unitary_aux_useful(b: int, d: int, n: int, l: int, ck: int, in_dtype: int, urep: int = 1) -> bool:
     """False when neither direction of the scan would touch an auxiliary buffer for this shape (the
-    vector-ALU kernels do not use it, e.g. n > 16 or inputs shared between batch elements), so that
-    the autograd wrapper does not allocate and keep b d l floats for nothing."""
+    vector-ALU kernels use it only for the segment states of a call that is split along the sequence), so
+    that the autograd wrapper does not allocate and keep a buffer for nothing."""
     lib = _lib.load()
     return bool(lib.aussm_unitary_kernel_mode(0, b, d, n, l, ck, in_dtype, urep, 1)
-                or lib.aussm_unitary_kernel_mode(1, b, d, n, l, ck, in_dtype, urep, 1))
+                or lib.aussm_unitary_kernel_mode(1, b, d, n, l, ck, in_dtype, urep, 1)
+                or lib.aussm_unitary_split_segments(b, d, n, l, ck) > 1)
 
 
 def unitary_fwd_raw(u, delta, theta, Bri, Cri, D=None, z=None, h0=None, want_state=False, ck=0, aux=None, ck_arg=0):
@@ -248,7 +249,9 @@ def unitary_scan(u: Tensor, delta: Tensor, theta: Tensor, Bc: Tensor, Cc: Tensor
         # matrix-core kernels, segment states of a launch that is split along L); no checkpoints are kept
         lib = _lib.load()
         ck = unitary_ck(b, d, n, l)
-        work = lib.aussm_unitary_aux_floats(b, d, n, l, ck) > b * d * l + _lib.AUX_PAD
+        # (the buffer of a shape that the matrix-core kernels serve starts with b d l floats that only a backward
+        # call would read; anything beyond them - segment states, operand images - is workspace of this call)
+        work = lib.aussm_unitary_aux_floats(b, d, n, l, ck) - _lib.AUX_PAD not in (0, b * d * l)
         aux = unitary_aux(theta, n, ck) if (work and u.shape[0] == b) else None
         y, hL, _ = unitary_fwd_raw(u, delta, theta, Bri, Cri, D, z, h0r, want_state=return_last_state,
                                    ck=0, aux=aux, ck_arg=ck if aux is not None else 0)

@@ -155,6 +155,9 @@ int aussm_unitary_bwd(const float* dy, const float* dhL,
  *    ssm_adaptive_unitary_forward.cu:122-162 one level up); the segment states live behind the
  *    per-(b,d,l) part of the buffer, during the call only.  Each call writes there: two calls
  *    that share one buffer must not overlap.  aussm_set_option(AUSSM_OPT_SPLIT_CAP, 0) switches the split off.
+ *    The vector-ALU kernels (more than 16 states, L not a multiple of 4, shared inputs, ...) split
+ *    the same way, with their own kernels for the segment states; the buffer of a shape that only
+ *    they serve has no per-(b,d,l) part and no operand images.
  * urep (>= 1, divides B): u and delta are [B / urep, D, L] and shared by urep consecutive batch
  * elements (theta, z, y, dy and every gradient stay [B, D, L]).  This is how the drop-in operator
  * runs its n states per channel, each with its own phase, as n batch elements of one launch without
@@ -167,7 +170,7 @@ size_t aussm_unitary_aux_floats(int B, int D, int N, int L, int ck);
  * 0 vector-ALU kernels, 2 / 3 / 5 matrix-core kernels that build their operands themselves,
  * 6 matrix-core kernels on operands prepared by a pre-pass.  have_aux: the call gets an auxiliary
  * buffer.  A caller can skip allocating that buffer when both directions answer 0 (the vector-ALU
- * kernels neither fill nor read it) and aussm_unitary_split_segments() answers 1. */
+ * kernels use it for the segment states of a split call only) and aussm_unitary_split_segments() answers 1. */
 int aussm_unitary_kernel_mode(int backward, int B, int D, int N, int L, int ck, int in_dtype, int urep, int have_aux);
 
 /* Number of segments a call of this shape is split into along L when it is given an auxiliary

@@ -72,12 +72,23 @@ def test_argument_checks_without_a_device():
     # few (batch, channel) pairs and a long sequence: room for the states of 64 segments of 256 steps
     assert lib.aussm_unitary_aux_floats(4, 256, 16, 16384, 256) == (4 * 256 * 16384 + 64 + 4 * 64 * 256 * (2 * 16 + 2)
                                                                     + img(4, 16384))
-    # ... which needs whole checkpoint blocks per segment, and states the matrix-core kernels serve
-    assert lib.aussm_unitary_aux_floats(4, 256, 16, 16384 + 4, 256) == 4 * 256 * (16384 + 4) + 64 + img(4, 16388)
+    # ... which needs whole checkpoint blocks per segment, and states the matrix-core kernels serve.  Where it does
+    # not apply, the segment area is what the vector-ALU kernels' split takes: ns segments of whole checkpoint blocks
+    # (the last one ragged), (2 n + 2) floats per (batch, segment, channel), rounded up to 64 floats
+    def gen(b, d, n, l, ck):
+        want = min(64, -(-256 // (b * -(-d // 64))))
+        ls = -(-(-(-l // want)) // ck) * ck
+        return -(-(b * -(-l // ls) * d * (2 * n + 2)) // 64) * 64
+    assert gen(4, 256, 16, 16388, 256) == 4 * 13 * 256 * 34
+    assert lib.aussm_unitary_aux_floats(4, 256, 16, 16384 + 4, 256) == (4 * 256 * (16384 + 4) + 64 + gen(4, 256, 16, 16388, 256)
+                                                                        + img(4, 16388))
     # (sizes do not depend on the option table: below the state size the matrix-core kernels take by default the images
     # are still provided for, because an option can ask for those kernels)
-    assert lib.aussm_unitary_aux_floats(4, 256, 4, 16384, 256) == 4 * 256 * 16384 + 64 + img(4, 16384)
-    assert lib.aussm_unitary_aux_floats(4, 256, 32, 16384, 256) == 4 * 256 * 16384 + 64
+    assert lib.aussm_unitary_aux_floats(4, 256, 4, 16384, 256) == (4 * 256 * 16384 + 64 + gen(4, 256, 4, 16384, 256)
+                                                                   + img(4, 16384))
+    # a shape only the vector-ALU kernels serve: no per-(b,d,l) part, no images
+    assert lib.aussm_unitary_aux_floats(4, 256, 32, 16384, 256) == 64 + gen(4, 256, 32, 16384, 256)
+    assert lib.aussm_unitary_aux_floats(32, 512, 32, 2048, 256) == 64
     lib.aussm_ssm_adaptive_unitary_workspace_floats.restype = ctypes.c_size_t
     w0 = lib.aussm_ssm_adaptive_unitary_workspace_floats(32, 256, 16, 720, 1)
     assert lib.aussm_set_option(5, 64) == 0 and lib.aussm_ssm_adaptive_unitary_workspace_floats(32, 256, 16, 720, 1) == w0
@@ -90,6 +101,8 @@ def test_argument_checks_without_a_device():
     assert lib.aussm_unitary_split_segments(16, 128, 16, 1024, 256) == 4
     assert lib.aussm_unitary_split_segments(16, 128, 16, 1024, 128) == 8
     assert lib.aussm_unitary_split_segments(32, 512, 16, 2048, 256) == 1
+    assert lib.aussm_unitary_split_segments(4, 256, 32, 16384, 256) == 16      # vector-ALU kernels: their own split
+    assert lib.aussm_unitary_split_segments(4, 256, 16, 16386, 256) == 13
     rc = lib.aussm_unitary_fwd_aux(one, one, one, one, one, null, null, null, one, null, null, ctypes.c_void_p(260),
                                    1, 1, 1, 32, 32, 0, 1, null)
     assert rc == -5

@@ -155,7 +155,57 @@ def test_sequence_split_over_workgroups(B, D, N, L, cap):
         _close(gt, wh.cpu(), k + " (split vs whole)", tol=2e-5)
 
 
-@pytest.mark.parametrize("B,D,N,L", [(2, 80, 16, 200), (1, 64, 7, 64), (1, 64, 16, 1024)])   # the last one is split along L
+@pytest.mark.parametrize("B,D,N,L,force", [
+    (1, 64, 32, 1024, False),      # more than 16 states
+    (2, 70, 24, 1000, False),      # ... ragged channel group, a last segment shorter than the others
+    (1, 40, 16, 1026, False),      # a length that is not a multiple of 4
+    (2, 33, 64, 777, False),       # odd everything
+    (1, 64, 16, 1024, True),       # a shape of the matrix-core kernels sent to the vector-ALU ones by option
+    (1, 64, 4, 2048, False),       # few states: the vector-ALU kernels by default
+])
+def test_vector_alu_kernels_split_along_the_sequence(B, D, N, L, force):
+    """The unitary scan on the vector-ALU kernels splits like the complex and real scans do: outputs, final state
+    and every gradient, with a carried-in state and an upstream gradient of the final state, against the CPU
+    oracle and against the same call with the split switched off."""
+    from aussm_amd import scan, _lib
+    lib = _lib.load()
+    ck = scan.unitary_ck(B, D, N, L)
+    assert lib.aussm_unitary_split_segments(B, D, N, L, ck) > 1, "the shape is meant to split"
+    p = _inputs(B, D, N, L, 5 + L + D, False)
+    g = torch.Generator().manual_seed(10)
+    dh = torch.complex(torch.randn(B, D, N, generator=g), torch.randn(B, D, N, generator=g))
+
+    def run(fn, dev):
+        lv = [p[k].clone().to(dev).requires_grad_(True) for k in NAMES]
+        h0 = p["h0"].clone().to(dev).requires_grad_(True)
+        y, hL = fn(*lv, None, h0)
+        loss = (y * p["dy"].to(dev)).sum() + (torch.view_as_real(hL) * torch.view_as_real(dh.to(dev))).sum()
+        loss.backward()
+        return [y.detach(), hL.detach()] + [t.grad for t in lv] + [h0.grad]
+
+    names = ("y", "hL") + tuple("d" + k for k in NAMES) + ("dh0",)
+    want = run(lambda *a: O.unitary_core_loop(*a), "cpu")
+    print(f"case vector-ALU split B={B} D={D} N={N} L={L} force={force}", flush=True)
+    forced = {"unitary_fwd": 0, "unitary_bwd": 0} if force else {}
+    with _opts(**forced):
+        assert lib.aussm_unitary_kernel_mode(0, B, D, N, L, ck, 0, 1, 1) == 0 and lib.aussm_unitary_kernel_mode(1, B, D, N, L, ck, 0, 1, 1) == 0
+        got = run(lambda *a: scan.unitary_scan(*a, return_last_state=True), "cuda")
+        torch.cuda.synchronize()
+    with _opts(split_cap=0, **forced):
+        whole = run(lambda *a: scan.unitary_scan(*a, return_last_state=True), "cuda")
+        torch.cuda.synchronize()
+    for k, w, gt, wh in zip(names, want, got, whole):
+        _close(gt, w, k, tol=1e-4)
+        _close(gt, wh.cpu(), k + " (split vs whole)", tol=2e-5)
+    # ... and without gradients (no checkpoints; the buffer is workspace only)
+    with torch.no_grad():
+        y, hL = scan.unitary_scan(*[p[k].cuda() for k in NAMES], None, p["h0"].cuda(), return_last_state=True)
+    _close(y, want[0], "y (no grad)", tol=1e-4)
+    _close(hL, want[1], "hL (no grad)", tol=1e-4)
+
+
+# (the third one is split along L on the matrix-core kernels, the fourth on the vector-ALU kernels)
+@pytest.mark.parametrize("B,D,N,L", [(2, 80, 16, 200), (1, 64, 7, 64), (1, 64, 16, 1024), (1, 64, 32, 1024)])
 def test_bf16_inputs_equal_the_float_run_on_the_same_values(B, D, N, L):
     """bfloat16 u / delta / B / C are widened exactly inside the matrix-core kernels: outputs and
     (float32) gradients must agree with the float32 call on the same, already rounded, values to
