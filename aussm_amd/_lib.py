@@ -47,6 +47,8 @@ _SIGNATURES = {
     "aussm_causal_conv1d_bwd": [_P] * 6 + [_I] * 4 + [_LL] * 2 + [_P],
     "aussm_swap_last2": [_P] * 2 + [_I] * 3 + [_LL] * 2 + [_P],
     "aussm_swap_last2_act": [_P] * 4 + [_I] * 3 + [_LL] * 4 + [_I] * 2 + [_P],
+    "aussm_gate_fwd": [_P] * 3 + [ctypes.c_size_t, _P],
+    "aussm_gate_bwd": [_P] * 5 + [ctypes.c_size_t, _P],
     "aussm_hbm_probe": [_P] * 5 + [_I] * 4 + [_P],
     "aussm_ssm_adaptive_unitary_fwd": [_P] * 16 + [_I] * 4 + [_P],
     "aussm_ssm_adaptive_unitary_bwd": [_P] * 30 + [_I] * 4 + [_P],

@@ -245,6 +245,16 @@ int run_conv_bwd(const ConvArgs& a, hipStream_t s) {
   return launch_status();
 }
 
+int run_gate(const float* dy, const float* ypre, const float* z, float* out, float* dz, size_t n, hipStream_t s) {
+  const size_t blocks = (n + 1023) / 1024;
+  const dim3 grid((unsigned)(blocks < 8192 ? blocks : 8192));
+  auto off16 = [](const void* q) { return q && (reinterpret_cast<uintptr_t>(q) & 15) != 0; };
+  const int vec = !(off16(dy) || off16(ypre) || off16(z) || off16(out) || off16(dz));
+  if (dz) hipLaunchKernelGGL(gate_bwd_kernel, grid, dim3(256), 0, s, dy, ypre, z, out, dz, n, vec);
+  else hipLaunchKernelGGL(gate_fwd_kernel, grid, dim3(256), 0, s, ypre, z, out, n, vec);
+  return launch_status();
+}
+
 int run_swap_last2(const SwapArgs& a, int B, hipStream_t s) {
   hipLaunchKernelGGL(swap_last2_kernel, dim3((unsigned)((a.C + 31) / 32), (unsigned)((a.R + 31) / 32), (unsigned)B), dim3(256), 0, s, a);
   return launch_status();

@@ -34,6 +34,8 @@ int run_hbm_probe(const float* a, const float* b, const float* c, float* o1, flo
 int run_conv_fwd(const ConvArgs& a, hipStream_t s);
 int run_conv_bwd(const ConvArgs& a, hipStream_t s);
 int run_swap_last2(const SwapArgs& a, int B, hipStream_t s);
+// dz null: out = ypre silu(z); else out = dy silu(z), dz = dy ypre silu'(z)
+int run_gate(const float* dy, const float* ypre, const float* z, float* out, float* dz, size_t n, hipStream_t s);
 
 // ---- k_xdl.hip: matrix-core unitary scans that prepare their operands themselves, and the
 // kernels of the split along L.  mode: operand pieces (2, 3; backward also 5 = three everywhere).

@@ -47,4 +47,40 @@ __global__ __launch_bounds__(256) void swap_last2_kernel(const SwapArgs p) {
   }
 }
 
+// The scans' output gate  y = y_pre silu(z)  (extension-cpp/extension_cpp/ops.py:226) and its two gradients
+//     dy_pre = dy silu(z),   dz = dy y_pre silu'(z)
+// as one pass each over contiguous tensors of n floats (vec: all of them 16-byte aligned), for the scan
+// whose backward kernel takes the gradient of the ungated output.
+__global__ __launch_bounds__(256) void gate_fwd_kernel(const float* __restrict__ ypre, const float* __restrict__ z,
+                                                       float* __restrict__ y, size_t n, int vec) {
+  const size_t stride = (size_t)gridDim.x * 256 * 4;
+  for (size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4; i < n; i += stride) {
+    if (vec && i + 4 <= n) {
+      const float4 a = *reinterpret_cast<const float4*>(ypre + i), g = *reinterpret_cast<const float4*>(z + i);
+      *reinterpret_cast<float4*>(y + i) = make_float4(a.x * siluf_(g.x), a.y * siluf_(g.y), a.z * siluf_(g.z), a.w * siluf_(g.w));
+    } else {
+      for (size_t j = i; j < n && j < i + 4; ++j) y[j] = ypre[j] * siluf_(z[j]);
+    }
+  }
+}
+__global__ __launch_bounds__(256) void gate_bwd_kernel(const float* __restrict__ dy, const float* __restrict__ ypre,
+                                                       const float* __restrict__ z, float* __restrict__ dypre,
+                                                       float* __restrict__ dz, size_t n, int vec) {
+  const size_t stride = (size_t)gridDim.x * 256 * 4;
+  for (size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4; i < n; i += stride) {
+    if (vec && i + 4 <= n) {
+      const float4 g = *reinterpret_cast<const float4*>(dy + i), a = *reinterpret_cast<const float4*>(ypre + i),
+                   v = *reinterpret_cast<const float4*>(z + i);
+      *reinterpret_cast<float4*>(dypre + i) = make_float4(g.x * siluf_(v.x), g.y * siluf_(v.y), g.z * siluf_(v.z), g.w * siluf_(v.w));
+      *reinterpret_cast<float4*>(dz + i) = make_float4(g.x * a.x * dsiluf_(v.x), g.y * a.y * dsiluf_(v.y),
+                                                       g.z * a.z * dsiluf_(v.z), g.w * a.w * dsiluf_(v.w));
+    } else {
+      for (size_t j = i; j < n && j < i + 4; ++j) {
+        dypre[j] = dy[j] * siluf_(z[j]);
+        dz[j] = dy[j] * ypre[j] * dsiluf_(z[j]);
+      }
+    }
+  }
+}
+
 }  // namespace aussm

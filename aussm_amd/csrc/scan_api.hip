@@ -656,6 +656,21 @@ int aussm_swap_last2_act(const float* x, const float* bias, const float* pre, fl
   return run_swap_last2(a, B, (hipStream_t)stream);
 }
 
+int aussm_gate_fwd(const float* y_pre, const float* z, float* y, size_t n, void* stream) {
+  if (!y_pre || !z || !y) return AUSSM_E_NULL;
+  if (n < 1) return AUSSM_E_SHAPE;
+  if (misaligned(y_pre, 4) || misaligned(z, 4) || misaligned(y, 4)) return AUSSM_E_ALIGN;
+  return run_gate(nullptr, y_pre, z, y, nullptr, n, (hipStream_t)stream);
+}
+
+int aussm_gate_bwd(const float* dy, const float* y_pre, const float* z, float* dy_pre, float* dz, size_t n, void* stream) {
+  if (!dy || !y_pre || !z || !dy_pre || !dz) return AUSSM_E_NULL;
+  if (n < 1) return AUSSM_E_SHAPE;
+  if (misaligned(dy, 4) || misaligned(y_pre, 4) || misaligned(z, 4) || misaligned(dy_pre, 4) || misaligned(dz, 4))
+    return AUSSM_E_ALIGN;
+  return run_gate(dy, y_pre, z, dy_pre, dz, n, (hipStream_t)stream);
+}
+
 // ---- the reference's operator extension_cpp::ssm_adaptive_unitary as fused kernels (dropin.h)
 
 // blocks of 16 states per channel, one per wavefront: 1, 2 or 4 (they have to divide the wavefronts of a workgroup)

@@ -24,7 +24,6 @@ from __future__ import annotations
 from typing import Optional
 
 import torch
-import torch.nn.functional as F
 
 from . import _lib
 from ._lib import check, ptr
@@ -212,6 +211,30 @@ class _UnitaryScanFn(torch.autograd.Function):
         return (du.to(u.dtype), ddelta.to(delta.dtype), dtheta, dB.to(Bri.dtype), dC.to(Cri.dtype), dD, dh0)
 
 
+class _GateFn(torch.autograd.Function):
+    """y = y_pre silu(z) behind the unitary scan, whose backward kernels take the gradient of the ungated output:
+    one pass forward, one backward (dy_pre = dy silu(z), dz = dy y_pre silu'(z)); reference
+    extension-cpp/extension_cpp/ops.py:226."""
+
+    @staticmethod
+    def forward(ctx, y_pre, z):
+        lib = _lib.load()
+        y_pre = y_pre.contiguous()
+        y = torch.empty_like(y_pre)
+        check(lib.aussm_gate_fwd(ptr(y_pre), ptr(z), ptr(y), y_pre.numel(), _stream()), "aussm_gate_fwd")
+        ctx.save_for_backward(y_pre, z)
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        lib = _lib.load()
+        y_pre, z = ctx.saved_tensors
+        dy = dy.contiguous()
+        dy_pre, dz = torch.empty_like(y_pre), torch.empty_like(z)
+        check(lib.aussm_gate_bwd(ptr(dy), ptr(y_pre), ptr(z), ptr(dy_pre), ptr(dz), dy.numel(), _stream()), "aussm_gate_bwd")
+        return dy_pre, dz
+
+
 def unitary_scan(u: Tensor, delta: Tensor, theta: Tensor, Bc: Tensor, Cc: Tensor, D: Optional[Tensor] = None,
                  z: Optional[Tensor] = None, h0: Optional[Tensor] = None, return_last_state: bool = False):
     """Adaptive-unitary scan.  u, delta, theta, z: (b, d, l); Bc, Cc: (b, n, l) complex64 (or
@@ -243,7 +266,7 @@ def unitary_scan(u: Tensor, delta: Tensor, theta: Tensor, Bc: Tensor, Cc: Tensor
     if needs_grad:
         y, hL = _UnitaryScanFn.apply(u, delta, theta, Bri, Cri, D, h0r)
         if z is not None:
-            y = y * F.silu(z)
+            y = _GateFn.apply(y, z)
     else:
         # no backward pass: the auxiliary buffer serves as workspace only (prepared operands of the
         # matrix-core kernels, segment states of a launch that is split along L); no checkpoints are kept

@@ -312,6 +312,16 @@ int aussm_swap_last2_act(const float* x, const float* bias, const float* pre, fl
                          long long xs_b, long long xs_r, long long ps_b, long long ps_r, int act, int deriv,
                          void* stream);
 
+/* The scans' output gate and its gradients as one pass each over contiguous tensors of n floats (16-byte
+ * aligned ones take the wide path; `y = y * F.silu(z)`, extension-cpp/extension_cpp/ops.py:226, and what autograd derives from it):
+ *   aussm_gate_fwd:  y = y_pre silu(z)
+ *   aussm_gate_bwd:  dy_pre = dy silu(z),  dz = dy y_pre silu'(z)
+ * The complex and real scans and the fused operator apply and differentiate their gate inside their kernels;
+ * the unitary core scan's backward kernels take the gradient of the ungated output, and a gated call with
+ * gradients runs these two around them (in place is allowed: y may be y_pre, dy_pre may be dy). */
+int aussm_gate_fwd(const float* y_pre, const float* z, float* y, size_t n, void* stream);
+int aussm_gate_bwd(const float* dy, const float* y_pre, const float* z, float* dy_pre, float* dz, size_t n, void* stream);
+
 /* ---------------------------------------------------------------------------------------
  * The reference's custom operator itself, as two calls: what
  *   torch.ops.extension_cpp.ssm_adaptive_unitary           (12 tensors -> y, next_hid_real, next_hid_imag)

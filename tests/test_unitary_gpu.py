@@ -125,3 +125,25 @@ def test_inputs_shared_by_consecutive_batch_elements(b, r, d, n, l):
             w, g = torch.view_as_real(w), torch.view_as_real(g)
         scale = max(1.0, float(w.abs().max()))
         torch.testing.assert_close(g.cpu() / scale, w / scale, atol=1e-4, rtol=1e-4, msg=lambda m: f"{name}: {m}")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("n,offset", [(4096, 0), (1027, 0), (1000, 1), (5, 3)])
+def test_gate_kernels(n, offset):
+    """aussm_gate_fwd / _bwd (y = y_pre silu(z) and its two gradients) against the formula in float64, aligned
+    and unaligned views, lengths that are not a multiple of four."""
+    from aussm_amd import scan, _lib
+    lib = _lib.load()
+    g = torch.Generator().manual_seed(n + offset)
+    base = [torch.randn(n + 8, generator=g).cuda() for _ in range(3)]
+    ypre, z, dy = (t[offset:offset + n] for t in base)
+    y, dyp, dz = (torch.empty(n + 8, device="cuda")[offset:offset + n] for _ in range(3))
+    print(f"case gate kernels n={n} offset={offset}", flush=True)
+    scan.check(lib.aussm_gate_fwd(scan.ptr(ypre), scan.ptr(z), scan.ptr(y), n, scan._stream()), "gate_fwd")
+    scan.check(lib.aussm_gate_bwd(scan.ptr(dy), scan.ptr(ypre), scan.ptr(z), scan.ptr(dyp), scan.ptr(dz), n, scan._stream()), "gate_bwd")
+    torch.cuda.synchronize()
+    a, v, d = ypre.double().cpu(), z.double().cpu(), dy.double().cpu()
+    sg = torch.sigmoid(v)
+    torch.testing.assert_close(y.double().cpu(), a * v * sg, atol=1e-6, rtol=1e-6)
+    torch.testing.assert_close(dyp.double().cpu(), d * v * sg, atol=1e-6, rtol=1e-6)
+    torch.testing.assert_close(dz.double().cpu(), d * a * sg * (1 + v * (1 - sg)), atol=1e-6, rtol=1e-6)
