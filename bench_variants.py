@@ -201,7 +201,7 @@ def main():
     ap.add_argument("--systems", default="SSMau-hip,SSMau-hip-composite,mamba-hip")
     ap.add_argument("--fused", default=None, metavar="b,d,n,L", nargs="?", const="32,256,16,720",
                     help="time the fused operator (extension_cpp::ssm_adaptive_unitary and its backward operator) at a shape, "
-                         "default BASELINE configuration 4's, with its matrix-pipe roofline")
+                         "default: the hybrid model benchmark's operator shape, with its matrix-pipe roofline")
     args = ap.parse_args()
     B, D, N, L = (int(v) for v in args.shape.split(","))
 

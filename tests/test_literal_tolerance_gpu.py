@@ -7,7 +7,7 @@ Where the literal bound cannot hold element-wise - at L = 2048 outputs reach |y|
 sequential-loop oracle is itself more than 1e-4 away from the float64 one on some elements - the test
 asserts instead that the HIP result is no further from float64 than 1.5 times the float32 oracle is
 (largest absolute error), and it prints the measured largest absolute and relative errors of both and
-the number of elements outside the literal bound, which is where the figures in the design notes come
+the number of elements outside the literal bound, which is where the published figures come
 from.  The fused operator gets the same treatment at its benchmark shape on a two-batch slice, directly
 against the loop oracle of the operator (factor 2: its phases are sums over 256 channels before they are
 sums over time, and its outputs reach |y| ~ 250 there)."""
@@ -79,7 +79,7 @@ def test_forward_outputs_literal_tolerance(name, B, D, N, L, _, variant):
 
 
 def test_fused_operator_at_its_benchmark_shape_against_the_loop_oracle():
-    """Two batch elements of b=32 d=256 n=16 L=720 (BASELINE configuration 4's operator shape): the three
+    """Two batch elements of b=32 d=256 n=16 L=720 (the operator shape of the hybrid model benchmark): the three
     outputs against adaptive_unitary_op_loop in float64, and all twelve gradients against its autograd
     (gradients normalised by the oracle gradient's largest magnitude, as everywhere)."""
     import aussm_amd.ops  # noqa: F401  (registers the operators)
