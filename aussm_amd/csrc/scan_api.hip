@@ -206,8 +206,10 @@ int launch_unitary_fwd(FwdArgs a, int in_dtype, hipStream_t s, AuxLayout ws) {
   // a call that does not fill the buffer marks it as not filled, and a call that does not prepare
   // images clears the note about the ones behind the buffer
   const bool fill = a.aux && a.hck && mode >= 2;
+  // (the prepared-operand kernel clears the fill tag itself, at its end: one launch less for a forward-only call)
+  const bool clear_in_kernel = a.aux && !fill && mode == 6;
   if (a.aux)
-    if (int e = run_aux_invalidate(ws.pad, !fill, mode != 6 && ws.stamp, s)) return e;
+    if (int e = run_aux_invalidate(ws.pad, !fill && !clear_in_kernel, mode != 6 && ws.stamp, s)) return e;
   if (!fill) a.aux = nullptr;
   if (!mode) {
     // vector-ALU kernel; with a segment area and few (batch, channel group) pairs, split along the sequence
@@ -250,7 +252,7 @@ int launch_unitary_fwd(FwdArgs a, int in_dtype, hipStream_t s, AuxLayout ws) {
     const bool with_bwd = a.hck != nullptr;
     PrepArgs pa{a.Bm, a.Cm, ws.fimg, with_bwd ? ws.img : nullptr, a.N, L, (L + XT - 1) / XT, nullptr, ImgStamp{}};
     if (int e = run_px_prep(pa, B, in_dtype, s)) return e;
-    const ImgNote note{ws.stamp, img_stamp(a.Bm, a.Cm, B, a.N, L, in_dtype, with_bwd)};
+    const ImgNote note{ws.stamp, img_stamp(a.Bm, a.Cm, B, a.N, L, in_dtype, with_bwd), clear_in_kernel ? ws.pad : nullptr};
     return run_px_fwd(a, ws.fimg, note, in_dtype, s);
   }
   return run_xdl_fwd(mode, a, in_dtype, s);

@@ -178,8 +178,9 @@ struct PrepArgs {
   ImgStamp want;
 };
 
-// Where a forward kernel that ran on freshly prepared images records what they were made from
-struct ImgNote { uint32_t* dst; ImgStamp stamp; };
+// Where a forward kernel that ran on freshly prepared images records what they were made from; clear: the
+// buffer's fill tag, set to zero by a call that is given the buffer and does not fill it (or null)
+struct ImgNote { uint32_t* dst; ImgStamp stamp; float* clear; };
 
 constexpr int CONV_MAX_K = 8;
 constexpr int CONV_ROWS = 128;   // (b, l) rows per workgroup of the weight-gradient kernel

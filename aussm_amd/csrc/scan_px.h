@@ -600,6 +600,7 @@ __global__ __launch_bounds__(512) void unitary_fwd_px_kernel(const FwdArgs p, co
   if (p.aux && blockIdx.x == 0 && tid == 0) p.aux[(size_t)(p.B / p.ns) * D * p.ld] = __uint_as_float(p.auxtag);
   // (the pre-pass that wrote the images has finished: this kernel read them)
   if (note.dst && blockIdx.x == 0 && tid < 8) note.dst[tid] = note.stamp.w[tid];
+  if (note.clear && blockIdx.x == 0 && tid == 0) *note.clear = 0.0f;
   if (p.hL && dok && hf == 0) {
     const f4 hr = s_h[0][cg][0][lane], hi = s_h[0][cg][1][lane];    // state after the last (possibly padding) chunk
 #pragma unroll
