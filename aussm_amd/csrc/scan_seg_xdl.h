@@ -22,8 +22,10 @@ namespace aussm {
 // ADJ = false: Z of each segment, chunks in forward order,  H <- P_T (H + B^T V).
 // ADJ = true:  Y of each segment, chunks in reverse order,  A <- conj(P_T) A + conj(C)^T Q.
 // Requires N <= 16, L % 4 == 0, 16-byte aligned tensors.  Tin: float or bf16_t (u, delta, B, C).
+// Four wavefronts per SIMD (128 registers): the launch of a split call (1024 light workgroups for 64 fine segments
+// of a batch of 4 x 4 channel groups) then fits the chip in one round instead of one and a third.
 template <int NP, bool ADJ, typename Tin = float>
-__global__ __launch_bounds__(256) void unitary_seg_state_kernel(const SegArgs p) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) void unitary_seg_state_kernel(const SegArgs p) {
   // row n: M[t(g, e)][n], real and imaginary parts (the imaginary part negated for ADJ: conj(C))
   __shared__ u4 s_mr[2][NP][XN * 4];
   __shared__ u4 s_mi[2][NP][XN * 4];
@@ -145,7 +147,7 @@ __global__ __launch_bounds__(256) void unitary_seg_state_kernel(const SegArgs p)
     for (int e = 0; e < 8; ++e) {
       const float ph = th[e >> 2][e & 3] + ((e >> 2) ? off_b : off_a);
       float sn, cs;
-      sincos_small(ph, &sn, &cs);
+      sincos_small_hw(ph, &sn, &cs);
       xr[e] = cs * x[e];        // x conj(P)
       xi[e] = -sn * x[e];
       if (e == 7) { c7 = cs; s7 = sn; }
