@@ -42,16 +42,17 @@ int run_seg_state(bool adjoint, const SegArgs& a, int in_dtype, unsigned grid, h
   return launch_status();
 }
 
-// (the chains are latency-bound and few: one wavefront per workgroup spreads them over the compute units)
 int run_seg_carry_fwd(float* seg, const float* ptot, const float* h0, float* hL, int B, int D, int N, int nf, hipStream_t s) {
   const size_t nst = (size_t)B * D * N;
-  hipLaunchKernelGGL(seg_carry_fwd_kernel, dim3((unsigned)((nst + 63) / 64)), dim3(64), 0, s, seg, ptot, h0, hL, B, D, N, nf);
+  if (nf > CARRY_SUBS * CARRY_RUN) return -2;
+  hipLaunchKernelGGL(seg_carry_kernel<false>, dim3((unsigned)((nst + 31) / 32)), dim3(32 * CARRY_SUBS), 0, s, seg, ptot, h0, hL, B, D, N, nf);
   return launch_status();
 }
 
 int run_seg_carry_bwd(float* seg, const float* ptot, const float* dhL, float* dh0, int B, int D, int N, int nf, hipStream_t s) {
   const size_t nst = (size_t)B * D * N;
-  hipLaunchKernelGGL(seg_carry_bwd_kernel, dim3((unsigned)((nst + 63) / 64)), dim3(64), 0, s, seg, ptot, dhL, dh0, B, D, N, nf);
+  if (nf > CARRY_SUBS * CARRY_RUN) return -2;
+  hipLaunchKernelGGL(seg_carry_kernel<true>, dim3((unsigned)((nst + 31) / 32)), dim3(32 * CARRY_SUBS), 0, s, seg, ptot, dhL, dh0, B, D, N, nf);
   return launch_status();
 }
 

@@ -4,7 +4,7 @@
 //   forward   1. core_fwd_kernel over the pairs from a zero state, outputs off: end state Z_k of every
 //                segment and the product q_k of its a_l (FwdArgs::ptot),
 //             2. the chain  h <- q_k h + Z_k  over the segments of each (batch, channel, state)
-//                (seg_carry_fwd_kernel for complex states, seg_carry_real_kernel here),
+//                (seg_carry_kernel for complex states, seg_carry_real_kernel here),
 //             3. core_fwd_kernel over the pairs, each from the state that enters it;
 //   backward  1. adjoint_seg_kernel: adjoint Y_k of the state entering every segment from a zero adjoint
 //                at its end (the reverse recurrence alone - no states are needed for it), and q_k,

@@ -204,73 +204,69 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
   }
 }
 
-constexpr int SEG_BATCH = 16;
-
-// Chains the segments of one (batch, channel, state): on entry seg[k] holds Z_k, on return the
-// state that enters segment k; the state after the last segment goes to hL (if wanted).
-__global__ __launch_bounds__(64) void seg_carry_fwd_kernel(float* __restrict__ seg, const float* __restrict__ ptot,
-                                     const float* __restrict__ h0, float* __restrict__ hL,
-                                     int B, int D, int N, int ns) {
-  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (idx >= (size_t)B * D * N) return;
-  const int n = (int)(idx % N);
-  const int d = (int)((idx / N) % D);
-  const int b = (int)(idx / ((size_t)N * D));
-  float hr = h0 ? h0[idx * 2] : 0.0f, hi = h0 ? h0[idx * 2 + 1] : 0.0f;
-  // batches of SEG_BATCH segments: all loads of a batch first (independent of the chain), then the chain
-  for (int k0 = 0; k0 < ns; k0 += SEG_BATCH) {
-    float2 z[SEG_BATCH], q[SEG_BATCH];
+// Chains the segments of one (batch, channel, state).  Forward (ADJ false): on entry seg[k] holds Z_k, on return the
+// state that enters segment k; the state after the last segment goes to `last` (if wanted); `first` is the state
+// before the first one (or null).  ADJ: on entry seg[k] holds Y_k, on return the adjoint that enters segment k at
+// its end, walking from the last segment with conj(q_k); `first` is the adjoint after the last segment, `last`
+// receives the adjoint of the initial state.
+// The chain is short and there are few of them (B D N), so one thread per chain leaves the chip waiting on its
+// loads: CARRY_SUBS threads share a chain - each composes its run of consecutive segments into one affine map
+// h -> Q h + Z, the maps of the runs before it (LDS) give the state that enters its run, and it walks the run
+// again writing every segment's incoming state.
+constexpr int CARRY_SUBS = 8;          // threads per chain
+constexpr int CARRY_RUN = 16;          // segments per thread at most: chains of up to 128 segments
+template <bool ADJ>
+__global__ __launch_bounds__(32 * CARRY_SUBS) void seg_carry_kernel(float* __restrict__ seg, const float* __restrict__ ptot,
+                                                                    const float* __restrict__ first, float* __restrict__ last,
+                                                                    int B, int D, int N, int ns) {
+  __shared__ float4 s_map[CARRY_SUBS][32];          // (Re Q, Im Q, Re Z, Im Z) of every run
+  const int cl = threadIdx.x & 31, sub = threadIdx.x >> 5;
+  const size_t idx = (size_t)blockIdx.x * 32 + cl;
+  const bool ok = idx < (size_t)B * D * N;
+  const size_t ic = ok ? idx : 0;
+  const int n = (int)(ic % N);
+  const int d = (int)((ic / N) % D);
+  const int b = (int)(ic / ((size_t)N * D));
+  const int per = (ns + CARRY_SUBS - 1) / CARRY_SUBS;
+  auto mul = [](float2 q, float hr, float hi) {          // q h, or conj(q) h for the adjoint
+    return ADJ ? make_float2(q.x * hr + q.y * hi, q.x * hi - q.y * hr) : make_float2(q.x * hr - q.y * hi, q.x * hi + q.y * hr);
+  };
+  float2 z[CARRY_RUN], q[CARRY_RUN];
+  size_t off[CARRY_RUN];
 #pragma unroll
-    for (int j = 0; j < SEG_BATCH; ++j) {
-      const int k = k0 + j < ns ? k0 + j : ns - 1;
-      const size_t v = ((size_t)b * ns + k) * D + d;
-      z[j] = *reinterpret_cast<const float2*>(seg + (v * N + n) * 2);
-      q[j] = *reinterpret_cast<const float2*>(ptot + v * 2);
-    }
+  for (int j = 0; j < CARRY_RUN; ++j) {
+    const int pos = sub * per + j;
+    const bool valid = j < per && pos < ns;
+    const int k = valid ? (ADJ ? ns - 1 - pos : pos) : 0;
+    const size_t v = ((size_t)b * ns + k) * D + d;
+    off[j] = valid ? (v * N + n) * 2 : ~(size_t)0;
+    z[j] = valid ? *reinterpret_cast<const float2*>(seg + (v * N + n) * 2) : make_float2(0.f, 0.f);
+    q[j] = valid ? *reinterpret_cast<const float2*>(ptot + v * 2) : make_float2(1.f, 0.f);
+  }
+  float Qr = 1.f, Qi = 0.f, Zr = 0.f, Zi = 0.f;
 #pragma unroll
-    for (int j = 0; j < SEG_BATCH; ++j) {
-      if (k0 + j < ns) {
-        const size_t v = ((size_t)b * ns + k0 + j) * D + d;
-        *reinterpret_cast<float2*>(seg + (v * N + n) * 2) = make_float2(hr, hi);
-        const float nr = q[j].x * hr - q[j].y * hi + z[j].x, ni = q[j].x * hi + q[j].y * hr + z[j].y;
-        hr = nr; hi = ni;
-      }
+  for (int j = 0; j < CARRY_RUN; ++j) {
+    const float2 a = mul(q[j], Qr, Qi), c = mul(q[j], Zr, Zi);
+    Qr = a.x; Qi = a.y; Zr = c.x + z[j].x; Zi = c.y + z[j].y;
+  }
+  s_map[sub][cl] = make_float4(Qr, Qi, Zr, Zi);
+  __syncthreads();
+  float hr = first ? first[ic * 2] : 0.0f, hi = first ? first[ic * 2 + 1] : 0.0f;
+  for (int s_ = 0; s_ < sub; ++s_) {
+    const float4 m = s_map[s_][cl];
+    // (the maps hold q's products already conjugated for the adjoint: plain complex multiplication here)
+    const float nr = m.x * hr - m.y * hi + m.z, ni = m.x * hi + m.y * hr + m.w;
+    hr = nr; hi = ni;
+  }
+#pragma unroll
+  for (int j = 0; j < CARRY_RUN; ++j) {
+    if (off[j] != ~(size_t)0) {
+      if (ok) *reinterpret_cast<float2*>(seg + off[j]) = make_float2(hr, hi);
+      const float2 a = mul(q[j], hr, hi);
+      hr = a.x + z[j].x; hi = a.y + z[j].y;
     }
   }
-  if (hL) { hL[idx * 2] = hr; hL[idx * 2 + 1] = hi; }
-}
-
-// The same for the adjoint, last segment first: on entry seg[k] holds Y_k, on return the adjoint
-// that enters segment k at its end; the adjoint of the initial state goes to dh0 (if wanted).
-__global__ __launch_bounds__(64) void seg_carry_bwd_kernel(float* __restrict__ seg, const float* __restrict__ ptot,
-                                     const float* __restrict__ dhL, float* __restrict__ dh0,
-                                     int B, int D, int N, int ns) {
-  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (idx >= (size_t)B * D * N) return;
-  const int n = (int)(idx % N);
-  const int d = (int)((idx / N) % D);
-  const int b = (int)(idx / ((size_t)N * D));
-  float ar = dhL ? dhL[idx * 2] : 0.0f, ai = dhL ? dhL[idx * 2 + 1] : 0.0f;
-  for (int k0 = ns - 1; k0 >= 0; k0 -= SEG_BATCH) {
-    float2 y[SEG_BATCH], q[SEG_BATCH];
-#pragma unroll
-    for (int j = 0; j < SEG_BATCH; ++j) {
-      const int k = k0 - j >= 0 ? k0 - j : 0;
-      const size_t v = ((size_t)b * ns + k) * D + d;
-      y[j] = *reinterpret_cast<const float2*>(seg + (v * N + n) * 2);
-      q[j] = *reinterpret_cast<const float2*>(ptot + v * 2);
-    }
-#pragma unroll
-    for (int j = 0; j < SEG_BATCH; ++j) {
-      if (k0 - j >= 0) {
-        const size_t v = ((size_t)b * ns + k0 - j) * D + d;
-        *reinterpret_cast<float2*>(seg + (v * N + n) * 2) = make_float2(ar, ai);
-        const float nr = q[j].x * ar + q[j].y * ai + y[j].x, ni = q[j].x * ai - q[j].y * ar + y[j].y;
-        ar = nr; ai = ni;
-      }
-    }
-  }
-  if (dh0) { dh0[idx * 2] = ar; dh0[idx * 2 + 1] = ai; }
+  if (last && ok && sub == CARRY_SUBS - 1) { last[idx * 2] = hr; last[idx * 2 + 1] = hi; }
 }
 
 }  // namespace aussm
