@@ -34,7 +34,18 @@ namespace aussm {
 template <typename Tin, bool CHECK>
 __global__ __launch_bounds__(256) void unitary_px_prep_kernel(const PrepArgs p) {
   constexpr int NP = PX_NP;
-  __shared__ XbBC<NP> s_bc;
+  // (the records the images do not hold - [Ci, Cr] and [-Bi, Br] - are formed in registers where the products
+  // need them: 48 KiB instead of 60 per workgroup, three workgroups per compute unit instead of two, so that one
+  // workgroup's stores - half of its life - overlap the others' loads and products)
+  struct PrepBC {
+    u4 cs_r[NP][XT * 4];   // row t: [ Cr[4g..], -Ci[4g..] ]
+    u4 bs[NP][XT * 4];     // row s: [ Br[4g..],  Bi[4g..] ]
+    u4 bt_r[NP][XN * 4];   // row n: Br[t(g,e)][n]
+    u4 bt_i[NP][XN * 4];
+    u4 ct_r[NP][XN * 4];   // row n: Cr[t(g,e)][n]
+    u4 ct_i[NP][XN * 4];
+  };
+  __shared__ PrepBC s_bc;
   __shared__ XbG<NP> s_g;
 
   // the images a forward call left behind are still those of these tensors: nothing to do
@@ -71,19 +82,13 @@ __global__ __launch_bounds__(256) void unitary_px_prep_kernel(const PrepArgs p) 
       x[k] = ok ? r.re() : 0.0f;
       x[4 + k] = ok ? r.im() : 0.0f;
     }
-    u4 pc[NP], pi[NP];
+    u4 pc[NP];
     split8<NP>(sk, x, pc);                  // [re, im]
-    rot_i<NP>(pc, pi);                      // [-im, re]
     const int o = xrec(m1_t, m1_g, XT);
 #pragma unroll
     for (int q = 0; q < NP; ++q) {
-      if (m1_isB) {
-        s_bc.bs[q][o] = pc[q];
-        s_bc.bs_c[q][o] = pi[q];
-      } else {
-        s_bc.cs_r[q][o] = u4{pc[q][0], pc[q][1], pc[q][2] ^ 0x80008000u, pc[q][3] ^ 0x80008000u};   // [re, -im]
-        s_bc.cs_i[q][o] = u4{pc[q][2], pc[q][3], pc[q][0], pc[q][1]};                                // [im, re]
-      }
+      if (m1_isB) s_bc.bs[q][o] = pc[q];
+      else s_bc.cs_r[q][o] = u4{pc[q][0], pc[q][1], pc[q][2] ^ 0x80008000u, pc[q][3] ^ 0x80008000u};   // [re, -im]
     }
   }
   {
@@ -124,7 +129,8 @@ __global__ __launch_bounds__(256) void unitary_px_prep_kernel(const PrepArgs p) 
     u4 a[NP], cr[NP], ci[NP];
     ldrec<NP>(s_bc.bs, xrec(16 * gst + dl, g, XT), a);
     ldrec<NP>(s_bc.cs_r, xrec(16 * gtt + dl, g, XT), cr);
-    ldrec<NP>(s_bc.cs_i, xrec(16 * gtt + dl, g, XT), ci);
+#pragma unroll
+    for (int q = 0; q < NP; ++q) ci[q] = u4{cr[q][2] ^ 0x80008000u, cr[q][3] ^ 0x80008000u, cr[q][0], cr[q][1]};   // [im, re]
     auto put_half = [&](u4 (*pr)[XT * 4], u4 (*pi)[XT * 4], int h, const f4& vr, const f4& vi) {
       uint32_t r0[NP], r1[NP], i0[NP], i1[NP];
       split2<NP>(sk, vr[0], vr[1], r0);
@@ -448,7 +454,11 @@ __global__ __launch_bounds__(512) void unitary_fwd_px_kernel(const FwdArgs p, co
     float vr[8], vi[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      sincos_small_hw(ph[e], &sn[e], &cs[e]);
+      // (the lane's last step through the polynomial: in lane group 3 it is the rotation of the whole chunk,
+      // which multiplies the carried state chunk after chunk - the hardware sine / cosine's 3e-7 against 9e-8
+      // would show after a few thousand steps; everywhere else an error of that size does not accumulate)
+      if (e == 7) sincos_small(ph[e], &sn[e], &cs[e]);
+      else sincos_small_hw(ph[e], &sn[e], &cs[e]);
       vr[e] = cs[e] * w[e];
       vi[e] = -sn[e] * w[e];
       uu[e] = un[e];
@@ -799,7 +809,8 @@ __global__ __launch_bounds__(512) void unitary_bwd_px_kernel(const UniBwdArgs p,
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       const float ph = th[e >> 2][e & 3] + ((e >> 2) ? off_b : off_a);
-      sincos_small_hw(ph, &sn[e], &cs[e]);
+      if (e == 7) sincos_small(ph, &sn[e], &cs[e]);       // (the chunk's rotation in lane group 3: see the forward kernel)
+      else sincos_small_hw(ph, &sn[e], &cs[e]);
       accD = fmaf(dy[e], uu[e], accD);
     }
   };

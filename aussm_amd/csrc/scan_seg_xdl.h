@@ -147,7 +147,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     for (int e = 0; e < 8; ++e) {
       const float ph = th[e >> 2][e & 3] + ((e >> 2) ? off_b : off_a);
       float sn, cs;
-      sincos_small_hw(ph, &sn, &cs);
+      if (e == 7) sincos_small(ph, &sn, &cs);       // (in lane group 3 the rotation of the whole chunk: it accumulates)
+      else sincos_small_hw(ph, &sn, &cs);
       xr[e] = cs * x[e];        // x conj(P)
       xi[e] = -sn * x[e];
       if (e == 7) { c7 = cs; s7 = sn; }
