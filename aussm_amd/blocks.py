@@ -38,6 +38,49 @@ def _causal_conv(conv1d: nn.Conv1d, x: torch.Tensor, l: int) -> torch.Tensor:
     return conv1d(x.transpose(1, 2))[:, :, :l].transpose(1, 2)
 
 
+class _LinearFn(torch.autograd.Function):
+    """`F.linear` whose weight gradient is formed in slices of the (batch x length) rows.  The blocks' weight
+    gradients are products with a short result (at most 1024 x 512) and a very long sum (b l = 23040 rows for the
+    (32, 720) batches of the time-series model): as ONE product the library GEMM runs them on a few dozen workgroups
+    (measured on an MI355X: 310 us for 1024 x 256, 12 GFLOP); as a batch of `_WGRAD_SLICES` products over slices of the
+    rows, summed afterwards, the same result takes 100 us and carries a third of the rounding error."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias):
+        ctx.save_for_backward(x, weight)
+        ctx.has_bias = bias is not None
+        return F.linear(x, weight, bias)
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, weight = ctx.saved_tensors
+        n, m = weight.shape
+        dx = dw = db = None
+        if ctx.needs_input_grad[0]:
+            dx = dy @ weight
+        d2 = dy.reshape(-1, n)
+        if ctx.needs_input_grad[1]:
+            x2 = x.reshape(-1, m)
+            s = _WGRAD_SLICES
+            dw = torch.bmm(d2.reshape(s, -1, n).transpose(1, 2), x2.reshape(s, -1, m)).sum(0)
+        if ctx.has_bias and ctx.needs_input_grad[2]:
+            db = d2.sum(0)
+        return dx, dw, db
+
+
+_WGRAD_SLICES = 8
+_WGRAD_MIN_ROWS = 4096
+
+
+def _linear(layer: nn.Linear, x: torch.Tensor) -> torch.Tensor:
+    """`layer(x)`; on the GPU, for inputs of many rows, with the weight gradient of `_LinearFn`."""
+    rows = x.numel() // max(x.shape[-1], 1)
+    if (x.is_cuda and x.dtype == torch.float32 and layer.weight.dtype == torch.float32 and rows >= _WGRAD_MIN_ROWS
+            and rows % _WGRAD_SLICES == 0 and torch.is_grad_enabled() and layer.weight.requires_grad):
+        return _LinearFn.apply(x, layer.weight, layer.bias)
+    return layer(x)
+
+
 def _swap_act(x: torch.Tensor, act: str, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """`_swap(act(x + bias))` in one pass on the GPU (the elementwise step rides on the layout change)."""
     if x.is_cuda and x.dtype == torch.float32:
@@ -127,17 +170,17 @@ class MambaBlock(nn.Module):
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         (b, l, d) = x.shape
-        x_and_z = self.in_proj(x)
+        x_and_z = _linear(self.in_proj, x)
         (x, z) = x_and_z.split(split_size=[self.args.d_inner, self.args.d_inner], dim=-1)
         x = _causal_conv(self.conv1d, x, l)
         y = self.ssm_mamba(x, z)
-        return self.out_proj(y)
+        return _linear(self.out_proj, y)
 
     def ssm_mamba(self, x, z):
         (b, l, d_in) = x.shape
-        x_proj = self.x_proj(x)
+        x_proj = _linear(self.x_proj, x)
         dt, B, C = x_proj.split([self.args.dt_rank, self.args.d_state, self.args.d_state], dim=-1)
-        dt = self.dt_proj(dt)
+        dt = _linear(self.dt_proj, dt)
         A = -torch.exp(self.A_log.float())
         y = self.scan_impl(
             _swap_act(x, "silu"),                       # x = F.silu(x), aussm.py:787
@@ -181,17 +224,17 @@ class SSMauBlock(nn.Module):
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         (b, l, d) = x.shape
-        x_and_z = self.in_proj(x)
+        x_and_z = _linear(self.in_proj, x)
         (x, z) = x_and_z.split(split_size=[self.args.d_model, self.args.d_model], dim=-1)
         if self.args.conv_1d:
             x = _causal_conv(self.conv1d, x, l)
         y = self.ssm_au(x, z)
-        return self.out_proj(y)
+        return _linear(self.out_proj, y)
 
     def ssm_au(self, x, z):
         b, l, d_in = x.shape
         n = self.args.d_state
-        dt = self.dt_proj(self.x_proj(x))
+        dt = _linear(self.dt_proj, _linear(self.x_proj, x))
         # dt = softplus(dt + self.dt_proj.bias) of aussm.py:879-880 happens inside the layout change below
         # "(n dstate1) dstate -> dstate1 n dstate"
         x_param = self.xA_proj.weight.view(n, d_in, d_in).permute(1, 0, 2)
@@ -280,7 +323,7 @@ class SSMTS(nn.Module):
                 {"params": self.output.parameters()}]
 
     def forward(self, input_ids, **kwargs):
-        x = self.embedding(input_ids)
+        x = _linear(self.embedding, input_ids)
         for layer in self.layers:
             x = layer(x)
-        return self.output(self.norm_f(x))
+        return _linear(self.output, self.norm_f(x))

@@ -126,11 +126,14 @@ def test_ssmts_hybrid_hip_matches_oracle_backend():
 
 
 @pytest.mark.gpu
-def test_ssmts_full_width_and_length_matches_oracle_backend():
+def test_ssmts_full_width_and_length_matches_oracle_backend(monkeypatch):
     """Benchmark configuration 4 at its full width and sequence length (d_model=256, l=720, layers a|m|a|m) on
     two sequences of the batch: outputs and every parameter gradient against the same seeded network running
     on the oracle's scans on the CPU.  (The batch size only multiplies the work; the full batch is
-    test_ssmts_full_size_step_runs.)  fp32 GEMMs of width 256-512 on both sides in different orders: 5e-4."""
+    test_ssmts_full_size_step_runs.)  fp32 GEMMs of width 256-512 on both sides in different orders: 5e-4.
+    The linear layers take the weight gradient they use at the full batch (slices of the rows, summed), which
+    1440 rows would not select by themselves."""
+    monkeypatch.setattr(blocks, "_WGRAD_MIN_ROWS", 1)
     x = torch.randn(2, 720, 21, generator=torch.Generator().manual_seed(4))
     print("case SSMTS d_model=256 layers=a|m|a|m x=(2,720,21) vs oracle backend", flush=True)
     _compare(lambda cpu: blocks.SSMTS(d_model=256, input_dim=21, output_dim=21, layers="a|m|a|m",
@@ -157,6 +160,26 @@ def test_ssmts_full_size_step_runs():
 
 def F_mse(a, b):
     return ((a - b) ** 2).mean()
+
+
+def test_linear_with_sliced_weight_gradient_is_linear_cpu():
+    """`_LinearFn` against torch's own `F.linear` in float64: output and the three gradients, for a 3-d input, an
+    input that is a slice of a wider tensor (the dt columns of x_proj's output) and a layer without bias."""
+    g = torch.Generator().manual_seed(11)
+    for (shape, n, bias, sl) in [((4, 6, 5), 7, True, None), ((2, 8, 9), 3, False, 4), ((16, 5), 2, True, None)]:
+        x = torch.randn(*shape, generator=g, dtype=torch.float64)
+        w = torch.randn(n, sl or shape[-1], generator=g, dtype=torch.float64)
+        b = torch.randn(n, generator=g, dtype=torch.float64) if bias else None
+        dy = torch.randn(*shape[:-1], n, generator=g, dtype=torch.float64)
+        res = []
+        for fn in (lambda a, ww, bb: blocks._LinearFn.apply(a, ww, bb), torch.nn.functional.linear):
+            leaves = [t.clone().requires_grad_(True) if t is not None else None for t in (x, w, b)]
+            inp = leaves[0][..., :sl] if sl else leaves[0]
+            y = fn(inp, leaves[1], leaves[2])
+            y.backward(dy)
+            res.append([y.detach()] + [t.grad for t in leaves if t is not None])
+        for a, want in zip(*res):
+            torch.testing.assert_close(a, want, atol=1e-12, rtol=1e-12)
 
 
 def test_rmsnorm_is_the_reference_formula_cpu():
