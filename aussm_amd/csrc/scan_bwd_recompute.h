@@ -238,8 +238,21 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
   if (ntiles > 1) { load_tile(fly, (ntiles - 2) * RT); load_start(st_fly, ntiles - 2); }
   else { load_start(st_fly, 0); }
 
+  // The walk consumes every B_t / C_t line of a tile through scalar loads that it waits for on the spot: the
+  // lines of the tile that comes next are touched a tile ahead, during the staging maths, so that those loads
+  // find them in the scalar cache.
+  constexpr int RB = (int)sizeof(Tbc) * C;
+  const bool full_group = active && n0 + NW <= N;          // wave-uniform
+  TileWarm<NW, RB, RT> warm;
+  if (full_group && ntiles * RT == L) {
+    warm.issue(gB, gC, row_base + (size_t)(ntiles - 1) * RT, ld);
+    warm.retire();
+  }
+
   for (int it = ntiles - 1; it >= 0; --it) {
     const int l0 = it * RT;
+    const bool warm_next = full_group && it > 0;
+    if (warm_next) warm.issue(gB, gC, row_base + l0 - RT, ld);
 
     // ---- stage
     float eu[E], edl[E], egy[E], eraw[E], egz[E];       // egz: dy silu'(z), for dz
@@ -271,6 +284,7 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
       edl[k] = dl;
       s_in[col * TS + row0 + k * RSTEP] = rec;
     }
+    if (warm_next) warm.retire();
     __syncthreads();
 
     float rres[NRES > 0 ? NRES : 1];

@@ -158,22 +158,25 @@ __device__ __forceinline__ uint32_t ld_touch(const void* p, size_t idx) {
 }
 
 // Warm the scalar cache with the B_t/C_t lines of the NW state rows starting at record `row`
-// (row stride L records) for one tile of TT timesteps.
+// (row stride L records) for one tile of TT timesteps: one dword per 64-byte line (rows of real fp32 records
+// have 16 steps per line, of complex ones 8 = TG).
 template <int NW, int REC_BYTES, int TT = T>
 struct TileWarm {
-  uint32_t v[2 * NW * (TT / TG)];
+  static constexpr int STEP = (64 / REC_BYTES > TG) ? 64 / REC_BYTES : TG;   // records between touches
+  static constexpr int NTOUCH = (TT + STEP - 1) / STEP;                       // touches per row
+  uint32_t v[2 * NW * NTOUCH];
   __device__ __forceinline__ void issue(const void* gB, const void* gC, size_t row, int L) {
 #pragma unroll
     for (int k = 0; k < NW; ++k)
 #pragma unroll
-      for (int g = 0; g < TT / TG; ++g) {
-        v[(2 * k) * (TT / TG) + g] = ld_touch<REC_BYTES>(gB, row + (size_t)k * L + g * TG);
-        v[(2 * k + 1) * (TT / TG) + g] = ld_touch<REC_BYTES>(gC, row + (size_t)k * L + g * TG);
+      for (int g = 0; g < NTOUCH; ++g) {
+        v[(2 * k) * NTOUCH + g] = ld_touch<REC_BYTES>(gB, row + (size_t)k * L + g * STEP);
+        v[(2 * k + 1) * NTOUCH + g] = ld_touch<REC_BYTES>(gC, row + (size_t)k * L + g * STEP);
       }
   }
   __device__ __forceinline__ void retire() {
 #pragma unroll
-    for (int i = 0; i < 2 * NW * (TT / TG); ++i) touch_uniform(v[i]);
+    for (int i = 0; i < 2 * NW * NTOUCH; ++i) touch_uniform(v[i]);
   }
 };
 

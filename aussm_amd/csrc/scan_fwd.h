@@ -236,6 +236,9 @@ __global__ __launch_bounds__(NT) void core_fwd_kernel(const FwdArgs p) {
               hr[k] = fmaf(a, hr[k], bc[t] * ry[t]);
               yacc[t] = fmaf(cc[t], hr[k], yacc[t]);
             }
+            // (keeps the next turn's wait for its scalar loads behind this turn's arithmetic: without the fence
+            // the compiler hoists it to the top of the turn, right behind the loads it waits for)
+            sched_fence();
           }
 #pragma unroll
           for (int t = 0; t < TG; ++t) {
@@ -291,6 +294,7 @@ __global__ __launch_bounds__(NT) void core_fwd_kernel(const FwdArgs p) {
               yacc[t] = fmaf(cc[2 * t], nr, yacc[t]);
               yacc[t] = fmaf(-cc[2 * t + 1], ni, yacc[t]);
             }
+            sched_fence();
           }
 #pragma unroll
           for (int t = 0; t < TG; ++t) {
