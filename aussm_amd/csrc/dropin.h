@@ -225,8 +225,7 @@ __global__ __launch_bounds__(NW * 64) void dropin_fwd_kernel(const DropinArgs p)
       hr[a] = row_last(her, lane);
       hi[a] = row_last(hei, lane);
     }
-    ysum += __shfl_xor(ysum, 16);
-    ysum += __shfl_xor(ysum, 32);
+    ysum = rows_sum(ysum);
     if (nb == 1) {
       if (p.y && iok && lok && g == 0) p.y[row + l] = silu_fast(zv) * (ysum + Di * ut);
     } else if (g == 0) {
@@ -418,10 +417,8 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(DROPIN_
       ar[a] = row_first(phr, lane);
       ai[a] = row_first(phi, lane);
     }
-    ysum += __shfl_xor(ysum, 16);
-    ysum += __shfl_xor(ysum, 32);
-    wsum += __shfl_xor(wsum, 16);
-    wsum += __shfl_xor(wsum, 32);
+    ysum = rows_sum(ysum);
+    wsum = rows_sum(wsum);
     if (nb > 1 && g == 0) s_yw[t & 1][wave][l_] = make_float2(ysum, wsum);
     if (t > t_first) tile_store<NT, NREC, KS>(sv, s_u[(t - 1) & 1], tid);
     if (nb > 1) {                                      // the channel's first wavefront adds the shares up

@@ -89,10 +89,7 @@ struct LaneTranspose16 {
     for (int s = 8; s >= 1; s >>= 1)
 #pragma unroll
       for (int i = 0; i < s; ++i) v[i] += v[i + s];
-    float t = v[0];
-    t += __shfl_xor(t, 16, 64);
-    t += __shfl_xor(t, 32, 64);
-    return t;
+    return rows_sum(v[0]);
   }
 };
 

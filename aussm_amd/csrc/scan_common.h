@@ -180,6 +180,64 @@ struct TileWarm {
   }
 };
 
+// ---- sums and moves across the four 16-lane rows of a wavefront (lane = 16 g + c) on the vector ALU.  gfx950 swaps
+// rows between two registers in one instruction (v_permlane16_swap: rows 1 and 3 of the first with rows 0 and 2 of
+// the second; v_permlane32_swap: the upper half of the first with the lower half of the second), so none of these
+// takes the LDS round trip of a lane shuffle (ds_bpermute), and the scans take two dependent steps instead of three.
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void rows_swap16(float& a, float& b) {
+  const u32x2 r = __builtin_amdgcn_permlane16_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+  a = __uint_as_float(r[0]); b = __uint_as_float(r[1]);
+}
+__device__ __forceinline__ void rows_swap32(float& a, float& b) {
+  const u32x2 r = __builtin_amdgcn_permlane32_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+  a = __uint_as_float(r[0]); b = __uint_as_float(r[1]);
+}
+// x = [x0 x1 x2 x3] by rows.  incl: row g gets x0 + .. + xg; tot: every row gets x0 + x1 + x2 + x3.
+__device__ __forceinline__ void rows_prefix(float x, int g, float* incl, float* tot) {
+  float a = x, b = x;
+  rows_swap16(a, b);                              // a = [x0 x0 x2 x2], b = [x1 x1 x3 x3]
+  const float pair = a + b;                       // [x0+x1, x0+x1, x2+x3, x2+x3]
+  float c = pair, d = pair;
+  rows_swap32(c, d);                              // c = x0+x1 in every row, d = x2+x3
+  float y = (g & 1) ? pair : x;
+  if (g >= 2) y += c;
+  *incl = y; *tot = c + d;
+}
+// incl: row g gets xg + .. + x3
+__device__ __forceinline__ void rows_suffix(float x, int g, float* incl, float* tot) {
+  float a = x, b = x;
+  rows_swap16(a, b);
+  const float pair = a + b;
+  float c = pair, d = pair;
+  rows_swap32(c, d);
+  float y = (g & 1) ? x : pair;
+  if (g < 2) y += d;
+  *incl = y; *tot = c + d;
+}
+__device__ __forceinline__ float rows_sum(float x) {
+  float a = x, b = x;
+  rows_swap16(a, b);
+  float c = a + b, d = c;
+  rows_swap32(c, d);
+  return c + d;
+}
+// the value of row 3 (row 0) of the same column, in every row
+__device__ __forceinline__ float rows_last(float x) {
+  float c = x, d = x;
+  rows_swap32(c, d);                              // d = [x2 x3 x2 x3]
+  float a = d, b = d;
+  rows_swap16(a, b);                              // b = [x3 x3 x3 x3]
+  return b;
+}
+__device__ __forceinline__ float rows_first(float x) {
+  float c = x, d = x;
+  rows_swap32(c, d);                              // c = [x0 x1 x0 x1]
+  float a = c, b = c;
+  rows_swap16(a, b);                              // a = [x0 x0 x0 x0]
+  return a;
+}
+
 // ---- staging geometry: a thread owns runs of FOUR consecutive timesteps of one channel row, so a
 // tile row of TT timesteps is covered by TT/4 neighbouring lanes with 16-byte accesses.
 template <int NT, int TT>

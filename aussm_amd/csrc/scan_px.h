@@ -384,14 +384,9 @@ __global__ __launch_bounds__(512) void unitary_fwd_px_kernel(const FwdArgs p, co
 #pragma unroll
     for (int st = 0; st < 2; ++st) { th[st][1] += th[st][0]; th[st][2] += th[st][1]; th[st][3] += th[st][2]; }
     // exclusive offsets over the order (st 0: g 0..3), (st 1: g 0..3)
-    float sa = th[0][3], sb = th[1][3];
-    {
-      float ta = __shfl_up(sa, 16), tb = __shfl_up(sb, 16);
-      if (g >= 1) { sa += ta; sb += tb; }
-      ta = __shfl_up(sa, 32); tb = __shfl_up(sb, 32);
-      if (g >= 2) { sa += ta; sb += tb; }
-    }
-    const float tot_a = __shfl(sa, 48 + dl);
+    float sa, sb, tot_a, tot_b_;
+    rows_prefix(th[0][3], g, &sa, &tot_a);
+    rows_prefix(th[1][3], g, &sb, &tot_b_);
     const float off_a = sa - th[0][3];
     const float off_b = tot_a + sb - th[1][3];
 #pragma unroll
@@ -467,7 +462,7 @@ __global__ __launch_bounds__(512) void unitary_fwd_px_kernel(const FwdArgs p, co
     split8<NP>(sk, vr, Vr);
     split8<NP>(sk, vi, Vi);
     // rotation over the whole chunk: the element (st 1, g 3, i 3) is timestep 31
-    const float cT = __shfl(cs[7], 48 + dl), sT = __shfl(sn[7], 48 + dl);
+    const float cT = rows_last(cs[7]), sT = rows_last(sn[7]);
     // ---- Z = B^T V  (four independent accumulation chains)
     f4 z0 = {0, 0, 0, 0}, z1 = {0, 0, 0, 0}, z2 = {0, 0, 0, 0}, z3 = {0, 0, 0, 0};
     {
@@ -796,14 +791,9 @@ __global__ __launch_bounds__(512) void unitary_bwd_px_kernel(const UniBwdArgs p,
     }
 #pragma unroll
     for (int st = 0; st < 2; ++st) { th[st][1] += th[st][0]; th[st][2] += th[st][1]; th[st][3] += th[st][2]; }
-    float sa = th[0][3], sb = th[1][3];
-    {
-      float ta = __shfl_up(sa, 16), tb = __shfl_up(sb, 16);
-      if (g >= 1) { sa += ta; sb += tb; }
-      ta = __shfl_up(sa, 32); tb = __shfl_up(sb, 32);
-      if (g >= 2) { sa += ta; sb += tb; }
-    }
-    const float tot_a = __shfl(sa, 48 + dl);
+    float sa, sb, tot_a, tot_b_;
+    rows_prefix(th[0][3], g, &sa, &tot_a);
+    rows_prefix(th[1][3], g, &sb, &tot_b_);
     const float off_a = sa - th[0][3];
     const float off_b = tot_a + sb - th[1][3];
 #pragma unroll
@@ -844,7 +834,7 @@ __global__ __launch_bounds__(512) void unitary_bwd_px_kernel(const UniBwdArgs p,
       }
       split8<NP>(sk, vr, Vr); split8<NP>(sk, vi, Vi); split8<NP>(sk, qr, Qr); split8<NP>(sk, qi, Qi);
     }
-    const float cT = __shfl(cs[7], 48 + dl), sT = __shfl(sn[7], 48 + dl);
+    const float cT = rows_last(cs[7]), sT = rows_last(sn[7]);
     // ---- Z = B^T V, then W = conj(C)^T Q  (four independent accumulation chains each; one after
     // the other so that only one set of operand records is live at a time)
     f4 z0 = {0, 0, 0, 0}, z1 = z0, z2 = z0, z3 = z0, w0 = z0, w1 = z0, w2 = z0, w3 = z0;
@@ -897,9 +887,7 @@ __global__ __launch_bounds__(512) void unitary_bwd_px_kernel(const UniBwdArgs p,
     float t = 0.0f;
 #pragma unroll
     for (int i = 0; i < 4; ++i) t -= ar[i] * ei[i] - ai[i] * er[i];   // - sum_n Im(conj(A') H_end): phase gradient at the last step
-    t += __shfl_xor(t, 16);
-    t += __shfl_xor(t, 32);
-    tq = t;
+    tq = rows_sum(t);
     f4 nAr, nAi;
     f4 pr, pi;                                            // what the next chunk takes as its end state
 #pragma unroll
@@ -977,14 +965,9 @@ __global__ __launch_bounds__(512) void unitary_bwd_px_kernel(const UniBwdArgs p,
       // suffix sums over the chunk: runs (st 1: g 3..0) then (st 0: g 3..0) in reverse time
       gth[2] += gth[3]; gth[1] += gth[2]; gth[0] += gth[1];
       gth[6] += gth[7]; gth[5] += gth[6]; gth[4] += gth[5];
-      float ra = gth[0], rb = gth[4];
-      {
-        float ta = __shfl_down(ra, 16), tb = __shfl_down(rb, 16);
-        if (g <= 2) { ra += ta; rb += tb; }
-        ta = __shfl_down(ra, 32); tb = __shfl_down(rb, 32);
-        if (g <= 1) { ra += ta; rb += tb; }
-      }
-      const float tot_b = __shfl(rb, dl);
+      float ra, rb, tot_a_, tot_b;
+      rows_suffix(gth[0], g, &ra, &tot_a_);
+      rows_suffix(gth[4], g, &rb, &tot_b);
       const float offb = rb - gth[4];
       const float offa = tot_b + ra - gth[0];
       if (dok && c >= 0) {
@@ -1231,8 +1214,7 @@ __global__ __launch_bounds__(512) void unitary_bwd_px_kernel(const UniBwdArgs p,
     }
   }
   if (p.dD && dok) {
-    accD += __shfl_xor(accD, 16);
-    accD += __shfl_xor(accD, 32);
+    accD = rows_sum(accD);
     if (g == 0) atomicAdd(p.dD + d, accD);
   }
 }
