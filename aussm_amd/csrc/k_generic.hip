@@ -86,10 +86,15 @@ static int rec_bwd_t(const RecBwdArgs& args, hipStream_t s) {
     const int nw = left <= 4 ? 1 : (left <= 8 ? 2 : 4);
     bool done = false;
 #ifndef AUSSM_REC_NARROW
-    // a full block of 16 states: eight wavefronts of two states, two wavefronts per SIMD (the gated complex scan
-    // needs a fourth partial sum per wavefront, which only fits with four wavefronts)
-    if (left > 8 && !(VAR == VAR_COMPLEX && a.z)) {
-      hipLaunchKernelGGL((recompute_bwd_kernel<VAR, 2, 512, Tin, float>), grid, dim3(512), 0, s, a);
+    // a full block of 16 states: eight wavefronts of two states, two wavefronts per SIMD (the complex scan with a
+    // gate gradient to return keeps a fourth partial sum per wavefront)
+    if (left > 8) {
+      if constexpr (VAR == VAR_COMPLEX) {
+        if (a.dz) hipLaunchKernelGGL((recompute_bwd_kernel<VAR, 2, 512, Tin, float, true>), grid, dim3(512), 0, s, a);
+        else hipLaunchKernelGGL((recompute_bwd_kernel<VAR, 2, 512, Tin, float, false>), grid, dim3(512), 0, s, a);
+      } else {
+        hipLaunchKernelGGL((recompute_bwd_kernel<VAR, 2, 512, Tin, float>), grid, dim3(512), 0, s, a);
+      }
       done = true;
     }
 #endif

@@ -67,7 +67,8 @@ __device__ __forceinline__ f32x8 ld_r8_tile(const Tin* p, size_t row, int t0, in
   else return ld_r8_safe(p, row, t0, L);
 }
 
-// Column sums of 16 products per lane (the workgroups of eight wavefronts: half the scratch per wavefront).
+// Column sums of 16 products per lane through LDS (the real scan's workgroups of eight wavefronts; the complex
+// scan's use `lanes_sum16`).
 // Lane (c = lane % 16, q = lane / 16) reads column c of the rows 16 (i / 4) + 4 q + i % 4, i = 0 .. 15: with a
 // row stride of 20 floats the two q of a 32-lane half are 16 banks apart, and the 16-byte row writes of
 // eight neighbouring lanes cover all banks.  finish() leaves the column's total in all four lanes.
@@ -97,9 +98,14 @@ struct LaneTranspose16 {
 // wavefront and reduce 32 products per lane transpose.  Workgroups of eight wavefronts (NT = 512, two
 // wavefronts per SIMD) fit with three planes of floats per wavefront instead of four-float records - complex:
 // (dw, dtheta, drho), real: (dw, ddelta, y_pre), so the gated complex scan stays with four wavefronts - and with
-// transposes of 16 products at a time.  (Adding the partial sums of two wavefronts into one slab with LDS float
-// atomics instead made the kernel 2.5 times slower: those run far below the rate of plain LDS writes.)
-template <int VAR, int NW, int NT, typename Tin, typename Tbc = Tin>
+// channel sums of 16 products at a time: through lane transposes in the real scan, on the vector ALU alone in the
+// complex scan (`lanes_sum16`: row swaps and DPP; through LDS this reduction was two fifths of the complex kernel's
+// time, while the real kernel, whose vector ALU is the busier, runs 4 % faster with the transposes).  The LDS the
+// complex scan saves holds a fourth plane, the read-out before the gate, so the gated complex scan runs here too.  (Adding the partial sums of
+// two wavefronts into one slab with LDS float atomics instead made the kernel 2.5 times slower: those run far below
+// the rate of plain LDS writes.)
+// PLANE4: the complex scan's workgroups of eight wavefronts with the fourth plane (calls that want dz).
+template <int VAR, int NW, int NT, typename Tin, typename Tbc = Tin, bool PLANE4 = false>
 __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
   static_assert(VAR == VAR_COMPLEX || VAR == VAR_REAL, "unitary has its own kernel");
   constexpr int C = (VAR == VAR_REAL) ? 1 : 2;
@@ -119,8 +125,12 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
 
   __shared__ float4 s_in[RT * TS];                         // complex (Re a, Im a, w, dy); real (delta, w, dy, -)
   __shared__ float4 s_part[WIDE ? 1 : NWV * RT * TS];      // per wavefront partial (dw, dtheta|ddelta, drho, y_pre)
-  __shared__ float s_slab[WIDE ? NWV * 3 * PLANE : 1];     // WIDE: per wavefront, three of those sums as planes
-  __shared__ __align__(16) float s_red[NWV * 64 * (WIDE ? RED16_RS : RED_RS)]; // lane-transpose scratch
+  constexpr int NPL = PLANE4 ? 4 : 3;                      // planes of a slab: gated complex (dw, dtheta, drho, y_pre)
+  static_assert(!PLANE4 || (VAR == VAR_COMPLEX && NT == 512), "the fourth plane is the gated complex scan's");
+  constexpr bool VALU_SUMS = WIDE && VAR == VAR_COMPLEX;   // channel sums without LDS
+  constexpr int SLAB = NPL * PLANE;                        // floats of a wavefront's slab
+  __shared__ float s_slab[WIDE ? NWV * SLAB : 1];   // WIDE: per wavefront, those sums as planes
+  __shared__ __align__(16) float s_red[VALU_SUMS ? 4 : NWV * 64 * (WIDE ? RED16_RS : RED_RS)];  // lane-transpose scratch
 
   const int tid = threadIdx.x, lane = tid & 63, wave = wave_index();
   const int wg = xcd_remap(blockIdx.x, gridDim.x);
@@ -141,9 +151,9 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
   const Tin* __restrict__ gdl = static_cast<const Tin*>(p.delta);
   const Tbc* __restrict__ gB = static_cast<const Tbc*>(p.Bm);
   const Tbc* __restrict__ gC = static_cast<const Tbc*>(p.Cm);
-  float* red = s_red + wave * 64 * (WIDE ? RED16_RS : RED_RS);
+  float* red = s_red + (VALU_SUMS ? 0 : wave * 64 * (WIDE ? RED16_RS : RED_RS));
   float4* part = s_part + (WIDE ? 0 : wave * RT * TS);
-  float* slab = s_slab + (WIDE ? wave * 3 * PLANE : 0);
+  float* slab = s_slab + (WIDE ? wave * SLAB : 0);
   const size_t row_base = ((size_t)b * N + n0) * ld + lbeg;
 
   // ---- per-lane constants and accumulators
@@ -406,9 +416,13 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
             for (int h = 0; h < C; ++h) {
 #pragma unroll
               for (int j = 0; j < 16; ++j) half[j] = vals[16 * h + j];
-              LaneTranspose16 xs;
-              xs.issue(half, red, lane);
-              rres[(g * NW + k) * C + h] = xs.finish();
+              if constexpr (VALU_SUMS) {
+                rres[(g * NW + k) * C + h] = lanes_sum16(half, lane);
+              } else {
+                LaneTranspose16 xs;
+                xs.issue(half, red, lane);
+                rres[(g * NW + k) * C + h] = xs.finish();
+              }
             }
 #pragma unroll
             for (int j = 0; j < RED_COLS; ++j) vals[j] = 0.f;
@@ -427,6 +441,7 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
             q[0] = kacc[t];
             q[PLANE] = xacc[t];
             q[2 * PLANE] = (VAR == VAR_COMPLEX) ? zacc[t] : yacc[t];
+            if constexpr (PLANE4) q[3 * PLANE] = yacc[t];
           }
         } else {
 #pragma unroll
@@ -452,8 +467,10 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
     sched_fence();
     if (active) {
       if constexpr (WIDE) {
-        // lanes 0 .. 15 hold the 16 columns: complex (dB | dC of a row: 8 steps x (re, im)), real (8 dB, 8 dC)
-        const int c = lane & 15;
+        // lane (g, c < 4) holds column 4 c + g of the 16: complex (dB | dC of a row: 8 steps x (re, im)), real (8 dB, 8 dC)
+        // (lanes_sum16), or lanes 0 .. 15 one column each (LaneTranspose16)
+        const int c = VALU_SUMS ? 4 * (lane & 3) + (lane >> 4) : (lane & 15);
+        const bool mine = VALU_SUMS ? (lane & 12) == 0 : lane < 16;
 #pragma unroll
         for (int g = 0; g < NGRP; ++g)
 #pragma unroll
@@ -464,10 +481,10 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
               const float v = rres[(g * NW + k) * C + h];
               if (VAR == VAR_REAL) {
                 float* dst = (c >> 3) ? p.dC : p.dB;
-                if (lane < 16 && n0 + k < N && t + (c & 7) < L) atomicAdd(dst + row_base + (size_t)k * ld + t + (c & 7), v);
+                if (mine && n0 + k < N && t + (c & 7) < L) atomicAdd(dst + row_base + (size_t)k * ld + t + (c & 7), v);
               } else {
                 float* dst = h ? p.dC : p.dB;
-                if (lane < 16 && n0 + k < N && t + (c >> 1) < L) atomicAdd(dst + 2 * (row_base + (size_t)k * ld + t) + c, v);
+                if (mine && n0 + k < N && t + (c >> 1) < L) atomicAdd(dst + 2 * (row_base + (size_t)k * ld + t) + c, v);
               }
             }
       } else {
@@ -504,8 +521,9 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
 #pragma unroll
       for (int w = 0; w < NSLAB; ++w) {
         if constexpr (WIDE) {
-          const float* q = s_slab + w * 3 * PLANE + col * TS + row0 + k * RSTEP;
-          pv[k][w] = (w < nwa) ? make_float4(q[0], q[PLANE], VAR == VAR_COMPLEX ? q[2 * PLANE] : 0.f, VAR == VAR_COMPLEX ? 0.f : q[2 * PLANE])
+          const float* q = s_slab + w * SLAB + col * TS + row0 + k * RSTEP;
+          pv[k][w] = (w < nwa) ? make_float4(q[0], q[PLANE], VAR == VAR_COMPLEX ? q[2 * PLANE] : 0.f,
+                                             VAR == VAR_COMPLEX ? (PLANE4 ? q[3 * PLANE] : 0.f) : q[2 * PLANE])
                                : make_float4(0.f, 0.f, 0.f, 0.f);
         } else {
           pv[k][w] = (w < nwa) ? s_part[(w * RT + col) * TS + row0 + k * RSTEP] : make_float4(0.f, 0.f, 0.f, 0.f);

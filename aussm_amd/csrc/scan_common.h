@@ -238,6 +238,35 @@ __device__ __forceinline__ float rows_first(float x) {
   return a;
 }
 
+// DPP moves inside a row of 16 lanes (every lane has a source for the patterns used here)
+template <int CTRL>
+__device__ __forceinline__ float dpp_perm(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+// Sums over the 64 lanes of 16 values per lane on the vector ALU alone (35 instructions, no LDS): lane (g, c) returns
+// the total of value 4 (c % 4) + g.  Two rounds of row swaps fold the four rows - 16 values, 8, 4: row g of q[j]
+// holds value 4 j + g summed over the rows -; two transposing steps inside the quads leave q[lane % 4]'s quad sums,
+// and two rotations by 4 and 8 lanes add the four quads of the row.
+__device__ __forceinline__ float lanes_sum16(const float (&v)[16], int lane) {
+  float q[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    float a0 = v[4 * j], b0 = v[4 * j + 1], a1 = v[4 * j + 2], b1 = v[4 * j + 3];
+    rows_swap16(a0, b0);
+    rows_swap16(a1, b1);
+    float c = a0 + b0, d = a1 + b1;
+    rows_swap32(c, d);
+    q[j] = c + d;
+  }
+  const bool b0 = lane & 1, b1 = lane & 2;
+  const float r01 = (b0 ? q[1] : q[0]) + dpp_perm<0xB1>(b0 ? q[0] : q[1]);   // quad_perm:[1,0,3,2]
+  const float r23 = (b0 ? q[3] : q[2]) + dpp_perm<0xB1>(b0 ? q[2] : q[3]);
+  float r = (b1 ? r23 : r01) + dpp_perm<0x4E>(b1 ? r01 : r23);               // quad_perm:[2,3,0,1]
+  r += dpp_perm<0x124>(r);                                                    // row_ror:4
+  r += dpp_perm<0x128>(r);                                                    // row_ror:8
+  return r;
+}
+
 // ---- staging geometry: a thread owns runs of FOUR consecutive timesteps of one channel row, so a
 // tile row of TT timesteps is covered by TT/4 neighbouring lanes with 16-byte accesses.
 template <int NT, int TT>
