@@ -60,9 +60,10 @@ __device__ __forceinline__ float row_suffix(float v) {   // inclusive, towards l
   v += dpp_mov0<0x108>(v);
   return v;
 }
-// value of the row's last / first lane in every lane of the row
-__device__ __forceinline__ float row_last(float v, int lane) { return __shfl(v, (lane & 48) | 15); }
-__device__ __forceinline__ float row_first(float v, int lane) { return __shfl(v, lane & 48); }
+// value of the row's last / first lane in every lane of the row (DPP row broadcast: one vector instruction, where a
+// lane shuffle is an LDS round trip on the chain that hands the state from tile to tile)
+__device__ __forceinline__ float row_last(float v, int) { return dpp_perm<0x15F>(v); }    // row_newbcast:15
+__device__ __forceinline__ float row_first(float v, int) { return dpp_perm<0x150>(v); }   // row_newbcast:0
 
 
 // x (d, n, d) -> operand records.  Record (v = i nb + sb, ks, piece, lane = (row = lane % 16, g = lane / 16))
