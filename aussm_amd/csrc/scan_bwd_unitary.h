@@ -96,8 +96,14 @@ __global__ __launch_bounds__(NT) void unitary_bwd_kernel(const UniBwdArgs p) {
   float2* part = s_part + wave * TT * TS;
   // lane -> element of the (row, 8 timesteps) output block of a turn: columns 0..15 are dB
   // (re, im interleaved), 16..31 dC; both halves of the wavefront add their half sum.
-  float* const red_dst = ((lane & 31) < 2 * TG) ? p.dB : p.dC;
-  const int red_off = lane & (2 * TG - 1);
+  // The sums over the channels of a turn's dB / dC products: through the LDS lane transpose, whose latency hides
+  // behind the next turn, or on the vector ALU alone (`lanes_sum16`).  Measured at B=32, D=512, L=2048: with eight
+  // states per wavefront (N = 64) the vector-ALU form is 10 % faster, with four or two (N = 32, 16) 2-5 % slower.
+  // (With lanes_sum16: lane (g, c) holds column 4 (c % 4) + g of dB for c / 4 == 0, of dC for c / 4 == 1.)
+  constexpr bool VALU_SUMS = NW >= 8;
+  float* const red_dst = VALU_SUMS ? ((lane & 4) ? p.dC : p.dB) : (((lane & 31) < 2 * TG) ? p.dB : p.dC);
+  const int red_off = VALU_SUMS ? 4 * (lane & 3) + (lane >> 4) : (lane & (2 * TG - 1));
+  const bool red_mine = VALU_SUMS ? (lane & 8) == 0 : true;
 
   auto load_ck = [&](int kb, float (&xr)[NW], float (&xi)[NW]) {
 #pragma unroll
@@ -266,10 +272,19 @@ __global__ __launch_bounds__(NT) void unitary_bwd_kernel(const UniBwdArgs p) {
             gr[k] = tg;
           }
           sched_fence();
-          // collect the previous turn's sums (turn (g, k-1), or (g+1, NW-1) across a group)
-          if (k > 0) rres[g * NW + k - 1] = xp.finish();
-          else if (g < NGRP - 1) rres[(g + 1) * NW + NW - 1] = xp.finish();
-          xp.issue(vals, red, lane);
+          if constexpr (VALU_SUMS) {
+            // the turn's 16 dB and 16 dC products summed over the channels on the vector ALU
+            float hb[16], hc[16];
+#pragma unroll
+            for (int j = 0; j < 16; ++j) { hb[j] = vals[j]; hc[j] = vals[16 + j]; }
+            const float sb = lanes_sum16(hb, lane), sc = lanes_sum16(hc, lane);
+            rres[g * NW + k] = (lane & 4) ? sc : sb;
+          } else {
+            // collect the previous turn's sums (turn (g, k-1), or (g+1, NW-1) across a group)
+            if (k > 0) rres[g * NW + k - 1] = xp.finish();
+            else if (g < NGRP - 1) rres[(g + 1) * NW + NW - 1] = xp.finish();
+            xp.issue(vals, red, lane);
+          }
         }
 #pragma unroll
         for (int t = 0; t < TG; ++t) {
@@ -277,7 +292,7 @@ __global__ __launch_bounds__(NT) void unitary_bwd_kernel(const UniBwdArgs p) {
           if (g > 0) { rc[t] = nc[t]; rs[t] = ns[t]; rw[t] = nw_[t]; rg[t] = ng[t]; }
         }
       }
-      rres[NW - 1] = xp.finish();   // the last turn was (g = 0, k = NW-1)
+      if constexpr (!VALU_SUMS) rres[NW - 1] = xp.finish();   // the last turn was (g = 0, k = NW-1)
     } else if (active) {
       // ---- general path (ragged tile or partial state group): one timestep at a time
       for (int t = tmax - 1; t >= 0; --t) {
@@ -343,7 +358,7 @@ __global__ __launch_bounds__(NT) void unitary_bwd_kernel(const UniBwdArgs p) {
       for (int g = 0; g < NGRP; ++g)
 #pragma unroll
         for (int k = 0; k < NW; ++k)
-          atomicAdd(red_dst + 2 * (brow + (size_t)k * ld + g * TG) + red_off, rres[g * NW + k]);
+          if (red_mine) atomicAdd(red_dst + 2 * (brow + (size_t)k * ld + g * TG) + red_off, rres[g * NW + k]);
     }
 
     // ---- epilogue: channel-wise gradients, coalesced along time
