@@ -3,7 +3,7 @@
 once with float32 inputs and once with bfloat16 u / delta / B / C (float32 phases, decay, skip,
 states, outputs and gradients): configuration 3 of the benchmark contract.
 
-    python bench_variants.py [--reps R] [--shape B,D,N,L] [--variants real,...] [--model | --only-model]
+    python bench_variants.py [--reps R] [--shape B,D,N,L] [--variants real,...] [--gate] [--model | --only-model]
     python bench_variants.py --scaling [--runs 50] [--bdn 16,32,64 --bdn 32,256,16] [--lengths 10,...]
 
 With --model it also times configuration 4 of the contract: one training step (forward, MSE loss,
@@ -194,6 +194,9 @@ def main():
     ap.add_argument("--model", action="store_true", help="also time the hybrid SSMTS training step (configuration 4)")
     ap.add_argument("--only-model", action="store_true", help="time only the SSMTS training step")
     ap.add_argument("--variants", default="unitary,complex,real", help="comma-separated subset of the variants")
+    ap.add_argument("--gate", action="store_true",
+                    help="time the complex and real scans with the gate z (y = y_pre silu(z), dz returned); the unitary core "
+                         "scan has no gate inside its kernels")
     ap.add_argument("--scaling", action="store_true", help="the sequence-length sweep of the reference's scaling benchmark")
     ap.add_argument("--runs", type=int, default=50, help="timed repetitions per point of the sweep (after 5 warm-ups)")
     ap.add_argument("--bdn", action="append", help="b,d,n of the sweep (repeatable)")
@@ -239,6 +242,7 @@ def main():
         rn = lambda *s: torch.randn(*s, generator=g, device=dev)
         std = N ** -0.5
         out = {"u": rn(B, D, L), "delta": torch.nn.functional.softplus(rn(B, D, L)), "Dskip": rn(D), "dy": rn(B, D, L)}
+        out["z"] = rn(B, D, L) if (args.gate and variant != "unitary") else None
         if variant == "real":
             out.update(A=-torch.exp(rn(D, N)), Bm=rn(B, N, L) * std, Cm=rn(B, N, L) * std)
         else:
@@ -259,12 +263,13 @@ def main():
                 ck = scan.REC_CK
 
                 def fwd():
-                    return scan.real_fwd_raw(u, delta, p["A"], Bm, Cm, p["Dskip"], ck=ck)
+                    return scan.real_fwd_raw(u, delta, p["A"], Bm, Cm, p["Dskip"], z=p["z"], ck=ck)
 
                 hck = fwd()[2]
 
                 def bwd():
-                    return scan.real_bwd_raw(p["dy"], None, u, delta, p["A"], Bm, Cm, p["Dskip"], None, False, None, hck)
+                    return scan.real_bwd_raw(p["dy"], None, u, delta, p["A"], Bm, Cm, p["Dskip"], None, False, None, hck,
+                                             z=p["z"])
             else:
                 Bri = torch.view_as_real(p["Bc"]).to(dt).contiguous()
                 Cri = torch.view_as_real(p["Cc"]).to(dt).contiguous()
@@ -284,17 +289,20 @@ def main():
                     ck = scan.REC_CK
 
                     def fwd():
-                        return scan.complex_fwd_raw(u, delta, p["rho"], p["theta"], Bri, Cri, p["Dskip"], ck=ck)
+                        return scan.complex_fwd_raw(u, delta, p["rho"], p["theta"], Bri, Cri, p["Dskip"], z=p["z"], ck=ck)
 
                     hck = fwd()[2]
 
                     def bwd():
                         return scan.complex_bwd_raw(p["dy"], None, u, delta, p["rho"], p["theta"], Bri, Cri, p["Dskip"],
-                                                    None, hck)
+                                                    None, hck, z=p["z"])
             t_f, t_b = timed(fwd), timed(bwd)
             b_f, b_b = algorithmic_bytes(variant, w, E, S)
+            gated = p["z"] is not None
+            if gated:                      # z read forward; z read and dz written backward
+                b_f, b_b = b_f + 4 * E, b_b + 8 * E
             print(json.dumps({
-                "variant": variant, "inputs": name, "shape": {"B": B, "D": D, "N": N, "L": L},
+                "variant": variant + (" (gated)" if gated else ""), "inputs": name, "shape": {"B": B, "D": D, "N": N, "L": L},
                 "fwd_us": round(t_f, 1), "bwd_us": round(t_b, 1),
                 "fwd_GBps": round(b_f / t_f / 1e3, 1), "bwd_GBps": round(b_b / t_b / 1e3, 1),
                 "fwd_bwd_frac_of_hbm_peak": round((b_f + b_b) / (t_f + t_b) / 1e3 / HBM_PEAK_GBS, 4),
