@@ -143,7 +143,6 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
   const int L = (ld - lbeg < p.L) ? ld - lbeg : p.L;        // steps of this segment
   const int n0 = p.nbase + wave * NW;
   const bool active = n0 < N;
-  const int nwa = (N - p.nbase + NW - 1) / NW;         // wavefronts of this launch that own existing states
   const int d = d0 + lane;
   const bool dok = d < D;
 
@@ -254,6 +253,16 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
   if (full_group && ntiles * RT == L) {
     warm.issue(gB, gC, row_base + (size_t)(ntiles - 1) * RT, ld);
     warm.retire();
+  }
+
+  // a wavefront that owns no state never writes its slab: it clears it once, so that the epilogue can add the
+  // slabs of all wavefronts without asking which of them exist (the first barrier of the loop orders the two)
+  if (!active) {
+    if constexpr (WIDE) {
+      for (int i = lane; i < SLAB; i += 64) slab[i] = 0.f;
+    } else {
+      for (int i = lane; i < RT * TS; i += 64) part[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+    }
   }
 
   for (int it = ntiles - 1; it >= 0; --it) {
@@ -522,11 +531,11 @@ __global__ __launch_bounds__(NT) void recompute_bwd_kernel(const RecBwdArgs p) {
       for (int w = 0; w < NSLAB; ++w) {
         if constexpr (WIDE) {
           const float* q = s_slab + w * SLAB + col * TS + row0 + k * RSTEP;
-          pv[k][w] = (w < nwa) ? make_float4(q[0], q[PLANE], VAR == VAR_COMPLEX ? q[2 * PLANE] : 0.f,
-                                             VAR == VAR_COMPLEX ? (PLANE4 ? q[3 * PLANE] : 0.f) : q[2 * PLANE])
-                               : make_float4(0.f, 0.f, 0.f, 0.f);
+          // (the slab of a wavefront without states holds zeros: it cleared it before the first tile)
+          pv[k][w] = make_float4(q[0], q[PLANE], VAR == VAR_COMPLEX ? q[2 * PLANE] : 0.f,
+                                 VAR == VAR_COMPLEX ? (PLANE4 ? q[3 * PLANE] : 0.f) : q[2 * PLANE]);
         } else {
-          pv[k][w] = (w < nwa) ? s_part[(w * RT + col) * TS + row0 + k * RSTEP] : make_float4(0.f, 0.f, 0.f, 0.f);
+          pv[k][w] = s_part[(w * RT + col) * TS + row0 + k * RSTEP];
         }
       }
     sched_fence();

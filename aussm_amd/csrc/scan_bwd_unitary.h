@@ -81,7 +81,6 @@ __global__ __launch_bounds__(NT) void unitary_bwd_kernel(const UniBwdArgs p) {
   const int n0 = wave * NW;
   const bool active = n0 < N;
   const bool full_group = active && n0 + NW <= N;
-  const int nwa = (N + NW - 1) / NW;
   const int d = d0 + lane;
   const bool dok = d < D;
 
@@ -183,6 +182,12 @@ __global__ __launch_bounds__(NT) void unitary_bwd_kernel(const UniBwdArgs p) {
   if (WARM && full_group && ntiles * TT == L) {
     warm.issue(gB, gC, row_base + (size_t)(ntiles - 1) * TT, ld);
     warm.retire();
+  }
+
+  // a wavefront that owns no state never writes its slab of partial sums: it clears it once, so that the epilogue
+  // can add the slabs of all wavefronts without asking which of them exist (the loop's first barrier orders the two)
+  if (!active) {
+    for (int i = lane; i < TT * TS; i += 64) part[i] = make_float2(0.f, 0.f);
   }
 
   for (int it = ntiles - 1; it >= 0; --it) {
@@ -368,7 +373,7 @@ __global__ __launch_bounds__(NT) void unitary_bwd_kernel(const UniBwdArgs p) {
     for (int k = 0; k < E; ++k)
 #pragma unroll
       for (int w = 0; w < NWV; ++w)
-        pv[k][w] = (w < nwa) ? s_part[(w * TT + col) * TS + row0 + k * RSTEP] : make_float2(0.f, 0.f);
+        pv[k][w] = s_part[(w * TT + col) * TS + row0 + k * RSTEP];   // (wavefronts without states hold zeros)
     sched_fence();
 #pragma unroll
     for (int k = 0; k < E; ++k) {

@@ -35,7 +35,6 @@ __global__ __launch_bounds__(NT) void core_fwd_kernel(const FwdArgs p) {
   const int L = (ld - lbeg < p.L) ? ld - lbeg : p.L;      // steps of this segment
   const int n0 = wave * NW;
   const bool active = n0 < N;                    // wave-uniform
-  const int nwa = (N + NW - 1) / NW;             // wavefronts that own states
   const int d = d0 + lane;
   const bool dok = d < D;
 
@@ -144,6 +143,13 @@ __global__ __launch_bounds__(NT) void core_fwd_kernel(const FwdArgs p) {
   // of a launch that wants it (a split launch chains its segments with it)
   const bool want_tot = p.ptot != nullptr && wave == 0;   // wave-uniform
   float fr = (VAR == VAR_REAL) ? 0.f : 1.f, fi = 0.f;
+
+  // a wavefront that owns no state never writes its slab of partial read-outs: it clears it once, so that the
+  // epilogue can add the slabs of all wavefronts without asking which of them exist (the first barrier of the loop
+  // orders the two)
+  if (!active) {
+    for (int i = lane; i < T * TSP; i += 64) s_part[wave * T * TSP + i] = 0.f;
+  }
 
   for (int l0 = 0; l0 < L; l0 += T) {
     const bool warm_next = WARM && full_group && l0 + 2 * T <= L;
@@ -368,7 +374,7 @@ __global__ __launch_bounds__(NT) void core_fwd_kernel(const FwdArgs p) {
         for (int i = 0; i < 4; ++i)
 #pragma unroll
           for (int w = 0; w < NWV; ++w)
-            pv[k][i][w] = (w < nwa && inrow[k]) ? s_part[(w * T + t0 + i) * TSP + srow[k]] : 0.f;
+            pv[k][i][w] = (SG::RP == CH || inrow[k]) ? s_part[(w * T + t0 + i) * TSP + srow[k]] : 0.f;
       sched_fence();
 #pragma unroll
       for (int k = 0; k < PASS; ++k) {
